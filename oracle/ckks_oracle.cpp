@@ -1,0 +1,823 @@
+// CPU oracle for the CKKS hot path.  TEST INFRASTRUCTURE ONLY: see ckks_oracle.h.
+// Plain C++17, unsigned __int128 for wide arithmetic, optional OpenMP over limbs / rows.
+// Every routine cites the file:line of haozetao/ckks_llm it restates.
+#include "ckks_oracle.h"
+
+#include <cmath>
+#include <cstring>
+#include <set>
+#include <string>
+#include <vector>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef unsigned __int128 u128;
+typedef uint64_t u64;
+
+// ------------------------------------------------------------------------------------------------
+// scalar modmath
+// ------------------------------------------------------------------------------------------------
+// Utils.cuh:33-38
+u64 orc_mulmod(u64 a, u64 b, u64 q) { return (u64)(((u128)a * b) % q); }
+// Utils.cuh:14-31
+u64 orc_powmod(u64 a, u64 e, u64 q) {
+    u64 r = 1;
+    while (e) {
+        if (e & 1) r = orc_mulmod(r, a, q);
+        a = orc_mulmod(a, a, q);
+        e >>= 1;
+    }
+    return r;
+}
+// Utils.cuh:48-53 (Fermat inverse; q prime)
+u64 orc_invmod(u64 a, u64 q) { return orc_powmod(a % q, q - 2, q); }
+// Utils.cuh:40-45
+u64 orc_xshoup(u64 x, u64 q) { return (u64)((((u128)x) << 64) / q); }
+
+// uint128.cuh:143-147
+static inline u64 csub_q(u64 a, u64 q) {
+    u64 t = a - q;
+    return t + (t >> 63) * q;
+}
+// uint128.cuh:169-179
+u64 orc_mulmod_shoup(u64 a, u64 b, u64 b_shoup, u64 q) {
+    u64 hi = (u64)(((u128)a * b_shoup) >> 64);
+    u64 r = a * b - hi * q;
+    return csub_q(r, q);
+}
+// Context_23.cuh:67-70 : mu = floor(2^128 / q) split in two words (q odd, so floor((2^128-1)/q) is the same number)
+void orc_barrett_mu(u64 q, u64* mu_hi, u64* mu_lo) {
+    u128 mu = (~(u128)0) / q;
+    *mu_hi = (u64)(mu >> 64);
+    *mu_lo = (u64)mu;
+}
+// uint128.cuh:182-212 : the quotient estimate drops the low word of a.lo*mu.lo exactly as the PTX does
+u64 orc_barrett128(u64 a_hi, u64 a_lo, u64 q, u64 mu_hi, u64 mu_lo) {
+    u64 tmp = (u64)(((u128)a_lo * mu_lo) >> 64);
+    u128 s = (u128)a_lo * mu_hi + tmp;       // mad.lo.cc / madc.hi
+    u64 tmp2 = (u64)s;
+    u64 res = (u64)(s >> 64);
+    u128 s2 = (u128)a_hi * mu_lo + tmp2;     // round 2
+    res += (u64)(s2 >> 64);                  // madc.hi with carry-in folded in s2
+    res += a_hi * mu_hi;                     // mad.lo
+    u64 r = a_lo - res * q;
+    return csub_q(r, q);
+}
+// uint128.cuh:214-225
+u64 orc_barrett64(u64 a, u64 q, u64 mu_hi) {
+    u64 s = (u64)(((u128)mu_hi * a) >> 64);
+    return csub_q(a - s * q, q);
+}
+
+// ------------------------------------------------------------------------------------------------
+// roots of unity and tables
+// ------------------------------------------------------------------------------------------------
+// Utils.cuh:63-77.  The loop bound is the reference's: i < sqrt(n) on the shrinking n, strict,
+// evaluated in double; a remaining cofactor > 2 is recorded as a "factor" even when it is a square.
+static void find_prime_factors(std::set<u64>& s, u64 number) {
+    while (number % 2 == 0) { s.insert(2); number /= 2; }
+    for (u64 i = 3; (double)i < std::sqrt((double)number); i++) {
+        while (number % i == 0) { s.insert(i); number /= i; }
+    }
+    if (number > 2) s.insert(number);
+}
+// Utils.cuh:79-96
+u64 orc_find_primitive_root(u64 q) {
+    std::set<u64> s;
+    u64 phi = q - 1;
+    find_prime_factors(s, phi);
+    for (u64 r = 2; r <= phi; r++) {
+        bool bad = false;
+        for (u64 f : s) if (orc_powmod(r, phi / f, q) == 1) { bad = true; break; }
+        if (!bad) return r;
+    }
+    return (u64)-1;
+}
+// Utils.cuh:98-109
+u64 orc_find_mth_root(u64 M, u64 q) {
+    u64 g = orc_find_primitive_root(q);
+    if ((q - 1) % M != 0) return (u64)-1;
+    return orc_powmod(g, (q - 1) / M, q);
+}
+// Utils.cuh:125-132
+uint32_t orc_bitrev(uint32_t x, int bits) {
+    uint32_t r = 0;
+    for (int i = 0; i < bits; i++) { r = (r << 1) | (x & 1); x >>= 1; }
+    return r;
+}
+static int ilog2(u64 n) { int l = 0; while ((1ull << l) < n) l++; return l; }
+
+// Utils.cuh:190-210 : psi[bitrev(i)] = psi^i, psiinv[bitrev(i)] = psi^-i, psiinv[1] *= n^-1, Shoup companions.
+void orc_fill_psi_tables(u64 psi, u64 q, uint32_t n, u64* psi_tab, u64* psiinv_tab, u64* psi_shoup, u64* psiinv_shoup) {
+    int lg = ilog2(n);
+    u64 psiinv = orc_invmod(psi, q);
+    u64 ninv = orc_invmod(n, q);
+    psi_tab[0] = psiinv_tab[0] = 1;
+    for (uint32_t i = 1; i < n; i++) {
+        uint32_t prev = orc_bitrev(i - 1, lg), next = orc_bitrev(i, lg);
+        psi_tab[next] = orc_mulmod(psi, psi_tab[prev], q);
+        psiinv_tab[next] = orc_mulmod(psiinv, psiinv_tab[prev], q);
+    }
+    psiinv_tab[1] = orc_mulmod(psiinv_tab[1], ninv, q);
+    if (psi_shoup) for (uint32_t i = 0; i < n; i++) psi_shoup[i] = orc_xshoup(psi_tab[i], q);
+    if (psiinv_shoup) for (uint32_t i = 0; i < n; i++) psiinv_shoup[i] = orc_xshoup(psiinv_tab[i], q);
+}
+
+// Forward negacyclic NTT, natural -> bit-reversed order, canonical output.
+// Loop shape: python/ntt.ipynb cell 2 (low_NTT); stage/twiddle rule psi[m+i]: ntt_60bit.cuh:320-346, :583-679.
+void orc_ntt_limb(u64* a, uint32_t n, u64 q, const u64* psi_tab) {
+    uint32_t t = n;
+    for (uint32_t m = 1; m < n; m <<= 1) {
+        t >>= 1;
+        for (uint32_t i = 0; i < m; i++) {
+            u64 w = psi_tab[m + i];
+            uint32_t j1 = 2 * i * t, j2 = j1 + t;
+            for (uint32_t j = j1; j < j2; j++) {
+                u64 U = a[j], V = orc_mulmod(a[j + t], w, q);
+                u64 s = U + V; if (s >= q) s -= q;
+                u64 d = U >= V ? U - V : U + q - V;
+                a[j] = s; a[j + t] = d;
+            }
+        }
+    }
+}
+// Inverse (Gentleman-Sande), bit-reversed -> natural order, scaled by n^-1, canonical output.
+// python/ntt.ipynb cell 2 (low_INNT); the reference folds n^-1 into psiinv[1] (Utils.cuh:200) for the (U-V) branch
+// of the last stage and multiplies the (U+V) branch by n_inv explicitly (ntt_60bit.cuh:890-893).
+void orc_intt_limb(u64* a, uint32_t n, u64 q, const u64* psiinv_tab, u64 n_inv) {
+    uint32_t t = 1;
+    for (uint32_t m = n; m > 1; m >>= 1) {
+        uint32_t h = m >> 1, j1 = 0;
+        for (uint32_t i = 0; i < h; i++) {
+            u64 w = psiinv_tab[h + i];
+            for (uint32_t j = j1; j < j1 + t; j++) {
+                u64 U = a[j], V = a[j + t];
+                u64 s = U + V; if (s >= q) s -= q;
+                u64 d = U >= V ? U - V : U + q - V;
+                a[j] = (h == 1) ? orc_mulmod(s, n_inv, q) : s;
+                a[j + t] = orc_mulmod(d, w, q);
+            }
+            j1 += 2 * t;
+        }
+        t <<= 1;
+    }
+}
+
+// Same transforms with the Shoup companions (uint128.cuh:169-179) instead of a 128-bit remainder; used by the
+// batched entry points so the oracle doubles as a timed CPU baseline.  Checked against the plain loops in tests.
+static void ntt_limb_shoup(u64* a, uint32_t n, u64 q, const u64* w, const u64* ws) {
+    uint32_t t = n;
+    for (uint32_t m = 1; m < n; m <<= 1) {
+        t >>= 1;
+        for (uint32_t i = 0; i < m; i++) {
+            u64 W = w[m + i], Ws = ws[m + i];
+            u64* x = a + 2 * (size_t)i * t; u64* y = x + t;
+            for (uint32_t j = 0; j < t; j++) {
+                u64 U = x[j], V = orc_mulmod_shoup(y[j], W, Ws, q);
+                u64 s = U + V; s = s >= q ? s - q : s;
+                u64 d = U >= V ? U - V : U + q - V;
+                x[j] = s; y[j] = d;
+            }
+        }
+    }
+}
+static void intt_limb_shoup(u64* a, uint32_t n, u64 q, const u64* w, const u64* ws, u64 n_inv, u64 n_inv_s) {
+    uint32_t t = 1;
+    for (uint32_t m = n; m > 1; m >>= 1) {
+        uint32_t h = m >> 1;
+        for (uint32_t i = 0; i < h; i++) {
+            u64 W = w[h + i], Ws = ws[h + i];
+            u64* x = a + 2 * (size_t)i * t; u64* y = x + t;
+            for (uint32_t j = 0; j < t; j++) {
+                u64 U = x[j], V = y[j];
+                u64 s = U + V; s = s >= q ? s - q : s;
+                u64 d = U >= V ? U - V : U + q - V;
+                x[j] = (h == 1) ? orc_mulmod_shoup(s, n_inv, n_inv_s, q) : s;
+                y[j] = orc_mulmod_shoup(d, W, Ws, q);
+            }
+        }
+        t <<= 1;
+    }
+}
+// Utils.cuh:255-285
+void orc_negacyclic_mul(const u64* a, const u64* b, u64* c, uint32_t n, u64 q) {
+    std::vector<u64> w(2 * (size_t)n, 0);
+    for (uint32_t i = 0; i < n; i++)
+        for (uint32_t j = 0; j < n; j++)
+            w[i + j] = (u64)(((u128)a[i] * b[j] + w[i + j]) % q);
+    for (uint32_t i = 0; i < n; i++) {
+        u64 lo = w[i], hi = w[i + n];
+        if (lo < hi) lo += q;
+        c[i] = (lo - hi) % q;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// context
+// ------------------------------------------------------------------------------------------------
+struct orc_ctx {
+    int logN = 0, p_num = 0, q_num = 0, t_num = 0, gamma = 0, L = 0, K = 0, dnum = 0;
+    int Ri_blockNum = 0, Qj_blockNum = 0;
+    long N = 0;
+    std::vector<u64> pqt, mu_hi, mu_lo, psi, psiinv_root, n_inv, n_inv_shoup, halfTmodpqti;
+    std::vector<u64> psi_table, psiinv_table, psi_shoup_table, psiinv_shoup_table;   // [prime][N]
+    // P -> q  (ModDown)
+    std::vector<u64> pHatVecModq;                          // [l<=L][K]
+    std::vector<u64> pHatInvVecModp, pHatInvVecModp_shoup; // [K]
+    std::vector<u64> PModqt, PModqt_shoup, PinvModq, PinvModq_shoup;
+    // Ri -> T
+    std::vector<u64> RiHatInv, RiHatInv_shoup;             // [Ri_blockNum][gamma]
+    std::vector<u64> RiHatModT;                            // [Ri_blockNum][t_num][gamma]
+    std::vector<u64> Rimodti;                              // [t_num][Ri_blockNum]
+    // Qj -> T
+    std::vector<u64> QjHatInv, QjHatInv_shoup;             // [L+1][Qj_blockNum][p_num]
+    std::vector<u64> QjHatModT;                            // [L+1][Qj_blockNum][t_num][p_num]
+    std::vector<u64> Qjmodti;                              // [L+1][Qj_blockNum][t_num]
+    // T -> PQ
+    std::vector<u64> THatInv, THatInv_shoup;               // [t_num]
+    std::vector<u64> THatModRi;                            // [K+L+1][t_num]
+    std::vector<u64> Tmodpqi;                              // [K+L+1]
+    // rescale
+    std::vector<u64> qiInvModql, qiInvModql_shoup;         // triangular, row l-1 at offset l(l-1)/2
+    // generic exact-conversion tables for the textbook hybrid switch: per level, per digit
+    const u64* psi_tab(int prime) const { return &psi_table[(size_t)prime * N]; }
+    const u64* psiinv_tab(int prime) const { return &psiinv_table[(size_t)prime * N]; }
+};
+
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// big-integer-free helpers: product of a list of primes modulo m
+static u64 prod_mod(const std::vector<u64>& v, int lo, int hi, int skip, u64 m) {
+    u64 r = 1;
+    for (int i = lo; i < hi; i++) { if (i == skip) continue; r = orc_mulmod(r, v[i] % m, m); }
+    return r;
+}
+
+// floor(T/2) mod m for T = prod t_i, without big integers: T is odd, so floor(T/2) = (T-1)/2 and
+// (T-1)/2 mod m = ((T mod 2m) - 1)/2 mod m  (Context_23.cuh:96-130 computes it with NTL::ZZ).
+static u64 half_prod_mod(const std::vector<u64>& t, u64 m) {
+    const u64 m2 = 2 * m;                      // m < 2^62 for every modulus this code handles
+    u64 r = 1;
+    for (u64 x : t) r = (u64)(((u128)r * (x % m2)) % m2);
+    return ((r - 1) / 2) % m;                  // r = T mod 2m is odd
+}
+
+orc_ctx* orc_ctx_create(int logN, const u64* p, int p_num, const u64* q, int q_num, const u64* t, int t_num, int gamma) {
+    orc_ctx* c = new orc_ctx();
+    c->logN = logN; c->N = 1L << logN;
+    c->p_num = p_num; c->q_num = q_num; c->t_num = t_num; c->gamma = gamma;
+    c->L = q_num - 1; c->K = p_num;
+    c->dnum = p_num ? q_num / p_num : 0;                                      // Context_23.cuh:29
+    c->Ri_blockNum = gamma ? ceil_div(p_num + q_num, gamma) : 0;              // :32
+    c->Qj_blockNum = p_num ? ceil_div(q_num, p_num) : 0;                      // :33
+    const long N = c->N; const int K = p_num, L = c->L;
+    for (int i = 0; i < p_num; i++) c->pqt.push_back(p[i]);
+    for (int i = 0; i < q_num; i++) c->pqt.push_back(q[i]);
+    for (int i = 0; i < t_num; i++) c->pqt.push_back(t[i]);
+    const int tot = (int)c->pqt.size();
+    std::vector<u64> pV(p, p + p_num), qV(q, q + q_num), tV(t, t + t_num);
+    c->mu_hi.resize(tot); c->mu_lo.resize(tot); c->psi.resize(tot); c->psiinv_root.resize(tot);
+    c->n_inv.resize(tot); c->n_inv_shoup.resize(tot);
+    for (int i = 0; i < tot; i++) {
+        u64 m = c->pqt[i];
+        orc_barrett_mu(m, &c->mu_hi[i], &c->mu_lo[i]);
+        c->psi[i] = orc_find_mth_root(2 * (u64)N, m);                         // Context_23.cuh:75,91,108
+        c->psiinv_root[i] = orc_invmod(c->psi[i], m);                         // :134-141
+        c->n_inv[i] = orc_invmod((u64)N, m);                                  // :144-151
+        c->n_inv_shoup[i] = orc_xshoup(c->n_inv[i], m);                       // :153-160
+        c->halfTmodpqti.push_back(t_num ? half_prod_mod(tV, m) : 0);          // :126-130
+    }
+    c->psi_table.resize((size_t)tot * N); c->psiinv_table.resize((size_t)tot * N);
+    c->psi_shoup_table.resize((size_t)tot * N); c->psiinv_shoup_table.resize((size_t)tot * N);
+#pragma omp parallel for schedule(dynamic)
+    for (int i = 0; i < tot; i++)                                             // Context_23.cuh:481-495
+        orc_fill_psi_tables(c->psi[i], c->pqt[i], (uint32_t)N, &c->psi_table[(size_t)i * N], &c->psiinv_table[(size_t)i * N],
+                            &c->psi_shoup_table[(size_t)i * N], &c->psiinv_shoup_table[(size_t)i * N]);
+
+    // ---- P x Q_l -> Q_l : Context_23.cuh:162-190 ----
+    for (int l = 0; l <= L; l++)
+        for (int i = 0; i < K; i++) c->pHatVecModq.push_back(prod_mod(pV, 0, K, i, qV[l]));
+    for (int i = 0; i < K; i++) {
+        u64 v = orc_invmod(prod_mod(pV, 0, K, i, pV[i]), pV[i]);
+        c->pHatInvVecModp.push_back(v); c->pHatInvVecModp_shoup.push_back(orc_xshoup(v, pV[i]));
+    }
+    // ---- Ri -> T : Context_23.cuh:232-283 ----
+    const int PQ = p_num + q_num;
+    if (gamma > 0 && t_num > 0) {
+        c->RiHatInv.assign((size_t)c->Ri_blockNum * gamma, 0); c->RiHatInv_shoup.assign((size_t)c->Ri_blockNum * gamma, 0);
+        c->RiHatModT.assign((size_t)c->Ri_blockNum * t_num * gamma, 0);
+        c->Rimodti.assign((size_t)t_num * c->Ri_blockNum, 0);
+        for (int i = 0; i < c->Ri_blockNum; i++) {
+            int lo = i * gamma, hi = std::min(lo + gamma, PQ);
+            for (int j = lo; j < hi; j++) {
+                u64 v = orc_invmod(prod_mod(c->pqt, lo, hi, j, c->pqt[j]), c->pqt[j]);
+                c->RiHatInv[(size_t)i * gamma + (j - lo)] = v;
+                c->RiHatInv_shoup[(size_t)i * gamma + (j - lo)] = orc_xshoup(v, c->pqt[j]);
+            }
+            for (int k = 0; k < t_num; k++) {
+                for (int j = lo; j < hi; j++)
+                    c->RiHatModT[(size_t)i * t_num * gamma + (size_t)k * gamma + (j - lo)] = prod_mod(c->pqt, lo, hi, j, tV[k]);
+                c->Rimodti[(size_t)k * c->Ri_blockNum + i] = prod_mod(c->pqt, lo, hi, -1, tV[k]);
+            }
+        }
+    }
+    // ---- Qj -> T : Context_23.cuh:286-351 ----
+    if (p_num > 0 && t_num > 0) {
+        const int B = c->Qj_blockNum;
+        c->QjHatInv.assign((size_t)(L + 1) * B * p_num, 0); c->QjHatInv_shoup.assign((size_t)(L + 1) * B * p_num, 0);
+        c->QjHatModT.assign((size_t)(L + 1) * B * t_num * p_num, 0);
+        c->Qjmodti.assign((size_t)(L + 1) * B * t_num, 0);
+        for (int l = 0; l <= L; l++) {
+            int nb = ceil_div(l + 1, p_num);
+            for (int i = 0; i < nb; i++) {
+                int lo = i * p_num, hi = std::min(lo + p_num, l + 1);
+                for (int j = lo; j < hi; j++) {
+                    u64 v = orc_invmod(prod_mod(qV, lo, hi, j, qV[j]), qV[j]);
+                    size_t o = (size_t)l * B * p_num + (size_t)i * p_num + (j - lo);
+                    c->QjHatInv[o] = v; c->QjHatInv_shoup[o] = orc_xshoup(v, qV[j]);
+                }
+                for (int k = 0; k < t_num; k++) {
+                    for (int j = lo; j < hi; j++)
+                        c->QjHatModT[(size_t)l * B * t_num * p_num + (size_t)i * t_num * p_num + (size_t)k * p_num + (j - lo)] =
+                            prod_mod(qV, lo, hi, j, tV[k]);
+                    c->Qjmodti[(size_t)l * B * t_num + (size_t)i * t_num + k] = prod_mod(qV, lo, hi, -1, tV[k]);
+                }
+            }
+        }
+    }
+    // ---- T -> PQ : Context_23.cuh:354-393 ----
+    for (int i = 0; i < t_num; i++) {
+        u64 v = orc_invmod(prod_mod(tV, 0, t_num, i, tV[i]), tV[i]);
+        c->THatInv.push_back(v); c->THatInv_shoup.push_back(orc_xshoup(v, tV[i]));
+    }
+    for (int i = 0; i < PQ; i++) {
+        for (int j = 0; j < t_num; j++) c->THatModRi.push_back(prod_mod(tV, 0, t_num, j, c->pqt[i]));
+        c->Tmodpqi.push_back(prod_mod(tV, 0, t_num, -1, c->pqt[i]));
+    }
+    // ---- P mod q,t ; P^-1 mod q : Context_23.cuh:397-421 ----
+    for (int i = 0; i <= L; i++) {
+        u64 v = prod_mod(pV, 0, K, -1, qV[i]);
+        c->PModqt.push_back(v); c->PModqt_shoup.push_back(orc_xshoup(v, qV[i]));
+        u64 w = orc_invmod(v, qV[i]);
+        c->PinvModq.push_back(w); c->PinvModq_shoup.push_back(orc_xshoup(w, qV[i]));
+    }
+    for (int i = 0; i < t_num; i++) {
+        u64 v = prod_mod(pV, 0, K, -1, tV[i]);
+        c->PModqt.push_back(v); c->PModqt_shoup.push_back(orc_xshoup(v, tV[i]));
+    }
+    // ---- rescale : Context_23.cuh:425-436, device layout :557-563 (row l-1 at offset l(l-1)/2) ----
+    for (int l = 1; l <= L; l++)
+        for (int j = 0; j < l; j++) {
+            u64 v = orc_invmod(qV[l], qV[j]);
+            c->qiInvModql.push_back(v); c->qiInvModql_shoup.push_back(orc_xshoup(v, qV[j]));
+        }
+    return c;
+}
+void orc_ctx_destroy(orc_ctx* c) { delete c; }
+
+int orc_ctx_info(const orc_ctx* c, const char* name) {
+    std::string n(name);
+    if (n == "logN") return c->logN;
+    if (n == "p_num") return c->p_num;
+    if (n == "q_num") return c->q_num;
+    if (n == "t_num") return c->t_num;
+    if (n == "gamma") return c->gamma;
+    if (n == "dnum") return c->dnum;
+    if (n == "Ri_blockNum") return c->Ri_blockNum;
+    if (n == "Qj_blockNum") return c->Qj_blockNum;
+    return -1;
+}
+long orc_ctx_get(const orc_ctx* c, const char* name, u64* out, long cap) {
+    std::string n(name);
+    const std::vector<u64>* v = nullptr;
+    if (n == "pqt") v = &c->pqt; else if (n == "mu_hi") v = &c->mu_hi; else if (n == "mu_lo") v = &c->mu_lo;
+    else if (n == "psi") v = &c->psi; else if (n == "psiinv") v = &c->psiinv_root;
+    else if (n == "n_inv") v = &c->n_inv; else if (n == "n_inv_shoup") v = &c->n_inv_shoup;
+    else if (n == "halfTmodpqti") v = &c->halfTmodpqti;
+    else if (n == "psi_table") v = &c->psi_table; else if (n == "psiinv_table") v = &c->psiinv_table;
+    else if (n == "psi_shoup_table") v = &c->psi_shoup_table; else if (n == "psiinv_shoup_table") v = &c->psiinv_shoup_table;
+    else if (n == "pHatVecModq") v = &c->pHatVecModq; else if (n == "pHatInvVecModp") v = &c->pHatInvVecModp;
+    else if (n == "PModqt") v = &c->PModqt; else if (n == "PinvModq") v = &c->PinvModq;
+    else if (n == "RiHatInv") v = &c->RiHatInv; else if (n == "RiHatModT") v = &c->RiHatModT; else if (n == "Rimodti") v = &c->Rimodti;
+    else if (n == "QjHatInv") v = &c->QjHatInv; else if (n == "QjHatModT") v = &c->QjHatModT; else if (n == "Qjmodti") v = &c->Qjmodti;
+    else if (n == "THatInv") v = &c->THatInv; else if (n == "THatModRi") v = &c->THatModRi; else if (n == "Tmodpqi") v = &c->Tmodpqi;
+    else if (n == "qiInvModql") v = &c->qiInvModql;
+    if (!v) return -1;
+    long cnt = (long)v->size();
+    if (out) { if (cap < cnt) return -1; std::memcpy(out, v->data(), cnt * sizeof(u64)); }
+    return cnt;
+}
+
+// ------------------------------------------------------------------------------------------------
+// batched NTT with the reference's addressing (Context_23.cuh:847-930; ntt_60bit.cuh:446-455, :913-934)
+// ------------------------------------------------------------------------------------------------
+static int ntt_batch(const orc_ctx* c, u64* a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                     int poly_mod_len, long batch_stride_limbs, int batch, bool inverse) {
+    const long N = c->N;
+    if (start_mod_idx < 0 || start_mod_idx + mod_num > (int)c->pqt.size()) return -1;
+    const long total = (long)batch * poly_num * mod_num;
+#pragma omp parallel for schedule(static)
+    for (long w = 0; w < total; w++) {
+        int j = (int)(w % mod_num); long r = w / mod_num;
+        int y = (int)(r % poly_num); int z = (int)(r / poly_num);
+        u64* limb = a + ((long)z * batch_stride_limbs + (long)y * poly_mod_len + start_poly_idx + j) * N;
+        int prime = start_mod_idx + j;
+        if (inverse) intt_limb_shoup(limb, (uint32_t)N, c->pqt[prime], c->psiinv_tab(prime), &c->psiinv_shoup_table[(size_t)prime * N],
+                                     c->n_inv[prime], c->n_inv_shoup[prime]);
+        else ntt_limb_shoup(limb, (uint32_t)N, c->pqt[prime], c->psi_tab(prime), &c->psi_shoup_table[(size_t)prime * N]);
+    }
+    return 0;
+}
+int orc_ntt_fwd(const orc_ctx* c, u64* a, int sp, int sm, int pn, int mn, int pml) { return ntt_batch(c, a, sp, sm, pn, mn, pml, 0, 1, false); }
+int orc_ntt_inv(const orc_ctx* c, u64* a, int sp, int sm, int pn, int mn, int pml) { return ntt_batch(c, a, sp, sm, pn, mn, pml, 0, 1, true); }
+int orc_ntt_fwd_ext(const orc_ctx* c, u64* a, int sp, int sm, int pn, int mn, int pml, int cmn, int bs) { return ntt_batch(c, a, sp, sm, pn, mn, pml, cmn, bs, false); }
+int orc_ntt_inv_ext(const orc_ctx* c, u64* a, int sp, int sm, int pn, int mn, int pml, int cmn, int bs) { return ntt_batch(c, a, sp, sm, pn, mn, pml, cmn, bs, true); }
+
+// ------------------------------------------------------------------------------------------------
+// basis conversion
+// ------------------------------------------------------------------------------------------------
+static inline u128 sub128_64(u128 a, u64 b) { return a - (u128)b; }          // uint128.cuh:273-283 (wraps mod 2^128)
+static inline u64 barrett_idx(const orc_ctx* c, u128 acc, int prime) {
+    return orc_barrett128((u64)(acc >> 64), (u64)acc, c->pqt[prime], c->mu_hi[prime], c->mu_lo[prime]);
+}
+
+// BasisConv.cuh:7-79
+int orc_modup_pq_to_t(const orc_ctx* c, u64* out, const u64* in, int l, int batch) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num;
+    if (g <= 0 || T <= 0 || l < 0 || l > c->L) return -1;
+    const int blockNum = ceil_div(P + l + 1, g);
+    for (int b = 0; b < batch; b++)
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int blk = 0; blk < blockNum; blk++)
+            for (long x = 0; x < N; x++) {
+                u64 rb[64]; double vv = 0; int cnt = 0;
+                for (int i = 0; i < g && i + blk * g < P + l + 1; i++, cnt++) {
+                    int pi = i + blk * g; u64 ri = c->pqt[pi];
+                    u64 ra = in[((long)pi + (long)b * (P + Q)) * N + x];
+                    rb[i] = orc_mulmod_shoup(ra, c->RiHatInv[(size_t)blk * g + i], c->RiHatInv_shoup[(size_t)blk * g + i], ri);
+                    vv += (double)rb[i] / (double)ri;                          // :33
+                }
+                int vf = (int)vv;                                              // :36
+                for (int k = 0; k < T; k++) {
+                    u128 acc = 0;
+                    for (int j = 0; j < cnt; j++) acc += (u128)rb[j] * c->RiHatModT[(size_t)blk * T * g + (size_t)k * g + j];
+                    acc = sub128_64(acc, (u64)vf * c->Rimodti[(size_t)k * c->Ri_blockNum + blk]);   // :54
+                    long oidx = (long)b * c->Ri_blockNum * T + (long)blk * T + k;                    // :52
+                    out[oidx * N + x] = barrett_idx(c, acc, P + Q + k);
+                }
+            }
+    return 0;
+}
+
+// BasisConv.cuh:84-179.  The reference indexes Qjmodti with the batch index folded in (:142,:153), which for
+// batch > 0 walks into the next level's table; every caller uses the table of level l, and so does this restatement.
+int orc_modup_qj_to_t(const orc_ctx* c, u64* out, const u64* in, int l, int batch) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num, T = c->t_num, B = c->Qj_blockNum;
+    if (P <= 0 || T <= 0 || l < 0 || l > c->L) return -1;
+    const int blockNum = ceil_div(l + 1, P);
+    const u64* hatinv = &c->QjHatInv[(size_t)l * B * P]; const u64* hatinv_s = &c->QjHatInv_shoup[(size_t)l * B * P];
+    const u64* hatT = &c->QjHatModT[(size_t)l * B * T * P]; const u64* qjmodt = &c->Qjmodti[(size_t)l * B * T];
+    for (int b = 0; b < batch; b++)
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int blk = 0; blk < blockNum; blk++)
+            for (long x = 0; x < N; x++) {
+                u64 rb[64]; double vv = 0; int cnt = 0;
+                for (int j = 0; j < P && j + blk * P < l + 1; j++, cnt++) {
+                    int iq = j + blk * P; u64 qi = c->pqt[P + iq];
+                    u64 ra = in[(long)b * Q * N + (long)iq * N + x];
+                    rb[j] = orc_mulmod_shoup(ra, hatinv[iq], hatinv_s[iq], qi);
+                    vv += (double)rb[j] / (double)qi;                          // :113-114
+                }
+                int vf = (int)vv;                                              // :152
+                for (int k = 0; k < T; k++) {
+                    u128 acc = 0;
+                    for (int j = 0; j < cnt; j++) acc += (u128)rb[j] * hatT[(size_t)blk * T * P + (size_t)k * P + j];
+                    acc = sub128_64(acc, (u64)vf * qjmodt[(size_t)blk * T + k]);
+                    long oidx = (long)b * B * T + (long)blk * T + k;
+                    out[oidx * N + x] = barrett_idx(c, acc, P + Q + k);
+                }
+            }
+    return 0;
+}
+
+// BasisConv.cuh:183-254
+int orc_modup_t_to_pql(const orc_ctx* c, u64* buf, const u64* in, int l, int batch) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum;
+    if (g <= 0 || T <= 0 || l < 0 || l > c->L) return -1;
+    const int blockNum = ceil_div(P + l + 1, g);
+    for (int b = 0; b < batch; b++)
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int blk = 0; blk < blockNum; blk++)
+            for (long x = 0; x < N; x++) {
+                u64 rb[64]; double vv = 0;
+                for (int i = 0; i < T; i++) {
+                    u64 t = c->pqt[P + Q + i];
+                    u64 ra = in[(long)b * RB * T * N + ((long)blk * T + i) * N + x];
+                    ra = ra + c->halfTmodpqti[P + Q + i];                      // :203
+                    rb[i] = orc_mulmod_shoup(ra, c->THatInv[i], c->THatInv_shoup[i], t);
+                    vv += (double)rb[i] / (double)t;                           // :209-210
+                }
+                int vf = (int)vv;
+                for (int j = 0; j < g && j + blk * g < P + l + 1; j++) {
+                    int ipq = j + blk * g; u64 ri = c->pqt[ipq];
+                    u128 acc = 0;
+                    for (int i = 0; i < T; i++) acc += (u128)rb[i] * c->THatModRi[(size_t)ipq * T + i];
+                    acc = sub128_64(acc, (u64)vf * c->Tmodpqi[ipq]);           // :232
+                    u64 r = barrett_idx(c, acc, ipq);
+                    r = r + ri - c->halfTmodpqti[ipq];                         // :236
+                    r = csub_q(r, ri);
+                    buf[(long)b * RB * T * N + (long)ipq * N + x] = r;         // :239
+                }
+            }
+    return 0;
+}
+
+// BasisConv.cuh:257-347
+int orc_moddown_pql_to_ql(const orc_ctx* c, u64* out, const u64* buf, int l, int batch) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum;
+    if (P <= 0 || l < 0 || l > c->L) return -1;
+    const long in_stride = (long)RB * T * N;
+    for (int b = 0; b < batch; b++)
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int iq = 0; iq <= l; iq++)
+            for (long x = 0; x < N; x++) {
+                u64 qi = c->pqt[P + iq];
+                u64 r;
+                if (P == 1) {                                                  // :261-283
+                    r = buf[b * in_stride + x] % qi;
+                } else {                                                       // :286-326
+                    u128 acc = 0;
+                    for (int i = 0; i < P; i++) {
+                        u64 ra = buf[b * in_stride + (long)i * N + x];
+                        u64 rb = orc_mulmod_shoup(ra, c->pHatInvVecModp[i], c->pHatInvVecModp_shoup[i], c->pqt[i]);
+                        acc += (u128)rb * c->pHatVecModq[(size_t)iq * P + i];
+                    }
+                    r = barrett_idx(c, acc, P + iq);
+                }
+                u64 v = qi - r + buf[b * in_stride + (long)(P + iq) * N + x];
+                out[(long)b * Q * N + (long)iq * N + x] = orc_mulmod_shoup(v, c->PinvModq[iq], c->PinvModq_shoup[iq], qi);
+            }
+    return 0;
+}
+
+// ExternalProduct.cuh:7-97
+int orc_external_product_t(const orc_ctx* c, u64* out, const u64* cT, const u64* swk, int l) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum;
+    if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L) return -1;
+    const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int blk = 0; blk < blockNum; blk++)
+        for (int k = 0; k < T; k++)
+            for (long x = 0; x < N; x++) {
+                u128 acc1 = 0, acc2 = 0;
+                for (int i = 0; i < cipher_blockNum; i++) {
+                    u64 ra = cT[((long)i * T + k) * N + x];
+                    long kidx = ((long)i * T * RB + (long)blk * T + k) * N + x;
+                    acc1 += (u128)ra * swk[kidx];
+                    acc2 += (u128)ra * swk[(long)RB * T * dnum * N + kidx];
+                }
+                long oidx = x + (long)blk * T * N + (long)k * N;
+                out[oidx] = barrett_idx(c, acc1, P + Q + k);
+                out[(long)RB * T * N + oidx] = barrett_idx(c, acc2, P + Q + k);
+            }
+    return 0;
+}
+
+// Scheme_23.cuh:321-385
+int orc_rescale(const orc_ctx* c, u64* cipher, int l) {
+    const long N = c->N; const int K = c->K, L = c->L;
+    if (l < 1 || l > L) return -1;
+    orc_ntt_inv(c, cipher, l, K + l, 2, 1, L + 1);                              // :372
+    std::vector<u64> rb((size_t)2 * (L + 1) * N, 0);
+    for (int z = 0; z < 2; z++)
+        for (int i = 0; i < l; i++) {
+            u64 q = c->pqt[K + i], mu_hi = c->mu_hi[K + i];
+            for (long x = 0; x < N; x++)                                       // mod_to_qi :356-367
+                rb[((size_t)z * (L + 1) + i) * N + x] = orc_barrett64(cipher[((size_t)z * (L + 1) + l) * N + x], q, mu_hi);
+        }
+    orc_ntt_fwd(c, rb.data(), 0, K, 2, l, L + 1);                               // :376
+    const u64* inv = &c->qiInvModql[(size_t)l * (l - 1) / 2]; const u64* inv_s = &c->qiInvModql_shoup[(size_t)l * (l - 1) / 2];
+    for (int z = 0; z < 2; z++)
+        for (int i = 0; i < l; i++) {
+            u64 q = c->pqt[K + i];
+            for (long x = 0; x < N; x++) {                                     // :339-354
+                size_t idx = ((size_t)z * (L + 1) + i) * N + x;
+                u64 ra = cipher[idx] + 2 * q - rb[idx];
+                ra = csub_q(ra, q);
+                cipher[idx] = orc_mulmod_shoup(ra, inv[i], inv_s[i], q);
+            }
+        }
+    return 0;
+}
+
+// KeySwitch_23.cuh:219-231
+int orc_keyswitch_23(const orc_ctx* c, u64* out, const u64* d2, const u64* swk, int l) {
+    const long N = c->N; const int K = c->K, L = c->L, T = c->t_num, RB = c->Ri_blockNum, g = c->gamma;
+    if (g <= 0 || T <= 0 || K <= 0 || l < 0 || l > L) return -1;
+    const int swk_blockNum = ceil_div(K + l + 1, g), cipher_blockNum = ceil_div(l + 1, K);
+    std::vector<u64> axax(d2, d2 + (size_t)(L + 1) * N);
+    std::vector<u64> up((size_t)N * T * c->Qj_blockNum, 0), ext((size_t)N * T * RB * 2, 0), buf((size_t)N * T * RB * 2, 0);
+    orc_ntt_inv(c, axax.data(), 0, K, 1, l + 1, L + 1);                         // :219
+    orc_modup_qj_to_t(c, up.data(), axax.data(), l, 1);                        // :221
+    orc_ntt_fwd(c, up.data(), 0, K + L + 1, cipher_blockNum, T, T);             // :223
+    orc_external_product_t(c, ext.data(), up.data(), swk, l);                  // :225
+    orc_ntt_inv_ext(c, ext.data(), 0, K + L + 1, swk_blockNum, T, T, RB * T, 2);// :226
+    orc_modup_t_to_pql(c, buf.data(), ext.data(), l, 2);                       // :228
+    orc_moddown_pql_to_ql(c, out, buf.data(), l, 2);                           // :229
+    orc_ntt_fwd(c, out, 0, K, 2, l + 1, L + 1);                                 // :231
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// textbook hybrid key switch over [P | Q_l], alpha = p_num primes per digit.
+// The reference has no such routine (its switch goes through the auxiliary basis T); this one applies the
+// reference's exact-conversion recipe (BasisConv.cuh:18-58: y_j = x_j * (D^_j)^-1 mod d_j,
+// v = trunc(sum (double)y_j/(double)d_j), out = sum y_j * (D^_j mod r) - v * (D mod r)) to a digit D of
+// alpha consecutive Q primes and every other prime r of [P | Q_l], and its ModDown (BasisConv.cuh:286-326).
+// ------------------------------------------------------------------------------------------------
+int orc_hybrid_modup(const orc_ctx* c, u64* digits_out, const u64* in, int l) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num;
+    if (P <= 0 || l < 0 || l > c->L) return -1;
+    const int dn = ceil_div(l + 1, P), W = P + Q;
+    for (int d = 0; d < dn; d++) {
+        int lo = d * P, hi = std::min(lo + P, l + 1), cnt = hi - lo;
+        std::vector<u64> hatinv(cnt), hatinv_s(cnt);
+        for (int j = lo; j < hi; j++) {
+            u64 qj = c->pqt[P + j];
+            hatinv[j - lo] = orc_invmod(prod_mod(c->pqt, P + lo, P + hi, P + j, qj), qj);
+            hatinv_s[j - lo] = orc_xshoup(hatinv[j - lo], qj);
+        }
+        std::vector<int> targets;
+        for (int r = 0; r < P + l + 1; r++) if (r < P + lo || r >= P + hi) targets.push_back(r);
+        std::vector<u64> hat((size_t)targets.size() * cnt), Dmod(targets.size());
+        for (size_t ti = 0; ti < targets.size(); ti++) {
+            u64 r = c->pqt[targets[ti]];
+            for (int j = lo; j < hi; j++) hat[ti * cnt + (j - lo)] = prod_mod(c->pqt, P + lo, P + hi, P + j, r);
+            Dmod[ti] = prod_mod(c->pqt, P + lo, P + hi, -1, r);
+        }
+        u64* o = digits_out + (long)d * W * N;
+#pragma omp parallel for schedule(static)
+        for (long x = 0; x < N; x++) {
+            u64 y[64]; double vv = 0;
+            for (int j = lo; j < hi; j++) {
+                u64 qj = c->pqt[P + j], xin = in[(long)j * N + x];
+                o[(long)(P + j) * N + x] = xin;
+                y[j - lo] = orc_mulmod_shoup(xin, hatinv[j - lo], hatinv_s[j - lo], qj);
+                vv += (double)y[j - lo] / (double)qj;
+            }
+            int vf = (int)vv;
+            for (size_t ti = 0; ti < targets.size(); ti++) {
+                u128 acc = 0;
+                for (int j = 0; j < cnt; j++) acc += (u128)y[j] * hat[ti * cnt + j];
+                acc = sub128_64(acc, (u64)vf * Dmod[ti]);
+                o[(long)targets[ti] * N + x] = barrett_idx(c, acc, targets[ti]);
+            }
+        }
+    }
+    return 0;
+}
+// evk: [2 (a,b)][dnum][P+Q] limbs (NTT domain); digits: [dn][P+Q] limbs (NTT domain); out: [2][P+Q] limbs.
+int orc_hybrid_inner_product(const orc_ctx* c, u64* out, const u64* digits, const u64* evk, int l) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num, W = P + Q;
+    if (P <= 0 || l < 0 || l > c->L) return -1;
+    const int dn = ceil_div(l + 1, P), dnum = ceil_div(Q, P);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int z = 0; z < 2; z++)
+        for (int r = 0; r < P + l + 1; r++)
+            for (long x = 0; x < N; x++) {
+                u128 acc = 0;
+                for (int d = 0; d < dn; d++)
+                    acc += (u128)digits[((long)d * W + r) * N + x] * evk[(((long)z * dnum + d) * W + r) * N + x];
+                out[((long)z * W + r) * N + x] = barrett_idx(c, acc, r);
+            }
+    return 0;
+}
+// in: [2][P+Q] limbs (coefficient domain) -> out: [2][Q] limbs; arithmetic of BasisConv.cuh:286-326.
+int orc_hybrid_moddown(const orc_ctx* c, u64* out, const u64* in, int l) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num, W = P + Q;
+    if (P <= 0 || l < 0 || l > c->L) return -1;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int z = 0; z < 2; z++)
+        for (int iq = 0; iq <= l; iq++) {
+            u64 qi = c->pqt[P + iq];
+            for (long x = 0; x < N; x++) {
+                u128 acc = 0;
+                for (int i = 0; i < P; i++) {
+                    u64 rb = orc_mulmod_shoup(in[((long)z * W + i) * N + x], c->pHatInvVecModp[i], c->pHatInvVecModp_shoup[i], c->pqt[i]);
+                    acc += (u128)rb * c->pHatVecModq[(size_t)iq * P + i];
+                }
+                u64 r = barrett_idx(c, acc, P + iq);
+                u64 v = qi - r + in[((long)z * W + P + iq) * N + x];
+                out[((long)z * Q + iq) * N + x] = orc_mulmod_shoup(v, c->PinvModq[iq], c->PinvModq_shoup[iq], qi);
+            }
+        }
+    return 0;
+}
+// in_ntt: Q limbs (NTT domain); out: [2][Q] limbs (NTT domain).
+int orc_hybrid_keyswitch(const orc_ctx* c, u64* out, const u64* in_ntt, const u64* evk, int l) {
+    const long N = c->N; const int P = c->p_num, Q = c->q_num, W = P + Q;
+    if (P <= 0 || l < 0 || l > c->L) return -1;
+    const int dn = ceil_div(l + 1, P);
+    std::vector<u64> in(in_ntt, in_ntt + (size_t)Q * N), dig((size_t)dn * W * N, 0), ip((size_t)2 * W * N, 0);
+    orc_ntt_inv(c, in.data(), 0, P, 1, l + 1, Q);
+    orc_hybrid_modup(c, dig.data(), in.data(), l);
+    orc_ntt_fwd(c, dig.data(), 0, 0, dn, P + l + 1, W);
+    orc_hybrid_inner_product(c, ip.data(), dig.data(), evk, l);
+    orc_ntt_inv(c, ip.data(), 0, 0, 2, P + l + 1, W);
+    orc_hybrid_moddown(c, out, ip.data(), l);
+    orc_ntt_fwd(c, out, 0, P, 2, l + 1, Q);
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// ring-packed PCMM
+// ------------------------------------------------------------------------------------------------
+struct orc_pcmm {
+    const orc_ctx* ctx; int N1, rank, np, nq;
+    std::vector<u64> pq, mu_hi, mu_lo;
+};
+// PCMM_Context.cuh:7-36
+orc_pcmm* orc_pcmm_create(const orc_ctx* c, int N1, int rank, const u64* p, int np, const u64* q, int nq) {
+    orc_pcmm* h = new orc_pcmm(); h->ctx = c; h->N1 = N1; h->rank = rank; h->np = np; h->nq = nq;
+    for (int i = 0; i < np; i++) h->pq.push_back(p[i]);
+    for (int i = 0; i < nq; i++) h->pq.push_back(q[i]);
+    h->mu_hi.resize(np + nq); h->mu_lo.resize(np + nq);
+    for (int i = 0; i < np + nq; i++) orc_barrett_mu(h->pq[i], &h->mu_hi[i], &h->mu_lo[i]);
+    return h;
+}
+void orc_pcmm_destroy(orc_pcmm* h) { delete h; }
+
+static inline u64 negate_modq(u64 a, u64 q) { return a == 0 ? 0 : q - a; }    // uint128.cuh:309-313
+
+// PCMM_Scheme.cuh:50-88 (the gather kernel only; coefficient-domain input)
+int orc_rlwe_decompose(const orc_pcmm* h, const u64* rlwe, u64* const* mlwe, int mlwe_num, int l) {
+    const orc_ctx* c = h->ctx; const long N = c->N; const int N1 = h->N1, k = h->rank, L = c->L, P = c->p_num;
+    if (mlwe_num > k || mlwe_num <= 0 || (long)N1 * k != N) return -1;
+    const int gap = k / mlwe_num;
+    for (int m = 0; m < mlwe_num; m++)
+        for (int im = 0; im <= l; im++) {
+            u64 q = c->pqt[P + im];
+            const u64* A = rlwe + N * im; const u64* B = rlwe + N * (L + 1 + im);
+            u64* ax = mlwe[m] + (long)N1 * (k + 1) * im; u64* bx = ax + (long)N1 * k;
+            for (int g = 0; g < N1; g++) {
+                long addr = (long)m * gap + (long)g * k; bool over = addr >= N;
+                ax[g] = over ? negate_modq(A[addr - N], q) : A[addr];
+                bx[g] = over ? negate_modq(B[addr - N], q) : B[addr];
+                for (int i = 1; i < k; i++) {
+                    if (g == 0) {
+                        addr = (long)(N1 - 1) * k + (k - i) + (long)m * gap; over = addr >= N;
+                        ax[g + (long)i * N1] = over ? A[addr - N] : negate_modq(A[addr], q);
+                    } else {
+                        addr = (long)(g - 1) * k + (k - i) + (long)m * gap; over = addr >= N;
+                        ax[g + (long)i * N1] = over ? negate_modq(A[addr - N], q) : A[addr];
+                    }
+                }
+            }
+        }
+    return 0;
+}
+
+// PPMM_kernel.cuh:12-31, 93-252.  Generalised from the reference's two ring-pack primes to mod_num primes:
+// the fused rescale divides by the LAST prime and uses (q_last)^-1 mod q_i, which for mod_num == 2 is exactly the
+// table row the reference hard-wires (l = 1, PPMM_kernel.cuh:298,310).
+int orc_ppmm(const orc_pcmm* h, const float* W, const u64* const* mlwe, u64* out, int M, int Kin, int mod_num,
+             double scaler, long col_begin, long col_count) {
+    const int N1 = h->N1, k = h->rank, np = h->np;
+    if (mod_num < 1 || mod_num > h->nq) return -1;
+    const long C = (long)(k + 1) * N1;
+    if (col_begin < 0 || col_begin + col_count > C) return -1;
+    std::vector<int64_t> A((size_t)M * Kin);
+    for (long i = 0; i < (long)M * Kin; i++) A[i] = (int64_t)((double)W[i] * scaler);   // :148 float*double -> int64 (trunc)
+    const u64 qlast = h->pq[np + mod_num - 1];
+    for (int im = mod_num - 1; im >= 0; im--) {
+        const u64 q = h->pq[np + im], mh = h->mu_hi[np + im], ml = h->mu_lo[np + im];
+        u64 qinv = 0, qinv_s = 0;
+        if (im != mod_num - 1) { qinv = orc_invmod(qlast, q); qinv_s = orc_xshoup(qinv, q); }   // Context_23.cuh:425-436
+#pragma omp parallel for schedule(static)
+        for (int m = 0; m < M; m++) {
+            std::vector<u64> a(Kin);
+            for (int n = 0; n < Kin; n++) { int64_t t = A[(size_t)m * Kin + n]; a[n] = t > 0 ? (u64)t : q + (u64)t; }   // :25
+            for (long cc = col_begin; cc < col_begin + col_count; cc++) {
+                u128 acc = 0;
+                for (int n = 0; n < Kin; n++) acc += (u128)a[n] * mlwe[n][(long)im * C + cc];
+                u64 r = orc_barrett128((u64)(acc >> 64), (u64)acc, q, mh, ml);
+                u64* o = out + (long)m * C * mod_num;
+                if (im == mod_num - 1) o[(long)im * C + cc] = r;                                 // :213-229
+                else {
+                    u64 temp = r + q - o[(long)(mod_num - 1) * C + cc];                          // :244
+                    o[(long)im * C + cc] = orc_mulmod_shoup(temp, qinv, qinv_s, q);              // :247
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

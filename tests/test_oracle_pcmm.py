@@ -1,0 +1,130 @@
+"""Pins the oracle's RLWE->MLWE gather and PPMM: notebook vectors, ring identity, big-int brute force."""
+import numpy as np
+import pytest
+
+from oracle import oracle_py as O
+from tests.helpers import negacyclic_mul, limbs_uniform
+from tests.params import CFG2_Q, REF_PARAMS
+
+
+def ring_down(poly, N, N1):
+    """ring_packing.ipynb cell 1 `ringDown`: sub-ring i takes coefficients i, i+k, i+2k, ..."""
+    k = N // N1
+    return [[poly[i + g * k] for g in range(N1)] for i in range(k)]
+
+
+def test_notebook_algebra_is_consistent(golden_nb):
+    """The test's own negacyclic algebra reproduces the numbers the notebook printed (cell 1): per-sub-ring
+    products, their sum ('inner product') and the extraction target."""
+    q = golden_nb["q"]
+    a, s = golden_nb["cell1_ax_big_ring"], golden_nb["cell0_sx_big_ring"]
+    a_down, s_down = ring_down(a, 32, 8), ring_down(s, 32, 8)
+    assert a_down == golden_nb["cell1_ax_down"]
+    prods = [negacyclic_mul(x, y, q) for x, y in zip(a_down, s_down)]
+    assert prods == golden_nb["cell1_products"]
+    ip = [sum(p[i] for p in prods) % q for i in range(8)]
+    assert ip == golden_nb["cell1_inner_product"] == golden_nb["cell1_target"]
+    tw_s = negacyclic_mul(golden_nb["cell1_twist"], s, q)
+    assert tw_s == golden_nb["cell1_twist_times_sx"]
+    assert ring_down(tw_s, 32, 8)[0] == golden_nb["cell1_target"]
+
+
+def make_small_ctx(q_list, logN=5, p=None):
+    # N = 32; every modulus must be 1 mod 64
+    return O.OracleContext(logN, p or [], q_list)
+
+
+def test_decompose_notebook_kat(golden_nb):
+    """Extract(twist(a)) returns the sub-rings of a (ring_packing.ipynb cells 1,3): the gather kernel applied to the
+    printed 'twist' polynomial must give the printed 'ax down' rows."""
+    q = golden_nb["q"]
+    ctx = make_small_ctx([q])
+    pc = O.OraclePCMM(ctx, 8, 4, [], [q])
+    rlwe = np.zeros((2, 1, 32), dtype=np.uint64)
+    rlwe[0, 0] = golden_nb["cell1_twist"]
+    rlwe[1, 0] = np.arange(32) * 2                      # cell 0: bx = [2i]
+    mlwe = [np.zeros((1, 5, 8), dtype=np.uint64)]
+    pc.rlweCipherDecompose(rlwe.reshape(-1), [m.reshape(-1) for m in mlwe], 0)
+    assert [[int(v) for v in row] for row in mlwe[0][0, :4]] == golden_nb["cell1_ax_down"]
+    assert [int(v) for v in mlwe[0][0, 4]] == [2 * (g * 4) for g in range(8)]
+
+
+@pytest.mark.parametrize("mlwe_num", [4, 2, 1])
+def test_decompose_ring_identity(mlwe_num):
+    """b_m + sum_i a_{m,i} * s_i  ==  ringDown(a*s + b)[m*gap]  for every extracted MLWE sample m
+    (decryption convention m = a*s + b, Scheme_23.cuh:125-126; PCMM_Scheme.cuh:546-552)."""
+    N, N1, k = 32, 8, 4
+    qs = [65537, 0xfff9c0001]
+    ctx = make_small_ctx(qs)
+    pc = O.OraclePCMM(ctx, N1, k, [], qs)
+    rng = np.random.default_rng(mlwe_num)
+    rlwe = limbs_uniform(3, qs, 2, N)                     # [2][L+1][N] coefficient domain
+    s = [int(v) for v in rng.integers(-1, 2, N)]
+    mlwe = [np.zeros((2, k + 1, N1), dtype=np.uint64) for _ in range(mlwe_num)]
+    pc.rlweCipherDecompose(rlwe.reshape(-1), [m.reshape(-1) for m in mlwe], 1)
+    gap = k // mlwe_num
+    for im, q in enumerate(qs):
+        a = [int(v) for v in rlwe[0, im]]
+        b = [int(v) for v in rlwe[1, im]]
+        big = negacyclic_mul(a, [v % q for v in s], q)
+        big = [(x + y) % q for x, y in zip(big, b)]
+        s_down = ring_down([v % q for v in s], N, N1)
+        for m in range(mlwe_num):
+            acc = [int(v) for v in mlwe[m][im, k]]
+            for i in range(k):
+                pr = negacyclic_mul([int(v) for v in mlwe[m][im, i]], s_down[i], q)
+                acc = [(x + y) % q for x, y in zip(acc, pr)]
+            assert acc == ring_down(big, N, N1)[m * gap]
+
+
+@pytest.mark.parametrize("mod_num", [2, 3, 1])
+def test_ppmm_bruteforce(mod_num):
+    N1, k, M, Kin = 4, 3, 5, 6
+    qs = CFG2_Q[:mod_num]
+    ctx = make_small_ctx(qs, logN=5)
+    pc = O.OraclePCMM(ctx, N1, k, [CFG2_Q[5]], qs)
+    C = (k + 1) * N1
+    rng = np.random.default_rng(mod_num)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    W[0, 0] = 0.0                                           # exercises the A == 0 -> q mapping (PPMM_kernel.cuh:25)
+    scaler = float(2 ** 26)
+    mlwe = [limbs_uniform(10 + n, qs, 1, C)[0] for n in range(Kin)]      # [mod][C]
+    out = np.zeros((M, mod_num, C), dtype=np.uint64)
+    pc.PPMM(W, [m.reshape(-1) for m in mlwe], out.reshape(-1), M, Kin, mod_num, scaler)
+    A = [[int(float(W[m, n]) * scaler) for n in range(Kin)] for m in range(M)]     # trunc toward zero
+    qlast = qs[-1]
+    for m in range(M):
+        for c in range(C):
+            last = sum(A[m][n] * int(mlwe[n][mod_num - 1, c]) for n in range(Kin)) % qlast
+            assert int(out[m, mod_num - 1, c]) == last
+            for im in range(mod_num - 1):
+                q = qs[im]
+                r = sum(A[m][n] * int(mlwe[n][im, c]) for n in range(Kin)) % q
+                assert int(out[m, im, c]) == (r - last) * pow(qlast, -1, q) % q
+    # column panel restriction computes the same numbers
+    out2 = np.zeros_like(out)
+    pc.PPMM(W, [m.reshape(-1) for m in mlwe], out2.reshape(-1), M, Kin, mod_num, scaler, 4, 8)
+    assert np.array_equal(out2[:, :, 4:12], out[:, :, 4:12]) and not out2[:, :, :4].any() and not out2[:, :, 12:].any()
+
+
+def test_ppmm_rescale_is_rounding_division():
+    """Two primes (the reference's shape): the fused rescale returns the exact quotient (X - [X]_q1) / q1 of the
+    integer X that both residues represent, so the output decodes to about X / q1."""
+    N1, k, M, Kin = 4, 1, 2, 3
+    qs = CFG2_Q[:2]
+    ctx = make_small_ctx(qs, logN=5)
+    pc = O.OraclePCMM(ctx, N1, k, [CFG2_Q[5]], qs)
+    C = (k + 1) * N1
+    rng = np.random.default_rng(0)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    scaler = float(2 ** 20)
+    small = [rng.integers(-1000, 1000, C) for _ in range(Kin)]
+    mlwe = [np.array([[int(v) % q for v in small[n]] for q in qs], dtype=np.uint64) for n in range(Kin)]
+    out = np.zeros((M, 2, C), dtype=np.uint64)
+    pc.PPMM(W, [m.reshape(-1) for m in mlwe], out.reshape(-1), M, Kin, 2, scaler)
+    A = [[int(float(W[m, n]) * scaler) for n in range(Kin)] for m in range(M)]
+    for m in range(M):
+        for c in range(C):
+            X = sum(A[m][n] * int(small[n][c]) for n in range(Kin))
+            want = (X - (X % qs[1])) // qs[1]
+            assert int(out[m, 0, c]) == want % qs[0]
