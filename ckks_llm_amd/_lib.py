@@ -1,0 +1,80 @@
+"""ctypes loader of the HIP library.  Fails loudly when the library is missing: there is no fallback path."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libckks_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def build_library(force=True, jobs=8):
+    """Compiles every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+    import subprocess
+    cmd = ["make", "-C", CSRC, "-j%d" % jobs]
+    if force:
+        cmd.append("-B")
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+_lib = None
+u64p = C.POINTER(C.c_uint64)
+vp = C.c_void_p
+
+
+def _declare(L):
+    i, l, d, sz = C.c_int, C.c_long, C.c_double, C.c_size_t
+    S = {
+        "ckks_last_error": (C.c_char_p, []), "ckks_version": (C.c_char_p, []),
+        "ckks_malloc": (i, [C.POINTER(vp), sz]), "ckks_free": (i, [vp]),
+        "ckks_memcpy_h2d": (i, [vp, vp, sz]), "ckks_memcpy_d2h": (i, [vp, vp, sz]), "ckks_memcpy_d2d": (i, [vp, vp, sz]),
+        "ckks_memset": (i, [vp, i, sz]), "ckks_sync": (i, []), "ckks_device_count": (i, [C.POINTER(i)]),
+        "ckks_timer_start": (i, [vp]), "ckks_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
+        "ckks_ctx_create": (i, [C.POINTER(vp), i, u64p, i, u64p, i, u64p, i, i]), "ckks_ctx_destroy": (i, [vp]),
+        "ckks_set_stream": (i, [vp, vp]), "ckks_ctx_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
+        "ckks_ctx_set_arith_mode": (i, [vp, i]),
+        "ckks_ctx_table": (i, [vp, C.c_char_p, u64p, sz, C.POINTER(sz)]),
+        "ckks_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "ckks_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
+        "ckks_ntt_fwd_ext": (i, [vp, vp, i, i, i, i, i, i, i]), "ckks_ntt_inv_ext": (i, [vp, vp, i, i, i, i, i, i, i]),
+        "ckks_modup_pq_to_t": (i, [vp, vp, vp, i, i]), "ckks_modup_qj_to_t": (i, [vp, vp, vp, i, i]),
+        "ckks_modup_t_to_pql": (i, [vp, vp, vp, i, i]), "ckks_moddown_pql_to_ql": (i, [vp, vp, vp, i, i]),
+        "ckks_external_product_t": (i, [vp, vp, vp, vp, i]), "ckks_rescale": (i, [vp, vp, vp, i]),
+        "ckks_keyswitch_23": (i, [vp, vp, vp, vp, i, vp, vp, vp]),
+        "ckks_hybrid_modup": (i, [vp, vp, vp, i]), "ckks_hybrid_inner_product": (i, [vp, vp, vp, vp, i]),
+        "ckks_hybrid_moddown": (i, [vp, vp, vp, i]), "ckks_hybrid_keyswitch": (i, [vp, vp, vp, vp, i, vp]),
+        "pcmm_ctx_create": (i, [C.POINTER(vp), vp, i, i, u64p, i, u64p, i]), "pcmm_ctx_destroy": (i, [vp]),
+        "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),
+        "pcmm_rlwe_decompose_ntt": (i, [vp, vp, C.POINTER(vp), i, i]),
+        "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
+        "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
+    }
+    missing = []
+    for name, (res, args) in S.items():
+        try:
+            f = getattr(L, name)
+        except AttributeError:
+            missing.append(name)
+            continue
+        f.restype, f.argtypes = res, args
+    return missing
+
+
+EXPORTS = None
+
+
+def load_library():
+    """Returns the loaded library; raises LibraryMissing if it was not built (run __graft_entry__.build())."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise LibraryMissing("HIP library not built: %s (run `python -c 'import __graft_entry__ as g; g.build()'`)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        missing = _declare(L)
+        if missing:
+            raise LibraryMissing("libckks_hip.so lacks symbols: %s" % ", ".join(missing))
+        _lib = L
+    return _lib

@@ -1,0 +1,245 @@
+"""Host-side mirror of the reference's interface for the hot path (names, argument order and error behaviour of
+Context_23 / PCMM_Context / PCMM_Scheme), calling the HIP library through its C ABI.
+
+Polynomial arguments are DeviceBuffer objects or raw device addresses (ints, e.g. torch.Tensor.data_ptr()).
+"""
+import ctypes as C
+
+import numpy as np
+
+from ._lib import load_library, u64p, vp
+
+
+class CkksError(RuntimeError):
+    pass
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = load_library().ckks_last_error().decode()
+        if rc == -4:
+            raise ValueError(msg or what)          # std::invalid_argument of the reference (KeySwitch_23.cuh:194-201)
+        raise CkksError("%s failed (%d): %s" % (what, rc, msg))
+
+
+def _addr(x):
+    if isinstance(x, DeviceBuffer):
+        return x.ptr
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    return int(x)
+
+
+def _arr(v):
+    return np.ascontiguousarray(np.array(list(v), dtype=np.uint64))
+
+
+class DeviceBuffer:
+    """Owns one device allocation (the cudaMalloc'd member of Ciphertext / Plaintext / Key_decomp / MLWECiphertext,
+    Ciphertext.cuh:26-31,88-99)."""
+
+    def __init__(self, nbytes):
+        self.L_ = load_library()
+        self.nbytes = int(nbytes)
+        p = vp()
+        _check(self.L_.ckks_malloc(C.byref(p), max(self.nbytes, 8)), "ckks_malloc")
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        b.upload(a)
+        return b
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a)
+        assert a.nbytes <= self.nbytes
+        _check(self.L_.ckks_memcpy_h2d(self.ptr, a.ctypes.data, a.nbytes), "ckks_memcpy_h2d")
+
+    def download(self, dtype=np.uint64, count=None, offset_bytes=0):
+        item = np.dtype(dtype).itemsize
+        if count is None:
+            count = (self.nbytes - offset_bytes) // item
+        out = np.empty(count, dtype=dtype)
+        _check(self.L_.ckks_memcpy_d2h(out.ctypes.data, self.ptr + offset_bytes, out.nbytes), "ckks_memcpy_d2h")
+        return out
+
+    def zero(self):
+        _check(self.L_.ckks_memset(self.ptr, 0, self.nbytes), "ckks_memset")
+
+    def free(self):
+        if self.ptr:
+            self.L_.ckks_sync()
+            self.L_.ckks_free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context_23:
+    """Context_23 (Context_23.h:19-279) for the hot path, with explicit prime lists instead of a logN switch."""
+
+    def __init__(self, logN, p, q, t=(), gamma=0):
+        self.L_ = load_library()
+        self.logN, self.N = logN, 1 << logN
+        self.pVec, self.qVec, self.tVec = list(p), list(q), list(t)
+        self.p_num, self.q_num, self.t_num, self.gamma = len(self.pVec), len(self.qVec), len(self.tVec), gamma
+        self.K, self.L = self.p_num, self.q_num - 1
+        pa, qa, ta = _arr(p), _arr(q), _arr(t)
+        h = vp()
+        _check(self.L_.ckks_ctx_create(C.byref(h), logN, pa.ctypes.data_as(u64p), len(pa), qa.ctypes.data_as(u64p), len(qa),
+                                       ta.ctypes.data_as(u64p), len(ta), gamma), "ckks_ctx_create")
+        self.h = h.value
+        self.dnum = self.info("dnum")
+        self.Ri_blockNum = self.info("Ri_blockNum")
+        self.Qj_blockNum = self.info("Qj_blockNum")
+
+    def __del__(self):
+        try:
+            if self.h:
+                self.L_.ckks_ctx_destroy(self.h)
+                self.h = None
+        except Exception:
+            pass
+
+    def info(self, name):
+        v = C.c_long()
+        _check(self.L_.ckks_ctx_info(self.h, name.encode(), C.byref(v)), "ckks_ctx_info")
+        return v.value
+
+    def table(self, name):
+        n = C.c_size_t()
+        _check(self.L_.ckks_ctx_table(self.h, name.encode(), None, 0, C.byref(n)), "ckks_ctx_table")
+        out = np.zeros(n.value, dtype=np.uint64)
+        _check(self.L_.ckks_ctx_table(self.h, name.encode(), out.ctypes.data_as(u64p), n.value, None), "ckks_ctx_table")
+        return out
+
+    def set_arith_mode(self, mode):
+        _check(self.L_.ckks_ctx_set_arith_mode(self.h, mode), "ckks_ctx_set_arith_mode")
+
+    def set_stream(self, stream_handle):
+        _check(self.L_.ckks_set_stream(self.h, stream_handle), "ckks_set_stream")
+
+    def sync(self):
+        _check(self.L_.ckks_sync(), "ckks_sync")
+
+    def timer_start(self):
+        _check(self.L_.ckks_timer_start(self.h), "ckks_timer_start")
+
+    def timer_stop(self):
+        ms = C.c_float()
+        _check(self.L_.ckks_timer_stop(self.h, C.byref(ms)), "ckks_timer_stop")
+        return ms.value
+
+    # -- Context_23.h:42-45
+    def ToNTTInplace(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len):
+        _check(self.L_.ckks_ntt_fwd(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ckks_ntt_fwd")
+
+    def FromNTTInplace(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len):
+        _check(self.L_.ckks_ntt_inv(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ckks_ntt_inv")
+
+    def ToNTTInplace_for_externalProduct(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                         cipher_mod_num, batch_size):
+        _check(self.L_.ckks_ntt_fwd_ext(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                        cipher_mod_num, batch_size), "ckks_ntt_fwd_ext")
+
+    def FromNTTInplace_for_externalProduct(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                           cipher_mod_num, batch_size):
+        _check(self.L_.ckks_ntt_inv_ext(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                        cipher_mod_num, batch_size), "ckks_ntt_inv_ext")
+
+    # -- Context_23.h:54-61
+    def modUpPQtoT_23(self, output, input, l, batch_size):
+        _check(self.L_.ckks_modup_pq_to_t(self.h, _addr(output), _addr(input), l, batch_size), "ckks_modup_pq_to_t")
+
+    def modUpQjtoT_23(self, output, input, l, batch_size):
+        _check(self.L_.ckks_modup_qj_to_t(self.h, _addr(output), _addr(input), l, batch_size), "ckks_modup_qj_to_t")
+
+    def modUpTtoPQl_23(self, modUp_TtoQj_buffer, exProduct_T_temp, l, batch_size):
+        _check(self.L_.ckks_modup_t_to_pql(self.h, _addr(modUp_TtoQj_buffer), _addr(exProduct_T_temp), l, batch_size), "ckks_modup_t_to_pql")
+
+    def modDownPQltoQl_23(self, output, modUp_TtoQj_buffer, l, batch_size):
+        _check(self.L_.ckks_moddown_pql_to_ql(self.h, _addr(output), _addr(modUp_TtoQj_buffer), l, batch_size), "ckks_moddown_pql_to_ql")
+
+    def external_product_T(self, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l):
+        _check(self.L_.ckks_external_product_t(self.h, _addr(output), _addr(cipher_modUp_QjtoT), _addr(swk_modUp_RitoT), l), "ckks_external_product_t")
+
+    def rescaleAndEqual(self, cipher, scratch, l):
+        _check(self.L_.ckks_rescale(self.h, _addr(cipher), _addr(scratch), l), "ckks_rescale")
+
+    def keyswitch_23(self, out, d2, swk, l, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer):
+        _check(self.L_.ckks_keyswitch_23(self.h, _addr(out), _addr(d2), _addr(swk), l, _addr(modUp_QjtoT_temp),
+                                         _addr(exProduct_T_temp), _addr(modUp_TtoQj_buffer)), "ckks_keyswitch_23")
+
+    # -- textbook hybrid key switch (no reference counterpart)
+    def hybrid_modup(self, digits, in_coeff, l):
+        _check(self.L_.ckks_hybrid_modup(self.h, _addr(digits), _addr(in_coeff), l), "ckks_hybrid_modup")
+
+    def hybrid_inner_product(self, ip, digits_ntt, evk, l):
+        _check(self.L_.ckks_hybrid_inner_product(self.h, _addr(ip), _addr(digits_ntt), _addr(evk), l), "ckks_hybrid_inner_product")
+
+    def hybrid_moddown(self, out, in_pq, l):
+        _check(self.L_.ckks_hybrid_moddown(self.h, _addr(out), _addr(in_pq), l), "ckks_hybrid_moddown")
+
+    def hybrid_keyswitch(self, out, in_ntt, evk, l, scratch):
+        _check(self.L_.ckks_hybrid_keyswitch(self.h, _addr(out), _addr(in_ntt), _addr(evk), l, _addr(scratch)), "ckks_hybrid_keyswitch")
+
+
+class PCMM_Context:
+    """PCMM_Context (pcmm/PCMM_Context.h:14-90)."""
+
+    def __init__(self, N1, mlwe_rank, p_ringpack, q_ringpack, context):
+        self.L_ = load_library()
+        self.context, self.N1, self.mlwe_rank = context, N1, mlwe_rank
+        self.p_ringpack, self.q_ringpack = list(p_ringpack), list(q_ringpack)
+        pa, qa = _arr(p_ringpack), _arr(q_ringpack)
+        h = vp()
+        _check(self.L_.pcmm_ctx_create(C.byref(h), context.h, N1, mlwe_rank, pa.ctypes.data_as(u64p), len(pa),
+                                       qa.ctypes.data_as(u64p), len(qa)), "pcmm_ctx_create")
+        self.h = h.value
+
+    def __del__(self):
+        try:
+            if self.h:
+                self.L_.pcmm_ctx_destroy(self.h)
+                self.h = None
+        except Exception:
+            pass
+
+
+class PCMM_Scheme:
+    """The rlweCipherDecompose / PPMM members of PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48)."""
+
+    def __init__(self, pcmm_context):
+        self.L_ = load_library()
+        self.pcmm_context = pcmm_context
+
+    @staticmethod
+    def _ptrs(bufs):
+        T = vp * len(bufs)
+        return T(*[_addr(b) for b in bufs])
+
+    def rlweCipherDecompose(self, rlwe_cipher, mlwe_cipher_decomposed, mlwe_num, offset, l, coeff_domain=False):
+        """PCMM_Scheme.cuh:90-125.  rlwe_cipher: [a | b] device buffer at level l; coeff_domain=True runs the gather only."""
+        bufs = mlwe_cipher_decomposed[offset:offset + mlwe_num]
+        f = self.L_.pcmm_rlwe_decompose if coeff_domain else self.L_.pcmm_rlwe_decompose_ntt
+        _check(f(self.pcmm_context.h, _addr(rlwe_cipher), self._ptrs(bufs), mlwe_num, l), "pcmm_rlwe_decompose")
+
+    def PPMM(self, plain_mat, mlwe_cipher_decomposed, out, mat_M, mat_N, mat_K, mlwe_num, mod_num, scaler):
+        """PPMM_kernel.cuh:254-349 (device part).  Shape errors are reported the way the reference does: a message and no
+        work (PPMM_kernel.cuh:256-263), here as ValueError."""
+        if mat_K != self.pcmm_context.N1:
+            raise ValueError("matrix K should be equal to N1!")
+        if mat_N != mlwe_num:
+            raise ValueError("matrix N should be equal to mlwe number!")
+        _check(self.L_.pcmm_ppmm(self.pcmm_context.h, _addr(plain_mat), self._ptrs(mlwe_cipher_decomposed[:mlwe_num]), _addr(out),
+                                 mat_M, mat_N, mod_num, float(scaler)), "pcmm_ppmm")
+
+    def PPMM_strided(self, plain_mat, mlwe_all, out, mat_M, mat_N, mod_num, scaler):
+        _check(self.L_.pcmm_ppmm_strided(self.pcmm_context.h, _addr(plain_mat), _addr(mlwe_all), _addr(out), mat_M, mat_N,
+                                         mod_num, float(scaler)), "pcmm_ppmm_strided")

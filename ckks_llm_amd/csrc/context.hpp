@@ -1,0 +1,93 @@
+// Internal definition of the context handle shared by the kernels' launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include <vector>
+
+#include "../../include/ckks_hip.h"
+#include "modarith.hpp"
+
+namespace ckks {
+
+// per-prime constants in device memory, indexed in pqt order
+struct PrimeConst {
+    u64 q, mu_hi, mu_lo;
+    u64 n_inv, n_inv_s;          // N^-1 and its Shoup word
+    u64 w1n, w1n_s;              // psiinv_table[1] (which already carries N^-1, Utils.cuh:200) and its Shoup word
+    double qd, qinv_d;           // (double)q and 1/q for the FP64 back end
+    double n_inv_d, w1n_d;       // balanced representatives of n_inv, w1n as doubles
+    int f64_ok;                  // prime small enough for the FP64 back end
+    int pad;
+};
+
+// one block of an exact RNS conversion (BasisConv.cuh:18-58): nsrc source primes -> ntgt target primes
+constexpr int CONV_MAX_SRC = 16;
+constexpr int CONV_MAX_TGT = 32;
+struct ConvBlock {
+    int nsrc, ntgt;
+    short src_prime[CONV_MAX_SRC], src_limb[CONV_MAX_SRC];
+    short tgt_prime[CONV_MAX_TGT], tgt_limb[CONV_MAX_TGT];
+    u64 hatinv[CONV_MAX_SRC], hatinv_s[CONV_MAX_SRC];   // (D/d_j)^-1 mod d_j
+    u64 hat[CONV_MAX_TGT][CONV_MAX_SRC];                // (D/d_j) mod r_k
+    u64 dmod[CONV_MAX_TGT];                             // D mod r_k
+    u64 add_in[CONV_MAX_SRC];                           // added to the input residue before scaling (T -> PQ centring)
+    u64 sub_out[CONV_MAX_TGT];                          // subtracted from the output residue (T -> PQ centring)
+    short copy_prime[CONV_MAX_SRC], copy_limb[CONV_MAX_SRC];  // ncopy source limbs passed through unchanged
+    int ncopy, pad;
+};
+
+struct ConvPlan {          // blocks of one map at one level, contiguous in device memory
+    int first = 0, count = 0;
+};
+
+}  // namespace ckks
+
+struct ckks_ctx {
+    int logN = 0, p_num = 0, q_num = 0, t_num = 0, gamma = 0, L = 0, K = 0, dnum = 0;
+    int Ri_blockNum = 0, Qj_blockNum = 0, nprimes = 0;
+    long N = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+
+    // host copies (reference names, reference layouts) for ckks_ctx_table and for launch-time decisions
+    std::vector<uint64_t> pqt, mu_hi, mu_lo, psi, psiinv, n_inv, n_inv_shoup, halfTmodpqti;
+    std::vector<uint64_t> psi_table, psiinv_table;                       // [prime][N]
+    std::vector<uint64_t> pHatVecModq, pHatInvVecModp, PModqt, PinvModq;
+    std::vector<uint64_t> RiHatInv, RiHatModT, Rimodti;
+    std::vector<uint64_t> QjHatInv, QjHatModT, Qjmodti;
+    std::vector<uint64_t> THatInv, THatModRi, Tmodpqi;
+    std::vector<uint64_t> qiInvModql;
+    std::vector<int> f64_ok;
+
+    // device tables
+    ckks::PrimeConst* d_primes = nullptr;
+    ulonglong2* d_tw_fwd = nullptr;       // [prime][N] (w, shoup(w)), index = reference psi_table index
+    ulonglong2* d_tw_inv = nullptr;       // [prime][N] from psiinv_table
+    double* d_twd_fwd = nullptr;          // [prime][N] balanced doubles, FP64 back end (0 entries for large primes)
+    double* d_twd_inv = nullptr;
+    ckks::ConvBlock* d_conv = nullptr;    // all conversion blocks
+    std::vector<ckks::ConvPlan> plan_pq_to_t, plan_qj_to_t, plan_t_to_pq, plan_hybrid;   // indexed by level l
+    // ModDown / rescale constants on device
+    uint64_t* d_pHatVecModq = nullptr;    // [L+1][K]
+    uint64_t* d_pHatInvVecModp = nullptr; // [K] then [K] Shoup words
+    uint64_t* d_PinvModq = nullptr;       // [L+1] then [L+1] Shoup words
+    uint64_t* d_qiInvModql = nullptr;     // triangular (+ Shoup words after)
+    size_t qiInv_count = 0;
+
+    int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
+};
+
+namespace ckks {
+void set_error(const std::string& s);
+int hip_fail(hipError_t e, const char* what);
+#define CKKS_HIP_TRY(expr)                                   \
+    do {                                                     \
+        hipError_t _e = (expr);                              \
+        if (_e != hipSuccess) return ckks::hip_fail(_e, #expr); \
+    } while (0)
+
+// launchers (ntt.hip, basisconv.hip)
+int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+               int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
+}  // namespace ckks

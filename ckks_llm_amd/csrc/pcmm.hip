@@ -1,0 +1,300 @@
+// Ring-packed plaintext x ciphertext matrix product (PPMM) and the RLWE -> MLWE gather for gfx950.
+//
+// Replaces PCMM_Context (pcmm/PCMM_Context.cuh:7-57), the gather kernel of PCMM_Scheme::rlweCipherDecompose
+// (pcmm/PCMM_Scheme.cuh:50-125) and pcmm_cuda_core_kernel / PCMM_Scheme::PPMM (pcmm/PPMM_kernel.cuh:93-349).
+//
+// PPMM semantics (per ring-pack prime q_i, i = mod_num-1 .. 0; C = (rank+1)*N1 columns):
+//     A[m][n]   = (int64) ((double) W[m][n] * scaler)                     truncation toward zero  (PPMM_kernel.cuh:148)
+//     r_i[m][c] = sum_n A[m][n] * Ct_n[i][c]  mod q_i                     (the reference maps A <= 0 to q + A, :25)
+//     out[m][last][c] = r_last ;  out[m][i][c] = (r_i + q_i - r_last) * q_last^-1 mod q_i   (fused rescale, :213-249)
+// The reference fixes mod_num = 2 (its rescale table offset is hard-wired to l = 1, :298); this implementation takes
+// any mod_num >= 1 and uses q_last^-1 mod q_i, which is the same constant when mod_num = 2.
+//
+// Two kernels compute it:
+//   * ppmm_mfma_kernel  - the dense path.  A is split once into DW balanced base-256 digits (int8 planes shared by
+//     all primes); residues are split on the fly into DC balanced digits (bytes of x + 0x80..80, each xor 0x80) while
+//     they are staged into LDS; v_mfma_i32_16x16x64_i8 accumulates the DW*DC digit products into DW+DC-1 int32
+//     anti-diagonal accumulators; the epilogue recombines them exactly and reduces modulo q_i.
+//   * ppmm_generic_kernel - one output per lane with 128-bit accumulation, for shapes the MFMA tiling does not cover
+//     (C not a multiple of 64, primes of 41 bits and more, |A| >= 2^31).
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "context.hpp"
+#include "host_math.hpp"
+
+struct pcmm_ctx {
+    ckks_ctx* ctx = nullptr;
+    int N1 = 0, rank = 0, np = 0, nq = 0;
+    std::vector<uint64_t> pq;
+    ckks::PrimeConst* d_pq = nullptr;        // ring-pack primes [p_ringpack | q_ringpack]
+    uint64_t** d_ptrs = nullptr;             // device copy of the caller's MLWE pointer table (PCMM_Scheme.cuh:16-18)
+    int ptr_cap = 0;
+    // workspace of the quantised plaintext matrix
+    long long* d_A = nullptr;                // [M][Kin] int64
+    int8_t* d_Adig = nullptr;                // [DW][Mpad][Kpad] balanced digits
+    size_t A_cap = 0, Adig_cap = 0;
+    unsigned long long* d_absmax = nullptr;
+};
+
+namespace ckks {
+
+// ------------------------------------------------------------------------------------------------------------
+// RLWE -> MLWE gather (PCMM_Scheme.cuh:50-88)
+// ------------------------------------------------------------------------------------------------------------
+struct GatherArgs {
+    const u64* rlwe;
+    u64* const* mlwe;
+    const PrimeConst* primes;   // context primes
+    long N;
+    int N1, rank, mlwe_num, L, p_num;
+};
+__global__ __launch_bounds__(256) void rlwe_gather_kernel(GatherArgs a) {
+    // one lane per output word: flat index over (row i in [0, rank], g in [0, N1))
+    const long flat = (long)blockIdx.x * 256 + threadIdx.x;
+    const int k = a.rank, N1 = a.N1;
+    if (flat >= (long)(k + 1) * N1) return;
+    const int i = (int)(flat / N1), g = (int)(flat % N1);
+    const int im = blockIdx.y, m = blockIdx.z;
+    const u64 q = a.primes[a.p_num + im].q;
+    const u64* A = a.rlwe + a.N * im;
+    const u64* B = a.rlwe + a.N * (a.L + 1 + im);
+    u64* dst = a.mlwe[m] + (long)N1 * (k + 1) * im;
+    const int gap = k / a.mlwe_num;
+    u64 v;
+    if (i == k) {                                           // b row
+        long addr = (long)m * gap + (long)g * k;
+        v = addr >= a.N ? negate_mod(B[addr - a.N], q) : B[addr];
+    } else if (i == 0) {
+        long addr = (long)m * gap + (long)g * k;
+        v = addr >= a.N ? negate_mod(A[addr - a.N], q) : A[addr];
+    } else if (g == 0) {
+        long addr = (long)(N1 - 1) * k + (k - i) + (long)m * gap;
+        v = addr >= a.N ? A[addr - a.N] : negate_mod(A[addr], q);
+    } else {
+        long addr = (long)(g - 1) * k + (k - i) + (long)m * gap;
+        v = addr >= a.N ? negate_mod(A[addr - a.N], q) : A[addr];
+    }
+    dst[(long)i * N1 + g] = v;
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// plaintext quantisation: A = (int64)(float * double), |A| maximum, balanced base-256 digit planes
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void quantise_kernel(const float* W, long long* A, unsigned long long* absmax, long count, double scaler) {
+    long i = (long)blockIdx.x * 256 + threadIdx.x;
+    unsigned long long m = 0;
+    if (i < count) {
+        long long v = (long long)((double)W[i] * scaler);
+        A[i] = v;
+        m = (unsigned long long)(v < 0 ? -v : v);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        unsigned long long o = __shfl_down(m, off);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m) atomicMax(absmax, m);
+}
+// digit d of A (balanced, in [-128, 127]): byte d of (A + 0x80..80) xor 0x80
+__global__ __launch_bounds__(256) void digits_kernel(const long long* A, int8_t* dig, int M, int Kin, int Mpad, int Kpad, int DW) {
+    long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)Mpad * Kpad) return;
+    int m = (int)(i / Kpad), n = (int)(i % Kpad);
+    unsigned long long biased = 0x8080808080808080ull;
+    if (m < M && n < Kin) biased += (unsigned long long)A[(long)m * Kin + n];
+    for (int d = 0; d < DW; d++) dig[(long)d * Mpad * Kpad + i] = (int8_t)(((biased >> (8 * d)) & 0xff) ^ 0x80);
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// generic kernel: one output per lane, 128-bit accumulation (the reference's arithmetic, PPMM_kernel.cuh:12-31)
+// ------------------------------------------------------------------------------------------------------------
+struct PpmmArgs {
+    const long long* A;           // [M][Kin]
+    const int8_t* Adig;           // [DW][Mpad][Kpad]
+    const u64* const* mlwe;       // Kin pointers (nullptr when strided)
+    const u64* mlwe_base;         // strided operand
+    long mlwe_stride;             // words between consecutive MLWE ciphertexts
+    u64* out;
+    const PrimeConst* pq;         // ring-pack primes, q part starts at np
+    const u64* qlast_inv;         // [mod_num] (q_last^-1 mod q_i), then Shoup words
+    long C;
+    int M, Kin, Mpad, Kpad, mod_num, np;
+};
+__device__ __forceinline__ const u64* mlwe_row(const PpmmArgs& a, int n) {
+    return a.mlwe ? a.mlwe[n] : a.mlwe_base + (long)n * a.mlwe_stride;
+}
+__global__ __launch_bounds__(256) void ppmm_generic_kernel(PpmmArgs a) {
+    const long c = (long)blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (c >= a.C) return;
+    u64* o = a.out + (long)m * a.C * a.mod_num;
+    u64 r_last = 0;
+    for (int im = a.mod_num - 1; im >= 0; im--) {
+        const PrimeConst& pr = a.pq[a.np + im];
+        u128w acc = {0, 0};
+        for (int n = 0; n < a.Kin; n++) {
+            long long t = a.A[(long)m * a.Kin + n];
+            u64 w = t > 0 ? (u64)t : pr.q + (u64)t;                       // PPMM_kernel.cuh:25
+            mac128(acc, w, mlwe_row(a, n)[(long)im * a.C + c]);
+        }
+        u64 r = barrett128(acc, pr.q, pr.mu_hi, pr.mu_lo);
+        if (im == a.mod_num - 1) {
+            r_last = r;
+            o[(long)im * a.C + c] = r;
+        } else {
+            u64 temp = r + pr.q - r_last;                                   // :244
+            o[(long)im * a.C + c] = mul_shoup(temp, a.qlast_inv[im], a.qlast_inv[a.mod_num + im], pr.q);
+        }
+    }
+}
+
+}  // namespace ckks
+
+using namespace ckks;
+namespace H = ckks_host;
+
+extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, const uint64_t* p, int np, const uint64_t* q, int nq) {
+    if (!out || !ctx || N1 <= 0 || rank <= 0 || nq < 1 || np < 0 || (np > 0 && !p) || !q) { set_error("pcmm_ctx_create: bad argument"); return CKKS_E_INVALID; }
+    if ((long)N1 * rank != ctx->N) { set_error("pcmm_ctx_create: N1 * mlwe_rank must equal N"); return CKKS_E_INVALID; }
+    pcmm_ctx* h = new pcmm_ctx();
+    h->ctx = ctx; h->N1 = N1; h->rank = rank; h->np = np; h->nq = nq;
+    for (int i = 0; i < np; i++) h->pq.push_back(p[i]);
+    for (int i = 0; i < nq; i++) h->pq.push_back(q[i]);
+    std::vector<PrimeConst> pc(h->pq.size());
+    for (size_t i = 0; i < h->pq.size(); i++) {
+        uint64_t m = h->pq[i];
+        if (m < 3 || (m & 1) == 0 || m >= (1ull << 62)) { delete h; set_error("pcmm_ctx_create: moduli must be odd and < 2^62"); return CKKS_E_INVALID; }
+        PrimeConst& P = pc[i];
+        memset(&P, 0, sizeof(P));
+        uint64_t hi, lo;
+        H::barrett_mu(m, hi, lo);
+        P.q = m; P.mu_hi = hi; P.mu_lo = lo; P.qd = (double)m; P.qinv_d = 1.0 / (double)m; P.f64_ok = m < (1ull << 41);
+    }
+    hipError_t e = hipMalloc((void**)&h->d_pq, pc.size() * sizeof(PrimeConst));
+    if (e == hipSuccess) e = hipMemcpy(h->d_pq, pc.data(), pc.size() * sizeof(PrimeConst), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void**)&h->d_absmax, sizeof(unsigned long long) + 2 * 64 * sizeof(uint64_t));
+    if (e != hipSuccess) { pcmm_ctx_destroy(h); return hip_fail(e, "pcmm_ctx_create"); }
+    *out = h;
+    return CKKS_OK;
+}
+extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
+    if (!h) return CKKS_OK;
+    (void)hipDeviceSynchronize();
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax};
+    for (void* p : ptrs) if (p) (void)hipFree(p);
+    delete h;
+    return CKKS_OK;
+}
+
+static int upload_ptrs(pcmm_ctx* h, const uint64_t* const* host_ptrs, int count) {
+    if (count > h->ptr_cap) {
+        if (h->d_ptrs) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_ptrs); h->d_ptrs = nullptr; }
+        int cap = std::max(count, 3072);                                   // PCMM_Scheme.cuh:16-18 sizes its table for 3072
+        CKKS_HIP_TRY(hipMalloc((void**)&h->d_ptrs, (size_t)cap * sizeof(uint64_t*)));
+        h->ptr_cap = cap;
+    }
+    CKKS_HIP_TRY(hipMemcpyAsync(h->d_ptrs, host_ptrs, (size_t)count * sizeof(uint64_t*), hipMemcpyHostToDevice, h->ctx->stream));
+    return CKKS_OK;
+}
+
+extern "C" int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l) {
+    if (!h || !rlwe || !mlwe_ptrs_host) return CKKS_E_INVALID;
+    ckks_ctx* c = h->ctx;
+    if (mlwe_num > h->rank) { set_error("rlweCipherDecompose extract number must be <= mlwe_rank"); return CKKS_E_INVALID; }   // PCMM_Scheme.cuh:103-106
+    if (mlwe_num <= 0 || l < 0 || l > c->L) { set_error("rlweCipherDecompose: bad mlwe_num or level"); return CKKS_E_INVALID; }
+    int rc = upload_ptrs(h, mlwe_ptrs_host, mlwe_num);
+    if (rc) return rc;
+    GatherArgs a;
+    a.rlwe = rlwe; a.mlwe = h->d_ptrs; a.primes = c->d_primes; a.N = c->N; a.N1 = h->N1; a.rank = h->rank; a.mlwe_num = mlwe_num;
+    a.L = c->L; a.p_num = c->p_num;
+    long per = (long)(h->rank + 1) * h->N1;
+    dim3 grid((unsigned)((per + 255) / 256), l + 1, mlwe_num), block(256);
+    hipLaunchKernelGGL(rlwe_gather_kernel, grid, block, 0, c->stream, a);
+    CKKS_HIP_TRY(hipGetLastError());
+    // the pointer table was copied asynchronously from the caller's host array: make sure it is consumed before returning
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
+    return CKKS_OK;
+}
+extern "C" int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l) {
+    if (!h || !rlwe) return CKKS_E_INVALID;
+    ckks_ctx* c = h->ctx;
+    if (l < 0 || l > c->L) { set_error("rlweCipherDecompose: bad level"); return CKKS_E_INVALID; }
+    int rc = launch_ntt(c, rlwe, 0, c->K, 2, l + 1, c->L + 1, 0, 1, true);             // PCMM_Scheme.cuh:107
+    if (rc) return rc;
+    if ((rc = pcmm_rlwe_decompose(h, rlwe, mlwe_ptrs_host, mlwe_num, l))) return rc;
+    return launch_ntt(c, rlwe, 0, c->K, 2, l + 1, c->L + 1, 0, 1, false);              // :124
+}
+
+namespace ckks { int launch_ppmm_mfma(pcmm_ctx* h, const PpmmArgs& a, int DW, int DC); }
+
+static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
+                       int M, int Kin, int mod_num, double scaler) {
+    if (!h || !W || !out || (!ptrs_host && !strided)) return CKKS_E_INVALID;
+    if (M <= 0 || Kin <= 0 || mod_num < 1 || mod_num > h->nq || mod_num > 64) { set_error("PPMM: bad shape or mod_num"); return CKKS_E_INVALID; }
+    ckks_ctx* c = h->ctx;
+    const long C = (long)(h->rank + 1) * h->N1;
+    int rc;
+    if (ptrs_host && (rc = upload_ptrs(h, ptrs_host, Kin))) return rc;
+    // workspace
+    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 63) / 64 * 64;
+    size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
+    if (needA > h->A_cap) {
+        if (h->d_A) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_A); h->d_A = nullptr; }
+        CKKS_HIP_TRY(hipMalloc((void**)&h->d_A, needA * sizeof(long long)));
+        h->A_cap = needA;
+    }
+    if (needD > h->Adig_cap) {
+        if (h->d_Adig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Adig); h->d_Adig = nullptr; }
+        CKKS_HIP_TRY(hipMalloc((void**)&h->d_Adig, needD));
+        h->Adig_cap = needD;
+    }
+    // q_last^-1 mod q_i and Shoup words, kept behind the |A| maximum word
+    std::vector<uint64_t> inv(2 * 64, 0);
+    const uint64_t qlast = h->pq[h->np + mod_num - 1];
+    uint64_t qmax = 0;
+    for (int i = 0; i < mod_num; i++) {
+        uint64_t qi = h->pq[h->np + i];
+        qmax = std::max(qmax, qi);
+        if (i < mod_num - 1) { inv[i] = H::invmod(qlast % qi, qi); inv[mod_num + i] = H::shoup(inv[i], qi); }
+    }
+    uint64_t* d_inv = (uint64_t*)(h->d_absmax + 1);
+    CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
+    CKKS_HIP_TRY(hipMemcpyAsync(d_inv, inv.data(), 2 * mod_num * sizeof(uint64_t), hipMemcpyHostToDevice, c->stream));
+    long count = (long)M * Kin;
+    hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, c->stream, W, h->d_A, h->d_absmax, count, scaler);
+    unsigned long long absmax = 0;
+    CKKS_HIP_TRY(hipMemcpyAsync(&absmax, h->d_absmax, sizeof(absmax), hipMemcpyDeviceToHost, c->stream));
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
+
+    PpmmArgs a;
+    a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = ptrs_host ? (const u64* const*)h->d_ptrs : nullptr; a.mlwe_base = strided;
+    a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.qlast_inv = d_inv; a.C = C; a.M = M; a.Kin = Kin;
+    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np;
+
+    // digit counts: DW digits cover |A| < 2^(8*DW-1); DC digits cover residues < 2^(8*DC-1)
+    int DW = 1; while (DW < 8 && absmax >= (1ull << (8 * DW - 1))) DW++;
+    int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;
+    static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
+    const bool mfma_ok = !force_generic && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
+                         (long)Kpad * 16384 * std::min(DW, DC) < (1l << 31) && absmax < qmax;
+    if (mfma_ok) {
+        long total = (long)Mpad * Kpad;
+        hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
+        rc = launch_ppmm_mfma(h, a, DW, DC);
+        if (rc) return rc;
+    } else {
+        dim3 grid((unsigned)((C + 255) / 256), M), block(256);
+        hipLaunchKernelGGL(ppmm_generic_kernel, grid, block, 0, c->stream, a);
+    }
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+
+extern "C" int pcmm_ppmm(pcmm_ctx* h, const float* W, const uint64_t* const* mlwe_ptrs_host, uint64_t* out, int M, int Kin, int mod_num, double scaler) {
+    return ppmm_common(h, W, mlwe_ptrs_host, nullptr, out, M, Kin, mod_num, scaler);
+}
+extern "C" int pcmm_ppmm_strided(pcmm_ctx* h, const float* W, const uint64_t* mlwe, uint64_t* out, int M, int Kin, int mod_num, double scaler) {
+    return ppmm_common(h, W, nullptr, mlwe, out, M, Kin, mod_num, scaler);
+}

@@ -1,0 +1,132 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of the CKKS arithmetic hot path:
+ * batched RNS negacyclic NTT / iNTT, RNS basis conversion for key switching, and the ring-packed
+ * plaintext x ciphertext matrix product (PPMM).
+ *
+ * The reference (haozetao/ckks_llm) has no FFI layer: its boundary for this path is a set of C++ member
+ * functions compiled into the caller.  Each entry point below replaces one of them and cites it; argument
+ * order and meaning follow the reference.  All polynomial pointers are DEVICE pointers to uint64_t in the
+ * reference's limb-major layout (limb = N consecutive words of one polynomial modulo one prime); prime
+ * indices are in "pqt order" [p_0..p_{K-1} | q_0..q_L | t_0..t_{tnum-1}] (Context_23.cuh:63-113).
+ *
+ * Every function returns 0 on success or a negative CKKS_E_* code; ckks_last_error() gives the text.
+ * A handle owns its device tables (the reference keeps them in process-global __constant__ symbols, so it can
+ * hold one context per process; here any number of contexts may coexist).  Work is issued on the stream set
+ * with ckks_set_stream (default: the null stream); calls on one handle from several host threads must be
+ * serialised by the caller, as in the reference.
+ */
+#ifndef CKKS_HIP_H
+#define CKKS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CKKS_OK 0
+#define CKKS_E_INVALID (-1)   /* bad argument (level, shape, unsupported size) */
+#define CKKS_E_HIP (-2)       /* a HIP runtime call failed */
+#define CKKS_E_NOMEM (-3)
+#define CKKS_E_STATE (-4)     /* e.g. missing key / level-0 operand: the C++ shell maps it to std::invalid_argument */
+
+typedef struct ckks_ctx ckks_ctx;
+typedef struct pcmm_ctx pcmm_ctx;
+
+const char* ckks_last_error(void);
+const char* ckks_version(void);
+
+/* ---- device memory and stream plumbing (cudaMalloc / cudaMemcpy / cudaDeviceSynchronize of the reference) ---- */
+int ckks_malloc(void** dev_ptr, size_t bytes);
+int ckks_free(void* dev_ptr);
+int ckks_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes);
+int ckks_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes);
+int ckks_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes);
+int ckks_memset(void* dst_dev, int value, size_t bytes);
+int ckks_sync(void);
+int ckks_device_count(int* count);
+/* HIP-event timing on the context's stream (replaces CUDATimer, TimeUtils.cuh:10-35) */
+int ckks_timer_start(ckks_ctx* ctx);
+int ckks_timer_stop(ckks_ctx* ctx, float* elapsed_ms);
+
+/* ---- context: Context_23::Context_23 + getPrimeCKKS + preComputeOnCPU + copyMemoryToGPU
+ *      (Context_23.cuh:12-472, 475-701; Params.cuh).  Primes are passed explicitly; gamma is the block width of
+ *      the [P|Q] -> T conversion (Params.cuh "gamma").  t_num may be 0 (no auxiliary basis), p_num may be 0. ---- */
+int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int p_num, const uint64_t* q, int q_num,
+                    const uint64_t* t, int t_num, int gamma);
+int ckks_ctx_destroy(ckks_ctx* ctx);
+int ckks_set_stream(ckks_ctx* ctx, void* hip_stream);
+/* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum" */
+int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
+/* host copy of a constant table, flattened in the reference's device layout (names as in ckks_oracle.h /
+ * Context_23.h: "pqt","psi","psi_table","psiinv_table","RiHatInv","QjHatModT",...). *count receives the length. */
+int ckks_ctx_table(const ckks_ctx* ctx, const char* name, uint64_t* host_out, size_t cap, size_t* count);
+
+/* ---- NTT: Context_23::ToNTTInplace / FromNTTInplace (Context_23.cuh:847-889; kernels ntt_60bit.cuh:421-901).
+ * Limb (y, j), y < poly_num, j < mod_num, lives at dev + (y*poly_mod_len + start_poly_idx + j)*N and is
+ * transformed modulo prime start_mod_idx + j.  Forward: natural -> bit-reversed order; inverse: bit-reversed ->
+ * natural order, scaled by N^-1.  Outputs are fully reduced. ---- */
+int ckks_ntt_fwd(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                 int poly_mod_len);
+int ckks_ntt_inv(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                 int poly_mod_len);
+/* Context_23::ToNTTInplace_for_externalProduct / FromNTTInplace_for_externalProduct (Context_23.cuh:891-930):
+ * same, repeated batch_size times with a stride of cipher_mod_num limbs. */
+int ckks_ntt_fwd_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                     int poly_mod_len, int cipher_mod_num, int batch_size);
+int ckks_ntt_inv_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                     int poly_mod_len, int cipher_mod_num, int batch_size);
+
+/* ---- basis conversion: Context_23::modUpPQtoT_23 / modUpQjtoT_23 / modUpTtoPQl_23 / modDownPQltoQl_23
+ *      (BasisConv.cuh:61-77, 161-179, 243-254, 328-347; strides as indexed at :25,:52,:110,:142,:201,:239,:304,:325) ---- */
+int ckks_modup_pq_to_t(ckks_ctx* ctx, uint64_t* out, const uint64_t* in, int l, int batch_size);
+int ckks_modup_qj_to_t(ckks_ctx* ctx, uint64_t* out, const uint64_t* in, int l, int batch_size);
+int ckks_modup_t_to_pql(ckks_ctx* ctx, uint64_t* buf, const uint64_t* in, int l, int batch_size);
+int ckks_moddown_pql_to_ql(ckks_ctx* ctx, uint64_t* out, const uint64_t* buf, int l, int batch_size);
+/* Context_23::external_product_T (ExternalProduct.cuh:85-97); swk laid out as Key_decomp (Key_decomp.cuh:19-24) */
+int ckks_external_product_t(ckks_ctx* ctx, uint64_t* out, const uint64_t* c_T, const uint64_t* swk_T, int l);
+/* Scheme_23::rescaleAndEqual (Scheme_23.cuh:369-385): cipher = [a: L+1 limbs | b: L+1 limbs], level l -> l-1.
+ * scratch: 2*(L+1)*N words (Scheme_23::rescale_buffer). */
+int ckks_rescale(ckks_ctx* ctx, uint64_t* cipher, uint64_t* scratch, int l);
+/* steps 2..9 of Scheme_23::mult_23 (KeySwitch_23.cuh:219-231): d2 (NTT domain, L+1 limbs, overwritten with its
+ * coefficient form) -> out = [a | b] (NTT domain).  Scratch buffers are the reference's
+ * modUp_QjtoT_temp (N*t_num*Qj_blockNum), exProduct_T_temp and modUp_TtoQj_buffer (N*t_num*Ri_blockNum*2 each). */
+int ckks_keyswitch_23(ckks_ctx* ctx, uint64_t* out, uint64_t* d2, const uint64_t* swk_T, int l,
+                      uint64_t* modUp_QjtoT_temp, uint64_t* exProduct_T_temp, uint64_t* modUp_TtoQj_buffer);
+
+/* ---- textbook hybrid key switch over [P | Q_l] with alpha = p_num primes per digit.  No counterpart in the
+ * reference (its switch goes through T); built from the reference's exact-conversion recipe (BasisConv.cuh:18-58)
+ * and ModDown (BasisConv.cuh:286-326).  digits: [ceil((l+1)/p_num)][p_num+q_num] limbs;
+ * evk: [2][ceil(q_num/p_num)][p_num+q_num] limbs (NTT domain); ip/in_pq: [2][p_num+q_num] limbs; out: [2][q_num]. ---- */
+int ckks_hybrid_modup(ckks_ctx* ctx, uint64_t* digits, const uint64_t* in_coeff, int l);
+int ckks_hybrid_inner_product(ckks_ctx* ctx, uint64_t* ip, const uint64_t* digits_ntt, const uint64_t* evk, int l);
+int ckks_hybrid_moddown(ckks_ctx* ctx, uint64_t* out, const uint64_t* in_pq_coeff, int l);
+/* whole switch: in_ntt (q_num limbs, NTT domain; overwritten with its coefficient form) -> out [2][q_num] NTT domain.
+ * scratch: (ceil((l+1)/p_num) + 2) * (p_num+q_num) * N words. */
+int ckks_hybrid_keyswitch(ckks_ctx* ctx, uint64_t* out, uint64_t* in_ntt, const uint64_t* evk, int l, uint64_t* scratch);
+
+/* ---- ring-packed PCMM ---- */
+/* PCMM_Context::PCMM_Context (PCMM_Context.cuh:7-57) */
+int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,
+                    const uint64_t* q_ringpack, int q_count);
+int pcmm_ctx_destroy(pcmm_ctx* h);
+/* the gather kernel of PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:50-88,115-119): rlwe = [a | b] with
+ * L+1 limbs each, COEFFICIENT domain; mlwe_ptrs_host: mlwe_num device pointers, each [(l+1)][(rank+1)][N1]. */
+int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l);
+/* PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:90-125): iNTT, gather, NTT back; rlwe in NTT domain. */
+int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l);
+/* PCMM_Scheme::PPMM device part (PPMM_kernel.cuh:93-252, launch :294-340):
+ * out[m][mod][c] = fused-rescaled sum_n trunc(W[m][n]*scaler) * mlwe[n][mod][c] mod q_mod, for mod_num ring-pack
+ * primes (the reference fixes mod_num = 2), c < (rank+1)*N1.  W: device fp32 row-major [M][Kin];
+ * mlwe_ptrs_host: Kin device pointers; out: device [M][mod_num][(rank+1)*N1]. */
+int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_host, uint64_t* out_dev, int M,
+              int Kin, int mod_num, double scaler);
+/* same contraction with the MLWE operands in one contiguous device array [Kin][mod_num][(rank+1)*N1] */
+int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev, uint64_t* out_dev, int M, int Kin,
+                      int mod_num, double scaler);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CKKS_HIP_H */

@@ -1,0 +1,161 @@
+"""GPU parity: batched NTT / iNTT through the C ABI against the CPU oracle, bit-exact."""
+import numpy as np
+import pytest
+
+from tests.gpu_common import Pair, to_dev, from_dev
+from tests.helpers import limbs_uniform
+from tests.params import CFG1_Q, CFG2_Q, CFG3_P, REF_PARAMS
+
+pytestmark = pytest.mark.gpu
+
+
+def check_fwd_inv(pair, primes_idx0, primes, poly_num, seed, mode=None):
+    """Forward vs oracle, inverse vs oracle, round trip; limbs (y, j) at (y*len + j)."""
+    if mode is not None:
+        pair.dev.set_arith_mode(mode)
+    N, mod_num = pair.N, len(primes)
+    data = limbs_uniform(seed, primes, poly_num, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, primes_idx0, poly_num, mod_num, mod_num)
+    buf = to_dev(data)
+    pair.dev.ToNTTInplace(buf, 0, primes_idx0, poly_num, mod_num, mod_num)
+    got = from_dev(buf, data.shape)
+    assert np.array_equal(got, want)
+    pair.dev.FromNTTInplace(buf, 0, primes_idx0, poly_num, mod_num, mod_num)
+    assert np.array_equal(from_dev(buf, data.shape), data)
+    # inverse of arbitrary (non-transform) data against the oracle
+    want_inv = data.copy()
+    pair.orc.FromNTTInplace(want_inv.reshape(-1), 0, primes_idx0, poly_num, mod_num, mod_num)
+    buf.upload(data)
+    pair.dev.FromNTTInplace(buf, 0, primes_idx0, poly_num, mod_num, mod_num)
+    assert np.array_equal(from_dev(buf, data.shape), want_inv)
+    buf.free()
+
+
+def test_config1_n4096_4primes_batch16():
+    """BASELINE config 1: N = 2^12, 4 primes < 2^36, batch of 16 polynomials, seed 1."""
+    pair = Pair(12, [], CFG1_Q)
+    for mode in (0, 1):       # FP64 back end, integer back end
+        check_fwd_inv(pair, 0, CFG1_Q, 16, seed=1, mode=mode)
+
+
+@pytest.mark.parametrize("logN", [8, 9, 10, 11, 13, 14, 15])
+def test_all_ring_sizes(logN):
+    q = CFG2_Q[:3]
+    pair = Pair(logN, [], q)
+    for mode in (0, 1):
+        check_fwd_inv(pair, 0, q, 3, seed=logN, mode=mode)
+
+
+def test_config2_one_ciphertext_n65536_24primes():
+    """BASELINE config 2: N = 2^16, 24 primes, one ciphertext = 2 polys x 24 limbs, seed 2."""
+    pair = Pair(16, [], CFG2_Q)
+    check_fwd_inv(pair, 0, CFG2_Q, 2, seed=2, mode=0)
+
+
+def test_n65536_integer_backend_and_large_primes():
+    """50-bit q/p and 60-bit t primes of the reference's logN = 16 set (Params.cuh:88-171) use the integer back end."""
+    P = REF_PARAMS[16]
+    p, q, t = P["p"][:1], P["q"][:2], P["t"][:2]
+    pair = Pair(16, p, q, t, gamma=2)
+    check_fwd_inv(pair, 0, p + q + t, 1, seed=3)
+    # 36-bit primes through the integer back end as well
+    pair2 = Pair(16, [], CFG2_Q[:2])
+    check_fwd_inv(pair2, 0, CFG2_Q[:2], 2, seed=4, mode=1)
+
+
+def test_reference_addressing_and_ext_variant():
+    """start_poly_idx / start_mod_idx / poly_mod_len addressing (ntt_60bit.cuh:446-455) and the batch stride of the
+    _for_externalProduct variants (ntt_60bit.cuh:913-934)."""
+    P = REF_PARAMS[14]
+    p, q, t = P["p"], P["q"][:4], P["t"][:3]
+    pair = Pair(12, p, q, t, gamma=3)
+    N, K = pair.N, len(p)
+    rng = np.random.default_rng(5)
+    buf_h = rng.integers(0, 1 << 35, size=(3, 7, N), dtype=np.uint64)          # 3 polys, poly_mod_len 7
+    want = buf_h.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 2, K + 1, 3, 3, 7)                  # limbs 2..4 of each poly, primes q1..q3
+    d = to_dev(buf_h)
+    pair.dev.ToNTTInplace(d, 2, K + 1, 3, 3, 7)
+    got = from_dev(d, buf_h.shape)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got[:, :2], buf_h[:, :2]) and np.array_equal(got[:, 5:], buf_h[:, 5:])
+    pair.dev.FromNTTInplace(d, 2, K + 1, 3, 3, 7)
+    assert np.array_equal(from_dev(d, buf_h.shape), buf_h)
+    # ext: batch 2, stride 9 limbs, 2 polys x 3 T-limbs
+    T0 = K + len(q)
+    e_h = rng.integers(0, 1 << 59, size=(2, 9, N), dtype=np.uint64)
+    for j in range(9):
+        e_h[:, j] %= np.uint64(t[j % 3])
+    want = e_h.copy()
+    pair.orc.ToNTTInplace_for_externalProduct(want.reshape(-1), 0, T0, 2, 3, 3, 9, 2)
+    d2 = to_dev(e_h)
+    pair.dev.ToNTTInplace_for_externalProduct(d2, 0, T0, 2, 3, 3, 9, 2)
+    assert np.array_equal(from_dev(d2, e_h.shape), want)
+    pair.orc.FromNTTInplace_for_externalProduct(want.reshape(-1), 0, T0, 2, 3, 3, 9, 2)
+    pair.dev.FromNTTInplace_for_externalProduct(d2, 0, T0, 2, 3, 3, 9, 2)
+    assert np.array_equal(from_dev(d2, e_h.shape), want) and np.array_equal(want, e_h)
+
+
+def test_tables_match_oracle():
+    P = REF_PARAMS[14]
+    pair = Pair(10, P["p"], P["q"], P["t"], P["gamma"])
+    for name in ["pqt", "mu_hi", "mu_lo", "psi", "psiinv", "n_inv", "n_inv_shoup", "halfTmodpqti", "psi_table",
+                 "psiinv_table", "psi_shoup_table", "psiinv_shoup_table", "pHatVecModq", "pHatInvVecModp", "PModqt",
+                 "PinvModq", "RiHatInv", "RiHatModT", "Rimodti", "QjHatInv", "QjHatModT", "Qjmodti", "THatInv",
+                 "THatModRi", "Tmodpqi", "qiInvModql"]:
+        assert np.array_equal(pair.dev.table(name), pair.orc.table(name)), name
+
+
+def test_edge_cases_and_errors():
+    from ckks_llm_amd import CkksError, Context_23
+    pair = Pair(10, [], CFG2_Q[:2])
+    d = to_dev(np.zeros((1, 2, pair.N), dtype=np.uint64))
+    pair.dev.ToNTTInplace(d, 0, 0, 0, 2, 2)          # empty batch: no work, no error
+    pair.dev.ToNTTInplace(d, 0, 0, 1, 0, 2)
+    assert not from_dev(d, (2, pair.N)).any()
+    pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)          # NTT(0) = 0
+    assert not from_dev(d, (2, pair.N)).any()
+    with pytest.raises(CkksError):
+        pair.dev.ToNTTInplace(d, 0, 1, 1, 2, 2)      # prime range outside the context
+    with pytest.raises(CkksError):
+        Context_23(10, [], [CFG2_Q[0] + 2])          # not 1 mod 2N
+    with pytest.raises(CkksError):
+        Context_23(17, [], CFG2_Q[:1])               # unsupported ring size
+    # maximal residues q-1 everywhere
+    data = np.stack([np.full(pair.N, q - 1, dtype=np.uint64) for q in CFG2_Q[:2]])[None]
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, 1, 2, 2)
+    d.upload(data)
+    pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)
+    assert np.array_equal(from_dev(d, data.shape), want)
+
+
+def test_full_size_properties_batch32():
+    """BASELINE config 2 at batch 32 (768 MiB): size-independent properties instead of a full oracle run:
+    round trip, linearity on a sampled pair, and oracle parity on one sampled ciphertext."""
+    pair = Pair(16, [], CFG2_Q)
+    N, L1, B = pair.N, 24, 32
+    rng = np.random.default_rng(2)
+    data = np.empty((2 * B, L1, N), dtype=np.uint64)
+    for j, q in enumerate(CFG2_Q):
+        data[:, j, :] = rng.integers(0, q, size=(2 * B, N), dtype=np.uint64)
+    d = to_dev(data)
+    pair.dev.ToNTTInplace(d, 0, 0, 2 * B, L1, L1)
+    got = from_dev(d, data.shape)
+    # parity on one sampled ciphertext (2 polys)
+    y = 17
+    want = data[y:y + 2].copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, 2, L1, L1)
+    assert np.array_equal(got[y:y + 2], want)
+    # linearity: NTT(a) + NTT(b) == NTT(a + b) for polys 0 and 1 (checked on the device transform of the sum)
+    s = np.empty((1, L1, N), dtype=np.uint64)
+    for j, q in enumerate(CFG2_Q):
+        s[0, j] = (data[0, j] + data[1, j]) % np.uint64(q)
+    ds = to_dev(s)
+    pair.dev.ToNTTInplace(ds, 0, 0, 1, L1, L1)
+    fs = from_dev(ds, s.shape)
+    for j, q in enumerate(CFG2_Q):
+        assert np.array_equal(fs[0, j], (got[0, j] + got[1, j]) % np.uint64(q))
+    pair.dev.FromNTTInplace(d, 0, 0, 2 * B, L1, L1)
+    assert np.array_equal(from_dev(d, data.shape), data)
