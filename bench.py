@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the CKKS hot path on one MI355X.
+
+Headline (BASELINE.json configs[1]): batched RNS NTT/iNTT at N = 2^16, 24 primes < 2^36, a batch of 32 ciphertexts
+(2 polynomials x 24 limbs each = 1536 limbs, 768 MiB of uniform u64 residues, seed 2), resident in HBM.
+One step = inverse transform then forward transform of the whole batch (the order ntt_throughput.cu:51-60 uses)
+= 2 * 1536 limb-transforms.  value = limb-transforms per second.
+
+Also measured and reported in the same JSON line:
+  roofline      - the slower of the two kernel launches of a forward transform, HIP events on the launch stream;
+                  algorithmic bytes = 16*N per limb-transform, half of it credited to each of the two launches
+  ppmm          - the ring-packed PPMM at the BERT-base shape (configs[3]), int8-MAC/s against the int8 MFMA peak
+  keyswitch     - one textbook hybrid key switch at configs[2]
+  cpu_baseline  - the CPU oracle (a port of the reference arithmetic, OpenMP) on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_I8_PEAK_TMACS = 2516.6          # 5.033 POP/s dense int8 = 2.5166e15 MAC/s
+
+
+def uniform_limbs(seed, primes, polys, N):
+    rng = np.random.default_rng(seed)
+    out = np.empty((polys, len(primes), N), dtype=np.uint64)
+    for j, q in enumerate(primes):
+        out[:, j, :] = rng.integers(0, q, size=(polys, N), dtype=np.uint64)
+    return out
+
+
+def bench_ntt(args, P):
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    logN, primes, cts = 16, P.CFG2_Q, args.batch
+    N, L1, polys = 1 << logN, len(primes), 2 * cts
+    limbs = polys * L1
+    ctx = Context_23(logN, [], primes)
+    # synthetic data: one ciphertext's worth of seeded residues, replicated over the batch (same distribution, bounded set-up time)
+    one = uniform_limbs(2, primes, 2, N)
+    buf = DeviceBuffer(8 * limbs * N)
+    for c in range(cts):
+        buf.L_.ckks_memcpy_h2d(buf.ptr + c * one.nbytes, one.ctypes.data, one.nbytes)
+    ctx.sync()
+
+    def step():
+        ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+        ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    # round trip must give the data back (bit-exact) - cheap end-to-end sanity on the timed buffer
+    back = buf.download(np.uint64, one.size).reshape(one.shape)
+    assert np.array_equal(back, one), "NTT round trip changed the data"
+    ms_per_step = dt / args.steps * 1e3
+    value = 2 * limbs * args.steps / dt
+
+    # per-kernel durations (HIP events between the two launches), averaged
+    reps = max(5, args.steps)
+    f1 = f2 = i1 = i2 = 0.0
+    for _ in range(reps):
+        a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, True)
+        i1 += a; i2 += b
+        a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, False)
+        f1 += a; f2 += b
+    f1, f2, i1, i2 = [x / reps for x in (f1, f2, i1, i2)]
+    alg_bytes_launch = 16.0 * N * limbs / 2.0          # half a transform per launch
+    dom_name, dom_ms = max([("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2)], key=lambda x: x[1])
+    achieved = alg_bytes_launch / (dom_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel_ms": {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)},
+                "transform_algorithmic_GBps": {"fwd": round(16.0 * N * limbs / ((f1 + f2) * 1e-3) / 1e9, 1),
+                                               "inv": round(16.0 * N * limbs / ((i1 + i2) * 1e-3) / 1e9, 1)},
+                "algorithmic_bytes_per_launch": alg_bytes_launch}
+    # one ciphertext (48 limbs, 24 MiB): the latency-oriented half of configs[1]
+    one_ct = {}
+    small = DeviceBuffer.from_numpy(one)
+    for _ in range(5):
+        ctx.ToNTTInplace(small, 0, 0, 2, L1, L1)
+        ctx.FromNTTInplace(small, 0, 0, 2, L1, L1)
+    ctx.timer_start()
+    R = 50
+    for _ in range(R):
+        ctx.ToNTTInplace(small, 0, 0, 2, L1, L1)
+    fw = ctx.timer_stop() / R
+    ctx.timer_start()
+    for _ in range(R):
+        ctx.FromNTTInplace(small, 0, 0, 2, L1, L1)
+    iv = ctx.timer_stop() / R
+    one_ct = {"fwd_us": round(fw * 1e3, 2), "inv_us": round(iv * 1e3, 2),
+              "fwd_limb_transforms_per_s": round(2 * L1 / (fw * 1e-3)), "inv_limb_transforms_per_s": round(2 * L1 / (iv * 1e-3))}
+    buf.free(); small.free()
+    return value, ms_per_step, roofline, one_ct, limbs
+
+
+def bench_cpu_baseline(P, seconds_target=12.0):
+    """Oracle (port of the reference arithmetic) on a bounded sample: forward+inverse of `limbs` limbs at N = 2^16."""
+    from oracle import oracle_py as O
+    primes = P.CFG2_Q
+    ctx = O.OracleContext(16, [], primes)
+    threads = O.lib().orc_max_threads()
+    polys = 4
+    data = uniform_limbs(2, primes, polys, 1 << 16)
+    flat = data.reshape(-1)
+    limbs = polys * len(primes)
+    # one untimed pass to size the sample
+    t0 = time.perf_counter()
+    ctx.FromNTTInplace(flat, 0, 0, polys, len(primes), len(primes))
+    ctx.ToNTTInplace(flat, 0, 0, polys, len(primes), len(primes))
+    once = time.perf_counter() - t0
+    reps = max(1, min(40, int(seconds_target / max(once, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ctx.FromNTTInplace(flat, 0, 0, polys, len(primes), len(primes))
+        ctx.ToNTTInplace(flat, 0, 0, polys, len(primes), len(primes))
+    dt = time.perf_counter() - t0
+    assert np.array_equal(flat.reshape(data.shape), uniform_limbs(2, primes, polys, 1 << 16))
+    return {"value": round(2 * limbs * reps / dt, 1), "unit": "limb-transforms/s", "cores": threads, "kind": "port",
+            "sample": "%d x (iNTT+NTT) of %d limbs (N=2^16, %d primes, %d polys), OpenMP over limbs" % (reps, limbs, len(primes), polys)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=32, help="ciphertexts per step (BASELINE configs[1]: 32)")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-extra", action="store_true", help="skip the PPMM / key-switch side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import tests.params as P
+    value, ms_per_step, roofline, one_ct, limbs = bench_ntt(args, P)
+    line = {
+        "metric": "NTT limb-transforms/s @N=2^16", "value": round(value, 1), "unit": "limb-transforms/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u64 residues (f64 butterflies for q < 2^41)", "data": "synthetic",
+        "config": {"workload": "configs[1]: RNS NTT+iNTT, N=2^16, 24 primes <2^36, batch of %d ciphertexts (%d limbs, %d MiB) per step"
+                               % (args.batch, limbs, limbs * 8 * 65536 >> 20), "limb_transforms_per_step": 2 * limbs},
+        "roofline": roofline, "one_ciphertext": one_ct,
+        "frac_of_hbm_roofline_whole_transform": round(value * 16 * 65536 / 1e9 / HBM_PEAK_GBS, 4),
+    }
+    if not args.skip_extra:
+        try:
+            import bench_extra
+            line.update(bench_extra.run(P))
+        except ImportError:
+            pass
+    if not args.skip_cpu:
+        line["cpu_baseline"] = bench_cpu_baseline(P)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -143,6 +143,13 @@ class Context_23:
     def FromNTTInplace(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len):
         _check(self.L_.ckks_ntt_inv(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ckks_ntt_inv")
 
+    def ntt_timed(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, inverse):
+        """One transform; returns the HIP-event durations (ms) of its two kernel launches."""
+        a, b = C.c_float(), C.c_float()
+        _check(self.L_.ckks_ntt_timed(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                      1 if inverse else 0, C.byref(a), C.byref(b)), "ckks_ntt_timed")
+        return a.value, b.value
+
     def ToNTTInplace_for_externalProduct(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
                                          cipher_mod_num, batch_size):
         _check(self.L_.ckks_ntt_fwd_ext(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,

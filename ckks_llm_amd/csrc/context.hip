@@ -306,6 +306,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
     }
     if (rc == CKKS_OK && hipEventCreate(&c->ev0) != hipSuccess) rc = CKKS_E_HIP;
     if (rc == CKKS_OK && hipEventCreate(&c->ev1) != hipSuccess) rc = CKKS_E_HIP;
+    if (rc == CKKS_OK && hipEventCreate(&c->ev_mid) != hipSuccess) rc = CKKS_E_HIP;
     if (rc != CKKS_OK) { ckks_ctx_destroy(c); return rc; }
     *out = c;
     return CKKS_OK;
@@ -319,6 +320,7 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     for (void* p : ptrs) if (p) (void)hipFree(p);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->ev_mid) (void)hipEventDestroy(c->ev_mid);
     delete c;
     return CKKS_OK;
 }
@@ -399,6 +401,23 @@ extern "C" int ckks_timer_stop(ckks_ctx* c, float* ms) {
     CKKS_HIP_TRY(hipEventRecord(c->ev1, c->stream));
     CKKS_HIP_TRY(hipEventSynchronize(c->ev1));
     CKKS_HIP_TRY(hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return CKKS_OK;
+}
+
+// Per-kernel timing of one transform: the two passes are separate launches; HIP events are recorded on the
+// context's stream before, between and after them.
+extern "C" int ckks_ntt_timed(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml, int inverse,
+                              float* first_pass_ms, float* second_pass_ms) {
+    if (!c || !first_pass_ms || !second_pass_ms) return CKKS_E_INVALID;
+    CKKS_HIP_TRY(hipEventRecord(c->ev0, c->stream));
+    c->ev_mid_armed = true;
+    int rc = ckks::launch_ntt(c, dev, sp, sm, pn, mn, pml, 0, 1, inverse != 0);
+    c->ev_mid_armed = false;
+    if (rc) return rc;
+    CKKS_HIP_TRY(hipEventRecord(c->ev1, c->stream));
+    CKKS_HIP_TRY(hipEventSynchronize(c->ev1));
+    CKKS_HIP_TRY(hipEventElapsedTime(first_pass_ms, c->ev0, c->ev_mid));
+    CKKS_HIP_TRY(hipEventElapsedTime(second_pass_ms, c->ev_mid, c->ev1));
     return CKKS_OK;
 }
 

@@ -48,7 +48,8 @@ struct ckks_ctx {
     int Ri_blockNum = 0, Qj_blockNum = 0, nprimes = 0;
     long N = 0;
     hipStream_t stream = nullptr;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr, ev_mid = nullptr;
+    bool ev_mid_armed = false;           // record ev_mid between the two passes of the next NTT (per-kernel timing)
 
     // host copies (reference names, reference layouts) for ckks_ctx_table and for launch-time decisions
     std::vector<uint64_t> pqt, mu_hi, mu_lo, psi, psiinv, n_inv, n_inv_shoup, halfTmodpqti;

@@ -320,9 +320,11 @@ static int launch_two_pass(ckks_ctx* c, const NttArgs& args, int limbs, bool inv
     dim3 gr(N1 / ROWS, limbs), br(C::U * ROWS);
     if (!inverse) {
         hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false>), gs, bs, 0, c->stream, args);
+        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
         hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false>), gr, br, 0, c->stream, args);
     } else {
         hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true>), gr, br, 0, c->stream, args);
+        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
         hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true>), gs, bs, 0, c->stream, args);
     }
     CKKS_HIP_TRY(hipGetLastError());

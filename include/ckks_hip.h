@@ -59,6 +59,9 @@ int ckks_ctx_destroy(ckks_ctx* ctx);
 int ckks_set_stream(ckks_ctx* ctx, void* hip_stream);
 /* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum" */
 int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
+/* 0 (default): FP64 butterflies for primes < 2^41, integer butterflies otherwise; 1: integer butterflies everywhere.
+ * Both give the same residues; the switch exists for testing and tuning. */
+int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
 /* host copy of a constant table, flattened in the reference's device layout (names as in ckks_oracle.h /
  * Context_23.h: "pqt","psi","psi_table","psiinv_table","RiHatInv","QjHatModT",...). *count receives the length. */
 int ckks_ctx_table(const ckks_ctx* ctx, const char* name, uint64_t* host_out, size_t cap, size_t* count);
@@ -77,6 +80,11 @@ int ckks_ntt_fwd_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start
                      int poly_mod_len, int cipher_mod_num, int batch_size);
 int ckks_ntt_inv_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                      int poly_mod_len, int cipher_mod_num, int batch_size);
+
+/* One transform with HIP-event timing of its two kernel launches (strided pass and row pass; the forward transform
+ * runs the strided pass first, the inverse the row pass first).  Replaces the cudaEvent pairs of ntt_throughput.cu:51-60. */
+int ckks_ntt_timed(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                   int poly_mod_len, int inverse, float* first_pass_ms, float* second_pass_ms);
 
 /* ---- basis conversion: Context_23::modUpPQtoT_23 / modUpQjtoT_23 / modUpTtoPQl_23 / modDownPQltoQl_23
  *      (BasisConv.cuh:61-77, 161-179, 243-254, 328-347; strides as indexed at :25,:52,:110,:142,:201,:239,:304,:325) ---- */

@@ -1,0 +1,166 @@
+"""GPU parity: RNS basis conversions, ModDown, external / inner product, rescale and both key-switch chains
+through the C ABI against the CPU oracle, bit-exact on every residue."""
+import numpy as np
+import pytest
+
+from ckks_llm_amd import DeviceBuffer
+from tests.gpu_common import Pair, to_dev, from_dev
+from tests.helpers import limbs_uniform
+from tests.params import CFG2_Q, CFG3_P, REF_PARAMS
+
+pytestmark = pytest.mark.gpu
+
+
+def ref_pair(params, logN):
+    P = REF_PARAMS[params]
+    return Pair(logN, P["p"], P["q"], P["t"], P["gamma"])
+
+
+@pytest.mark.parametrize("params,logN", [(13, 10), (14, 12), (15, 11), (16, 10)])
+def test_four_conversion_maps(params, logN):
+    pair = ref_pair(params, logN)
+    o, d, N = pair.orc, pair.dev, pair.N
+    K, Q, T, RB, QB = o.p_num, o.q_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum
+    pq = o.p + o.q
+    for l in sorted({o.L, o.L - 1, o.L // 2, 0}):
+        batch = 2
+        # [P|Q] -> T  (modUpPQtoT_23)
+        inp = limbs_uniform(100 + l, pq, batch, N)
+        want = np.zeros((batch, RB * T, N), dtype=np.uint64)
+        o.modUpPQtoT_23(want.reshape(-1), inp.reshape(-1), l, batch)
+        dout = to_dev(np.zeros_like(want))
+        din = to_dev(inp)
+        d.modUpPQtoT_23(dout, din, l, batch)
+        assert np.array_equal(from_dev(dout, want.shape), want), ("pq_to_t", l)
+        # Q digit -> T  (modUpQjtoT_23); corner values in the first columns
+        inq = limbs_uniform(200 + l, o.q, batch, N)
+        inq[:, :, 0] = 0
+        for j, q in enumerate(o.q):
+            inq[:, j, 1] = q - 1
+            inq[:, j, 2] = 1
+        want = np.zeros((batch, QB * T, N), dtype=np.uint64)
+        o.modUpQjtoT_23(want.reshape(-1), inq.reshape(-1), l, batch)
+        dout2 = to_dev(np.zeros_like(want))
+        d.modUpQjtoT_23(dout2, to_dev(inq), l, batch)
+        assert np.array_equal(from_dev(dout2, want.shape), want), ("qj_to_t", l)
+        # T -> [P|Q_l]  (modUpTtoPQl_23), then ModDown (modDownPQltoQl_23)
+        int_ = np.zeros((batch, RB * T, N), dtype=np.uint64)
+        rng = np.random.default_rng(300 + l)
+        for k in range(RB * T):
+            int_[:, k, :] = rng.integers(0, o.t[k % T], size=(batch, N), dtype=np.uint64)
+        int_[:, :, 0] = 0
+        want = np.zeros((batch, RB * T, N), dtype=np.uint64)
+        o.modUpTtoPQl_23(want.reshape(-1), int_.reshape(-1), l, batch)
+        dbuf = to_dev(np.zeros_like(want))
+        d.modUpTtoPQl_23(dbuf, to_dev(int_), l, batch)
+        got = from_dev(dbuf, want.shape)
+        assert np.array_equal(got[:, :K + l + 1], want[:, :K + l + 1]), ("t_to_pql", l)
+        wdown = np.zeros((batch, Q, N), dtype=np.uint64)
+        o.modDownPQltoQl_23(wdown.reshape(-1), want.reshape(-1), l, batch)
+        ddown = to_dev(np.zeros_like(wdown))
+        d.modDownPQltoQl_23(ddown, to_dev(want), l, batch)
+        assert np.array_equal(from_dev(ddown, wdown.shape)[:, :l + 1], wdown[:, :l + 1]), ("moddown", l)
+
+
+@pytest.mark.parametrize("params", [14, 15])
+def test_external_product_and_keyswitch_23(params):
+    pair = ref_pair(params, 12)
+    o, d, N = pair.orc, pair.dev, pair.N
+    K, Q, T, RB, QB, dnum, L = o.p_num, o.q_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum, o.dnum, o.L
+    swk = limbs_uniform(7, o.t, 2 * dnum * RB, N)                     # [2][dnum][RB][T][N] uniform in T
+    dswk = to_dev(swk)
+    for l in (L, L - 1, 1):
+        cT = limbs_uniform(8 + l, o.t, QB, N)
+        want = np.zeros((2, RB * T, N), dtype=np.uint64)
+        o.external_product_T(want.reshape(-1), cT.reshape(-1), swk.reshape(-1), l)
+        dout = to_dev(np.zeros_like(want))
+        d.external_product_T(dout, to_dev(cT), dswk, l)
+        nblk = -(-(K + l + 1) // o.gamma)
+        got = from_dev(dout, want.shape)
+        assert np.array_equal(got[:, :nblk * T], want[:, :nblk * T]), ("external_product", l)
+        # whole chain (steps 2..9 of mult_23)
+        d2 = np.zeros((Q, N), dtype=np.uint64)
+        d2[:l + 1] = limbs_uniform(20 + l, o.q[:l + 1], 1, N)[0]
+        wout = np.zeros((2, Q, N), dtype=np.uint64)
+        o.keyswitch_23(wout.reshape(-1), d2.reshape(-1), swk.reshape(-1), l)
+        dd2, do = to_dev(d2), to_dev(np.zeros_like(wout))
+        s1 = DeviceBuffer(8 * N * T * QB)
+        s2 = DeviceBuffer(8 * N * T * RB * 2)
+        s3 = DeviceBuffer(8 * N * T * RB * 2)
+        s1.zero(); s2.zero(); s3.zero()
+        d.keyswitch_23(do, dd2, dswk, l, s1, s2, s3)
+        assert np.array_equal(from_dev(do, wout.shape)[:, :l + 1], wout[:, :l + 1]), ("keyswitch_23", l)
+
+
+def test_rescale():
+    pair = ref_pair(14, 12)
+    o, d, N = pair.orc, pair.dev, pair.N
+    L = o.L
+    for l in (L, 1):
+        c = limbs_uniform(30 + l, o.q, 2, N)
+        want = c.copy()
+        o.rescaleAndEqual(want.reshape(-1), l)
+        dc = to_dev(c)
+        scratch = DeviceBuffer(8 * 2 * (L + 1) * N)
+        d.rescaleAndEqual(dc, scratch, l)
+        got = from_dev(dc, c.shape)
+        assert np.array_equal(got[:, :l + 1], want[:, :l + 1])
+        assert np.array_equal(got[:, l + 1:], c[:, l + 1:])
+    with pytest.raises(ValueError):
+        d.rescaleAndEqual(dc, scratch, 0)                   # level-0 operand (Scheme_23.cuh:192-194 behaviour)
+
+
+@pytest.mark.parametrize("logN,nq,np_", [(12, 6, 2), (10, 7, 3), (12, 24, 6)])
+def test_hybrid_keyswitch_stages(logN, nq, np_):
+    """Textbook hybrid switch over [P|Q_l] (BASELINE config 3 shape at reduced N): every stage and the whole chain."""
+    q, p = CFG2_Q[:nq], CFG3_P[:np_]
+    pair = Pair(logN, p, q)
+    o, d, N = pair.orc, pair.dev, pair.N
+    W = np_ + nq
+    dnum = -(-nq // np_)
+    evk = limbs_uniform(3, p + q, 2 * dnum, N)                          # [2][dnum][W][N], seed 3
+    devk = to_dev(evk)
+    for l in (nq - 1, nq - 2, 0):
+        dn = -(-(l + 1) // np_)
+        inp = np.zeros((nq, N), dtype=np.uint64)
+        inp[:l + 1] = limbs_uniform(40 + l, q[:l + 1], 1, N)[0]
+        wdig = np.zeros((dn, W, N), dtype=np.uint64)
+        o.hybrid_modup(wdig.reshape(-1), inp.reshape(-1), l)
+        ddig = to_dev(np.zeros_like(wdig))
+        d.hybrid_modup(ddig, to_dev(inp), l)
+        assert np.array_equal(from_dev(ddig, wdig.shape)[:, :np_ + l + 1], wdig[:, :np_ + l + 1]), ("modup", l)
+        wip = np.zeros((2, W, N), dtype=np.uint64)
+        o.hybrid_inner_product(wip.reshape(-1), wdig.reshape(-1), evk.reshape(-1), l)
+        dip = to_dev(np.zeros_like(wip))
+        d.hybrid_inner_product(dip, to_dev(wdig), devk, l)
+        assert np.array_equal(from_dev(dip, wip.shape)[:, :np_ + l + 1], wip[:, :np_ + l + 1]), ("inner", l)
+        wout = np.zeros((2, nq, N), dtype=np.uint64)
+        o.hybrid_moddown(wout.reshape(-1), wip.reshape(-1), l)
+        dout = to_dev(np.zeros_like(wout))
+        d.hybrid_moddown(dout, to_dev(wip), l)
+        assert np.array_equal(from_dev(dout, wout.shape)[:, :l + 1], wout[:, :l + 1]), ("moddown", l)
+        # whole switch
+        wks = np.zeros((2, nq, N), dtype=np.uint64)
+        o.hybrid_keyswitch(wks.reshape(-1), inp.reshape(-1), evk.reshape(-1), l)
+        dks = to_dev(np.zeros_like(wks))
+        scratch = DeviceBuffer(8 * (dn + 2) * W * N)
+        scratch.zero()
+        d.hybrid_keyswitch(dks, to_dev(inp), devk, l, scratch)
+        assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), ("keyswitch", l)
+
+
+def test_config3_full_size_keyswitch():
+    """BASELINE config 3 at full size: N = 2^16, 24 Q + 6 P primes, dnum = 4, seed 3; parity with the oracle on the
+    whole switch output (every residue)."""
+    q, p = CFG2_Q, CFG3_P
+    pair = Pair(16, p, q)
+    o, d, N = pair.orc, pair.dev, pair.N
+    W, nq, np_, l = 30, 24, 6, 23
+    evk = limbs_uniform(3, p + q, 2 * 4, N)
+    inp = limbs_uniform(33, q, 1, N)[0]
+    wks = np.zeros((2, nq, N), dtype=np.uint64)
+    o.hybrid_keyswitch(wks.reshape(-1), inp.copy().reshape(-1), evk.reshape(-1), l)
+    dks = to_dev(np.zeros_like(wks))
+    scratch = DeviceBuffer(8 * (4 + 2) * W * N)
+    d.hybrid_keyswitch(dks, to_dev(inp), to_dev(evk), l, scratch)
+    assert np.array_equal(from_dev(dks, wks.shape), wks)

@@ -1,0 +1,102 @@
+"""GPU parity: RLWE -> MLWE gather and PPMM through the C ABI against the CPU oracle, bit-exact."""
+import os
+
+import numpy as np
+import pytest
+
+from ckks_llm_amd import DeviceBuffer, PCMM_Context, PCMM_Scheme
+from oracle import oracle_py as O
+from tests.gpu_common import Pair, to_dev, from_dev
+from tests.helpers import limbs_uniform
+from tests.params import CFG2_Q, CFG3_P, REF_PARAMS
+
+pytestmark = pytest.mark.gpu
+
+
+def make(logN, N1, q_ctx, p_ctx, p_rp, q_rp):
+    pair = Pair(logN, p_ctx, q_ctx)
+    rank = pair.N // N1
+    dev = PCMM_Scheme(PCMM_Context(N1, rank, p_rp, q_rp, pair.dev))
+    orc = O.OraclePCMM(pair.orc, N1, rank, p_rp, q_rp)
+    return pair, dev, orc, rank
+
+
+@pytest.mark.parametrize("logN,N1,mlwe_num", [(10, 128, 8), (10, 128, 2), (12, 256, 16), (10, 64, 1)])
+def test_rlwe_decompose(logN, N1, mlwe_num):
+    q = CFG2_Q[:3]
+    pair, dev, orc, rank = make(logN, N1, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
+    N, L = pair.N, len(q) - 1
+    for l in (L, 0):
+        rlwe = limbs_uniform(l + 1, q, 2, N)                                  # [2][L+1][N], coefficient domain
+        rlwe[:, :, 0] = 0                                                     # negate(0) = 0 corner
+        per = (L + 1) * (rank + 1) * N1
+        want = [np.zeros(per, dtype=np.uint64) for _ in range(mlwe_num)]
+        orc.rlweCipherDecompose(rlwe.reshape(-1), want, l)
+        bufs = [DeviceBuffer(8 * per) for _ in range(mlwe_num)]
+        for b in bufs:
+            b.zero()
+        dev.rlweCipherDecompose(to_dev(rlwe), bufs, mlwe_num, 0, l, coeff_domain=True)
+        for m in range(mlwe_num):
+            assert np.array_equal(bufs[m].download(), want[m]), (l, m)
+        # NTT-domain entry point (PCMM_Scheme.cuh:107-124): iNTT, gather, NTT back
+        rl_ntt = rlwe.copy()
+        pair.orc.ToNTTInplace(rl_ntt.reshape(-1), 0, 1, 2, l + 1, L + 1)
+        d_rl = to_dev(rl_ntt)
+        for b in bufs:
+            b.zero()
+        dev.rlweCipherDecompose(d_rl, bufs, mlwe_num, 0, l)
+        for m in range(mlwe_num):
+            assert np.array_equal(bufs[m].download(), want[m]), ("ntt", l, m)
+        assert np.array_equal(from_dev(d_rl, rl_ntt.shape), rl_ntt)
+    with pytest.raises(Exception):
+        dev.rlweCipherDecompose(to_dev(rlwe), bufs * (rank + 1), rank + 1, 0, L, coeff_domain=True)
+
+
+def run_ppmm(dev, orc, rank, N1, M, Kin, mod_num, qs, scaler, seed, strided=False, w_std=0.02):
+    C = (rank + 1) * N1
+    rng = np.random.default_rng(seed)
+    W = rng.normal(0, w_std, (M, Kin)).astype(np.float32)
+    W[0, 0] = 0.0
+    mlwe = [limbs_uniform(seed * 1000 + n, qs[:mod_num], 1, C)[0] for n in range(Kin)]
+    want = np.zeros((M, mod_num, C), dtype=np.uint64)
+    orc.PPMM(W, [m.reshape(-1) for m in mlwe], want.reshape(-1), M, Kin, mod_num, scaler)
+    dW = DeviceBuffer.from_numpy(W)
+    dout = DeviceBuffer(want.nbytes)
+    dout.zero()
+    if strided:
+        dall = to_dev(np.stack(mlwe))
+        dev.PPMM_strided(dW, dall, dout, M, Kin, mod_num, scaler)
+    else:
+        bufs = [to_dev(m) for m in mlwe]
+        dev.PPMM(dW, bufs, dout, M, Kin, N1, Kin, mod_num, scaler)
+    got = from_dev(dout, want.shape)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("mod_num", [1, 2, 3])
+def test_ppmm_small_36bit(mod_num):
+    """C = 9*128 = 1152 columns (multiple of 64): the MFMA path when it is built, 36-bit primes."""
+    q = CFG2_Q[:4]
+    pair, dev, orc, rank = make(10, 128, q, CFG3_P[:1], [CFG3_P[0]], q[:3])
+    run_ppmm(dev, orc, rank, 128, 48, 40, mod_num, q, float(2 ** 26), seed=mod_num)
+    run_ppmm(dev, orc, rank, 128, 130, 64, mod_num, q, float(2 ** 26), seed=10 + mod_num, strided=True)
+
+
+def test_ppmm_reference_shape_50bit_primes():
+    """The reference's own shape: two 50-bit ring-pack primes {q0, q1}, p_ringpack = {p_last}
+    (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284)."""
+    P = REF_PARAMS[15]
+    q = P["q"][:2]
+    pair, dev, orc, rank = make(10, 128, q, P["p"][:1], [P["p"][0]], q)
+    scaler = float(int(q[1] * float(2 ** 49) / float(2 ** 49)))
+    run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1)
+    run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1)
+
+
+def test_ppmm_shape_errors():
+    q = CFG2_Q[:2]
+    pair, dev, orc, rank = make(10, 128, q, [], [], q)
+    with pytest.raises(ValueError):
+        dev.PPMM(0, [], 0, 4, 4, 64, 4, 2, 1.0)            # mat_K != N1  (PPMM_kernel.cuh:256-259)
+    with pytest.raises(ValueError):
+        dev.PPMM(0, [], 0, 4, 4, 128, 5, 2, 1.0)           # mat_N != mlwe_num (:260-263)
