@@ -1,0 +1,83 @@
+"""Side measurements printed in bench.py's JSON line: PPMM at the BERT-base shape (BASELINE configs[3]) against the
+int8 MFMA roofline and one textbook hybrid key switch (configs[2]) against the HBM roofline."""
+import numpy as np
+
+MFMA_I8_PEAK_MACS = 2.5166e15      # 5.033 POP/s dense int8
+HBM_PEAK = 8.0e12
+
+
+def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3):
+    from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
+    primes = P.CFG2_Q[:L]
+    ctx = Context_23(16, [], primes)
+    rank = (1 << 16) // N1
+    C = (rank + 1) * N1
+    sch = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, ctx))
+    rng = np.random.default_rng(4)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    dW = DeviceBuffer.from_numpy(W)
+    # synthetic MLWE operands: 16 distinct seeded ciphertexts of uniform residues, copied into Kin separate buffers
+    seeds = []
+    rng5 = np.random.default_rng(5)
+    for s in range(16):
+        a = np.empty((L, C), dtype=np.uint64)
+        for j, q in enumerate(primes):
+            a[j] = rng5.integers(0, q, C, dtype=np.uint64)
+        seeds.append(DeviceBuffer.from_numpy(a))
+    per = 8 * L * C
+    bufs = []
+    for n in range(Kin):
+        b = DeviceBuffer(per)
+        b.L_.ckks_memcpy_d2d(b.ptr, seeds[n % 16].ptr, per)
+        bufs.append(b)
+    out = DeviceBuffer(8 * M * L * C)
+    scaler = float(2 ** 26)
+    sch.PPMM(dW, bufs, out, M, Kin, N1, Kin, L, scaler)      # warm-up (also allocates the workspace)
+    ctx.sync()
+    best = 1e30
+    for _ in range(reps):
+        ctx.timer_start()
+        sch.PPMM(dW, bufs, out, M, Kin, N1, Kin, L, scaler)
+        best = min(best, ctx.timer_stop())
+    DW, DC, path = sch.pcmm_context.info("last_DW"), sch.pcmm_context.info("last_DC"), sch.pcmm_context.info("last_path")
+    word_macs = float(M) * Kin * C * L
+    macs = word_macs * DW * DC
+    res = {"workload": "configs[3]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (M, Kin, N1, L, C),
+           "ms": round(best, 3), "word_MAC_per_s": round(word_macs / (best * 1e-3), 1), "int8_MAC_per_s": round(macs / (best * 1e-3), 1),
+           "D_w": DW, "D_c": DC, "kernel": "int8 MFMA" if path == 1 else "generic u128",
+           "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
+                        "unit": "TMAC/s (int8)", "frac": round(macs / (best * 1e-3) / MFMA_I8_PEAK_MACS, 4)}}
+    for b in bufs + seeds + [out, dW]:
+        b.free()
+    return res
+
+
+def bench_keyswitch(P, reps=10):
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    q, p = P.CFG2_Q, P.CFG3_P
+    ctx = Context_23(16, p, q)
+    N, W, nq, l, dn = 1 << 16, 30, 24, 23, 4
+    rng = np.random.default_rng(3)
+    evk = np.empty((2 * dn, W, N), dtype=np.uint64)
+    for j, m in enumerate(p + q):
+        evk[:, j, :] = rng.integers(0, m, size=(2 * dn, N), dtype=np.uint64)
+    inp = np.empty((nq, N), dtype=np.uint64)
+    for j, m in enumerate(q):
+        inp[j] = rng.integers(0, m, N, dtype=np.uint64)
+    devk, dinp, dout = DeviceBuffer.from_numpy(evk), DeviceBuffer.from_numpy(inp), DeviceBuffer(8 * 2 * nq * N)
+    scratch = DeviceBuffer(8 * (dn + 2) * W * N)
+    for _ in range(3):
+        ctx.hybrid_keyswitch(dout, dinp, devk, l, scratch)
+    ctx.timer_start()
+    for _ in range(reps):
+        ctx.hybrid_keyswitch(dout, dinp, devk, l, scratch)
+    ms = ctx.timer_stop() / reps
+    stage_bytes = 1008 * 8 * N           # stage-sum of minimal limb moves: ModUp 24+96, NTT 2*120, IP 360+60, iNTT 2*60, ModDown 60+48
+    return {"workload": "configs[2]: hybrid key switch N=2^16, 24 Q + 6 P primes, dnum=4", "us": round(ms * 1e3, 1),
+            "keyswitch_per_s": round(1e3 / ms, 1),
+            "roofline": {"bound": "hbm", "achieved": round(stage_bytes / (ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(stage_bytes / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": stage_bytes}}
+
+
+def run(P):
+    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P)}

@@ -48,6 +48,7 @@ def _declare(L):
         "ckks_hybrid_modup": (i, [vp, vp, vp, i]), "ckks_hybrid_inner_product": (i, [vp, vp, vp, vp, i]),
         "ckks_hybrid_moddown": (i, [vp, vp, vp, i]), "ckks_hybrid_keyswitch": (i, [vp, vp, vp, vp, i, vp]),
         "pcmm_ctx_create": (i, [C.POINTER(vp), vp, i, i, u64p, i, u64p, i]), "pcmm_ctx_destroy": (i, [vp]),
+        "pcmm_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_rlwe_decompose_ntt": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),

@@ -210,6 +210,11 @@ class PCMM_Context:
                                        qa.ctypes.data_as(u64p), len(qa)), "pcmm_ctx_create")
         self.h = h.value
 
+    def info(self, name):
+        v = C.c_long()
+        _check(self.L_.pcmm_info(self.h, name.encode(), C.byref(v)), "pcmm_info")
+        return v.value
+
     def __del__(self):
         try:
             if self.h:

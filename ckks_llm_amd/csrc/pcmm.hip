@@ -22,22 +22,8 @@
 #include <cstring>
 #include <vector>
 
-#include "context.hpp"
+#include "pcmm.hpp"
 #include "host_math.hpp"
-
-struct pcmm_ctx {
-    ckks_ctx* ctx = nullptr;
-    int N1 = 0, rank = 0, np = 0, nq = 0;
-    std::vector<uint64_t> pq;
-    ckks::PrimeConst* d_pq = nullptr;        // ring-pack primes [p_ringpack | q_ringpack]
-    uint64_t** d_ptrs = nullptr;             // device copy of the caller's MLWE pointer table (PCMM_Scheme.cuh:16-18)
-    int ptr_cap = 0;
-    // workspace of the quantised plaintext matrix
-    long long* d_A = nullptr;                // [M][Kin] int64
-    int8_t* d_Adig = nullptr;                // [DW][Mpad][Kpad] balanced digits
-    size_t A_cap = 0, Adig_cap = 0;
-    unsigned long long* d_absmax = nullptr;
-};
 
 namespace ckks {
 
@@ -110,21 +96,7 @@ __global__ __launch_bounds__(256) void digits_kernel(const long long* A, int8_t*
 // ------------------------------------------------------------------------------------------------------------
 // generic kernel: one output per lane, 128-bit accumulation (the reference's arithmetic, PPMM_kernel.cuh:12-31)
 // ------------------------------------------------------------------------------------------------------------
-struct PpmmArgs {
-    const long long* A;           // [M][Kin]
-    const int8_t* Adig;           // [DW][Mpad][Kpad]
-    const u64* const* mlwe;       // Kin pointers (nullptr when strided)
-    const u64* mlwe_base;         // strided operand
-    long mlwe_stride;             // words between consecutive MLWE ciphertexts
-    u64* out;
-    const PrimeConst* pq;         // ring-pack primes, q part starts at np
-    const u64* qlast_inv;         // [mod_num] (q_last^-1 mod q_i), then Shoup words
-    long C;
-    int M, Kin, Mpad, Kpad, mod_num, np;
-};
-__device__ __forceinline__ const u64* mlwe_row(const PpmmArgs& a, int n) {
-    return a.mlwe ? a.mlwe[n] : a.mlwe_base + (long)n * a.mlwe_stride;
-}
+__device__ __forceinline__ const u64* mlwe_row(const PpmmArgs& a, int n) { return a.mlwe[n]; }
 __global__ __launch_bounds__(256) void ppmm_generic_kernel(PpmmArgs a) {
     const long c = (long)blockIdx.x * 256 + threadIdx.x;
     const int m = blockIdx.y;
@@ -145,7 +117,7 @@ __global__ __launch_bounds__(256) void ppmm_generic_kernel(PpmmArgs a) {
             o[(long)im * a.C + c] = r;
         } else {
             u64 temp = r + pr.q - r_last;                                   // :244
-            o[(long)im * a.C + c] = mul_shoup(temp, a.qlast_inv[im], a.qlast_inv[a.mod_num + im], pr.q);
+            o[(long)im * a.C + c] = mul_shoup(temp, a.consts[im], a.consts[PPMM_MAX_MODS + im], pr.q);
         }
     }
 }
@@ -174,7 +146,7 @@ extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, 
     }
     hipError_t e = hipMalloc((void**)&h->d_pq, pc.size() * sizeof(PrimeConst));
     if (e == hipSuccess) e = hipMemcpy(h->d_pq, pc.data(), pc.size() * sizeof(PrimeConst), hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMalloc((void**)&h->d_absmax, sizeof(unsigned long long) + 2 * 64 * sizeof(uint64_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&h->d_absmax, sizeof(unsigned long long) * (1 + PPMM_CONST_WORDS));
     if (e != hipSuccess) { pcmm_ctx_destroy(h); return hip_fail(e, "pcmm_ctx_create"); }
     *out = h;
     return CKKS_OK;
@@ -227,7 +199,6 @@ extern "C" int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* co
     return launch_ntt(c, rlwe, 0, c->K, 2, l + 1, c->L + 1, 0, 1, false);              // :124
 }
 
-namespace ckks { int launch_ppmm_mfma(pcmm_ctx* h, const PpmmArgs& a, int DW, int DC); }
 
 static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
                        int M, int Kin, int mod_num, double scaler) {
@@ -236,7 +207,14 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     ckks_ctx* c = h->ctx;
     const long C = (long)(h->rank + 1) * h->N1;
     int rc;
-    if (ptrs_host && (rc = upload_ptrs(h, ptrs_host, Kin))) return rc;
+    std::vector<const uint64_t*> strided_ptrs;
+    if (!ptrs_host) {               // contiguous operand: same kernels through a generated pointer table
+        strided_ptrs.resize(Kin);
+        for (int n = 0; n < Kin; n++) strided_ptrs[n] = strided + (size_t)n * mod_num * C;
+        ptrs_host = strided_ptrs.data();
+    }
+    if ((rc = upload_ptrs(h, ptrs_host, Kin))) return rc;
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
     // workspace
     const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 63) / 64 * 64;
     size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
@@ -250,18 +228,25 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         CKKS_HIP_TRY(hipMalloc((void**)&h->d_Adig, needD));
         h->Adig_cap = needD;
     }
-    // q_last^-1 mod q_i and Shoup words, kept behind the |A| maximum word
-    std::vector<uint64_t> inv(2 * 64, 0);
+    // per-call epilogue constants, kept behind the |A| maximum word
+    std::vector<uint64_t> cst(PPMM_CONST_WORDS, 0);
     const uint64_t qlast = h->pq[h->np + mod_num - 1];
-    uint64_t qmax = 0;
+    uint64_t qmax = 0, qmin = ~0ull;
+    auto dbits = [](uint64_t x, uint64_t m) { double d = x > m / 2 ? -(double)(m - x) : (double)x; uint64_t b; memcpy(&b, &d, 8); return b; };
     for (int i = 0; i < mod_num; i++) {
         uint64_t qi = h->pq[h->np + i];
-        qmax = std::max(qmax, qi);
-        if (i < mod_num - 1) { inv[i] = H::invmod(qlast % qi, qi); inv[mod_num + i] = H::shoup(inv[i], qi); }
+        qmax = std::max(qmax, qi); qmin = std::min(qmin, qi);
+        if (i < mod_num - 1) {
+            cst[i] = H::invmod(qlast % qi, qi);
+            cst[PPMM_MAX_MODS + i] = H::shoup(cst[i], qi);
+            cst[4 * PPMM_MAX_MODS + i] = dbits(cst[i], qi);
+        }
+        cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 24, qi), qi);
+        cst[3 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 48, qi), qi);
     }
-    uint64_t* d_inv = (uint64_t*)(h->d_absmax + 1);
+    uint64_t* d_cst = (uint64_t*)(h->d_absmax + 1);
     CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
-    CKKS_HIP_TRY(hipMemcpyAsync(d_inv, inv.data(), 2 * mod_num * sizeof(uint64_t), hipMemcpyHostToDevice, c->stream));
+    CKKS_HIP_TRY(hipMemcpyAsync(d_cst, cst.data(), PPMM_CONST_WORDS * sizeof(uint64_t), hipMemcpyHostToDevice, c->stream));
     long count = (long)M * Kin;
     hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, c->stream, W, h->d_A, h->d_absmax, count, scaler);
     unsigned long long absmax = 0;
@@ -269,8 +254,8 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
 
     PpmmArgs a;
-    a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = ptrs_host ? (const u64* const*)h->d_ptrs : nullptr; a.mlwe_base = strided;
-    a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.qlast_inv = d_inv; a.C = C; a.M = M; a.Kin = Kin;
+    a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
+    a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
     a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np;
 
     // digit counts: DW digits cover |A| < 2^(8*DW-1); DC digits cover residues < 2^(8*DC-1)
@@ -278,11 +263,12 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
     const bool mfma_ok = !force_generic && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
-                         (long)Kpad * 16384 * std::min(DW, DC) < (1l << 31) && absmax < qmax;
+                         (long)Kpad * 16384 * std::min(std::max(DW, 3), 5) < (1l << 31) && absmax < qmin && qmin > (1ull << 25);
+    h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
         hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
-        rc = launch_ppmm_mfma(h, a, DW, DC);
+        rc = launch_ppmm_mfma_impl(c->stream, a, DW);
         if (rc) return rc;
     } else {
         dim3 grid((unsigned)((C + 255) / 256), M), block(256);
@@ -292,6 +278,14 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     return CKKS_OK;
 }
 
+extern "C" int pcmm_info(const pcmm_ctx* h, const char* name, long* value) {
+    if (!h || !name || !value) return CKKS_E_INVALID;
+    std::string n(name);
+    if (n == "last_path") *value = h->last_path; else if (n == "last_DW") *value = h->last_DW; else if (n == "last_DC") *value = h->last_DC;
+    else if (n == "last_absmax") *value = (long)h->last_absmax; else if (n == "N1") *value = h->N1; else if (n == "mlwe_rank") *value = h->rank;
+    else { set_error("pcmm_info: unknown name " + n); return CKKS_E_INVALID; }
+    return CKKS_OK;
+}
 extern "C" int pcmm_ppmm(pcmm_ctx* h, const float* W, const uint64_t* const* mlwe_ptrs_host, uint64_t* out, int M, int Kin, int mod_num, double scaler) {
     return ppmm_common(h, W, mlwe_ptrs_host, nullptr, out, M, Kin, mod_num, scaler);
 }

@@ -1,0 +1,47 @@
+// Internal types shared by the PCMM launchers and kernels.
+#pragma once
+#include <vector>
+
+#include "context.hpp"
+
+struct pcmm_ctx {
+    ckks_ctx* ctx = nullptr;
+    int N1 = 0, rank = 0, np = 0, nq = 0;
+    std::vector<uint64_t> pq;
+    ckks::PrimeConst* d_pq = nullptr;        // ring-pack primes [p_ringpack | q_ringpack]
+    uint64_t** d_ptrs = nullptr;             // device copy of the caller's MLWE pointer table (PCMM_Scheme.cuh:16-18)
+    int ptr_cap = 0;
+    // workspace of the quantised plaintext matrix
+    long long* d_A = nullptr;                // [M][Kin] int64
+    int8_t* d_Adig = nullptr;                // [DW][Mpad][Kpad] balanced digits
+    size_t A_cap = 0, Adig_cap = 0;
+    int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
+    unsigned long long last_absmax = 0;
+    unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
+};
+
+namespace ckks {
+
+// per-call constants of the PPMM epilogue, one row of PPMM_MAX_MODS words each:
+//   [0] q_last^-1 mod q_i   [1] its Shoup word   [2] 2^24 mod q_i   [3] 2^48 mod q_i   [4] q_last^-1 mod q_i
+//   rows 2..4 are balanced representatives stored as IEEE double bit patterns (FP64 epilogue)
+constexpr int PPMM_MAX_MODS = 64;
+constexpr int PPMM_CONST_ROWS = 5;
+constexpr int PPMM_CONST_WORDS = PPMM_MAX_MODS * PPMM_CONST_ROWS;
+
+struct PpmmArgs {
+    const long long* A;           // [M][Kin]
+    const int8_t* Adig;           // [DW][Mpad][Kpad]
+    const u64* const* mlwe;       // Kin pointers (nullptr when strided)
+    const u64* mlwe_base;         // strided operand
+    long mlwe_stride;             // words between consecutive MLWE ciphertexts
+    u64* out;
+    const PrimeConst* pq;         // ring-pack primes, q part starts at np
+    const u64* consts;            // PPMM_CONST_WORDS words, see above
+    long C;
+    int M, Kin, Mpad, Kpad, mod_num, np;
+};
+
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW);
+
+}  // namespace ckks

@@ -119,6 +119,9 @@ int ckks_hybrid_keyswitch(ckks_ctx* ctx, uint64_t* out, uint64_t* in_ntt, const 
 int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,
                     const uint64_t* q_ringpack, int q_count);
 int pcmm_ctx_destroy(pcmm_ctx* h);
+/* "N1", "mlwe_rank", and facts about the last PPMM call: "last_path" (1 = int8 MFMA kernel, 0 = generic 128-bit kernel),
+ * "last_DW" / "last_DC" (base-256 digits of the plaintext matrix / of the residues), "last_absmax" (max |A|). */
+int pcmm_info(const pcmm_ctx* h, const char* name, long* value);
 /* the gather kernel of PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:50-88,115-119): rlwe = [a | b] with
  * L+1 limbs each, COEFFICIENT domain; mlwe_ptrs_host: mlwe_num device pointers, each [(l+1)][(rank+1)][N1]. */
 int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l);

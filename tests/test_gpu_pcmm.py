@@ -71,6 +71,7 @@ def run_ppmm(dev, orc, rank, N1, M, Kin, mod_num, qs, scaler, seed, strided=Fals
         dev.PPMM(dW, bufs, dout, M, Kin, N1, Kin, mod_num, scaler)
     got = from_dev(dout, want.shape)
     assert np.array_equal(got, want)
+    return dev.pcmm_context.info("last_path")
 
 
 @pytest.mark.parametrize("mod_num", [1, 2, 3])
@@ -78,8 +79,11 @@ def test_ppmm_small_36bit(mod_num):
     """C = 9*128 = 1152 columns (multiple of 64): the MFMA path when it is built, 36-bit primes."""
     q = CFG2_Q[:4]
     pair, dev, orc, rank = make(10, 128, q, CFG3_P[:1], [CFG3_P[0]], q[:3])
-    run_ppmm(dev, orc, rank, 128, 48, 40, mod_num, q, float(2 ** 26), seed=mod_num)
-    run_ppmm(dev, orc, rank, 128, 130, 64, mod_num, q, float(2 ** 26), seed=10 + mod_num, strided=True)
+    assert run_ppmm(dev, orc, rank, 128, 48, 40, mod_num, q, float(2 ** 26), seed=mod_num) == 1          # MFMA kernel
+    assert run_ppmm(dev, orc, rank, 128, 130, 64, mod_num, q, float(2 ** 26), seed=10 + mod_num, strided=True) == 1
+    # 4 plaintext digits (|A| up to 2^30) and a K that is not a multiple of the MFMA depth
+    assert run_ppmm(dev, orc, rank, 128, 16, 100, mod_num, q, float(2 ** 33), seed=20 + mod_num) == 1
+    assert dev.pcmm_context.info("last_DW") == 4
 
 
 def test_ppmm_reference_shape_50bit_primes():
@@ -89,8 +93,8 @@ def test_ppmm_reference_shape_50bit_primes():
     q = P["q"][:2]
     pair, dev, orc, rank = make(10, 128, q, P["p"][:1], [P["p"][0]], q)
     scaler = float(int(q[1] * float(2 ** 49) / float(2 ** 49)))
-    run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1)
-    run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1)
+    assert run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1) == 0          # generic kernel
+    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1) == 0
 
 
 def test_ppmm_shape_errors():
