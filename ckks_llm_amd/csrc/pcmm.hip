@@ -216,7 +216,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     if ((rc = upload_ptrs(h, ptrs_host, Kin))) return rc;
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
     // workspace
-    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 63) / 64 * 64;
+    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 127) / 128 * 128;   // K padded to an even number of 64-deep MFMA steps
     size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
     if (needA > h->A_cap) {
         if (h->d_A) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_A); h->d_A = nullptr; }
