@@ -154,7 +154,7 @@ extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, 
 extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     if (!h) return CKKS_OK;
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax};
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     delete h;
     return CKKS_OK;
@@ -207,16 +207,25 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     ckks_ctx* c = h->ctx;
     const long C = (long)(h->rank + 1) * h->N1;
     int rc;
-    std::vector<const uint64_t*> strided_ptrs;
-    if (!ptrs_host) {               // contiguous operand: same kernels through a generated pointer table
-        strided_ptrs.resize(Kin);
-        for (int n = 0; n < Kin; n++) strided_ptrs[n] = strided + (size_t)n * mod_num * C;
-        ptrs_host = strided_ptrs.data();
+    // Row-pointer table on the device, padded to Kpad entries: rows of the K padding point to a zero buffer, so the dense
+    // kernel needs no bounds checks along K.  A contiguous operand goes through a generated table.
+    const int Kpad_tab = (Kin + 191) / 192 * 192;
+    size_t zero_words = (size_t)mod_num * C;
+    if (Kpad_tab > Kin && zero_words > h->zero_cap) {
+        if (h->d_zero) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_zero); h->d_zero = nullptr; }
+        CKKS_HIP_TRY(hipMalloc((void**)&h->d_zero, zero_words * sizeof(uint64_t)));
+        CKKS_HIP_TRY(hipMemset(h->d_zero, 0, zero_words * sizeof(uint64_t)));
+        h->zero_cap = zero_words;
     }
-    if ((rc = upload_ptrs(h, ptrs_host, Kin))) return rc;
+    std::vector<const uint64_t*> tab(Kpad_tab);
+    for (int n = 0; n < Kpad_tab; n++)
+        tab[n] = n >= Kin ? h->d_zero : (ptrs_host ? ptrs_host[n] : strided + (size_t)n * mod_num * C);
+    bool aligned16 = true;
+    for (int n = 0; n < Kin; n++) aligned16 = aligned16 && (((uintptr_t)tab[n]) & 15) == 0;
+    if ((rc = upload_ptrs(h, tab.data(), Kpad_tab))) return rc;
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
     // workspace
-    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 127) / 128 * 128;   // K padded to an even number of 64-deep MFMA steps
+    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 191) / 192 * 192;   // K padded to a multiple of three 64-deep MFMA steps (LDS ring of three slots)
     size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
     if (needA > h->A_cap) {
         if (h->d_A) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_A); h->d_A = nullptr; }
@@ -262,13 +271,20 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     int DW = 1; while (DW < 8 && absmax >= (1ull << (8 * DW - 1))) DW++;
     int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
-    const bool mfma_ok = !force_generic && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
+    const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
                          (long)Kpad * 16384 * std::min(std::max(DW, 3), 5) < (1l << 31) && absmax < qmin && qmin > (1ull << 25);
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
         hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
-        rc = launch_ppmm_mfma_impl(c->stream, a, DW);
+        size_t need = ppmm_bdig_bytes(a);
+        if (need > h->Bdig_cap) {
+            if (h->d_Bdig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Bdig); h->d_Bdig = nullptr; h->Bdig_cap = 0; }
+            hipError_t e = hipMalloc((void**)&h->d_Bdig, need);
+            if (e != hipSuccess) { set_error("PPMM: cannot allocate the residue digit planes"); return CKKS_E_NOMEM; }
+            h->Bdig_cap = need;
+        }
+        rc = launch_ppmm_mfma_impl(c->stream, a, DW, h->d_Bdig);
         if (rc) return rc;
     } else {
         dim3 grid((unsigned)((C + 255) / 256), M), block(256);

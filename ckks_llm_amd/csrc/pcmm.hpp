@@ -15,6 +15,10 @@ struct pcmm_ctx {
     long long* d_A = nullptr;                // [M][Kin] int64
     int8_t* d_Adig = nullptr;                // [DW][Mpad][Kpad] balanced digits
     size_t A_cap = 0, Adig_cap = 0;
+    int8_t* d_Bdig = nullptr;                // residue digit planes [prime][K step][digit][column][64]
+    size_t Bdig_cap = 0;
+    uint64_t* d_zero = nullptr;              // zero rows the K padding of the row-pointer table points to
+    size_t zero_cap = 0;
     int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
     unsigned long long last_absmax = 0;
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
@@ -42,6 +46,7 @@ struct PpmmArgs {
     int M, Kin, Mpad, Kpad, mod_num, np;
 };
 
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW);
+size_t ppmm_bdig_bytes(const PpmmArgs& a);
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig);
 
 }  // namespace ckks

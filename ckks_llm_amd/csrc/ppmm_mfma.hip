@@ -4,19 +4,12 @@
 //
 // Exact integer product through base-256 balanced digits:
 //     A[m][n]  = sum_{d<DW} a_d[m][n] * 256^d ,  a_d in [-128,127]   (int8 planes built once per call, shared by all primes)
-//     Ct[n][c] = sum_{j<DC} b_j[n][c] * 256^j ,  b_j in [-128,127]   (bytes of (x + 0x8080808080) xor 0x80, made while staging)
+//     Ct[n][c] = sum_{j<DC} b_j[n][c] * 256^j ,  b_j in [-128,127]   (bytes of (x + 0x8080808080) xor 0x80, int8 planes built once per call)
 //     sum_n A*Ct = sum_{e<DW+DC-1} 256^e * S_e ,   S_e = sum_{d+j=e} sum_n a_d*b_j    (int32, |S_e| <= min(DW,DC)*Kin*2^14)
 // One v_mfma_i32_16x16x64_i8 per (d, j, 16x16 tile, 64 k) accumulates into the anti-diagonal accumulator S_{d+j}.
 // The epilogue recombines the S_e without rounding in FP64 (three diagonals at a time fit 48 bits), reduces modulo q_i
 // (q_i < 2^39) and applies the fused rescale (PPMM_kernel.cuh:213-249).
 //
-// Work decomposition: workgroup = 256 lanes = 4 waves owns a 128 (M) x 64 (columns) output tile for ALL primes
-// (prime loop outermost, as in the reference: the rescale operand r_last is the lane's own earlier store); each wave owns a
-// 64 x 32 sub-tile = 4 x 2 MFMA tiles x (DW+DC-1) accumulators.  K advances 64 at a time through double-buffered LDS:
-//   A digits : global int8 planes -> LDS [d][row][64]            (16 B per lane, rows of 64 B)
-//   residues : 16 consecutive-k u64 per lane (one column), digit-split and byte-transposed in registers -> LDS [j][col][64]
-// so that every MFMA operand is one ds_read_b128.  Workgroups that share a column panel are numbered so that they land on
-// the same XCD (ids congruent mod 8) back to back: the panel is fetched from HBM once and re-read from that XCD's L2.
 #include <type_traits>
 
 #include "pcmm.hpp"
@@ -26,7 +19,6 @@ namespace ckks {
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int MT = 128, CT = 64, KS = 64;        // workgroup tile and K step
-constexpr int WM = 64, WC = 32;                  // wave tile
 constexpr int DCMAX = 5;
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -47,26 +39,74 @@ __device__ __forceinline__ double balance_f64(double x, double q, double qinv) {
     return __builtin_fma(-__builtin_rint(x * qinv), q, x);
 }
 
-// Pipeline (global step s = prime iteration * ksteps + K step, parity p = s & 1; ksteps is even):
-//   at the start of step s   : A[p], B[p] hold the digits of step s; RAW[(s+1)&1] holds the raw residues of step s+1
-//   during step s            : asynchronous loads  A(s+1) -> A[p^1],  raw(s+2) -> RAW[p]      (nothing in registers)
-//                              MFMAs of step s on A[p], B[p]  interleaved with  digit split of RAW[p^1] -> B[p^1]
-//   end of step s            : wait for the loads, ONE workgroup barrier
-// With four plaintext digits the LDS cannot hold two raw buffers; then raw(s+1) is loaded during step s and split after
-// its MFMAs (OVERLAP = false).
-// Every LDS buffer is a separate __shared__ object addressed with a compile-time parity, so that the compiler can tell
-// that the asynchronous writes of a step never alias the operands the step's MFMAs read (otherwise it waits for the
-// loads before the first LDS read and the overlap is lost).
+// ------------------------------------------------------------------------------------------------------------
+// Pass 1: residue digit planes.  Every residue is read ONCE, split into DC balanced base-256 digits and written in the
+// order the MFMA kernel stages it:  Bdig[prime][K step][digit][column][64 k]  (k contiguous, 64 B per column).
+// One workgroup (256 lanes) handles 64 k x 64 columns: coalesced 512 B row reads, a byte transpose in registers,
+// LDS to gather the 4 waves' quarter rows, then 16 B per lane coalesced writes.
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __restrict__ bdig) {
+    constexpr int DC = DCMAX;
+    __shared__ __align__(16) int8_t tile[DC][CT][KS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const unsigned c0 = blockIdx.x * CT;
+    const int ks = blockIdx.y, im = blockIdx.z;
+    const long col_word = (long)im * a.C + c0 + lane;
+    uint4 dig[DC];
+    unsigned* dw = reinterpret_cast<unsigned*>(dig);
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        u64 y[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) y[i] = a.mlwe[ks * KS + 16 * wave + 4 * g + i][col_word] + 0x8080808080ull;   // bytes = digit + 128
+        const unsigned x0 = (unsigned)y[0], x1 = (unsigned)y[1], x2 = (unsigned)y[2], x3 = (unsigned)y[3];
+        const unsigned t0 = __byte_perm(x0, x1, 0x5140), t1 = __byte_perm(x0, x1, 0x7362);
+        const unsigned t2 = __byte_perm(x2, x3, 0x5140), t3 = __byte_perm(x2, x3, 0x7362);
+        dw[0 * 4 + g] = __byte_perm(t0, t2, 0x5410) ^ 0x80808080u;
+        dw[1 * 4 + g] = __byte_perm(t0, t2, 0x7632) ^ 0x80808080u;
+        dw[2 * 4 + g] = __byte_perm(t1, t3, 0x5410) ^ 0x80808080u;
+        dw[3 * 4 + g] = __byte_perm(t1, t3, 0x7632) ^ 0x80808080u;
+        const unsigned h01 = __byte_perm((unsigned)(y[0] >> 32), (unsigned)(y[1] >> 32), 0x0040);
+        const unsigned h23 = __byte_perm((unsigned)(y[2] >> 32), (unsigned)(y[3] >> 32), 0x0040);
+        dw[4 * 4 + g] = __byte_perm(h01, h23, 0x5410) ^ 0x80808080u;
+    }
+    // LDS chunk index xor-swizzled with the column so that the 64-byte-strided 16-byte stores spread over the banks
+#pragma unroll
+    for (int jj = 0; jj < DC; jj++) *reinterpret_cast<uint4*>(&tile[jj][lane][16 * (wave ^ ((lane >> 1) & 3))]) = dig[jj];
+    __syncthreads();
+    int8_t* dst = bdig + (((long)im * gridDim.y + ks) * gridDim.x + blockIdx.x) * (long)(DC * CT * KS);
+#pragma unroll
+    for (int t = 0; t < DC * CT * KS / (256 * 16); t++) {
+        const int flat = (t * 256 + tid) * 16;                  // byte offset in [digit][column][64]
+        const int jj = flat / (CT * KS), col = (flat / KS) % CT, chunk = (flat % KS) / 16;
+        *reinterpret_cast<uint4*>(dst + flat) = *reinterpret_cast<const uint4*>(&tile[jj][col][16 * (chunk ^ ((col >> 1) & 3))]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Pass 2: the contraction.  A workgroup of 512 lanes = 8 waves (two per SIMD, so that one wave's waits and epilogue overlap
+// the other's MFMAs) owns a 128 (M) x 64 (columns) output tile for all primes; wave (wm, wc) owns the 32 x 32 sub-tile at
+// rows 32*wm, columns 32*wc = 2 x 2 MFMA tiles x (DW+DC-1) accumulators.
+// K advances 64 per step through a three-deep LDS ring filled by asynchronous global->LDS loads issued two steps ahead
+// (plaintext digit slabs of 16 rows x 64 B, residue digit slabs of 16 columns x 64 B; 1 KiB per wave instruction, nothing
+// held in registers).  The ring runs across prime boundaries: global step s = prime iteration * ksteps + K step, slot s % 3.
+// Every ring slot is a separate __shared__ object addressed with a compile-time index (the K loop is unrolled by 3 and
+// ksteps is a multiple of 3), so that the compiler can tell that the asynchronous writes of a step never alias the
+// operands its MFMAs read; otherwise it waits for the loads before the first LDS read and the overlap is lost.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int NWAVES = 8;
+
 template <int DW>
-__global__ __launch_bounds__(256) void ppmm_mfma_kernel(PpmmArgs a, int c_tiles, int m_tiles) {
+__global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_tiles) {
     constexpr int DC = DCMAX, ND = DW + DC - 1;
-    constexpr bool OVERLAP = DW <= 3;
+    constexpr int A_SLABS = DW * 8, B_SLABS = DC * 4;            // 1 KiB slabs per step
+    constexpr int A_PER_WAVE = (A_SLABS + NWAVES - 1) / NWAVES, B_PER_WAVE = (B_SLABS + NWAVES - 1) / NWAVES;
     __shared__ __align__(16) int8_t lds_a0[DW][MT][KS];
     __shared__ __align__(16) int8_t lds_a1[DW][MT][KS];
-    __shared__ __align__(16) int8_t lds_b0[DC][CT][KS];       // 16-byte chunks xor-swizzled by column
+    __shared__ __align__(16) int8_t lds_a2[DW][MT][KS];
+    __shared__ __align__(16) int8_t lds_b0[DC][CT][KS];
     __shared__ __align__(16) int8_t lds_b1[DC][CT][KS];
-    __shared__ __align__(16) u64 lds_raw0[KS][CT];
-    __shared__ __align__(16) u64 lds_raw1[OVERLAP ? KS : 1][CT];
+    __shared__ __align__(16) int8_t lds_b2[DC][CT][KS];
 
     // XCD-aware tile numbering: ids congruent mod 8 share an XCD; consecutive ones there share the column panel
     const unsigned id = blockIdx.x, xcd = id & 7, j = id >> 3;
@@ -81,133 +121,62 @@ __global__ __launch_bounds__(256) void ppmm_mfma_kernel(PpmmArgs a, int c_tiles,
     const int lr = lane & 15, lg = lane >> 4;
     const int ksteps = a.Kpad / KS;
     const long plane = (long)a.Mpad * a.Kpad;
-    const int8_t* a_tile = a.Adig + (long)m0 * a.Kpad;                   // uniform
-    const unsigned a_lane_off = (unsigned)(lane >> 2) * (unsigned)a.Kpad + 16u * (lane & 3);   // row lane/4, chunk lane%4 of a 16-row slab
-    const unsigned b_wr = (unsigned)lane * KS + 16u * (wave ^ ((lane >> 1) & 3));
+    // plaintext digits: slab (d, rr) = rows 16*rr..+15 of digit d, 64 B each; lane -> row lane/4, 16-byte chunk lane%4
+    const int8_t* a_lane = a.Adig + (long)(m0 + (lane >> 2)) * a.Kpad + 16 * (lane & 3);
+    // residue digits: [prime][K step][digit][column][64]; slab (jj, cc) = columns 16*cc..+15 of digit jj = 1 KiB contiguous
+    const long b_step = (long)c_tiles * (DC * CT * KS);                 // bytes per (prime, K step)
+    const int8_t* b_lane = bdig + (long)c_tile * (DC * CT * KS) + 16 * lane;
 
-    // Row pointers of the caller's MLWE table for one K step: lanes 0..15 of each wave fetch the 16 rows the wave stages
-    // (rows 2*slab, 2*slab+1 for slab = wave + 4t) with ONE vector load, issued a whole step ahead of their use; they are
-    // moved to scalar registers when needed.  (A scalar load of the table is not available to the compiler here: the
-    // table lives in ordinary global memory that it cannot prove unwritten.)
-    auto fetch_row_ptrs = [&](int ks) -> u64 {
-        const int t = (lane >> 1) & 7, half = lane & 1;
-        int k = ks * KS + 2 * (wave + 4 * t) + half;
-        k = k < a.Kin ? k : a.Kin - 1;             // K padding: read a valid row; it is zeroed at the digit split
-        return (u64)(uintptr_t)a.mlwe[k];
-    };
-    // DW*8 slabs of plaintext digits (16 rows x 64 B), 1 KiB each, dealt round-robin to the 4 waves
-    auto issue_a = [&](int ks, int8_t (*dst)[MT][KS]) {
+    auto issue = [&](int ks, int im, int8_t (*adst)[MT][KS], int8_t (*bdst)[CT][KS]) {
 #pragma unroll
-        for (int t = 0; t < DW * 2; t++) {
-            const int slab = wave + 4 * t, d = slab >> 3, rr = slab & 7;
-            async_copy16(a_tile + d * plane + (long)(rr * 16) * a.Kpad + ks * KS + a_lane_off, &dst[d][rr * 16][0]);
+        for (int t = 0; t < A_PER_WAVE; t++) {
+            int slab = wave + NWAVES * t;
+            slab = slab < A_SLABS ? slab : A_SLABS - 1;                  // surplus lanes re-load the last slab (same bytes)
+            const int d = slab >> 3, rr = slab & 7;
+            async_copy16(a_lane + d * plane + (long)(rr * 16) * a.Kpad + ks * KS, &adst[d][rr * 16][0]);
         }
-    };
-    // 32 slabs of raw residues (2 rows x 64 columns x 8 B), 1 KiB each
-    auto issue_raw = [&](unsigned col_word, u64 row_ptrs, u64 (*dst)[CT]) {
-        const unsigned lo = (unsigned)row_ptrs, hi = (unsigned)(row_ptrs >> 32);
+        const int8_t* bsrc = b_lane + ((long)im * ksteps + ks) * b_step;
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const int slab = wave + 4 * t;                                 // rows 2*slab (lanes 0..31), 2*slab+1 (lanes 32..63)
-            // readlane returns a signed int: convert each half to unsigned before widening, or the low half sign-extends
-            // into the high half of the address
-            const u64 pa = ((u64)(unsigned)__builtin_amdgcn_readlane((int)hi, 2 * t) << 32) | (u64)(unsigned)__builtin_amdgcn_readlane((int)lo, 2 * t);
-            const u64 pb = ((u64)(unsigned)__builtin_amdgcn_readlane((int)hi, 2 * t + 1) << 32) | (u64)(unsigned)__builtin_amdgcn_readlane((int)lo, 2 * t + 1);
-            const u64* p = (const u64*)(uintptr_t)(lane < 32 ? pa : pb) + col_word + 2 * (lane & 31);
-            async_copy16(p, &dst[2 * slab][0]);
+        for (int t = 0; t < B_PER_WAVE; t++) {
+            int slab = wave + NWAVES * t;
+            slab = slab < B_SLABS ? slab : B_SLABS - 1;
+            async_copy16(bsrc + slab * 1024, &bdst[0][0][0] + slab * 1024);
         }
-    };
-    // digit split of the raw residues of K step ks: lane = column, this wave's 16 rows
-    auto split_digits = [&](int ks, const u64 (*src)[CT], int8_t (*dst)[CT][KS]) {
-        const int kbase = ks * KS + 16 * wave;
-        uint4 dig[DC];
-        unsigned* dw = reinterpret_cast<unsigned*>(dig);
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            u64 y[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const u64 v = src[16 * wave + 4 * g + i][lane];
-                // bytes of x + 0x8080808080 are (digit + 128); rows of the K padding contribute zero digits
-                y[i] = (kbase + 4 * g + i < a.Kin ? v : 0) + 0x8080808080ull;
-            }
-            const unsigned x0 = (unsigned)y[0], x1 = (unsigned)y[1], x2 = (unsigned)y[2], x3 = (unsigned)y[3];
-            const unsigned t0 = __byte_perm(x0, x1, 0x5140), t1 = __byte_perm(x0, x1, 0x7362);
-            const unsigned t2 = __byte_perm(x2, x3, 0x5140), t3 = __byte_perm(x2, x3, 0x7362);
-            dw[0 * 4 + g] = __byte_perm(t0, t2, 0x5410) ^ 0x80808080u;
-            dw[1 * 4 + g] = __byte_perm(t0, t2, 0x7632) ^ 0x80808080u;
-            dw[2 * 4 + g] = __byte_perm(t1, t3, 0x5410) ^ 0x80808080u;
-            dw[3 * 4 + g] = __byte_perm(t1, t3, 0x7632) ^ 0x80808080u;
-            const unsigned h01 = __byte_perm((unsigned)(y[0] >> 32), (unsigned)(y[1] >> 32), 0x0040);
-            const unsigned h23 = __byte_perm((unsigned)(y[2] >> 32), (unsigned)(y[3] >> 32), 0x0040);
-            dw[4 * 4 + g] = __byte_perm(h01, h23, 0x5410) ^ 0x80808080u;
-        }
-#pragma unroll
-        for (int jj = 0; jj < DC; jj++) *reinterpret_cast<uint4*>(&dst[jj][0][0] + b_wr) = dig[jj];
     };
     auto wait_loads = [&]() {
         __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): this wave's asynchronous loads have landed in LDS
         __syncthreads();                            // ... and so have everybody else's
     };
 
-    // (ks1, im1) / (ks2, im2): K step and prime of the next / next-but-one global step, advanced without divisions;
-    // im < 0 means "past the end".
+    // (ks2, im2): K step and prime of global step s+2, advanced without divisions; past the end the loads re-fetch valid
+    // data into slots nobody reads again, so that a step has no branches.
     auto advance = [&](int& ks, int& im) { if (++ks == ksteps) { ks = 0; --im; } };
-    auto col_word_of = [&](int im) { return (unsigned)(im < 0 ? 0 : im) * (unsigned)a.C + c0; };   // word offset in one MLWE ciphertext (< 2^32)
-    int ks1 = 0, im1 = a.mod_num - 1, ks2, im2;
-    u64 ptrs_next;
-
-    // ---- prologue ----
-    issue_a(0, lds_a0);
-    issue_raw(col_word_of(im1), fetch_row_ptrs(0), lds_raw0);
-    advance(ks1, im1);
-    ks2 = ks1; im2 = im1;
-    advance(ks2, im2);                                  // (ks1, im1) = step 1, (ks2, im2) = step 2
-    if (OVERLAP) {
-        if (im1 >= 0) issue_raw(col_word_of(im1), fetch_row_ptrs(ks1), lds_raw1);
-        ptrs_next = fetch_row_ptrs(im2 >= 0 ? ks2 : 0);          // rows of raw(2), issued by step 0
-    } else {
-        ptrs_next = fetch_row_ptrs(im1 >= 0 ? ks1 : 0);          // rows of raw(1), issued by step 0
-    }
+    int ks2 = 0, im2 = a.mod_num - 1;
+    issue(ks2, im2, lds_a0, lds_b0);
+    advance(ks2, im2);
+    issue(ks2, im2 < 0 ? 0 : im2, lds_a1, lds_b1);
+    advance(ks2, im2);
     wait_loads();
-    split_digits(0, lds_raw0, lds_b0);
-    __syncthreads();
 
-    v4i acc[ND][4][2];
-    // one K step with compile-time buffer parity P
-    auto kstep = [&](auto parity) {
-        constexpr int P = decltype(parity)::value;
-        int8_t (*A_cur)[MT][KS] = P ? lds_a1 : lds_a0;
-        int8_t (*A_nxt)[MT][KS] = P ? lds_a0 : lds_a1;
-        int8_t (*B_cur)[CT][KS] = P ? lds_b1 : lds_b0;
-        int8_t (*B_nxt)[CT][KS] = P ? lds_b0 : lds_b1;
-        // Branch-free on purpose: past the last step the loads re-fetch valid data into buffers nobody reads again, so the
-        // whole step is one basic block and the loads / digit split can be interleaved with the MFMAs.
-        const int ksn = im1 >= 0 ? ks1 : 0;
-        issue_a(ksn, A_nxt);
-        if (OVERLAP) {
-            issue_raw(col_word_of(im2), ptrs_next, P ? lds_raw1 : lds_raw0);                    // raw(s+2) -> RAW[p]
-            int ks3 = ks2, im3 = im2;
-            advance(ks3, im3);
-            ptrs_next = fetch_row_ptrs(im3 >= 0 ? ks3 : 0);              // rows of raw(s+3), used by the next step
-            split_digits(ksn, P ? lds_raw0 : lds_raw1, B_nxt);          // RAW[p^1] -> B[p^1], overlaps the MFMAs below
-        } else {
-            issue_raw(col_word_of(im1), ptrs_next, lds_raw0);                                   // raw(s+1)
-            ptrs_next = fetch_row_ptrs(im2 >= 0 ? ks2 : 0);
-        }
+    v4i acc[ND][2][2];
+    // one K step reading ring slot R (compile time), refilling slot (R + 2) % 3 for step s + 2
+    auto kstep = [&](auto slot) {
+        constexpr int R = decltype(slot)::value, W = (R + 2) % 3;
+        int8_t (*A_cur)[MT][KS] = R == 0 ? lds_a0 : R == 1 ? lds_a1 : lds_a2;
+        int8_t (*B_cur)[CT][KS] = R == 0 ? lds_b0 : R == 1 ? lds_b1 : lds_b2;
+        int8_t (*A_nxt)[MT][KS] = W == 0 ? lds_a0 : W == 1 ? lds_a1 : lds_a2;
+        int8_t (*B_nxt)[CT][KS] = W == 0 ? lds_b0 : W == 1 ? lds_b1 : lds_b2;
+        issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
         v4i bf[2][DC];
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            const unsigned col = wc * WC + nt * 16 + lr;
-            const unsigned rd = col * KS + 16u * (lg ^ ((col >> 1) & 3));
+        for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][0][0] + rd);
-        }
+            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16 + lr][16 * lg]);
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) {
+        for (int mt = 0; mt < 2; mt++) {
             v4i af[DW];
 #pragma unroll
-            for (int d = 0; d < DW; d++) af[d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * WM + mt * 16 + lr][16 * lg]);
+            for (int d = 0; d < DW; d++) af[d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + mt * 16 + lr][16 * lg]);
 #pragma unroll
             for (int nt = 0; nt < 2; nt++)
 #pragma unroll
@@ -216,31 +185,19 @@ __global__ __launch_bounds__(256) void ppmm_mfma_kernel(PpmmArgs a, int c_tiles,
                     for (int jj = 0; jj < DC; jj++)
                         acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
         }
-        if (OVERLAP) {
-            // scheduling pattern for the block above: after each MFMA issue up to three other instructions
-            // (address arithmetic, asynchronous loads, digit split) while the matrix pipe works
-#pragma unroll
-            for (int i = 0; i < 4 * 2 * DW * DC; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
-                __builtin_amdgcn_sched_group_barrier(0x7f6, 3, 0);      // up to three non-MFMA instructions
-            }
-            wait_loads();
-        } else {
-            wait_loads();
-            split_digits(ksn, lds_raw0, B_nxt);
-            __syncthreads();
-        }
-        advance(ks1, im1);
+        // the loads issued one step ago (for step s+1) must have landed; the ones just issued may stay in flight
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (A_PER_WAVE + B_PER_WAVE));      // vmcnt(loads of one step)
+        __syncthreads();
         advance(ks2, im2);
     };
 
-    // r_last (residues modulo the last prime, < 2^39) of this lane's 32 outputs, kept in registers for the fused rescale
+    // r_last (residues modulo the last prime, < 2^39) of this lane's 16 outputs, kept in registers for the fused rescale
     // of the other primes: low words, and the 7 high bits packed four to a word.
-    unsigned rl_lo[4][4][2], rl_hi[4][2];
+    unsigned rl_lo[2][4][2], rl_hi[2][2];
     auto epilogue = [&](int im, auto last_c, auto full_c) {
         constexpr bool LAST = decltype(last_c)::value, FULL = decltype(full_c)::value;
         // The output addressing starts from a value the optimiser cannot hoist above the K loop (it would otherwise keep
-        // 32 row pointers alive across the loop and spill them).
+        // the row pointers alive across the loop).
         long row_stride = (long)a.mod_num * a.C;
         asm volatile("" : "+s"(row_stride));
         const PrimeConst& pr = a.pq[a.np + im];
@@ -248,10 +205,10 @@ __global__ __launch_bounds__(256) void ppmm_mfma_kernel(PpmmArgs a, int c_tiles,
         const double c24 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^24 mod q
         const double c48 = __longlong_as_double((long long)a.consts[3 * PPMM_MAX_MODS + im]);   // 2^48 mod q
         const double qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
-        const int mrow = m0 + wm * WM + 4 * lg;
-        u64* obase = a.out + (long)im * a.C + c0 + wc * WC + lr;
+        const int mrow = m0 + wm * 32 + 4 * lg;
+        u64* obase = a.out + (long)im * a.C + c0 + wc * 32 + lr;
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) {
+        for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int row = mrow + mt * 16 + r;
@@ -297,36 +254,40 @@ __global__ __launch_bounds__(256) void ppmm_mfma_kernel(PpmmArgs a, int c_tiles,
 #pragma unroll
         for (int e = 0; e < ND; e++)
 #pragma unroll
-            for (int mt = 0; mt < 4; mt++)
+            for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++) acc[e][mt][nt] = v4i{0, 0, 0, 0};
 
-        for (int ks = 0; ks < ksteps; ks += 2) {
+        for (int ks = 0; ks < ksteps; ks += 3) {
             kstep(std::integral_constant<int, 0>{});
             kstep(std::integral_constant<int, 1>{});
+            kstep(std::integral_constant<int, 2>{});
         }
 
         // ---- end of a prime: exact recombination, reduction mod q, fused rescale ----
         // Straight-line code (the prime-position and M-padding cases are resolved once, outside the unrolled loops) so that
-        // the 32 independent output chains of a lane can be interleaved.
+        // the independent output chains of a lane can be interleaved.
         const bool last = im == a.mod_num - 1, full = m0 + MT <= a.M;
         if (last) { if (full) epilogue(im, std::true_type{}, std::true_type{}); else epilogue(im, std::true_type{}, std::false_type{}); }
         else      { if (full) epilogue(im, std::false_type{}, std::true_type{}); else epilogue(im, std::false_type{}, std::false_type{}); }
     }
 }
 
+size_t ppmm_bdig_bytes(const PpmmArgs& a) { return (size_t)a.mod_num * a.Kpad * a.C * DCMAX; }
+
 template <int DW>
-static int launch_dw(hipStream_t stream, const PpmmArgs& a) {
+static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig) {
     const int c_tiles = (int)(a.C / CT), m_tiles = a.Mpad / MT;
+    hipLaunchKernelGGL(ppmm_pack_kernel, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
     const unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
-    hipLaunchKernelGGL(ppmm_mfma_kernel<DW>, dim3(blocks), dim3(256), 0, stream, a, c_tiles, m_tiles);
+    hipLaunchKernelGGL(ppmm_mfma_kernel<DW>, dim3(blocks), dim3(64 * NWAVES), 0, stream, a, (const int8_t*)bdig, c_tiles, m_tiles);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
 
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW) {
-    if (DW <= 3) return launch_dw<3>(stream, a);
-    return launch_dw<4>(stream, a);
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig) {
+    if (DW <= 3) return launch_dw<3>(stream, a, bdig);
+    return launch_dw<4>(stream, a, bdig);
 }
 
 }  // namespace ckks
