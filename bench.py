@@ -144,7 +144,7 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
-    import tests.params as P
+    import ckks_llm_amd.params as P
     value, ms_per_step, roofline, one_ct, limbs = bench_ntt(args, P)
     line = {
         "metric": "NTT limb-transforms/s @N=2^16", "value": round(value, 1), "unit": "limb-transforms/s", "n_gpus": 1,
