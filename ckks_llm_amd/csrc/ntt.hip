@@ -23,6 +23,8 @@
 //            |x| < 2^8 * q < 2^49 inside a pass and every integer involved stays below 2^53.
 // Between the two passes of one transform the buffer holds back-end specific words (lazy residues in [0,4q) /
 // [0,2q) for IntArith, raw double bit patterns for F64Arith); after the second pass it holds canonical residues.
+#include <cstdlib>
+
 #include "context.hpp"
 
 namespace ckks {
@@ -179,12 +181,14 @@ struct NttArgs {
     const void* tw;            // [prime][N] twiddles of the back end in use
     int start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len;
     long batch_stride_limbs;
+    unsigned limb_base, limbs_total;      // this launch covers limbs limb_base .. limb_base + gridDim.y - 1 of limbs_total
 };
 
 // limb index of this block -> base pointer and prime.  Limbs are ordered prime-major so that consecutive
 // workgroups reuse one prime's twiddle table while it is hot in L2.
 __device__ __forceinline__ u64* limb_ptr(const NttArgs& a, unsigned limb, long N, int& prime) {
-    unsigned per_mod = gridDim.y / a.mod_num;          // poly_num * batch
+    limb += a.limb_base;
+    unsigned per_mod = a.limbs_total / a.mod_num;      // poly_num * batch
     unsigned j = limb / per_mod, r = limb % per_mod;
     unsigned y = r % a.poly_num, z = r / a.poly_num;
     prime = a.start_mod_idx + (int)j;
@@ -311,21 +315,28 @@ __global__ __launch_bounds__(RowCfg<SB>::U * (RowCfg<SB>::ROWS < (1 << SA) ? Row
 }
 
 template <class AR, int SA, int SB>
-static int launch_two_pass(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse) {
+static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
     constexpr int N1 = 1 << SA, N2 = 1 << SB, CW = N2 < 16 ? N2 : 16;
     constexpr int RA = 1 << s1_of(SA);
     typedef RowCfg<SB> C;
     constexpr int ROWS = C::ROWS < N1 ? C::ROWS : N1;
-    dim3 gs(N2 / CW, limbs), bs((N1 / RA) * CW);
-    dim3 gr(N1 / ROWS, limbs), br(C::U * ROWS);
-    if (!inverse) {
-        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false>), gs, bs, 0, c->stream, args);
-        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false>), gr, br, 0, c->stream, args);
-    } else {
-        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true>), gr, br, 0, c->stream, args);
-        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true>), gs, bs, 0, c->stream, args);
+    static const int chunk_env = getenv("CKKS_NTT_CHUNK") ? atoi(getenv("CKKS_NTT_CHUNK")) : 0;
+    const int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs;
+    args.limbs_total = (unsigned)limbs;
+    for (int base = 0; base < limbs; base += chunk) {
+        const int n = limbs - base < chunk ? limbs - base : chunk;
+        args.limb_base = (unsigned)base;
+        dim3 gs(N2 / CW, n), bs((N1 / RA) * CW);
+        dim3 gr(N1 / ROWS, n), br(C::U * ROWS);
+        if (!inverse) {
+            hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false>), gs, bs, 0, c->stream, args);
+            if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
+            hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false>), gr, br, 0, c->stream, args);
+        } else {
+            hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true>), gr, br, 0, c->stream, args);
+            if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
+            hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true>), gs, bs, 0, c->stream, args);
+        }
     }
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;

@@ -12,11 +12,11 @@
 //
 // Two kernels compute it:
 //   * ppmm_mfma_kernel  - the dense path.  A is split once into DW balanced base-256 digits (int8 planes shared by
-//     all primes); residues are split on the fly into DC balanced digits (bytes of x + 0x80..80, each xor 0x80) while
-//     they are staged into LDS; v_mfma_i32_16x16x64_i8 accumulates the DW*DC digit products into DW+DC-1 int32
-//     anti-diagonal accumulators; the epilogue recombines them exactly and reduces modulo q_i.
+//     all primes); a first pass splits every residue into DC balanced digits (bytes of x + 0x80..80, each xor 0x80)
+//     laid out as the MFMA operand slabs; v_mfma_i32_16x16x64_i8 accumulates the DW*DC digit products into DW+DC-1
+//     int32 anti-diagonal accumulators; the epilogue recombines them exactly and reduces modulo q_i.
 //   * ppmm_generic_kernel - one output per lane with 128-bit accumulation, for shapes the MFMA tiling does not cover
-//     (C not a multiple of 64, primes of 41 bits and more, |A| >= 2^31).
+//     (C not a multiple of 64, primes of 40 bits and more, |A| >= 2^31, DW * Kin > 2^14).
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
@@ -250,8 +250,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             cst[PPMM_MAX_MODS + i] = H::shoup(cst[i], qi);
             cst[4 * PPMM_MAX_MODS + i] = dbits(cst[i], qi);
         }
-        cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 24, qi), qi);
-        cst[3 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 48, qi), qi);
+        cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 32, qi), qi);
     }
     uint64_t* d_cst = (uint64_t*)(h->d_absmax + 1);
     CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
@@ -272,7 +271,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
     const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
-                         (long)Kpad * 16384 * std::min(std::max(DW, 3), 5) < (1l << 31) && absmax < qmin && qmin > (1ull << 25);
+                         (long)Kpad * (DW <= 3 ? 3 : 4) <= 16384 && absmax < qmin && qmin > (1ull << 25);
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;

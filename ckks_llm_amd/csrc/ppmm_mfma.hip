@@ -7,7 +7,7 @@
 //     Ct[n][c] = sum_{j<DC} b_j[n][c] * 256^j ,  b_j in [-128,127]   (bytes of (x + 0x8080808080) xor 0x80, int8 planes built once per call)
 //     sum_n A*Ct = sum_{e<DW+DC-1} 256^e * S_e ,   S_e = sum_{d+j=e} sum_n a_d*b_j    (int32, |S_e| <= min(DW,DC)*Kin*2^14)
 // One v_mfma_i32_16x16x64_i8 per (d, j, 16x16 tile, 64 k) accumulates into the anti-diagonal accumulator S_{d+j}.
-// The epilogue recombines the S_e without rounding in FP64 (three diagonals at a time fit 48 bits), reduces modulo q_i
+// The epilogue recombines the S_e without rounding in FP64 (four diagonals at a time stay below 2^53), reduces modulo q_i
 // (q_i < 2^39) and applies the fused rescale (PPMM_kernel.cuh:213-249).
 //
 #include <type_traits>
@@ -21,12 +21,16 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int MT = 128, CT = 64, KS = 64;        // workgroup tile and K step
 constexpr int DCMAX = 5;
 
-typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 // 16 bytes per lane from global memory straight into LDS (no registers held while the load is in flight):
-// lane l of the wave writes lds_base + 16*l.  lds_base must be wave-uniform.
+// lane l of the wave writes lds_base + 16*l.  lds_base must be wave-uniform (it travels in M0).
+// Written as inline assembly on purpose: when the compiler sees LDS-DMA loads it makes every later LDS read that it cannot
+// prove disjoint wait for ALL outstanding loads (vmcnt(0)), which serialises the ring.  Here the waits are explicit: a
+// vmcnt(n) before the workgroup barrier that publishes a slot.  The compiler's own vmcnt bookkeeping stays safe because
+// loads complete in order: extra loads in flight can only make one of its waits longer, never shorter.
 __device__ __forceinline__ void async_copy16(const void* g, void* lds_base) {
-    __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds_base, 16, 0, 0);
+    const unsigned l = (unsigned)(size_t)(lptr_t)lds_base;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory");
 }
 
 __device__ __forceinline__ double mulmod_f64(double a, double w, double q, double qinv) {
@@ -119,13 +123,18 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);          // wave-uniform
     const int wm = wave >> 1, wc = wave & 1;
     const int lr = lane & 15, lg = lane >> 4;
+    const int frag_off = 16 * (lg ^ (((lr >> 1) + (lr >> 3)) & 3));                   // swizzled position of this lane's operand chunk
     const int ksteps = a.Kpad / KS;
     const long plane = (long)a.Mpad * a.Kpad;
     // plaintext digits: slab (d, rr) = rows 16*rr..+15 of digit d, 64 B each; lane -> row lane/4, 16-byte chunk lane%4
-    const int8_t* a_lane = a.Adig + (long)(m0 + (lane >> 2)) * a.Kpad + 16 * (lane & 3);
+    // LDS position (lane & 3) of slab row r = lane/4 receives the 16-byte chunk (lane & 3) ^ swz(r), swz(r) = ((r >> 1) + (r >> 3)) & 3:
+    // lanes reading one chunk of consecutive rows (64 B apart) then hit distinct 16-byte bank groups both within every aligned
+    // 8 lanes (128 B of banks) and within every aligned 16 lanes (256 B of banks).
+    const int swz_ld = (((lane >> 2) >> 1) + ((lane >> 2) >> 3)) & 3;
+    const int8_t* a_lane = a.Adig + (long)(m0 + (lane >> 2)) * a.Kpad + 16 * ((lane & 3) ^ swz_ld);
     // residue digits: [prime][K step][digit][column][64]; slab (jj, cc) = columns 16*cc..+15 of digit jj = 1 KiB contiguous
     const long b_step = (long)c_tiles * (DC * CT * KS);                 // bytes per (prime, K step)
-    const int8_t* b_lane = bdig + (long)c_tile * (DC * CT * KS) + 16 * lane;
+    const int8_t* b_lane = bdig + (long)c_tile * (DC * CT * KS) + 16 * (lane ^ swz_ld);
 
     auto issue = [&](int ks, int im, int8_t (*adst)[MT][KS], int8_t (*bdst)[CT][KS]) {
 #pragma unroll
@@ -166,17 +175,19 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
         int8_t (*B_cur)[CT][KS] = R == 0 ? lds_b0 : R == 1 ? lds_b1 : lds_b2;
         int8_t (*A_nxt)[MT][KS] = W == 0 ? lds_a0 : W == 1 ? lds_a1 : lds_a2;
         int8_t (*B_nxt)[CT][KS] = W == 0 ? lds_b0 : W == 1 ? lds_b1 : lds_b2;
+        // The refill of slot W is issued before any operand read of this step: an LDS read placed behind an asynchronous
+        // load in program order makes the compiler wait for every load in flight.
         issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
         v4i bf[2][DC];
 #pragma unroll
         for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16 + lr][16 * lg]);
+            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16 + lr][frag_off]);
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) {
             v4i af[DW];
 #pragma unroll
-            for (int d = 0; d < DW; d++) af[d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + mt * 16 + lr][16 * lg]);
+            for (int d = 0; d < DW; d++) af[d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + mt * 16 + lr][frag_off]);
 #pragma unroll
             for (int nt = 0; nt < 2; nt++)
 #pragma unroll
@@ -202,8 +213,7 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
         asm volatile("" : "+s"(row_stride));
         const PrimeConst& pr = a.pq[a.np + im];
         const double q = pr.qd, qinv = pr.qinv_d;
-        const double c24 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^24 mod q
-        const double c48 = __longlong_as_double((long long)a.consts[3 * PPMM_MAX_MODS + im]);   // 2^48 mod q
+        const double c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
         const double qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
         const int mrow = m0 + wm * 32 + 4 * lg;
         u64* obase = a.out + (long)im * a.C + c0 + wc * 32 + lr;
@@ -216,17 +226,15 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
                 u64* orow = obase + (long)(FULL || row < a.M ? row : a.M - 1) * row_stride;
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++) {
-                    double y[3] = {0.0, 0.0, 0.0};
+                    // Horner inside each group of four diagonals: y_g = sum_{i<4} 256^i S_{4g+i}; |S_e| <= DW * Kpad * 2^14 and the
+                    // launcher admits DW * Kpad < 2^15 only, so |y_g| < 2^53 and every step is exact
+                    double y0 = (double)acc[3][mt][nt][r], y1 = (double)acc[ND - 1][mt][nt][r];
 #pragma unroll
-                    for (int e = ND - 1; e >= 0; e--) {
-                        // Horner inside each group of three diagonals: y_g = S_3g + 256*S_3g+1 + 65536*S_3g+2  (|y_g| < 2^48, exact)
-                        const int g = e / 3;
-                        y[g] = __builtin_fma(y[g], 256.0, (double)acc[e][mt][nt][r]);
-                    }
-                    double t = balance_f64(y[0], q, qinv);
-                    if (ND > 3) t += mulmod_f64(y[1], c24, q, qinv);
-                    if (ND > 6) t += mulmod_f64(y[2], c48, q, qinv);
-                    t = balance_f64(t, q, qinv);                                           // in (-0.51 q, 0.51 q)
+                    for (int e = 2; e >= 0; e--) y0 = __builtin_fma(y0, 256.0, (double)acc[e][mt][nt][r]);
+#pragma unroll
+                    for (int e = ND - 2; e >= 4; e--) y1 = __builtin_fma(y1, 256.0, (double)acc[e][mt][nt][r]);
+                    // |y0 + (y1 * 2^32 mod q)| < 2^53 + 0.51 q: one exact addition, one reduction to (-0.51 q, 0.51 q)
+                    double t = balance_f64(y0 + mulmod_f64(y1, c32, q, qinv), q, qinv);
                     double res;
                     if (LAST) {
                         res = t;
@@ -238,7 +246,8 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
                         res = mulmod_f64(t - rlast, qli, q, qinv);
                     }
                     res = res < 0.0 ? res + q : res;
-                    const u64 ures = (u64)(long long)res;
+                    // res is an integer in [0, q): adding 2^52 leaves it in the low mantissa bits
+                    const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFull;
                     if (LAST) {
                         rl_lo[mt][r][nt] = (unsigned)ures;
                         rl_hi[mt][nt] = (r == 0 ? 0u : rl_hi[mt][nt]) | ((unsigned)(ures >> 32) << (8 * r));
