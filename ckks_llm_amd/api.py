@@ -122,6 +122,14 @@ class Context_23:
     def set_arith_mode(self, mode):
         _check(self.L_.ckks_ctx_set_arith_mode(self.h, mode), "ckks_ctx_set_arith_mode")
 
+    def set_ntt_mode(self, mode):
+        """0: automatic, 1: two launches per transform, 2: one fused launch wherever that kernel exists."""
+        _check(self.L_.ckks_ctx_set_ntt_mode(self.h, mode), "ckks_ctx_set_ntt_mode")
+
+    def check(self):
+        """Synchronise the context's stream; raises if a bounded wait of the one-launch transform ran out."""
+        _check(self.L_.ckks_ctx_check(self.h), "ckks_ctx_check")
+
     def set_stream(self, stream_handle):
         _check(self.L_.ckks_set_stream(self.h, stream_handle), "ckks_set_stream")
 

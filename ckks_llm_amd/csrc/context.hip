@@ -304,6 +304,11 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         std::vector<u64> z = c->qiInvModql; z.insert(z.end(), qiInv_s.begin(), qiInv_s.end());
         up(upload(&c->d_qiInvModql, z));
     }
+    if (rc == CKKS_OK) {
+        if (hipMalloc(&c->d_ntt_sched, ckks::ntt_sched_bytes()) != hipSuccess || hipMemset(c->d_ntt_sched, 0, ckks::ntt_sched_bytes()) != hipSuccess) rc = CKKS_E_NOMEM;
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) c->cu_count = cus;
+    }
     if (rc == CKKS_OK && hipEventCreate(&c->ev0) != hipSuccess) rc = CKKS_E_HIP;
     if (rc == CKKS_OK && hipEventCreate(&c->ev1) != hipSuccess) rc = CKKS_E_HIP;
     if (rc == CKKS_OK && hipEventCreate(&c->ev_mid) != hipSuccess) rc = CKKS_E_HIP;
@@ -316,7 +321,7 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     if (!c) return CKKS_OK;
     (void)hipDeviceSynchronize();
     void* ptrs[] = {c->d_primes, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
-                    c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql};
+                    c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_sched};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
@@ -338,7 +343,7 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
     else if (n == "p_num") *value = c->p_num; else if (n == "q_num") *value = c->q_num; else if (n == "t_num") *value = c->t_num;
     else if (n == "gamma") *value = c->gamma; else if (n == "dnum") *value = c->dnum;
     else if (n == "Ri_blockNum") *value = c->Ri_blockNum; else if (n == "Qj_blockNum") *value = c->Qj_blockNum;
-    else if (n == "arith_mode") *value = c->arith_mode;
+    else if (n == "arith_mode") *value = c->arith_mode; else if (n == "ntt_mode") *value = c->ntt_mode;
     else { ckks::set_error("ckks_ctx_info: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
@@ -347,6 +352,29 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
 extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
     if (!c || mode < 0 || mode > 1) return CKKS_E_INVALID;
     c->arith_mode = mode;
+    return CKKS_OK;
+}
+
+// test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = the fused launch wherever it exists (N >= 2^15)
+extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
+    if (!c || mode < 0 || mode > 2) return CKKS_E_INVALID;
+    c->ntt_mode = mode;
+    return CKKS_OK;
+}
+
+// Waits for the context's stream and reports a scheduler wait of the fused NTT kernel that ran out (the transforms of
+// that launch are then incomplete).  The flag is cleared by the call.
+extern "C" int ckks_ctx_check(ckks_ctx* c) {
+    if (!c) return CKKS_E_INVALID;
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
+    unsigned err = 0;
+    char* word = (char*)c->d_ntt_sched + ckks::ntt_sched_error_offset();
+    CKKS_HIP_TRY(hipMemcpy(&err, word, sizeof(err), hipMemcpyDeviceToHost));
+    if (err) {
+        CKKS_HIP_TRY(hipMemset(c->d_ntt_sched, 0, ckks::ntt_sched_bytes()));
+        ckks::set_error("fused NTT: a scheduler wait ran out; the last transforms are incomplete");
+        return CKKS_E_UNAVAILABLE;
+    }
     return CKKS_OK;
 }
 

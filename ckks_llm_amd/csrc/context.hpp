@@ -77,6 +77,9 @@ struct ckks_ctx {
     size_t qiInv_count = 0;
 
     int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
+    int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: fused launch wherever it exists
+    int cu_count = 256;
+    void* d_ntt_sched = nullptr;          // scheduler words of the fused NTT kernel (zero between launches)
 };
 
 namespace ckks {
@@ -89,6 +92,8 @@ int hip_fail(hipError_t e, const char* what);
     } while (0)
 
 // launchers (ntt.hip, basisconv.hip)
+size_t ntt_sched_bytes();
+size_t ntt_sched_error_offset();
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
 }  // namespace ckks

@@ -30,6 +30,7 @@ extern "C" {
 #define CKKS_E_HIP (-2)       /* a HIP runtime call failed */
 #define CKKS_E_NOMEM (-3)
 #define CKKS_E_STATE (-4)     /* e.g. missing key / level-0 operand: the C++ shell maps it to std::invalid_argument */
+#define CKKS_E_UNAVAILABLE (-5) /* a code path that this build has switched off, or a device-side wait that ran out */
 
 typedef struct ckks_ctx ckks_ctx;
 typedef struct pcmm_ctx pcmm_ctx;
@@ -62,6 +63,14 @@ int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
 /* 0 (default): FP64 butterflies for primes < 2^41, integer butterflies otherwise; 1: integer butterflies everywhere.
  * Both give the same residues; the switch exists for testing and tuning. */
 int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
+/* 0 (default) and 1: two launches per transform.  2: both passes in one launch with the limb held in the XCD's L2 between
+ * them - switched off in this build (its launches did not complete on MI355X), transforms then return CKKS_E_UNAVAILABLE.
+ * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
+int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
+/* Synchronises the context's stream and returns CKKS_E_UNAVAILABLE if a bounded scheduler wait of the one-launch transform
+ * ran out (its outputs are then incomplete); clears the condition.  Plays the part of the reference's
+ * cudaDeviceSynchronize + cudaGetLastError checks (Utils.cuh CUDA_CHECK). */
+int ckks_ctx_check(ckks_ctx* ctx);
 /* host copy of a constant table, flattened in the reference's device layout (names as in ckks_oracle.h /
  * Context_23.h: "pqt","psi","psi_table","psiinv_table","RiHatInv","QjHatModT",...). *count receives the length. */
 int ckks_ctx_table(const ckks_ctx* ctx, const char* name, uint64_t* host_out, size_t cap, size_t* count);

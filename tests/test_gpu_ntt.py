@@ -97,6 +97,55 @@ def test_reference_addressing_and_ext_variant():
     assert np.array_equal(from_dev(d2, e_h.shape), want) and np.array_equal(want, e_h)
 
 
+@pytest.mark.skip(reason="the one-launch transform is switched off: its launches did not complete on MI355X (ended by the "
+                         "test time-out twice, the second time with all scheduler waits bounded to 20 ms); cause not shown yet")
+@pytest.mark.parametrize("logN,polys,mode", [(16, 9, 0), (16, 5, 1), (15, 7, 0), (15, 3, 1)])
+def test_one_launch_transform_matches_two_launch_and_oracle(logN, polys, mode):
+    """The fused kernel (both passes in one launch, inter-pass data in L2, ticket scheduler) against the oracle and
+    against the two-launch path, both directions, both arithmetic back ends; two launches in a row reuse the
+    scheduler words the kernel restores at exit."""
+    q = CFG2_Q[:5]
+    pair = Pair(logN, [], q)
+    N, L1 = pair.N, len(q)
+    pair.dev.set_arith_mode(mode)
+    data = limbs_uniform(40 + logN, q, polys, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, L1, L1)
+    want_inv = data.copy()
+    pair.orc.FromNTTInplace(want_inv.reshape(-1), 0, 0, polys, L1, L1)
+    pair.dev.set_ntt_mode(2)
+    buf = to_dev(data)
+    pair.dev.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+    pair.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), want)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    pair.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), data)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    pair.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), want_inv)
+    # a sub-range of limbs with the reference addressing: primes 1..3 of polys 0..polys-1
+    buf.upload(data)
+    pair.dev.ToNTTInplace(buf, 1, 1, polys, 3, L1)
+    pair.dev.check()
+    got = from_dev(buf, data.shape)
+    assert np.array_equal(got[:, 1:4], want[:, 1:4]) and np.array_equal(got[:, 0], data[:, 0]) and np.array_equal(got[:, 4], data[:, 4])
+    buf.free()
+
+
+def test_one_launch_mode_reports_that_it_is_switched_off():
+    from ckks_llm_amd import CkksError
+    pair = Pair(15, [], CFG2_Q[:2])
+    d = to_dev(np.zeros((1, 2, pair.N), dtype=np.uint64))
+    pair.dev.set_ntt_mode(2)
+    with pytest.raises(CkksError):
+        pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)
+    pair.dev.set_ntt_mode(0)
+    pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)
+    pair.dev.check()
+    assert not from_dev(d, (2, pair.N)).any()
+
+
 def test_tables_match_oracle():
     P = REF_PARAMS[14]
     pair = Pair(10, P["p"], P["q"], P["t"], P["gamma"])
@@ -158,4 +207,5 @@ def test_full_size_properties_batch32():
     for j, q in enumerate(CFG2_Q):
         assert np.array_equal(fs[0, j], (got[0, j] + got[1, j]) % np.uint64(q))
     pair.dev.FromNTTInplace(d, 0, 0, 2 * B, L1, L1)
+    pair.dev.check()
     assert np.array_equal(from_dev(d, data.shape), data)
