@@ -123,7 +123,8 @@ class Context_23:
         _check(self.L_.ckks_ctx_set_arith_mode(self.h, mode), "ckks_ctx_set_arith_mode")
 
     def set_ntt_mode(self, mode):
-        """0: automatic, 1: two launches per transform, 2: one fused launch wherever that kernel exists."""
+        """0: automatic, 1: two launches per transform, 2: ticket-scheduled one-launch transform (switched off),
+        3: one workgroup per limb wherever that kernel exists (N >= 2^15)."""
         _check(self.L_.ckks_ctx_set_ntt_mode(self.h, mode), "ckks_ctx_set_ntt_mode")
 
     def check(self):

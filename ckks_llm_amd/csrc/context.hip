@@ -355,9 +355,10 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
     return CKKS_OK;
 }
 
-// test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = the fused launch wherever it exists (N >= 2^15)
+// test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = ticket-scheduled one-launch transform (switched off),
+// 3 = one workgroup per limb wherever that kernel exists (N >= 2^15)
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
-    if (!c || mode < 0 || mode > 2) return CKKS_E_INVALID;
+    if (!c || mode < 0 || mode > 3) return CKKS_E_INVALID;
     c->ntt_mode = mode;
     return CKKS_OK;
 }

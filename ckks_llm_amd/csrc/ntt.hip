@@ -220,11 +220,11 @@ struct StridedCfg {
 
 template <class AR, int SA, int SB, bool INVERSE, bool COHERENT>
 __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                             typename AR::V* lds) {
+                                             typename AR::V* lds, unsigned tid) {
     typedef StridedCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     typedef typename AR::V V;
-    const unsigned cl = threadIdx.x % CW, g = threadIdx.x / CW;
+    const unsigned cl = tid % CW, g = tid / CW;
     u64* col = limb + tile * CW + cl;
     V v[R];
     if (!INVERSE) {
@@ -267,7 +267,7 @@ __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pas
     int prime;
     u64* limb = limb_ptr(a, blockIdx.y, N, prime);
     const AR ar(a.primes[prime]);
-    strided_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds);
+    strided_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -285,11 +285,11 @@ __device__ __forceinline__ int padded(int pos) { return pos + (pos >> 4); }
 
 template <class AR, int SA, int SB, bool INVERSE, bool COHERENT>
 __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                         typename AR::V* lds) {
+                                         typename AR::V* lds, unsigned tid) {
     typedef RowCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     typedef typename AR::V V;
-    const unsigned u = threadIdx.x % U, rl = threadIdx.x / U;
+    const unsigned u = tid % U, rl = tid / U;
     const unsigned row = tile * ROWS + rl;
     u64* rp = limb + (long)row * N2;
     V* lrow = lds + rl * C::PITCH;
@@ -338,7 +338,52 @@ __global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass(NttArg
     int prime;
     u64* limb = limb_ptr(a, blockIdx.y, N, prime);
     const AR ar(a.primes[prime]);
-    row_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds);
+    row_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x);
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Whole-limb transform: one workgroup carries one limb through both passes in one launch.
+//
+// The workgroup is GROUPS groups of 256 lanes; each group takes every GROUPS-th tile of the first pass, the workgroup waits
+// until all its stores have left the compute unit, then the groups take the tiles of the second pass.  Nothing is exchanged
+// between workgroups, so there is no synchronisation beyond the workgroup barrier.  Between the passes the limb is not
+// read back from HBM: its lines are still in the XCD's L2 or, once displaced from there, in the memory-side cache, because
+// only (resident workgroups) x N x 8 bytes are in that state at any time.  The second-pass loads bypass the L1, which may
+// still hold pre-transform copies of the same lines from the first pass of this very workgroup.
+// ------------------------------------------------------------------------------------------------------------
+template <class AR, int SA, int SB, bool INVERSE, int GROUPS>
+__global__ __launch_bounds__(256 * GROUPS) void ntt_limb_kernel(NttArgs a) {
+    typedef StridedCfg<SA, SB> CS;
+    typedef RowCfg<SA, SB> CR;
+    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES, "whole-limb kernel: tile shapes must agree");
+    static_assert(CS::TILES % GROUPS == 0, "whole-limb kernel: tiles must divide among the groups");
+    constexpr int TILES = CS::TILES;
+    constexpr long N = 1l << (SA + SB);
+    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
+    typedef typename AR::TW TW;
+    __shared__ typename AR::V lds_all[GROUPS][LDS_WORDS];
+    const unsigned grp = threadIdx.x / 256, tid = threadIdx.x % 256;
+    typename AR::V* lds = lds_all[grp];
+    int prime;
+    u64* limb = limb_ptr(a, blockIdx.x, N, prime);
+    const AR ar(a.primes[prime]);
+    const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
+#pragma unroll 1
+    for (int t = grp; t < TILES; t += GROUPS) {
+        if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, t, tw, ar, lds, tid);
+        else row_tile<AR, SA, SB, true, false>(limb, t, tw, ar, lds, tid);
+        __syncthreads();
+    }
+    // every store of the first pass has been acknowledged by the L2 before any lane starts the second pass
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+#pragma unroll 1
+    for (int t = grp; t < TILES; t += GROUPS) {
+        if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, t, tw, ar, lds, tid);
+        else strided_tile<AR, SA, SB, true, true>(limb, t, tw, ar, lds, tid);
+        __syncthreads();
+    }
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -439,16 +484,16 @@ __global__ __launch_bounds__(256) void ntt_fused_kernel(NttArgs a, NttSched* sch
         const AR ar(a.primes[prime]);
         const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
         if (!second) {
-            if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds);
-            else row_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds);
+            if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
+            else row_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
             // all stores of this tile have reached the L2 before the completion count moves
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
             if (threadIdx.x == 0) atomicAdd(&sched->done[limb_id], 1u);
         } else {
-            if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, tile, tw, ar, lds);
-            else strided_tile<AR, SA, SB, true, true>(limb, tile, tw, ar, lds);
+            if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, tile, tw, ar, lds, threadIdx.x);
+            else strided_tile<AR, SA, SB, true, true>(limb, tile, tw, ar, lds, threadIdx.x);
             __syncthreads();
         }
     }
@@ -509,6 +554,22 @@ static int launch_fused(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
     return CKKS_OK;
 }
 
+template <class AR, int SA, int SB>
+static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
+    static const int groups_env = getenv("CKKS_NTT_GROUPS") ? atoi(getenv("CKKS_NTT_GROUPS")) : 0;
+    args.limb_base = 0;
+    args.limbs_total = (unsigned)limbs;
+    if (groups_env == 2) {
+        if (!inverse) hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, false, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
+        else hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, true, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
+    } else {
+        if (!inverse) hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, false, 4>), dim3(limbs), dim3(1024), 0, c->stream, args);
+        else hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, true, 4>), dim3(limbs), dim3(1024), 0, c->stream, args);
+    }
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+
 // the word of the scheduler block that a bounded wait sets when it runs out
 size_t ntt_sched_error_offset() { return offsetof(NttSched, error); }
 
@@ -520,6 +581,12 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
     if (c->ntt_mode == 2) {
         set_error("NTT: the one-launch transform is switched off in this build (its launches did not complete on MI355X)");
         return CKKS_E_UNAVAILABLE;
+    }
+    // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
+    // (the limbs in flight, 0.5 MiB per resident workgroup, exceed the L2 by far), so the automatic mode does not pick it.
+    if (!c->ev_mid_armed && c->ntt_mode == 3) {
+        if (c->logN == 16) return launch_whole_limb<AR, 8, 8>(c, args, limbs, inverse);
+        if (c->logN == 15) return launch_whole_limb<AR, 8, 7>(c, args, limbs, inverse);
     }
     constexpr bool fused_enabled = false;
     if (fused_enabled && c->d_ntt_sched && !c->ev_mid_armed && limbs >= 96) {

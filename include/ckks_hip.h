@@ -63,8 +63,10 @@ int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
 /* 0 (default): FP64 butterflies for primes < 2^41, integer butterflies otherwise; 1: integer butterflies everywhere.
  * Both give the same residues; the switch exists for testing and tuning. */
 int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
-/* 0 (default) and 1: two launches per transform.  2: both passes in one launch with the limb held in the XCD's L2 between
- * them - switched off in this build (its launches did not complete on MI355X), transforms then return CKKS_E_UNAVAILABLE.
+/* How a transform is launched.  0 (default) and 1: two launches, one per pass.  3: one workgroup carries a limb through
+ * both passes in one launch (N >= 2^15; same residues, slower at large batches).  2: both passes in one launch with the
+ * limb held in the XCD's L2 between them under a ticket scheduler - switched off in this build (its launches did not
+ * complete on MI355X): transforms then return CKKS_E_UNAVAILABLE.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
 /* Synchronises the context's stream and returns CKKS_E_UNAVAILABLE if a bounded scheduler wait of the one-launch transform

@@ -133,6 +133,34 @@ def test_one_launch_transform_matches_two_launch_and_oracle(logN, polys, mode):
     buf.free()
 
 
+@pytest.mark.parametrize("logN,polys,mode", [(16, 9, 0), (16, 5, 1), (15, 7, 0), (15, 3, 1)])
+def test_whole_limb_transform_matches_oracle(logN, polys, mode):
+    """One workgroup per limb, both passes in one launch (ntt_mode 3): against the oracle, both directions, both arithmetic
+    back ends, and with the reference's sub-range addressing."""
+    q = CFG2_Q[:5]
+    pair = Pair(logN, [], q)
+    N, L1 = pair.N, len(q)
+    pair.dev.set_arith_mode(mode)
+    data = limbs_uniform(40 + logN, q, polys, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, L1, L1)
+    want_inv = data.copy()
+    pair.orc.FromNTTInplace(want_inv.reshape(-1), 0, 0, polys, L1, L1)
+    pair.dev.set_ntt_mode(3)
+    buf = to_dev(data)
+    pair.dev.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+    assert np.array_equal(from_dev(buf, data.shape), want)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    assert np.array_equal(from_dev(buf, data.shape), data)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    assert np.array_equal(from_dev(buf, data.shape), want_inv)
+    buf.upload(data)
+    pair.dev.ToNTTInplace(buf, 1, 1, polys, 3, L1)
+    got = from_dev(buf, data.shape)
+    assert np.array_equal(got[:, 1:4], want[:, 1:4]) and np.array_equal(got[:, 0], data[:, 0]) and np.array_equal(got[:, 4], data[:, 4])
+    buf.free()
+
+
 def test_one_launch_mode_reports_that_it_is_switched_off():
     from ckks_llm_amd import CkksError
     pair = Pair(15, [], CFG2_Q[:2])
@@ -209,3 +237,9 @@ def test_full_size_properties_batch32():
     pair.dev.FromNTTInplace(d, 0, 0, 2 * B, L1, L1)
     pair.dev.check()
     assert np.array_equal(from_dev(d, data.shape), data)
+    # the two-launch path and the whole-limb path give the same residues on the whole batch
+    for m in (1, 3):
+        pair.dev.set_ntt_mode(m)
+        pair.dev.ToNTTInplace(d, 0, 0, 2 * B, L1, L1)
+        assert np.array_equal(from_dev(d, data.shape), got), m
+        pair.dev.FromNTTInplace(d, 0, 0, 2 * B, L1, L1)
