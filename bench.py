@@ -25,6 +25,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes moved by ONE pass launch of the default workload (1536 limbs), from the rocprofv3 counters FETCH_SIZE and
+# WRITE_SIZE of that launch, each scaled by what the same counter reads for a device-to-device copy of known size in the
+# same run (FETCH_SIZE reads 0.502 of the bytes copied, WRITE_SIZE 1.000): 768 MiB read + 12 MiB twiddles, 768 MiB written.
+NTT_PASS_TRAFFIC_BYTES_1536_LIMBS = 1.623e9
 MFMA_I8_PEAK_TMACS = 2516.6          # 5.033 POP/s dense int8 = 2.5166e15 MAC/s
 
 
@@ -80,11 +84,18 @@ def bench_ntt(args, P):
     dom_name, dom_ms = max([("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2)], key=lambda x: x[1])
     achieved = alg_bytes_launch / (dom_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": NTT_PASS_TRAFFIC_BYTES_1536_LIMBS if limbs == 1536 else None,
                 "kernel_ms": {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)},
                 "transform_algorithmic_GBps": {"fwd": round(16.0 * N * limbs / ((f1 + f2) * 1e-3) / 1e9, 1),
                                                "inv": round(16.0 * N * limbs / ((i1 + i2) * 1e-3) / 1e9, 1)},
                 "algorithmic_bytes_per_launch": alg_bytes_launch}
+    if args.batch_only:
+        # reference point for the traffic counters: one device-to-device copy of known size in the same process
+        half = 4 * limbs * N
+        buf.L_.ckks_memcpy_d2d(buf.ptr + half, buf.ptr, half)
+        ctx.sync()
+        buf.free()
+        return value, ms_per_step, roofline, None, limbs
     # one ciphertext (48 limbs, 24 MiB): the latency-oriented half of configs[1]
     one_ct = {}
     small = DeviceBuffer.from_numpy(one)
@@ -140,6 +151,9 @@ def main():
     ap.add_argument("--batch", type=int, default=32, help="ciphertexts per step (BASELINE configs[1]: 32)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extra", action="store_true", help="skip the PPMM / key-switch side measurements")
+    ap.add_argument("--batch-only", action="store_true",
+                    help="profiling aid: only the batched NTT launches (no one-ciphertext, PPMM, key-switch or CPU legs), plus one "
+                         "device-to-device copy of half the batch as the reference point of the traffic counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -155,6 +169,9 @@ def main():
         "roofline": roofline, "one_ciphertext": one_ct,
         "frac_of_hbm_roofline_whole_transform": round(value * 16 * 65536 / 1e9 / HBM_PEAK_GBS, 4),
     }
+    if args.batch_only:
+        del line["one_ciphertext"]
+        args.skip_extra = args.skip_cpu = True
     if not args.skip_extra:
         try:
             import bench_extra
