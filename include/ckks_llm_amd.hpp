@@ -1,0 +1,266 @@
+// C++ host mirror of the reference's classes for the NTT -> key switch -> PCMM path, on top of the C ABI (ckks_hip.h).
+//
+// Same class names, member names, argument order and addressing as the reference's headers, so that code written
+// against Context_23.h / Scheme_23.h / pcmm/PCMM_Scheme.h compiles against this header with
+// `using namespace ckks_llm_amd;`.  Differences, all deliberate:
+//   * primes are passed to the constructor (the reference selects a compiled-in set by logN, Context_23.cuh:12-113);
+//   * tables live in the handle, not in process-global __constant__ symbols, so several contexts can coexist;
+//   * scales are long double (the reference uses NTL::RR only for this bookkeeping, Ciphertext.cuh:23);
+//   * C-ABI error codes become exceptions: std::invalid_argument where the reference throws it
+//     (KeySwitch_23.cuh:194-201, Scheme_23.cuh:192-194), std::runtime_error for everything the reference never checks.
+// Header-only, no HIP headers needed: any C++17 host compiler can build against it and link libckks_hip.so.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <iostream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ckks_hip.h"
+
+namespace ckks_llm_amd {
+
+typedef uint64_t uint64_tt;
+
+inline void check(int rc, const char* what) {
+    if (rc == CKKS_OK) return;
+    std::string msg = std::string(what) + ": " + ckks_last_error();
+    if (rc == CKKS_E_STATE) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
+}
+
+inline uint64_tt* device_alloc_words(size_t words) {
+    void* p = nullptr;
+    check(ckks_malloc(&p, sizeof(uint64_tt) * (words ? words : 1)), "ckks_malloc");
+    return static_cast<uint64_tt*>(p);
+}
+inline void device_release(uint64_tt*& p) {
+    if (!p) return;
+    ckks_sync();                       // the reference synchronises around every cudaFree (Ciphertext.cuh:88-99)
+    ckks_free(p);
+    p = nullptr;
+}
+
+// Context_23 (Context_23.h:19-279): prime sets, tables, NTT and basis conversion.
+class Context_23 {
+public:
+    long logN, N;
+    int p_num, q_num, t_num, gamma, K, L, dnum, Ri_blockNum, Qj_blockNum;
+    std::vector<uint64_tt> pVec, qVec, tVec;
+    ckks_ctx* handle = nullptr;
+
+    Context_23(long logN, const std::vector<uint64_tt>& p, const std::vector<uint64_tt>& q,
+               const std::vector<uint64_tt>& t = {}, int gamma = 0)
+        : logN(logN), N(1l << logN), p_num((int)p.size()), q_num((int)q.size()), t_num((int)t.size()), gamma(gamma),
+          K((int)p.size()), L((int)q.size() - 1), pVec(p), qVec(q), tVec(t) {
+        check(ckks_ctx_create(&handle, (int)logN, p.data(), p_num, q.data(), q_num, t.data(), t_num, gamma), "Context_23");
+        dnum = (int)info("dnum");
+        Ri_blockNum = (int)info("Ri_blockNum");
+        Qj_blockNum = (int)info("Qj_blockNum");
+    }
+    Context_23(const Context_23&) = delete;
+    Context_23& operator=(const Context_23&) = delete;
+    ~Context_23() { if (handle) ckks_ctx_destroy(handle); }
+
+    long info(const char* name) const {
+        long v = 0;
+        check(ckks_ctx_info(handle, name, &v), "ckks_ctx_info");
+        return v;
+    }
+
+    // Context_23.h:42-45
+    void ToNTTInplace(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len) {
+        check(ckks_ntt_fwd(handle, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ToNTTInplace");
+    }
+    void FromNTTInplace(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len) {
+        check(ckks_ntt_inv(handle, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "FromNTTInplace");
+    }
+    void ToNTTInplace_for_externalProduct(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                                          int poly_mod_len, int cipher_mod_num, int batch_size) {
+        check(ckks_ntt_fwd_ext(handle, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, cipher_mod_num,
+                               batch_size), "ToNTTInplace_for_externalProduct");
+    }
+    void FromNTTInplace_for_externalProduct(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                                            int poly_mod_len, int cipher_mod_num, int batch_size) {
+        check(ckks_ntt_inv_ext(handle, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, cipher_mod_num,
+                               batch_size), "FromNTTInplace_for_externalProduct");
+    }
+    // Context_23.h:54-61
+    void modUpPQtoT_23(uint64_tt* output, const uint64_tt* input, int l, int batch_size) {
+        check(ckks_modup_pq_to_t(handle, output, input, l, batch_size), "modUpPQtoT_23");
+    }
+    void modUpQjtoT_23(uint64_tt* output, const uint64_tt* input, int l, int batch_size) {
+        check(ckks_modup_qj_to_t(handle, output, input, l, batch_size), "modUpQjtoT_23");
+    }
+    void modUpTtoPQl_23(uint64_tt* modUp_TtoQj_buffer, const uint64_tt* exProduct_T_temp, int l, int batch_size) {
+        check(ckks_modup_t_to_pql(handle, modUp_TtoQj_buffer, exProduct_T_temp, l, batch_size), "modUpTtoPQl_23");
+    }
+    void modDownPQltoQl_23(uint64_tt* output, const uint64_tt* modUp_TtoQj_buffer, int l, int batch_size) {
+        check(ckks_moddown_pql_to_ql(handle, output, modUp_TtoQj_buffer, l, batch_size), "modDownPQltoQl_23");
+    }
+    void external_product_T(uint64_tt* output, const uint64_tt* cipher_modUp_QjtoT, const uint64_tt* swk_modUp_RitoT, int l) {
+        check(ckks_external_product_t(handle, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l), "external_product_T");
+    }
+};
+
+// Ciphertext (Ciphertext.cuh:5-99): one device buffer [a: L+1 limbs | b: L+1 limbs].
+class Ciphertext {
+public:
+    uint64_tt* ax_device = nullptr;
+    uint64_tt* bx_device = nullptr;
+    uint64_tt* cipher_device = nullptr;
+    int N = 0, l = 0, L = 0, slots = 0;
+    long double scale = 0;
+
+    Ciphertext() {}
+    Ciphertext(int N, int L, int l, int slots, long double scale) : N(N), l(l), L(L), slots(slots), scale(scale) {
+        cipher_device = device_alloc_words((size_t)N * (L + 1) * 2);
+        ax_device = cipher_device;
+        bx_device = cipher_device + (size_t)N * (L + 1);
+    }
+    Ciphertext(const Ciphertext& c) : Ciphertext(c.N, c.L, c.l, c.slots, c.scale) {
+        check(ckks_memcpy_d2d(cipher_device, c.cipher_device, sizeof(uint64_tt) * (size_t)N * (L + 1) * 2), "Ciphertext copy");
+    }
+    Ciphertext& operator=(const Ciphertext&) = delete;
+    virtual ~Ciphertext() { device_release(cipher_device); }
+};
+
+// MLWECiphertext (pcmm/MLWECiphertext.cuh:6-78): [(L+1) moduli][a_0 .. a_{k-1}, b][N1].
+class MLWECiphertext {
+public:
+    uint64_tt* cipher_device = nullptr;
+    int N1 = 0, L = 0, l = 0, k = 0;
+    long double scale = 0;
+
+    MLWECiphertext() {}
+    MLWECiphertext(int N1, int L, int l, int k, long double scale) : N1(N1), L(L), l(l), k(k), scale(scale) {
+        cipher_device = device_alloc_words((size_t)N1 * (L + 1) * (k + 1));
+    }
+    MLWECiphertext(const MLWECiphertext&) = delete;
+    MLWECiphertext& operator=(const MLWECiphertext&) = delete;
+    virtual ~MLWECiphertext() { device_release(cipher_device); }
+};
+
+// The members of Scheme_23 on the path (Scheme_23.h:113-182): rescale and the key-switch chain of mult_23.
+class Scheme_23 {
+public:
+    Context_23& context;
+    // Scheme_23::mallocMemory (Scheme_23.cuh:7-51): scratch owned by the scheme
+    uint64_tt* rescale_buffer = nullptr;
+    uint64_tt* modUp_QjtoT_temp = nullptr;
+    uint64_tt* exProduct_T_temp = nullptr;
+    uint64_tt* modUp_TtoQj_buffer = nullptr;
+
+    explicit Scheme_23(Context_23& context) : context(context) {
+        const size_t N = (size_t)context.N;
+        rescale_buffer = device_alloc_words(2 * N * (context.L + 1));
+        if (context.t_num > 0) {
+            modUp_QjtoT_temp = device_alloc_words(N * context.t_num * context.Qj_blockNum);
+            exProduct_T_temp = device_alloc_words(N * context.t_num * context.Ri_blockNum * 2);
+            modUp_TtoQj_buffer = device_alloc_words(N * context.t_num * context.Ri_blockNum * 2);
+        }
+    }
+    Scheme_23(const Scheme_23&) = delete;
+    ~Scheme_23() {
+        device_release(rescale_buffer);
+        device_release(modUp_QjtoT_temp);
+        device_release(exProduct_T_temp);
+        device_release(modUp_TtoQj_buffer);
+    }
+
+    // Scheme_23::rescaleAndEqual (Scheme_23.cuh:369-385); throws std::invalid_argument on level 0 (:192-194 style)
+    void rescaleAndEqual(Ciphertext& cipher) {
+        check(ckks_rescale(context.handle, cipher.cipher_device, rescale_buffer, cipher.l), "rescaleAndEqual");
+        cipher.scale /= (long double)context.qVec[cipher.l];
+        cipher.l -= 1;
+    }
+    // steps 2..9 of Scheme_23::mult_23 (KeySwitch_23.cuh:219-231): d2 (NTT domain, L+1 limbs) -> out = [a | b].
+    // A null key throws std::invalid_argument as the missing rotation / relinearisation key does (:198-201).
+    void keySwitch_23(uint64_tt* out, uint64_tt* d2, const uint64_tt* swk, int l) {
+        check(ckks_keyswitch_23(context.handle, out, d2, swk, l, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer), "keySwitch_23");
+    }
+};
+
+// PCMM_Context (pcmm/PCMM_Context.h:14-90)
+class PCMM_Context {
+public:
+    Context_23& context;
+    int N1, mlwe_rank, ringpack_p_count, ringpack_q_count, ringpack_pq_count;
+    std::vector<uint64_tt> p_ringpack, q_ringpack;
+    pcmm_ctx* handle = nullptr;
+
+    PCMM_Context(int N1, int mlwe_rank, const std::vector<uint64_tt>& p_ringpack, const std::vector<uint64_tt>& q_ringpack,
+                 Context_23& context)
+        : context(context), N1(N1), mlwe_rank(mlwe_rank), ringpack_p_count((int)p_ringpack.size()),
+          ringpack_q_count((int)q_ringpack.size()), ringpack_pq_count((int)(p_ringpack.size() + q_ringpack.size())),
+          p_ringpack(p_ringpack), q_ringpack(q_ringpack) {
+        check(pcmm_ctx_create(&handle, context.handle, N1, mlwe_rank, p_ringpack.data(), ringpack_p_count, q_ringpack.data(),
+                              ringpack_q_count), "PCMM_Context");
+    }
+    PCMM_Context(const PCMM_Context&) = delete;
+    ~PCMM_Context() { if (handle) pcmm_ctx_destroy(handle); }
+    long info(const char* name) const {
+        long v = 0;
+        check(pcmm_info(handle, name, &v), "pcmm_info");
+        return v;
+    }
+};
+
+// The rlweCipherDecompose / PPMM members of PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48).
+class PCMM_Scheme {
+public:
+    PCMM_Context& pcmm_context;
+    Scheme_23& scheme;
+    uint64_tt* ppmm_output = nullptr;          // [mat_M][ringpack_q_count][(rank+1)*N1] (PCMM_Scheme.cuh:20)
+    size_t ppmm_output_words = 0;
+
+    PCMM_Scheme(PCMM_Context& pcmm_context, Scheme_23& scheme) : pcmm_context(pcmm_context), scheme(scheme) {}
+    PCMM_Scheme(const PCMM_Scheme&) = delete;
+    ~PCMM_Scheme() { device_release(ppmm_output); }
+
+    // PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:90-125).  Shape errors print and return, as the reference (:103-106).
+    void rlweCipherDecompose(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,
+                             uint64_tt offset) {
+        if (mlwe_num > (uint64_tt)pcmm_context.mlwe_rank) {
+            std::cout << "rlweCipherDecompose extract number muse <= mlwe_rank" << std::endl;
+            return;
+        }
+        if (offset + mlwe_num > mlwe_cipher_decomposed.size()) throw std::invalid_argument("rlweCipherDecompose: offset + mlwe_num exceeds the vector");
+        std::vector<uint64_tt*> ptrs(mlwe_num);
+        for (uint64_tt i = 0; i < mlwe_num; i++) ptrs[i] = mlwe_cipher_decomposed[offset + i]->cipher_device;
+        check(pcmm_rlwe_decompose_ntt(pcmm_context.handle, rlwe_cipher.cipher_device, ptrs.data(), (int)mlwe_num, rlwe_cipher.l),
+              "rlweCipherDecompose");
+    }
+
+    // PCMM_Scheme::PPMM (PPMM_kernel.cuh:254-349): plain_mat is a DEVICE pointer to mat_M x mat_N fp32, row-major.
+    // scaler = (long)(q_ringpack[1] * 2^49 / scale) (:283-284); afterwards row i of the product (first modulus) is copied
+    // back into mlwe_cipher_decomposed[i] and its scale becomes scale * scaler / q_ringpack[1] (:345-348).
+    void PPMM(float* plain_mat, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, int mat_M, int mat_N, int mat_K, int mlwe_num) {
+        if (mat_K != pcmm_context.N1) { std::cout << "matrix K should be equal to N1!" << std::endl; return; }
+        if (mat_N != mlwe_num) { std::cout << "matrix N should be equal to mlwe number!" << std::endl; return; }
+        const int mod_num = pcmm_context.ringpack_q_count;
+        const size_t C = (size_t)pcmm_context.N1 * (pcmm_context.mlwe_rank + 1);
+        const size_t need = (size_t)mat_M * mod_num * C;
+        if (need > ppmm_output_words) {
+            device_release(ppmm_output);
+            ppmm_output = device_alloc_words(need);
+            ppmm_output_words = need;
+        }
+        std::vector<const uint64_tt*> ptrs(mlwe_num);
+        for (int i = 0; i < mlwe_num; i++) ptrs[i] = mlwe_cipher_decomposed[i]->cipher_device;
+        const long double target_scale = (long double)(1ll << 49);
+        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * target_scale / mlwe_cipher_decomposed[0]->scale);
+        last_scaler = scaler;
+        check(pcmm_ppmm(pcmm_context.handle, plain_mat, ptrs.data(), ppmm_output, mat_M, mat_N, mod_num, (double)scaler), "PPMM");
+        const int rows = mat_M < mlwe_num ? mat_M : mlwe_num;
+        for (int i = 0; i < rows; i++) {
+            mlwe_cipher_decomposed[i]->scale = mlwe_cipher_decomposed[i]->scale * scaler / (long double)pcmm_context.q_ringpack[1];
+            check(ckks_memcpy_d2d(mlwe_cipher_decomposed[i]->cipher_device, ppmm_output + (size_t)i * C * mod_num, sizeof(uint64_tt) * C),
+                  "PPMM copy back");
+        }
+    }
+    long last_scaler = 0;
+};
+
+}  // namespace ckks_llm_amd

@@ -1,0 +1,139 @@
+// Parity test of the C++ host mirror (include/ckks_llm_amd.hpp) in the style of the reference's own test programs
+// (test_rlwe_decomp.cu, ntt_throughput.cu): build objects, call the member functions, compare - but against the CPU
+// oracle, bit for bit, and with assertions instead of prints.  Needs a GPU.  Exit code 0 = all checks passed.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <unistd.h>
+#include <random>
+#include <vector>
+
+#include "../../include/ckks_llm_amd.hpp"
+#include "../../oracle/ckks_oracle.h"
+
+using namespace ckks_llm_amd;
+
+static int failures = 0;
+#define EXPECT(cond, what)                                                      \
+    do {                                                                        \
+        if (!(cond)) { printf("FAIL %s (line %d)\n", what, __LINE__); failures++; } \
+        else printf("ok   %s\n", what);                                         \
+    } while (0)
+
+static std::vector<uint64_tt> uniform_limbs(std::mt19937_64& rng, const std::vector<uint64_tt>& primes, int polys, long N) {
+    std::vector<uint64_tt> v((size_t)polys * primes.size() * N);
+    for (int y = 0; y < polys; y++)
+        for (size_t j = 0; j < primes.size(); j++)
+            for (long i = 0; i < N; i++) v[((size_t)y * primes.size() + j) * N + i] = rng() % primes[j];
+    return v;
+}
+static void upload(uint64_tt* dev, const std::vector<uint64_tt>& h) { check(ckks_memcpy_h2d(dev, h.data(), h.size() * 8), "h2d"); }
+static std::vector<uint64_tt> download(const uint64_tt* dev, size_t words) {
+    std::vector<uint64_tt> h(words);
+    check(ckks_memcpy_d2h(h.data(), dev, words * 8), "d2h");
+    return h;
+}
+
+static int run() {
+    // the four largest primes below 2^36 that are 1 mod 2^13 (N = 2^12), as in BASELINE config 1
+    const std::vector<uint64_tt> q = {0xffffee001ull, 0xffffc4001ull, 0xffffbe001ull, 0xffffba001ull};
+    const int logN = 12;
+    const long N = 1l << logN;
+    std::mt19937_64 rng(7);
+
+    Context_23 context(logN, {}, q);
+    orc_ctx* orc = orc_ctx_create(logN, nullptr, 0, q.data(), (int)q.size(), nullptr, 0, 0);
+    Scheme_23 scheme(context);
+
+    // ---- ToNTTInplace / FromNTTInplace on a ciphertext (2 polys x 4 limbs), reference addressing ----
+    Ciphertext ct((int)N, context.L, context.L, (int)(N / 2), (long double)(1ll << 40));
+    std::vector<uint64_tt> h = uniform_limbs(rng, q, 2, N), want = h;
+    upload(ct.cipher_device, h);
+    context.ToNTTInplace(ct.cipher_device, 0, context.K, 2, context.L + 1, context.L + 1);
+    orc_ntt_fwd(orc, want.data(), 0, 0, 2, (int)q.size(), (int)q.size());
+    EXPECT(download(ct.cipher_device, h.size()) == want, "ToNTTInplace == oracle");
+    context.FromNTTInplace(ct.cipher_device, 0, context.K, 2, context.L + 1, context.L + 1);
+    EXPECT(download(ct.cipher_device, h.size()) == h, "FromNTTInplace(ToNTTInplace(x)) == x");
+
+    // ---- rescaleAndEqual: level L -> L-1 against the oracle, then std::invalid_argument at level 0 ----
+    upload(ct.cipher_device, want);                       // NTT-domain content
+    std::vector<uint64_tt> want_rs = want;
+    orc_rescale(orc, want_rs.data(), context.L);
+    scheme.rescaleAndEqual(ct);
+    EXPECT(download(ct.cipher_device, h.size()) == want_rs && ct.l == context.L - 1, "rescaleAndEqual == oracle, level drops");
+    Ciphertext ct0((int)N, context.L, 0, (int)(N / 2), 1.0L);
+    bool threw = false;
+    try { scheme.rescaleAndEqual(ct0); } catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw, "rescaleAndEqual on level 0 throws std::invalid_argument");
+
+    // ---- rlweCipherDecompose + PPMM (N1 = 128, rank 32: N = N1 * rank), two ring-pack primes ----
+    const int N1 = 128, rank = 32, mlwe_num = 16, M = 16;
+    const std::vector<uint64_tt> q_rp = {q[0], q[1]};
+    PCMM_Context pcmm_context(N1, rank, {}, q_rp, context);
+    PCMM_Scheme pcmm_scheme(pcmm_context, scheme);
+    orc_pcmm* orc_p = orc_pcmm_create(orc, N1, rank, nullptr, 0, q_rp.data(), 2);
+    Ciphertext rlwe((int)N, context.L, 1, (int)(N / 2), (long double)(1ll << 36));     // level 1: primes q0, q1
+    std::vector<uint64_tt> rl = uniform_limbs(rng, q, 2, N);
+    upload(rlwe.cipher_device, rl);
+    std::vector<MLWECiphertext*> mlwe;
+    for (int i = 0; i < mlwe_num; i++) mlwe.push_back(new MLWECiphertext(N1, 1, 1, rank, rlwe.scale));
+    pcmm_scheme.rlweCipherDecompose(rlwe, mlwe, mlwe_num, 0);
+    // oracle: iNTT of the level-1 limbs, gather
+    std::vector<uint64_tt> rl_coeff = rl;
+    orc_ntt_inv(orc, rl_coeff.data(), 0, 0, 2, 2, (int)q.size());
+    const size_t mlwe_words = (size_t)2 * (rank + 1) * N1;
+    std::vector<std::vector<uint64_tt>> om(mlwe_num, std::vector<uint64_tt>(mlwe_words));
+    std::vector<uint64_tt*> omp(mlwe_num);
+    for (int i = 0; i < mlwe_num; i++) omp[i] = om[i].data();
+    orc_rlwe_decompose(orc_p, rl_coeff.data(), omp.data(), mlwe_num, 1);
+    bool same = true;
+    for (int i = 0; i < mlwe_num; i++) same = same && download(mlwe[i]->cipher_device, mlwe_words) == om[i];
+    EXPECT(same, "rlweCipherDecompose == oracle");
+    EXPECT(download(rlwe.cipher_device, rl.size()) == rl, "rlweCipherDecompose leaves the RLWE ciphertext in NTT form");
+
+    std::vector<float> W((size_t)M * mlwe_num);
+    std::normal_distribution<float> nd(0.f, 0.02f);
+    for (float& w : W) w = nd(rng);
+    void* Wd = nullptr;
+    check(ckks_malloc(&Wd, W.size() * 4), "malloc W");
+    check(ckks_memcpy_h2d(Wd, W.data(), W.size() * 4), "h2d W");
+    const long double scale0 = mlwe[0]->scale;
+    const long scaler = (long)((long double)q_rp[1] * (long double)(1ll << 49) / scale0);
+    const size_t C = (size_t)(rank + 1) * N1;
+    std::vector<uint64_tt> oout((size_t)M * 2 * C);
+    std::vector<const uint64_tt*> ocp(mlwe_num);
+    for (int i = 0; i < mlwe_num; i++) ocp[i] = om[i].data();
+    orc_ppmm(orc_p, W.data(), ocp.data(), oout.data(), M, mlwe_num, 2, (double)scaler, 0, (long)C);
+    pcmm_scheme.PPMM((float*)Wd, mlwe, M, mlwe_num, N1, mlwe_num);
+    EXPECT(pcmm_scheme.last_scaler == scaler, "PPMM scaler = q_ringpack[1] * 2^49 / scale");
+    same = true;
+    for (int i = 0; i < M; i++) {
+        std::vector<uint64_tt> row = download(mlwe[i]->cipher_device, C);
+        same = same && std::memcmp(row.data(), oout.data() + (size_t)i * 2 * C, C * 8) == 0;
+    }
+    EXPECT(same, "PPMM rows copied back == oracle (first modulus, fused rescale)");
+    EXPECT(download(pcmm_scheme.ppmm_output, oout.size()) == oout, "PPMM output buffer == oracle (all moduli)");
+    const long double want_scale = scale0 * scaler / (long double)q_rp[1];
+    EXPECT(mlwe[0]->scale == want_scale, "PPMM updates the scale as the reference");
+    // shape errors: message and no work, as the reference
+    std::vector<uint64_tt> before = download(mlwe[0]->cipher_device, C);
+    pcmm_scheme.PPMM((float*)Wd, mlwe, M, mlwe_num, N1 + 1, mlwe_num);
+    pcmm_scheme.PPMM((float*)Wd, mlwe, M, mlwe_num - 1, N1, mlwe_num);
+    EXPECT(download(mlwe[0]->cipher_device, C) == before, "PPMM shape errors do no work");
+
+    for (MLWECiphertext* m : mlwe) delete m;
+    ckks_free(Wd);
+    orc_pcmm_destroy(orc_p);
+    orc_ctx_destroy(orc);
+    return failures;
+}
+
+int main() {
+    setvbuf(stdout, nullptr, _IONBF, 0);
+    const int failed = run();          // every device object is released when run() returns
+    printf(failed ? "FAILED: %d check(s)\n" : "all C++ mirror checks passed\n", failed);
+    fflush(stdout);
+    // leave without running the exit handlers of the HIP runtime and of the oracle's OpenMP runtime: their relative order
+    // at process exit is not defined and has crashed once after all checks had passed
+    _exit(failed ? 1 : 0);
+}
