@@ -79,6 +79,8 @@ struct ckks_ctx {
     int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
     int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: fused launch wherever it exists
     int cu_count = 256;
+    void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
+    size_t ntt_mid_cap = 0;
     void* d_ntt_sched = nullptr;          // scheduler words of the fused NTT kernel (zero between launches)
 };
 

@@ -25,6 +25,7 @@
 // [0,2q) for IntArith, raw double bit patterns for F64Arith); after the second pass it holds canonical residues.
 #include <cstddef>
 #include <cstdlib>
+#include <type_traits>
 
 #include "context.hpp"
 
@@ -44,6 +45,8 @@ struct IntArith {
     __device__ __forceinline__ V from_mid(u64 x) const { return x; }
     __device__ __forceinline__ u64 to_mid_fwd(V x) const { return x; }          // lazy [0,4q)
     __device__ __forceinline__ u64 to_mid_inv(V x) const { return x; }          // lazy [0,2q)
+    __device__ __forceinline__ u64 enc40(V x) const { return x; }               // the compact inter-pass form is FP64-only
+    __device__ __forceinline__ V dec40(unsigned lo, unsigned) const { return lo; }
     __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return csub(csub(x, q2), q); }
     // Harvey lazy butterflies; ranges as ntt_60bit.cuh:293-318
     __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
@@ -85,6 +88,11 @@ struct F64Arith {
         return (u64)(long long)r;
     }
     __device__ __forceinline__ u64 to_mid_inv(V x) const { return (u64)__double_as_longlong(balance(x)); }
+    // 40-bit form of a balanced value (q < 2^39, so |r| < 2^38.1): r + 2^39 read from the low mantissa bits of r + 2^52 + 2^39
+    __device__ __forceinline__ u64 enc40(V x) const { return (u64)__double_as_longlong(balance(x) + 4504149383184384.0) & 0xFFFFFFFFFFull; }
+    __device__ __forceinline__ V dec40(unsigned lo, unsigned hi8) const {
+        return __longlong_as_double((long long)(0x4330000000000000ull | ((u64)hi8 << 32) | lo)) - 4504149383184384.0;
+    }
     __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon(balance(x)); }
     __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
         double t = mulmod(y, w);
@@ -183,7 +191,18 @@ struct NttArgs {
     int start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len;
     long batch_stride_limbs;
     unsigned limb_base, limbs_total;      // this launch covers limbs limb_base .. limb_base + gridDim.y - 1 of limbs_total
+    char* mid;                            // compact inter-pass buffer (MID_LIMB_BYTES per limb of the launch) or nullptr
 };
+
+// Compact inter-pass form (N = 2^16, FP64 back end, q < 2^39): 5 bytes per value instead of 8, in a separate buffer laid out
+// for BOTH passes: piece (cb, rb) = the 16 x 16 block of columns 16cb.. and rows 16rb.., 1280 bytes:
+//   lo words  [r_local][c_local]            1024 B
+//   hi bytes  forward transforms: [r_local / 4][c_local] dwords, byte r_local % 4; inverse transforms: [r_local][c_local]   256 B
+// The strided pass (tile = cb) touches pieces (cb, 0..15), the row pass (tile = rb) pieces (0..15, rb); in all four access
+// patterns 16 lanes cover 64 contiguous bytes.
+constexpr int MID_PIECE_BYTES = 1280;
+constexpr long MID_LIMB_BYTES = 256l * MID_PIECE_BYTES;
+__device__ __forceinline__ char* mid_piece(char* mid_limb, unsigned cb, unsigned rb) { return mid_limb + (cb * 16 + rb) * MID_PIECE_BYTES; }
 
 // limb index of this block -> base pointer and prime.  Limbs are ordered prime-major so that consecutive
 // workgroups reuse one prime's twiddle table while it is hot in L2.
@@ -218,9 +237,9 @@ struct StridedCfg {
     static constexpr int THREADS = G * CW, TILES = N2 / CW, LDS_WORDS = N1 * CW;
 };
 
-template <class AR, int SA, int SB, bool INVERSE, bool COHERENT>
+template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false>
 __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                             typename AR::V* lds, unsigned tid) {
+                                             typename AR::V* lds, unsigned tid, char* mid_limb = nullptr) {
     typedef StridedCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     typedef typename AR::V V;
@@ -237,11 +256,33 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
         fwd_packed<AR, SA, S1>(v, tw, 1u, g, ar);
+        if constexpr (COMPACT) {
+            // lane (cl, g) holds rows 16g .. 16g+15 of column cl: piece (tile, g)
+            char* piece = mid_piece(mid_limb, tile, g);
+            unsigned hi[4] = {0, 0, 0, 0};
 #pragma unroll
-        for (int j = 0; j < R; j++) col[(long)(g * R + j) * N2] = ar.to_mid_fwd(v[j]);
+            for (int j = 0; j < R; j++) {
+                const u64 e = ar.enc40(v[j]);
+                *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
+                hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
+            }
+#pragma unroll
+            for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) col[(long)(g * R + j) * N2] = ar.to_mid_fwd(v[j]);
+        }
     } else {
+        if constexpr (COMPACT) {
+            const char* piece = mid_piece(mid_limb, tile, g);
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(col + (long)(g * R + j) * N2));
+            for (int j = 0; j < R; j++)
+                v[j] = ar.dec40(*reinterpret_cast<const unsigned*>(piece + (j * 16 + cl) * 4),
+                                *reinterpret_cast<const unsigned char*>(piece + 1024 + j * 16 + cl));
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(col + (long)(g * R + j) * N2));
+        }
         inv_packed<AR, SA, S1>(v, tw, 1u, g, ar);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[(g * R + j) * CW + cl] = v[j];
@@ -260,14 +301,15 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
     }
 }
 
-template <class AR, int SA, int SB, bool INVERSE>
+template <class AR, int SA, int SB, bool INVERSE, bool COMPACT = false>
 __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pass(NttArgs a) {
     constexpr long N = 1l << (SA + SB);
     __shared__ typename AR::V lds[StridedCfg<SA, SB>::LDS_WORDS];
     int prime;
     u64* limb = limb_ptr(a, blockIdx.y, N, prime);
     const AR ar(a.primes[prime]);
-    strided_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x);
+    strided_tile<AR, SA, SB, INVERSE, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
+                                                      COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -283,9 +325,9 @@ struct RowCfg {
 };
 __device__ __forceinline__ int padded(int pos) { return pos + (pos >> 4); }
 
-template <class AR, int SA, int SB, bool INVERSE, bool COHERENT>
+template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false>
 __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                         typename AR::V* lds, unsigned tid) {
+                                         typename AR::V* lds, unsigned tid, char* mid_limb = nullptr) {
     typedef RowCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     typedef typename AR::V V;
@@ -296,8 +338,19 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
     const unsigned tw_off = N1 + row;
     V v[R];
     if (!INVERSE) {
+        if constexpr (COMPACT) {
+            // lane (u, rl) takes columns u + 16j of row 16*tile + rl: element (rl, u) of piece (j, tile)
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(rp + u + j * U));
+            for (int j = 0; j < R; j++) {
+                const char* piece = mid_piece(mid_limb, j, tile);
+                const unsigned lo = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
+                const unsigned hi = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
+                v[j] = ar.dec40(lo, (hi >> (8 * (rl & 3))) & 0xffu);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(rp + u + j * U));
+        }
         fwd_spread<AR, SB, S1>(v, tw, tw_off, ar);
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];
@@ -326,19 +379,32 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lrow[padded(u + j * U)];
         inv_spread<AR, SB, S1, 0>(v, tw, tw_off, ar);
+        if constexpr (COMPACT) {
+            // inverse transforms keep the hi bytes as bytes [r_local][c_local]: a wave (16 columns x 4 rows of a piece) stores
+            // 64 contiguous bytes per instruction and needs no cross-lane packing
 #pragma unroll
-        for (int j = 0; j < R; j++) rp[u + j * U] = ar.to_mid_inv(v[j]);
+            for (int j = 0; j < R; j++) {
+                char* piece = mid_piece(mid_limb, j, tile);
+                const u64 e = ar.enc40(v[j]);
+                *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
+                *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) rp[u + j * U] = ar.to_mid_inv(v[j]);
+        }
     }
 }
 
-template <class AR, int SA, int SB, bool INVERSE>
+template <class AR, int SA, int SB, bool INVERSE, bool COMPACT = false>
 __global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass(NttArgs a) {
     constexpr long N = 1l << (SA + SB);
     __shared__ typename AR::V lds[RowCfg<SA, SB>::LDS_WORDS];
     int prime;
     u64* limb = limb_ptr(a, blockIdx.y, N, prime);
     const AR ar(a.primes[prime]);
-    row_tile<AR, SA, SB, INVERSE, false>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x);
+    row_tile<AR, SA, SB, INVERSE, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
+                                                  COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -512,27 +578,52 @@ __global__ __launch_bounds__(256) void ntt_fused_kernel(NttArgs a, NttSched* sch
 
 size_t ntt_sched_bytes() { return sizeof(NttSched); }
 
-template <class AR, int SA, int SB>
-static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
+// launches of one chunk of limbs; COMPACT selects the 5-byte inter-pass buffer
+template <class AR, int SA, int SB, bool COMPACT>
+static void launch_passes(ckks_ctx* c, const NttArgs& args, int n, bool inverse) {
     typedef StridedCfg<SA, SB> CS;
     typedef RowCfg<SA, SB> CR;
+    dim3 gs(CS::TILES, n), bs(CS::THREADS);
+    dim3 gr(CR::TILES, n), br(CR::THREADS);
+    if (!inverse) {
+        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT>), gs, bs, 0, c->stream, args);
+        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
+        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false, COMPACT>), gr, br, 0, c->stream, args);
+    } else {
+        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true, COMPACT>), gr, br, 0, c->stream, args);
+        if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
+        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true, COMPACT>), gs, bs, 0, c->stream, args);
+    }
+}
+
+template <class AR, int SA, int SB>
+static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok) {
+    constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
     static const int chunk_env = getenv("CKKS_NTT_CHUNK") ? atoi(getenv("CKKS_NTT_CHUNK")) : 0;
-    const int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs;
+    int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs;
+    const bool compact = CAN_COMPACT && compact_ok && c->ntt_mode != 1;
+    if (compact) {
+        // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
+        const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
+        if (chunk > max_limbs) chunk = max_limbs;
+        const size_t need = (size_t)chunk * MID_LIMB_BYTES;
+        if (need > c->ntt_mid_cap) {
+            if (c->d_ntt_mid) { (void)hipDeviceSynchronize(); (void)hipFree(c->d_ntt_mid); c->d_ntt_mid = nullptr; c->ntt_mid_cap = 0; }
+            if (hipMalloc(&c->d_ntt_mid, need) != hipSuccess) { set_error("NTT: cannot allocate the inter-pass buffer"); return CKKS_E_NOMEM; }
+            c->ntt_mid_cap = need;
+        }
+        args.mid = (char*)c->d_ntt_mid;
+    } else {
+        args.mid = nullptr;
+    }
     args.limbs_total = (unsigned)limbs;
     for (int base = 0; base < limbs; base += chunk) {
         const int n = limbs - base < chunk ? limbs - base : chunk;
         args.limb_base = (unsigned)base;
-        dim3 gs(CS::TILES, n), bs(CS::THREADS);
-        dim3 gr(CR::TILES, n), br(CR::THREADS);
-        if (!inverse) {
-            hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false>), gs, bs, 0, c->stream, args);
-            if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-            hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false>), gr, br, 0, c->stream, args);
-        } else {
-            hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true>), gr, br, 0, c->stream, args);
-            if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-            hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true>), gs, bs, 0, c->stream, args);
+        if constexpr (CAN_COMPACT) {
+            if (compact) { launch_passes<AR, SA, SB, true>(c, args, n, inverse); continue; }
         }
+        launch_passes<AR, SA, SB, false>(c, args, n, inverse);
     }
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
@@ -547,6 +638,7 @@ static int launch_fused(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
     if (blocks > tiles) blocks = tiles;
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
+    args.mid = nullptr;
     NttSched* sched = (NttSched*)c->d_ntt_sched;
     if (!inverse) hipLaunchKernelGGL((ntt_fused_kernel<AR, SA, SB, false, 1>), dim3((unsigned)blocks), dim3(256), 0, c->stream, args, sched);
     else hipLaunchKernelGGL((ntt_fused_kernel<AR, SA, SB, true, 1>), dim3((unsigned)blocks), dim3(256), 0, c->stream, args, sched);
@@ -559,6 +651,7 @@ static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse)
     static const int groups_env = getenv("CKKS_NTT_GROUPS") ? atoi(getenv("CKKS_NTT_GROUPS")) : 0;
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
+    args.mid = nullptr;
     if (groups_env == 2) {
         if (!inverse) hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, false, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
         else hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, true, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
@@ -574,7 +667,7 @@ static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse)
 size_t ntt_sched_error_offset() { return offsetof(NttSched, error); }
 
 template <class AR>
-static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse) {
+static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok) {
     // The one-launch transform (ntt_fused_kernel) is switched off: on MI355X its launches did not complete (the process had to
     // be ended by a test time-out, twice, the second time with every scheduler wait bounded to 20 ms), and the cause has not
     // been shown yet.  Mode 2 therefore reports an error instead of launching it; the automatic mode uses two launches.
@@ -594,15 +687,15 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
         if (c->logN == 15) return launch_fused<AR, 8, 7>(c, args, limbs, inverse);
     }
     switch (c->logN) {
-        case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse);
-        case 9:  return launch_two_pass<AR, 5, 4>(c, args, limbs, inverse);
-        case 10: return launch_two_pass<AR, 5, 5>(c, args, limbs, inverse);
-        case 11: return launch_two_pass<AR, 6, 5>(c, args, limbs, inverse);
-        case 12: return launch_two_pass<AR, 6, 6>(c, args, limbs, inverse);
-        case 13: return launch_two_pass<AR, 7, 6>(c, args, limbs, inverse);
-        case 14: return launch_two_pass<AR, 7, 7>(c, args, limbs, inverse);
-        case 15: return launch_two_pass<AR, 8, 7>(c, args, limbs, inverse);
-        case 16: return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse);
+        case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse, compact_ok);
+        case 9:  return launch_two_pass<AR, 5, 4>(c, args, limbs, inverse, compact_ok);
+        case 10: return launch_two_pass<AR, 5, 5>(c, args, limbs, inverse, compact_ok);
+        case 11: return launch_two_pass<AR, 6, 5>(c, args, limbs, inverse, compact_ok);
+        case 12: return launch_two_pass<AR, 6, 6>(c, args, limbs, inverse, compact_ok);
+        case 13: return launch_two_pass<AR, 7, 6>(c, args, limbs, inverse, compact_ok);
+        case 14: return launch_two_pass<AR, 7, 7>(c, args, limbs, inverse, compact_ok);
+        case 15: return launch_two_pass<AR, 8, 7>(c, args, limbs, inverse, compact_ok);
+        case 16: return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
         default: set_error("NTT: logN must be in [8, 16]"); return CKKS_E_INVALID;
     }
 }
@@ -617,8 +710,11 @@ int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx
     }
     long limbs = (long)poly_num * mod_num * batch;
     if (limbs > 65535) { set_error("NTT: more than 65535 limbs in one call"); return CKKS_E_INVALID; }
-    bool f64 = c->arith_mode == 0;
-    for (int j = 0; j < mod_num && f64; j++) f64 = c->f64_ok[start_mod_idx + j] != 0;
+    bool f64 = c->arith_mode == 0, compact_ok = true;
+    for (int j = 0; j < mod_num; j++) {
+        f64 = f64 && c->f64_ok[start_mod_idx + j] != 0;
+        compact_ok = compact_ok && c->pqt[start_mod_idx + j] < (1ull << 39);
+    }
     NttArgs args;
     args.data = (u64*)dev;
     args.primes = c->d_primes;
@@ -630,10 +726,10 @@ int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx
     args.batch_stride_limbs = batch_stride_limbs;
     if (f64) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
-        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse);
+        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok);
     }
     args.tw = inverse ? (const void*)c->d_tw_inv : (const void*)c->d_tw_fwd;
-    return dispatch_logn<IntArith>(c, args, (int)limbs, inverse);
+    return dispatch_logn<IntArith>(c, args, (int)limbs, inverse, false);
 }
 
 }  // namespace ckks

@@ -64,6 +64,31 @@ def test_n65536_integer_backend_and_large_primes():
     check_fwd_inv(pair2, 0, CFG2_Q[:2], 2, seed=4, mode=1)
 
 
+def test_n65536_inter_pass_formats():
+    """N = 2^16, FP64 back end: primes below 2^39 take the 5-byte inter-pass buffer, 40-bit primes the in-place 8-byte form, and
+    ntt_mode 1 forces the in-place form; all against the oracle.  A batch wider than one launch chunk is not needed: chunks
+    only re-use the buffer in stream order."""
+    from ckks_llm_amd.params import small_primes
+    q40 = small_primes(40, 1 << 17, 2)
+    assert all((1 << 39) <= p < (1 << 41) for p in q40)
+    pair = Pair(16, [], CFG2_Q[:3] + q40)
+    check_fwd_inv(pair, 0, CFG2_Q[:3], 3, seed=21, mode=0)            # compact
+    check_fwd_inv(pair, 3, q40, 2, seed=22, mode=0)                   # FP64, in place
+    check_fwd_inv(pair, 0, CFG2_Q[:3] + q40, 1, seed=23, mode=0)      # mixed call: in place
+    pair.dev.set_ntt_mode(1)
+    check_fwd_inv(pair, 0, CFG2_Q[:3], 3, seed=24, mode=0)            # forced in place
+    # maximal and minimal residues through the 40-bit codec
+    N = pair.N
+    pair.dev.set_ntt_mode(0)
+    data = np.stack([np.full(N, p - 1, dtype=np.uint64) for p in CFG2_Q[:3]])[None].copy()
+    data[0, :, ::2] = 0
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, 1, 3, 5)
+    d = to_dev(data)
+    pair.dev.ToNTTInplace(d, 0, 0, 1, 3, 5)
+    assert np.array_equal(from_dev(d, data.shape), want)
+
+
 def test_reference_addressing_and_ext_variant():
     """start_poly_idx / start_mod_idx / poly_mod_len addressing (ntt_60bit.cuh:446-455) and the batch stride of the
     _for_externalProduct variants (ntt_60bit.cuh:913-934)."""
