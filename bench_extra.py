@@ -79,5 +79,43 @@ def bench_keyswitch(P, reps=10):
                          "frac": round(stage_bytes / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": stage_bytes}}
 
 
+def bench_packing(P, N1=128, reps=5):
+    """MLWE -> RLWE packing after PPMM (PCMM_Scheme::mlweCipherPacking): rank = 512 samples of N1 = 128 into one ciphertext at
+    N = 2^16, one special prime and q0.  Algorithmic bytes: samples in, the embedded polynomials out and through one NTT,
+    embedded 'a' polynomials and keys into the inner product, and the small tail (4 limbs through iNTT, ModDown, NTT)."""
+    from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
+    p0, q = P.CFG3_P[0], P.CFG2_Q[:2]
+    ctx = Context_23(16, [p0], q)
+    N = 1 << 16
+    rank = N // N1
+    sch = PCMM_Scheme(PCMM_Context(N1, rank, [p0], q, ctx))
+    rng = np.random.default_rng(6)
+    sample = DeviceBuffer.from_numpy(rng.integers(0, q[0], size=(rank + 1) * N1, dtype=np.uint64))
+    bufs = []
+    for _ in range(rank):
+        b = DeviceBuffer(8 * (rank + 1) * N1)
+        b.L_.ckks_memcpy_d2d(b.ptr, sample.ptr, b.nbytes)
+        bufs.append(b)
+    keys = DeviceBuffer(8 * rank * 4 * N)
+    one_key = np.empty((4, N), dtype=np.uint64)
+    for j, pr in enumerate((p0, q[0], p0, q[0])):
+        one_key[j] = rng.integers(0, pr, N, dtype=np.uint64)
+    k0 = DeviceBuffer.from_numpy(one_key)
+    for i in range(rank):
+        keys.L_.ckks_memcpy_d2d(keys.ptr + i * one_key.nbytes, k0.ptr, one_key.nbytes)
+    out, embed, mult = DeviceBuffer(8 * 2 * 2 * N), DeviceBuffer(8 * (rank + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    sch.mlweCipherPacking(out, bufs, rank, 0, keys, embed, mult)
+    ctx.timer_start()
+    for _ in range(reps):
+        sch.mlweCipherPacking(out, bufs, rank, 0, keys, embed, mult)
+    ms = ctx.timer_stop() / reps
+    limb = 8.0 * N
+    alg = 8.0 * rank * (rank + 1) * N1 + (rank + 1) * 2 * limb + 2 * (rank * 2) * limb + rank * 6 * limb + 4 * limb * 6
+    return {"workload": "mlweCipherPacking: 512 MLWE samples (N1=128) -> 1 RLWE ciphertext, N=2^16, primes [p0|q0]", "ms": round(ms, 3),
+            "packings_per_s": round(1e3 / ms, 1),
+            "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
+
+
 def run(P):
-    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P)}
+    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P), "packing": bench_packing(P)}

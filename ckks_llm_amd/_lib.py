@@ -51,6 +51,7 @@ def _declare(L):
         "pcmm_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_rlwe_decompose_ntt": (i, [vp, vp, C.POINTER(vp), i, i]),
+        "pcmm_mlwe_pack": (i, [vp, vp, C.POINTER(vp), i, vp, vp, vp]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
     }

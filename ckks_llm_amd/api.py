@@ -251,6 +251,15 @@ class PCMM_Scheme:
         f = self.L_.pcmm_rlwe_decompose if coeff_domain else self.L_.pcmm_rlwe_decompose_ntt
         _check(f(self.pcmm_context.h, _addr(rlwe_cipher), self._ptrs(bufs), mlwe_num, l), "pcmm_rlwe_decompose")
 
+    def mlweCipherPacking(self, rlwe_cipher, mlwe_cipher_decomposed, mlwe_num, offset, repacking_keys, embeded_mlwe_buffer,
+                          mult_key_output):
+        """PCMM_Scheme.cuh:361-425.  rlwe_cipher: [a | b] device buffer (limb 0 of both polynomials is written, NTT domain);
+        repacking_keys: rank keys [a | b] over [p0 | q0] in one device buffer; the two scratch buffers are the reference's
+        embeded_mlwe_buffer ((rank+1)*2*N words) and the 4*N words it borrows from the scheme for the key product."""
+        bufs = mlwe_cipher_decomposed[offset:offset + mlwe_num]
+        _check(self.L_.pcmm_mlwe_pack(self.pcmm_context.h, _addr(rlwe_cipher), self._ptrs(bufs), mlwe_num, _addr(repacking_keys),
+                                      _addr(embeded_mlwe_buffer), _addr(mult_key_output)), "pcmm_mlwe_pack")
+
     def PPMM(self, plain_mat, mlwe_cipher_decomposed, out, mat_M, mat_N, mat_K, mlwe_num, mod_num, scaler):
         """PPMM_kernel.cuh:254-349 (device part).  Shape errors are reported the way the reference does: a message and no
         work (PPMM_kernel.cuh:256-263), here as ValueError."""

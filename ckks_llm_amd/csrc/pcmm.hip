@@ -200,6 +200,120 @@ extern "C" int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* co
 }
 
 
+// ------------------------------------------------------------------------------------------------------------
+// MLWE -> RLWE packing: PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425)
+//   embed  : k+1 big polynomials over [p0, q0]; coefficient n*k + m*gap of big polynomial i is coefficient n of row i of MLWE
+//            sample m (zero elsewhere), lifted to p0 around zero (mlweCipherEmbedding_new_kernel, :309-340)
+//   NTT of the k "a" polynomials, inner product with the k repacking keys (mlweCipherMultRepackingKey_kernel, :262-289),
+//   iNTT, division by p0 (ringpacking_ModDown_kernel, :291-306), + (0, b), NTT.
+// All three kernels stream: one pass over their inputs, coalesced on both sides.
+// ------------------------------------------------------------------------------------------------------------
+struct EmbedArgs {
+    const u64* const* mlwe;       // mlwe_num pointers, each [(k+1)][N1] (one modulus)
+    u64* embed;                   // [(k+1)][2][N]
+    long N;
+    int N1, rank, mlwe_num;
+    u64 p0, q0;
+};
+constexpr int EMBED_ROWS = 8;     // coefficients n of the small ring per workgroup
+__global__ __launch_bounds__(256) void mlwe_embed_kernel(EmbedArgs a) {
+    extern __shared__ u64 tile[];                       // [EMBED_ROWS][rank]
+    const int k = a.rank, i = blockIdx.y, n0 = blockIdx.x * EMBED_ROWS, gap = k / a.mlwe_num;
+    for (int t = threadIdx.x; t < EMBED_ROWS * k; t += 256) tile[t] = 0;
+    __syncthreads();
+    // 8 lanes read 64 contiguous bytes of one sample; the tile turns (sample, n) into (n, position inside the big coefficient group)
+    for (int t = threadIdx.x; t < EMBED_ROWS * a.mlwe_num; t += 256) {
+        const int m = t / EMBED_ROWS, j = t % EMBED_ROWS;
+        tile[j * k + m * gap] = a.mlwe[m][(long)i * a.N1 + n0 + j];
+    }
+    __syncthreads();
+    u64* big = a.embed + (long)i * 2 * a.N;
+    for (int t = threadIdx.x; t < EMBED_ROWS * k; t += 256) {
+        const u64 v = tile[t];
+        const long pos = (long)n0 * k + t;              // (n0 + t / k) * k + t % k
+        big[a.N + pos] = v;                                                         // mod q0
+        big[pos] = v > a.q0 / 2 ? (a.p0 - (a.q0 - v)) % a.p0 : v;                   // mod p0, lifted around zero (:335-339)
+    }
+}
+
+struct RepackArgs {
+    const u64* embed;             // [(k+1)][2][N], the first k polynomials in NTT form
+    const u64* keys;              // [k][a: 2 limbs | b: 2 limbs][N]
+    u64* acc;                     // [2][2][N]
+    u64* rlwe;                    // [a: L+1 limbs | b: L+1 limbs]
+    const PrimeConst* pq;         // ring-pack primes [p0, q0, ...]
+    long N;
+    int rank, L;
+    u64 pinv, pinv_s;             // p0^-1 mod q0 and its Shoup word
+};
+__global__ __launch_bounds__(256) void repack_mult_kernel(RepackArgs a) {
+    const long x = (long)blockIdx.x * 256 + threadIdx.x;
+    const int im = blockIdx.y;
+    const PrimeConst pr = a.pq[im];
+    u128w sa = {0, 0}, sb = {0, 0};
+    const u64* e = a.embed + (long)im * a.N + x;
+    const u64* ka = a.keys + (long)im * a.N + x;
+    const u64* kb = ka + 2 * a.N;
+#pragma unroll 4
+    for (int i = 0; i < a.rank; i++) {
+        const u64 c = e[(long)i * 2 * a.N];
+        mac128(sa, c, ka[(long)i * 4 * a.N]);
+        mac128(sb, c, kb[(long)i * 4 * a.N]);
+    }
+    a.acc[(long)im * a.N + x] = barrett128(sa, pr.q, pr.mu_hi, pr.mu_lo);
+    a.acc[(long)(2 + im) * a.N + x] = barrett128(sb, pr.q, pr.mu_hi, pr.mu_lo);
+}
+__global__ __launch_bounds__(256) void repack_moddown_kernel(RepackArgs a) {
+    const long x = (long)blockIdx.x * 256 + threadIdx.x;
+    const int y = blockIdx.y;
+    const u64 q0 = a.pq[1].q;
+    const u64* in = a.acc + (long)y * 2 * a.N;
+    u64 ra = in[x] % q0;                                                            // :300
+    ra = q0 - ra + in[a.N + x];
+    u64 r = mul_shoup(ra, a.pinv, a.pinv_s, q0);
+    if (y == 1) r = csub(r + a.embed[(long)a.rank * 2 * a.N + a.N + x], q0);        // + (0, b), poly_arithmetic.cuh:111-121
+    a.rlwe[(long)y * a.N * (a.L + 1) + x] = r;
+}
+
+extern "C" int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* const* mlwe_ptrs_host, int mlwe_num,
+                              const uint64_t* repacking_keys, uint64_t* embed_scratch, uint64_t* mult_scratch) {
+    if (!h || !rlwe_out || !mlwe_ptrs_host || !repacking_keys || !embed_scratch || !mult_scratch) return CKKS_E_INVALID;
+    ckks_ctx* c = h->ctx;
+    const int k = h->rank, N1 = h->N1, K = c->K;
+    if (h->np != 1 || h->nq != 2) {
+        set_error("mlweCipherPacking: one special ring-pack prime and two ring-pack moduli are supported (the reference's embedding overlaps otherwise)");
+        return CKKS_E_INVALID;
+    }
+    if (mlwe_num <= 0 || mlwe_num > k || k % mlwe_num || (long)N1 * k != c->N || N1 % EMBED_ROWS || K < 1 || c->N % 256) {
+        set_error("mlweCipherPacking: bad mlwe_num or ring shape");
+        return CKKS_E_INVALID;
+    }
+    if (c->pqt[K - 1] != h->pq[0] || c->pqt[K] != h->pq[1]) {
+        set_error("mlweCipherPacking: the ring-pack primes must be the context's last special prime and q0");
+        return CKKS_E_INVALID;
+    }
+    if ((size_t)EMBED_ROWS * k * sizeof(u64) > 64 * 1024) { set_error("mlweCipherPacking: rank too large"); return CKKS_E_INVALID; }
+    int rc = upload_ptrs(h, mlwe_ptrs_host, mlwe_num);
+    if (rc) return rc;
+    EmbedArgs ea;
+    ea.mlwe = (const u64* const*)h->d_ptrs; ea.embed = embed_scratch; ea.N = c->N; ea.N1 = N1; ea.rank = k; ea.mlwe_num = mlwe_num;
+    ea.p0 = h->pq[0]; ea.q0 = h->pq[1];
+    hipLaunchKernelGGL(mlwe_embed_kernel, dim3(N1 / EMBED_ROWS, k + 1), dim3(256), (size_t)EMBED_ROWS * k * sizeof(u64), c->stream, ea);
+    if ((rc = launch_ntt(c, embed_scratch, 0, K - 1, k, 2, 2, 0, 1, false))) return rc;            // :389
+    RepackArgs ra;
+    ra.embed = embed_scratch; ra.keys = repacking_keys; ra.acc = mult_scratch; ra.rlwe = rlwe_out; ra.pq = h->d_pq; ra.N = c->N;
+    ra.rank = k; ra.L = c->L;
+    ra.pinv = H::invmod(h->pq[0] % h->pq[1], h->pq[1]); ra.pinv_s = H::shoup(ra.pinv, h->pq[1]);
+    hipLaunchKernelGGL(repack_mult_kernel, dim3((unsigned)(c->N / 256), 2), dim3(256), 0, c->stream, ra);
+    if ((rc = launch_ntt(c, mult_scratch, 0, K - 1, 2, 2, 2, 0, 1, true))) return rc;              // :405
+    hipLaunchKernelGGL(repack_moddown_kernel, dim3((unsigned)(c->N / 256), 2), dim3(256), 0, c->stream, ra);
+    CKKS_HIP_TRY(hipGetLastError());
+    if ((rc = launch_ntt(c, rlwe_out, 0, K, 2, 1, c->L + 1, 0, 1, false))) return rc;              // :419
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the pointer table came from the caller's host array
+    return CKKS_OK;
+}
+
+
 static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
                        int M, int Kin, int mod_num, double scaler) {
     if (!h || !W || !out || (!ptrs_host && !strided)) return CKKS_E_INVALID;

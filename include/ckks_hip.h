@@ -138,6 +138,16 @@ int pcmm_info(const pcmm_ctx* h, const char* name, long* value);
 int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l);
 /* PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:90-125): iNTT, gather, NTT back; rlwe in NTT domain. */
 int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* const* mlwe_ptrs_host, int mlwe_num, int l);
+/* PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425; kernels :262-340): packs mlwe_num MLWE ciphertexts (the rows PPMM
+ * leaves behind: one modulus, [(rank+1)][N1] words each, coefficient domain, mlwe_num divides rank) into one RLWE ciphertext
+ * rlwe_out = [a: L+1 limbs | b: L+1 limbs], of which limb 0 of both polynomials is written, NTT domain, level 0.
+ * repacking_keys: rank keys over the primes [p0 | q0] (p0 = the context's last special prime = the ring-pack special prime,
+ * q0 = the first ring-pack modulus), key i at keys + i*4*N = [a mod p0 | a mod q0 | b mod p0 | b mod q0], NTT domain
+ * (PCMM_Scheme::addRepakcingKey, :152-224).  embed_scratch: (rank+1)*2*N words (PCMM_Scheme::embeded_mlwe_buffer, :12);
+ * mult_scratch: 4*N words (the reference borrows Scheme_23::modUp_TtoQj_buffer, :394).
+ * The reference's embedding is only meaningful for one special prime and two ring-pack moduli; other contexts get CKKS_E_INVALID. */
+int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* const* mlwe_ptrs_host, int mlwe_num,
+                   const uint64_t* repacking_keys, uint64_t* embed_scratch, uint64_t* mult_scratch);
 /* PCMM_Scheme::PPMM device part (PPMM_kernel.cuh:93-252, launch :294-340):
  * out[m][mod][c] = fused-rescaled sum_n trunc(W[m][n]*scaler) * mlwe[n][mod][c] mod q_mod, for mod_num ring-pack
  * primes (the reference fixes mod_num = 2), c < (rank+1)*N1.  W: device fp32 row-major [M][Kin];

@@ -215,9 +215,35 @@ public:
     uint64_tt* ppmm_output = nullptr;          // [mat_M][ringpack_q_count][(rank+1)*N1] (PCMM_Scheme.cuh:20)
     size_t ppmm_output_words = 0;
 
-    PCMM_Scheme(PCMM_Context& pcmm_context, Scheme_23& scheme) : pcmm_context(pcmm_context), scheme(scheme) {}
+    uint64_tt* embeded_mlwe_buffer = nullptr;  // (rank+1) big polynomials over [p0 | q0] (PCMM_Scheme.cuh:12)
+    uint64_tt* mult_key_output = nullptr;      // 4 limbs; the reference borrows scheme.modUp_TtoQj_buffer (PCMM_Scheme.cuh:394)
+    uint64_tt* repackingKeys = nullptr;        // rank keys [a | b] over [p0 | q0], NTT domain, one buffer (PCMM_Scheme.cuh:166-176)
+
+    PCMM_Scheme(PCMM_Context& pcmm_context, Scheme_23& scheme) : pcmm_context(pcmm_context), scheme(scheme) {
+        const size_t N = (size_t)scheme.context.N;
+        embeded_mlwe_buffer = device_alloc_words((size_t)(pcmm_context.mlwe_rank + 1) * N * (pcmm_context.ringpack_pq_count - 1));
+        mult_key_output = device_alloc_words(2 * N * (pcmm_context.ringpack_pq_count - 1));
+    }
     PCMM_Scheme(const PCMM_Scheme&) = delete;
-    ~PCMM_Scheme() { device_release(ppmm_output); }
+    ~PCMM_Scheme() {
+        device_release(ppmm_output);
+        device_release(embeded_mlwe_buffer);
+        device_release(mult_key_output);
+    }
+
+    // PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425): k MLWE samples -> 1 RLWE ciphertext with the repacking keys
+    // (the reference generates them in addRepakcingKey from the secret keys; here the caller installs them in repackingKeys).
+    void mlweCipherPacking(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,
+                           uint64_tt offset) {
+        if (!repackingKeys) throw std::invalid_argument("mlweCipherPacking: repacking keys not exists");
+        if (offset + mlwe_num > mlwe_cipher_decomposed.size()) throw std::invalid_argument("mlweCipherPacking: offset + mlwe_num exceeds the vector");
+        std::vector<const uint64_tt*> ptrs(mlwe_num);
+        for (uint64_tt i = 0; i < mlwe_num; i++) ptrs[i] = mlwe_cipher_decomposed[offset + i]->cipher_device;
+        check(pcmm_mlwe_pack(pcmm_context.handle, rlwe_cipher.cipher_device, ptrs.data(), (int)mlwe_num, repackingKeys,
+                             embeded_mlwe_buffer, mult_key_output), "mlweCipherPacking");
+        rlwe_cipher.l = pcmm_context.ringpack_q_count - 1 - 1;                       // :407-409
+        rlwe_cipher.scale = mlwe_cipher_decomposed[0]->scale;
+    }
 
     // PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:90-125).  Shape errors print and return, as the reference (:103-106).
     void rlweCipherDecompose(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,

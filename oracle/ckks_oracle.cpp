@@ -814,6 +814,75 @@ int orc_ppmm(const orc_pcmm* h, const float* W, const u64* const* mlwe, u64* out
     return 0;
 }
 
+// PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425) with its kernels: mlweCipherEmbedding_new_kernel (:309-358),
+// mlweCipherMultRepackingKey_kernel (:262-289), ringpacking_ModDown_kernel (:291-306).
+//   mlwe[m]   : [(nq-1) moduli][(rank+1)][N1]  (the PPMM output rows after the fused rescale), coefficient domain
+//   keys      : rank switching keys, key i at keys + i*N*mod_num*2 = [a: mod_num limbs | b: mod_num limbs], NTT domain,
+//               mod_num = np + nq - 1 limbs over the context primes K-np .. K-np+mod_num-1 (PCMM_Scheme.cuh:166-171)
+//   rlwe_out  : [a: L+1 limbs | b: L+1 limbs]; limbs 0 .. nq-2 of both are written (NTT domain), level nq-2
+// The reference's embedding writes the lifted value of modulus idx_mod to limb idx_mod and the value itself to limb
+// np + idx_mod (:333-339), which only makes sense for one special prime and one remaining modulus; that is what is accepted.
+int orc_mlwe_pack(const orc_pcmm* h, u64* rlwe_out, const u64* const* mlwe, int mlwe_num, const u64* keys) {
+    const orc_ctx* c = h->ctx; const long N = c->N; const int N1 = h->N1, k = h->rank, np = h->np, nq = h->nq, K = c->p_num, L = c->L;
+    if (np != 1 || nq != 2 || mlwe_num <= 0 || mlwe_num > k || k % mlwe_num || (long)N1 * k != N || K < np) return -1;
+    const int mod_num = np + nq - 1, first_prime = K - np;
+    for (int i = 0; i < mod_num; i++) if (c->pqt[first_prime + i] != h->pq[i]) return -1;
+    const int gap = k / mlwe_num;
+    const u64 p0 = h->pq[0];
+    // embedding + centred lift q -> p (:309-340); the buffer starts zeroed (:386)
+    std::vector<u64> embed((size_t)(k + 1) * mod_num * N, 0);
+    for (int m = 0; m < mlwe_num; m++)
+        for (int im = 0; im < nq - 1; im++) {
+            const u64 qi = h->pq[np + im];
+            for (int i = 0; i <= k; i++)
+                for (int n = 0; n < N1; n++) {
+                    const u64 v = mlwe[m][(long)im * N1 * (k + 1) + (long)i * N1 + n];
+                    u64* big = embed.data() + (size_t)i * N * mod_num;
+                    const long pos = (long)n * k + (long)m * gap;
+                    big[(long)(np + im) * N + pos] = v;
+                    big[(long)im * N + pos] = v > qi / 2 ? (p0 - (qi - v)) % p0 : v;
+                }
+        }
+    // NTT of the k "a" polynomials over [p0, q0] (:389)
+    orc_ntt_fwd(c, embed.data(), 0, first_prime, k, mod_num, mod_num);
+    // sum_i a_i * key_i (:262-289): 128-bit accumulation, one Barrett reduction
+    std::vector<u64> acc((size_t)2 * mod_num * N);
+    for (int im = 0; im < mod_num; im++) {
+        const u64 q = h->pq[im], mh = h->mu_hi[im], ml = h->mu_lo[im];
+#pragma omp parallel for schedule(static)
+        for (long x = 0; x < N; x++) {
+            u128 sa = 0, sb = 0;
+            for (int i = 0; i < k; i++) {
+                const u64 ca = embed[(size_t)i * N * mod_num + (size_t)im * N + x];
+                const u64* key = keys + (size_t)i * N * mod_num * 2;
+                sa += (u128)ca * key[(size_t)im * N + x];
+                sb += (u128)ca * key[(size_t)(im + mod_num) * N + x];
+            }
+            acc[(size_t)im * N + x] = orc_barrett128((u64)(sa >> 64), (u64)sa, q, mh, ml);
+            acc[(size_t)(mod_num + im) * N + x] = orc_barrett128((u64)(sb >> 64), (u64)sb, q, mh, ml);
+        }
+    }
+    orc_ntt_inv(c, acc.data(), 0, first_prime, 2, mod_num, mod_num);                         // :405
+    // ModDown pq -> q (:291-306) and + (0, b) (:417)
+    for (int y = 0; y < 2; y++)
+        for (int im = 0; im < nq - 1; im++) {
+            const u64 qi = h->pq[np + im];
+            const u64 pinv = orc_invmod(p0 % qi, qi), pinv_s = orc_xshoup(pinv, qi);          // PCMM_Context.cuh:47-56
+            const u64* in = acc.data() + (size_t)y * N * mod_num;
+            u64* out = rlwe_out + (size_t)y * N * (L + 1) + (size_t)im * N;
+            const u64* bpoly = embed.data() + (size_t)k * N * mod_num + (size_t)(np + im) * N;
+            for (long x = 0; x < N; x++) {
+                u64 ra = in[(size_t)im * N + x] % qi;
+                ra = qi - ra + in[(size_t)(np + im) * N + x];
+                u64 r = orc_mulmod_shoup(ra, pinv, pinv_s, qi);
+                if (y == 1) { r += bpoly[x]; if (r >= qi) r -= qi; }
+                out[x] = r;
+            }
+        }
+    orc_ntt_fwd(c, rlwe_out, 0, K, 2, nq - 1, L + 1);                                        // :419
+    return 0;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -107,6 +107,11 @@ int orc_rlwe_decompose(const orc_pcmm*, const uint64_t* rlwe, uint64_t* const* m
 int orc_ppmm(const orc_pcmm*, const float* W, const uint64_t* const* mlwe, uint64_t* out, int M, int Kin,
              int mod_num, double scaler, long col_begin, long col_count);
 
+/* PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425): mlwe_num MLWE ciphertexts [(nq-1)][(rank+1)][N1] (coefficient
+ * domain) -> one RLWE ciphertext [a | b] (L+1 limbs each, limbs 0..nq-2 written, NTT domain) with rank repacking keys
+ * (key i at keys + i*N*mod_num*2 = [a | b], mod_num = np+nq-1 limbs, NTT domain).  One special prime, two ring-pack moduli. */
+int orc_mlwe_pack(const orc_pcmm*, uint64_t* rlwe_out, const uint64_t* const* mlwe, int mlwe_num, const uint64_t* keys);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

@@ -59,6 +59,7 @@ def lib():
             "orc_pcmm_create": (vp, [vp, i, i, P64, i, P64, i]), "orc_pcmm_destroy": (None, [vp]),
             "orc_rlwe_decompose": (i, [vp, P64, C.POINTER(P64), i, i]),
             "orc_ppmm": (i, [vp, C.POINTER(C.c_float), C.POINTER(P64), P64, i, i, i, d, l, l]),
+            "orc_mlwe_pack": (i, [vp, P64, C.POINTER(P64), i, P64]),
             "orc_max_threads": (i, []),
         }
         for name, (res, args) in sig.items():
@@ -179,6 +180,13 @@ class OraclePCMM:
         rc = self.L_.orc_rlwe_decompose(self.h, _ptr(rlwe_coeff), self._ptrs(mlwe), len(mlwe), l)
         if rc:
             raise ValueError("orc_rlwe_decompose: %d" % rc)
+
+    def mlweCipherPacking(self, rlwe_out, mlwe, keys):
+        """PCMM_Scheme.cuh:361-425 on host arrays: mlwe list of [(nq-1)][(rank+1)][N1] coefficient-domain arrays, keys
+        [rank][2][mod_num][N] (NTT domain); writes limbs 0..nq-2 of both polynomials of rlwe_out ([2][L+1][N], NTT domain)."""
+        rc = self.L_.orc_mlwe_pack(self.h, _ptr(rlwe_out), self._ptrs(mlwe), len(mlwe), _ptr(keys))
+        if rc:
+            raise ValueError("orc_mlwe_pack: %d" % rc)
 
     def PPMM(self, W, mlwe, out, M, Kin, mod_num, scaler, col_begin=0, col_count=None):
         C_ = (self.rank + 1) * self.N1

@@ -121,6 +121,11 @@ static int run() {
     pcmm_scheme.PPMM((float*)Wd, mlwe, M, mlwe_num - 1, N1, mlwe_num);
     EXPECT(download(mlwe[0]->cipher_device, C) == before, "PPMM shape errors do no work");
 
+    // mlweCipherPacking without repacking keys: std::invalid_argument, as a missing key in the reference (KeySwitch_23.cuh:198-201)
+    threw = false;
+    try { pcmm_scheme.mlweCipherPacking(rlwe, mlwe, mlwe_num, 0); } catch (const std::invalid_argument&) { threw = true; }
+    EXPECT(threw, "mlweCipherPacking without keys throws std::invalid_argument");
+
     for (MLWECiphertext* m : mlwe) delete m;
     ckks_free(Wd);
     orc_pcmm_destroy(orc_p);

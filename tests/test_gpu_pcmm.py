@@ -104,3 +104,46 @@ def test_ppmm_shape_errors():
         dev.PPMM(0, [], 0, 4, 4, 64, 4, 2, 1.0)            # mat_K != N1  (PPMM_kernel.cuh:256-259)
     with pytest.raises(ValueError):
         dev.PPMM(0, [], 0, 4, 4, 128, 5, 2, 1.0)           # mat_N != mlwe_num (:260-263)
+
+
+@pytest.mark.parametrize("logN,N1,mlwe_num", [(12, 128, 32), (12, 128, 8), (10, 64, 16), (16, 128, 512)])
+def test_mlwe_packing(logN, N1, mlwe_num):
+    """mlweCipherPacking through the C ABI against the oracle: embedding, lift to the special prime, NTT, inner product with the
+    repacking keys, iNTT, division by the special prime, + (0, b), NTT - bit-exact on random samples and random keys (the
+    oracle itself is pinned by a decrypt identity with real keys)."""
+    p0, q = CFG3_P[0], CFG2_Q[:2]
+    pair, dev, orc, rank = make(logN, N1, q, [p0], [p0], q)
+    N = pair.N
+    assert rank % mlwe_num == 0
+    rng = np.random.default_rng(logN * 1000 + mlwe_num)
+    mlwe = [rng.integers(0, q[0], size=(1, rank + 1, N1), dtype=np.uint64) for _ in range(mlwe_num)]
+    for m in mlwe[:2]:
+        m[0, :, 0] = q[0] - 1                              # largest residues: the lift's upper branch
+        m[0, :, 1] = q[0] // 2 + 1
+        m[0, :, 2] = q[0] // 2
+    keys = np.empty((rank, 4, N), dtype=np.uint64)
+    for j, pr in enumerate((p0, q[0], p0, q[0])):
+        keys[:, j, :] = rng.integers(0, pr, size=(rank, N), dtype=np.uint64)
+    want = np.zeros((2, 2, N), dtype=np.uint64)
+    orc.mlweCipherPacking(want.reshape(-1), [m.reshape(-1) for m in mlwe], keys.reshape(-1))
+    bufs = [DeviceBuffer.from_numpy(m) for m in mlwe]
+    dkeys = DeviceBuffer.from_numpy(keys)
+    dout = DeviceBuffer(want.nbytes); dout.zero()
+    embed, mult = DeviceBuffer(8 * (rank + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    dev.mlweCipherPacking(dout, bufs, mlwe_num, 0, dkeys, embed, mult)
+    got = dout.download(np.uint64).reshape(want.shape)
+    assert np.array_equal(got[:, 0], want[:, 0])
+    assert not got[:, 1].any()                             # limbs above the level are not touched
+
+
+def test_mlwe_packing_errors():
+    from ckks_llm_amd import CkksError
+    q = CFG2_Q[:3]
+    pair, dev, orc, rank = make(10, 64, q, CFG3_P[:1], [CFG3_P[0]], q)          # three ring-pack moduli: not supported
+    b = DeviceBuffer(8 * 17 * 64)
+    big = DeviceBuffer(8 * 17 * 2 * 1024)
+    with pytest.raises(CkksError):
+        dev.mlweCipherPacking(big, [b], 1, 0, big, big, big)
+    pair, dev, orc, rank = make(10, 64, q[:2], CFG3_P[:1], [CFG3_P[0]], q[:2])
+    with pytest.raises(CkksError):
+        dev.mlweCipherPacking(big, [b] * 3, 3, 0, big, big, big)                  # 3 does not divide the rank

@@ -128,3 +128,59 @@ def test_ppmm_rescale_is_rounding_division():
             X = sum(A[m][n] * int(small[n][c]) for n in range(Kin))
             want = (X - (X % qs[1])) // qs[1]
             assert int(out[m, 0, c]) == want % qs[0]
+
+
+@pytest.mark.parametrize("mlwe_num", [16, 4])
+def test_packing_decrypt_identity(mlwe_num):
+    """mlweCipherPacking (PCMM_Scheme.cuh:361-425) pinned end to end on a small ring: decompose an RLWE ciphertext of mu into
+    MLWE samples, build repacking keys the way addRepakcingKey does (key_i = (a_i, -a_i*s + p0*iota(s_i)), s_i[n] = s[i + n*k],
+    PCMM_Scheme.cuh:128-224, ringSwitch.cuh:7-19; noise left out), pack, decrypt with s: the result is mu on the positions
+    n*k + m*gap and 0 elsewhere, up to the rounding of the ModDown.  A wrong embedding position, lift, key slot or sign breaks it."""
+    from tests.params import CFG3_P
+    logN, N, N1, k = 8, 256, 16, 16
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    ctx = O.OracleContext(logN, [P0], [Q0, Q1])
+    pc = O.OraclePCMM(ctx, N1, k, [P0], [Q0, Q1])
+    rng = np.random.default_rng(100 + mlwe_num)
+    s = [int(v) for v in rng.integers(-1, 2, N)]
+    mu = [int(v) for v in rng.integers(-(1 << 20), 1 << 20, N)]
+    a = [int(v) for v in rng.integers(0, Q0, N)]
+    a_s = negacyclic_mul(a, [v % Q0 for v in s], Q0)
+    b = [(m - x) % Q0 for m, x in zip(mu, a_s)]                       # decryption convention mu = a*s + b
+    rlwe = np.zeros((2, 2, N), dtype=np.uint64)                         # [a | b], L + 1 = 2 limbs, level 0 in use
+    rlwe[0, 0], rlwe[1, 0] = a, b
+    mlwe = [np.zeros((1, k + 1, N1), dtype=np.uint64) for _ in range(mlwe_num)]
+    pc.rlweCipherDecompose(rlwe.reshape(-1), [m.reshape(-1) for m in mlwe], 0)
+    # repacking keys over [P0, Q0], coefficient domain first
+    keys = np.zeros((k, 2, 2, N), dtype=np.uint64)
+    for i in range(k):
+        iota = [0] * N
+        for n in range(N1):
+            iota[n * k] = s[i + n * k]
+        for j, q in enumerate((P0, Q0)):
+            ai = [int(v) for v in rng.integers(0, q, N)]
+            ais = negacyclic_mul(ai, [v % q for v in s], q)
+            keys[i, 0, j] = ai
+            keys[i, 1, j] = [(-x + P0 * t) % q for x, t in zip(ais, iota)]
+        for y in range(2):
+            ctx.ToNTTInplace(keys[i, y].reshape(-1), 0, 0, 1, 2, 2)      # primes [P0, Q0] = context primes 0, 1
+    out = np.zeros((2, 2, N), dtype=np.uint64)
+    pc.mlweCipherPacking(out.reshape(-1), [m.reshape(-1) for m in mlwe], keys.reshape(-1))
+    ctx.FromNTTInplace(out.reshape(-1), 0, 1, 2, 1, 2)                   # limb 0 of both polynomials, prime Q0
+    a2, b2 = [int(v) for v in out[0, 0]], [int(v) for v in out[1, 0]]
+    dec = [(x + y) % Q0 for x, y in zip(negacyclic_mul(a2, [v % Q0 for v in s], Q0), b2)]
+    gap = k // mlwe_num
+    worst = 0
+    for pos in range(N):
+        want = mu[pos] if (pos % k) % gap == 0 else 0
+        d = (dec[pos] - want) % Q0
+        d = d - Q0 if d > Q0 // 2 else d
+        worst = max(worst, abs(d))
+    assert worst <= N, worst
+
+
+def test_packing_rejects_what_the_reference_cannot_do():
+    ctx = O.OracleContext(8, [CFG2_Q[5]], CFG2_Q[:3])
+    pc = O.OraclePCMM(ctx, 16, 16, [CFG2_Q[5]], CFG2_Q[:3])               # two remaining moduli: the reference's embedding overlaps
+    with pytest.raises(ValueError):
+        pc.mlweCipherPacking(np.zeros(2 * 3 * 256, dtype=np.uint64), [np.zeros(2 * 17 * 16, dtype=np.uint64)], np.zeros(16 * 2 * 3 * 256, dtype=np.uint64))
