@@ -59,6 +59,63 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel(ConvArgs a) {
     }
 }
 
+// ---- the same conversion in FP64 for bases whose primes are all below 2^41 ----
+// On this part a 64 x 64 -> 128-bit integer product costs more than ten quarter-rate 32-bit multiplies, a double FMA is one
+// full-rate instruction: with u128 accumulation the conversions are bound by integer multiplies, not by memory.  Here every
+// value is an exact integer held in a double (|.| < 2^53 throughout) and a*w mod q is the two-product form used by the NTT, so
+// the words written are the same.  y_j is brought to its canonical representative before it enters v and the sum, because the
+// reference's v = (int) sum y_j / d_j and sum y_j * hat_j are functions of that representative.
+__device__ __forceinline__ double u2d(u64 x) {                       // exact for x < 2^52
+    return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0;
+}
+__device__ __forceinline__ u64 d2u(double x) {                       // exact integer 0 <= x < 2^52
+    return (u64)__double_as_longlong(x + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
+}
+__device__ __forceinline__ double mulmod_d(double a, double w, double q, double qinv) {      // in (-0.51 q, 0.51 q)
+    const double h = a * w, l = __builtin_fma(a, w, -h), c = __builtin_rint(h * qinv);
+    return __builtin_fma(-c, q, h) + l;
+}
+__device__ __forceinline__ double canon_d(double r, double q, double qinv) {                 // any |r| < 2^52 -> [0, q)
+    r = __builtin_fma(-__builtin_rint(r * qinv), q, r);
+    return r < 0.0 ? r + q : r;
+}
+
+// The targets of a block are shared out over CONV_TGT_PARTS workgroups (each recomputes the cheap y_j): a lane that walked
+// through all 24+ targets alone left the launch with too few, too long lanes to cover the memory latency.
+constexpr int CONV_TGT_PARTS = 4;
+template <int MAXS>
+__global__ __launch_bounds__(CONV_THREADS) void conv_kernel_f64(ConvArgs a) {
+    const int blk = blockIdx.y / CONV_TGT_PARTS, part = blockIdx.y % CONV_TGT_PARTS;
+    const ConvBlock& __restrict__ b = a.blocks[blk];
+    const long x = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
+    const u64* in = a.in + (long)blockIdx.z * a.in_batch_stride;
+    u64* out = a.out + (long)blockIdx.z * a.out_batch_stride + (long)blk * a.out_block_stride;
+    const int nsrc = b.nsrc;
+    double y[MAXS];
+    double vv = 0.0;
+#pragma unroll
+    for (int j = 0; j < MAXS; j++) {
+        y[j] = 0.0;
+        if (j < nsrc) {
+            const PrimeConst& ps = a.primes[b.src_prime[j]];
+            const u64 xin = in[(long)b.src_limb[j] * a.N + x];
+            if (j < b.ncopy && part == 0) out[(long)b.copy_limb[j] * a.N + x] = xin;
+            y[j] = canon_d(mulmod_d(u2d(xin), b.hatinv_d[j], ps.qd, ps.qinv_d), ps.qd, ps.qinv_d);
+            vv += y[j] / ps.qd;
+        }
+    }
+    const double v = (double)(int)vv;
+    const int per = (b.ntgt + CONV_TGT_PARTS - 1) / CONV_TGT_PARTS, k_end = min(b.ntgt, (part + 1) * per);
+    for (int k = part * per; k < k_end; k++) {
+        const PrimeConst& pr = a.primes[b.tgt_prime[k]];
+        double acc = -v * b.dmod_d[k];                               // |v| <= nsrc, |dmod| <= q/2: exact
+#pragma unroll
+        for (int j = 0; j < MAXS; j++)
+            if (j < nsrc) acc += mulmod_d(y[j], b.hat_d[k][j], pr.qd, pr.qinv_d);
+        out[(long)b.tgt_limb[k] * a.N + x] = d2u(canon_d(acc, pr.qd, pr.qinv_d));
+    }
+}
+
 static int launch_conv(ckks_ctx* c, const ConvPlan& plan, u64* out, const u64* in, int batch, long in_bs, long out_bs,
                        long out_block_stride, int centred, int max_src) {
     if (plan.count == 0 || batch <= 0) return CKKS_OK;
@@ -67,6 +124,14 @@ static int launch_conv(ckks_ctx* c, const ConvPlan& plan, u64* out, const u64* i
     a.N = c->N; a.in_batch_stride = in_bs; a.out_batch_stride = out_bs; a.out_block_stride = out_block_stride;
     a.centred = centred;
     dim3 grid((unsigned)(c->N / CONV_THREADS), plan.count, batch), block(CONV_THREADS);
+    if (plan.f64_ok && !centred && c->arith_mode == 0) {
+        grid.y *= CONV_TGT_PARTS;
+        if (max_src <= 4) hipLaunchKernelGGL(conv_kernel_f64<4>, grid, block, 0, c->stream, a);
+        else if (max_src <= 8) hipLaunchKernelGGL(conv_kernel_f64<8>, grid, block, 0, c->stream, a);
+        else hipLaunchKernelGGL(conv_kernel_f64<CONV_MAX_SRC>, grid, block, 0, c->stream, a);
+        CKKS_HIP_TRY(hipGetLastError());
+        return CKKS_OK;
+    }
     if (max_src <= 4) hipLaunchKernelGGL(conv_kernel<4>, grid, block, 0, c->stream, a);
     else if (max_src <= 8) hipLaunchKernelGGL(conv_kernel<8>, grid, block, 0, c->stream, a);
     else hipLaunchKernelGGL(conv_kernel<CONV_MAX_SRC>, grid, block, 0, c->stream, a);
@@ -107,11 +172,55 @@ __global__ __launch_bounds__(CONV_THREADS) void moddown_kernel(ModDownArgs a) {
     u64 v = pq.q - r + in[(long)(a.K + iq) * a.N + x];
     a.out[(long)blockIdx.z * a.out_batch_stride + (long)iq * a.N + x] = mul_shoup(v, a.PinvModq[iq], a.PinvModq[a.q_num + iq], pq.q);
 }
+constexpr int MODDOWN_TGTS = 4;        // output primes per lane: the special-prime residues are read and scaled once for all of them
+template <int MAXK>
+__global__ __launch_bounds__(CONV_THREADS) void moddown_kernel_f64(ModDownArgs a, int q_count) {
+    const long x = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
+    const u64* in = a.in + (long)blockIdx.z * a.in_batch_stride;
+    double rb[MAXK];
+#pragma unroll
+    for (int i = 0; i < MAXK; i++) {
+        rb[i] = 0.0;
+        if (i < a.K) {
+            const PrimeConst& pp = a.primes[i];
+            // the canonical representative of rb enters the sums (there is no v term to absorb another one)
+            rb[i] = a.K == 1 ? u2d(in[x])
+                             : canon_d(mulmod_d(u2d(in[(long)i * a.N + x]), u2d(a.pHatInv[i]), pp.qd, pp.qinv_d), pp.qd, pp.qinv_d);
+        }
+    }
+    const int iq_end = min(q_count, (int)(blockIdx.y + 1) * MODDOWN_TGTS);
+    for (int iq = blockIdx.y * MODDOWN_TGTS; iq < iq_end; iq++) {
+        const PrimeConst& pq = a.primes[a.K + iq];
+        double r;
+        if (a.K == 1) {
+            r = canon_d(rb[0], pq.qd, pq.qinv_d);                         // in[x] % q
+        } else {
+            double acc = 0.0;
+#pragma unroll
+            for (int i = 0; i < MAXK; i++)
+                if (i < a.K) acc += mulmod_d(rb[i], u2d(a.pHatVecModq[(long)iq * a.K + i]), pq.qd, pq.qinv_d);
+            r = canon_d(acc, pq.qd, pq.qinv_d);
+        }
+        const double v = pq.qd - r + u2d(in[(long)(a.K + iq) * a.N + x]);
+        a.out[(long)blockIdx.z * a.out_batch_stride + (long)iq * a.N + x] =
+            d2u(canon_d(mulmod_d(v, u2d(a.PinvModq[iq]), pq.qd, pq.qinv_d), pq.qd, pq.qinv_d));
+    }
+}
 static int launch_moddown(ckks_ctx* c, u64* out, const u64* in, int l, int batch, long in_bs, long out_bs) {
     ModDownArgs a;
     a.in = in; a.out = out; a.primes = c->d_primes; a.pHatVecModq = c->d_pHatVecModq; a.pHatInv = c->d_pHatInvVecModp;
     a.PinvModq = c->d_PinvModq; a.N = c->N; a.in_batch_stride = in_bs; a.out_batch_stride = out_bs; a.K = c->K; a.q_num = c->q_num;
     dim3 grid((unsigned)(c->N / CONV_THREADS), l + 1, batch), block(CONV_THREADS);
+    bool f64 = c->arith_mode == 0;
+    for (int i = 0; i < c->K + l + 1 && f64; i++) f64 = c->f64_ok[i] != 0;
+    if (f64) {
+        grid.y = (unsigned)((l + 1 + MODDOWN_TGTS - 1) / MODDOWN_TGTS);
+        if (c->K <= 4) hipLaunchKernelGGL(moddown_kernel_f64<4>, grid, block, 0, c->stream, a, l + 1);
+        else if (c->K <= 8) hipLaunchKernelGGL(moddown_kernel_f64<8>, grid, block, 0, c->stream, a, l + 1);
+        else hipLaunchKernelGGL(moddown_kernel_f64<16>, grid, block, 0, c->stream, a, l + 1);
+        CKKS_HIP_TRY(hipGetLastError());
+        return CKKS_OK;
+    }
     if (c->K <= 4) hipLaunchKernelGGL(moddown_kernel<4>, grid, block, 0, c->stream, a);
     else if (c->K <= 8) hipLaunchKernelGGL(moddown_kernel<8>, grid, block, 0, c->stream, a);
     else hipLaunchKernelGGL(moddown_kernel<16>, grid, block, 0, c->stream, a);

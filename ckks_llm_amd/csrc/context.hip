@@ -65,6 +65,18 @@ static void fill_conv_block(ckks::ConvBlock& b, const std::vector<u64>& pqt, con
         for (int j = 0; j < b.nsrc; j++) b.hat[k][j] = H::prod_mod(sp, 0, b.nsrc, j, r);
         b.dmod[k] = H::prod_mod(sp, 0, b.nsrc, -1, r);
     }
+    // FP64 tables for the conversion kernel's double-precision path (all primes of the block below 2^41)
+    b.f64_ok = 1;
+    for (int i : src) if (pqt[i] >= (1ull << 41)) b.f64_ok = 0;
+    for (int i : tgt) if (pqt[i] >= (1ull << 41)) b.f64_ok = 0;
+    if (b.f64_ok) {
+        for (int j = 0; j < b.nsrc; j++) b.hatinv_d[j] = balanced_double(b.hatinv[j], sp[j]);
+        for (int k = 0; k < b.ntgt; k++) {
+            const u64 r = pqt[tgt[k]];
+            for (int j = 0; j < b.nsrc; j++) b.hat_d[k][j] = balanced_double(b.hat[k][j], r);
+            b.dmod_d[k] = balanced_double(b.dmod[k], r);
+        }
+    }
 }
 
 extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int p_num, const uint64_t* q, int q_num,
@@ -284,6 +296,12 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
             }
         }
     }
+
+    for (auto* plans : {&c->plan_pq_to_t, &c->plan_qj_to_t, &c->plan_t_to_pq, &c->plan_hybrid})
+        for (ckks::ConvPlan& pl : *plans) {
+            pl.f64_ok = pl.count > 0;
+            for (int b = 0; b < pl.count; b++) pl.f64_ok = pl.f64_ok && blocks[pl.first + b].f64_ok;
+        }
 
     // ---- upload ----
     int rc = CKKS_OK;

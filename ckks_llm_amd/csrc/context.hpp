@@ -34,11 +34,16 @@ struct ConvBlock {
     u64 add_in[CONV_MAX_SRC];                           // added to the input residue before scaling (T -> PQ centring)
     u64 sub_out[CONV_MAX_TGT];                          // subtracted from the output residue (T -> PQ centring)
     short copy_prime[CONV_MAX_SRC], copy_limb[CONV_MAX_SRC];  // ncopy source limbs passed through unchanged
-    int ncopy, pad;
+    int ncopy;
+    int f64_ok;                                         // every prime of the block is below 2^41: the FP64 tables below are filled
+    double hatinv_d[CONV_MAX_SRC];                      // balanced representatives as doubles
+    double hat_d[CONV_MAX_TGT][CONV_MAX_SRC];
+    double dmod_d[CONV_MAX_TGT];
 };
 
 struct ConvPlan {          // blocks of one map at one level, contiguous in device memory
     int first = 0, count = 0;
+    bool f64_ok = false;   // all blocks can take the FP64 kernel
 };
 
 }  // namespace ckks

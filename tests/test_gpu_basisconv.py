@@ -110,11 +110,14 @@ def test_rescale():
         d.rescaleAndEqual(dc, scratch, 0)                   # level-0 operand (Scheme_23.cuh:192-194 behaviour)
 
 
-@pytest.mark.parametrize("logN,nq,np_", [(12, 6, 2), (10, 7, 3), (12, 24, 6)])
-def test_hybrid_keyswitch_stages(logN, nq, np_):
-    """Textbook hybrid switch over [P|Q_l] (BASELINE config 3 shape at reduced N): every stage and the whole chain."""
+@pytest.mark.parametrize("arith_mode", [0, 1])
+@pytest.mark.parametrize("logN,nq,np_", [(12, 6, 2), (10, 7, 3), (12, 24, 6), (10, 3, 1)])
+def test_hybrid_keyswitch_stages(logN, nq, np_, arith_mode):
+    """Textbook hybrid switch over [P|Q_l] (BASELINE config 3 shape at reduced N): every stage and the whole chain, with the
+    FP64 conversion / ModDown kernels (arith_mode 0: these primes are below 2^41) and with the integer ones (arith_mode 1)."""
     q, p = CFG2_Q[:nq], CFG3_P[:np_]
     pair = Pair(logN, p, q)
+    pair.dev.set_arith_mode(arith_mode)
     o, d, N = pair.orc, pair.dev, pair.N
     W = np_ + nq
     dnum = -(-nq // np_)
