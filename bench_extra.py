@@ -117,5 +117,31 @@ def bench_packing(P, N1=128, reps=5):
                          "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
 
 
+def bench_decompose(P, N1=128, L1=12, reps=5):
+    """RLWE -> MLWE decomposition in front of PPMM (PCMM_Scheme::rlweCipherDecompose): one ciphertext at N = 2^16 with 12 primes
+    into rank = 512 samples.  The output is rank times the input; algorithmic bytes = input read once + output written once."""
+    from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
+    primes = P.CFG2_Q[:L1]
+    ctx = Context_23(16, [], primes)
+    N = 1 << 16
+    rank = N // N1
+    sch = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, ctx))
+    rng = np.random.default_rng(7)
+    rl = np.empty((2, L1, N), dtype=np.uint64)
+    for j, q in enumerate(primes):
+        rl[:, j] = rng.integers(0, q, (2, N), dtype=np.uint64)
+    d = DeviceBuffer.from_numpy(rl)
+    bufs = [DeviceBuffer(8 * L1 * (rank + 1) * N1) for _ in range(rank)]
+    sch.rlweCipherDecompose(d, bufs, rank, 0, L1 - 1)
+    ctx.timer_start()
+    for _ in range(reps):
+        sch.rlweCipherDecompose(d, bufs, rank, 0, L1 - 1)
+    ms = ctx.timer_stop() / reps
+    alg = 8.0 * rank * L1 * (rank + 1) * N1 + 2 * L1 * 8.0 * N * 3        # samples out; ciphertext through iNTT, gather, NTT
+    return {"workload": "rlweCipherDecompose: 1 RLWE ciphertext (N=2^16, 12 primes) -> 512 MLWE samples (N1=128)", "ms": round(ms, 3),
+            "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
+
+
 def run(P):
-    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P), "packing": bench_packing(P)}
+    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P), "decompose": bench_decompose(P), "packing": bench_packing(P)}

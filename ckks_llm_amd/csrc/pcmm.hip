@@ -66,6 +66,40 @@ __global__ __launch_bounds__(256) void rlwe_gather_kernel(GatherArgs a) {
     dst[(long)i * N1 + g] = v;
 }
 
+// The same gather through LDS.  Row i of sample m is the negacyclic polynomial a read at positions g*k + (m*gap - i), g = 0..N1-1
+// (positions below zero wrap to the top with a sign change), so for a tile of G consecutive g every row needs the contiguous
+// window [g0*k - (k-1), (g0+G)*k): it is loaded once, coalesced, into LDS (one pad word per k so that lanes on consecutive g hit
+// different banks) and every output row segment (G words = 64 or 128 contiguous bytes) is written from there.  The output is
+// k times larger than the input; the kernel is bound by its writes.
+constexpr int GATHER_M_CHUNK = 8;          // samples per workgroup
+template <int G>
+__global__ __launch_bounds__(256) void rlwe_gather_tiled_kernel(GatherArgs a) {
+    extern __shared__ u64 win[];                                     // (G + 1) * (k + 1) words
+    const int k = a.rank, N1 = a.N1, im = blockIdx.y, g0 = blockIdx.x * G;
+    const int gap = k / a.mlwe_num;
+    const u64 q = a.primes[a.p_num + im].q;
+    const u64* A = a.rlwe + a.N * im;
+    const u64* B = a.rlwe + a.N * (a.L + 1 + im);
+    // window position u = p - g0*k + k, p = polynomial position; LDS index u + u / k
+    for (int u = threadIdx.x + 1; u < (G + 1) * k; u += 256) {
+        const long p = (long)g0 * k + u - k;
+        win[u + u / k] = p >= 0 ? A[p] : negate_mod(A[a.N + p], q);
+    }
+    __syncthreads();
+    const int gl = threadIdx.x % G, slot = threadIdx.x / G;
+    constexpr int SLOTS = 256 / G;
+    const int m_end = min(a.mlwe_num, (int)(blockIdx.z + 1) * GATHER_M_CHUNK);
+    for (int m = blockIdx.z * GATHER_M_CHUNK; m < m_end; m++) {
+        u64* dst = a.mlwe[m] + (long)N1 * (k + 1) * im + g0 + gl;
+        const int base = gl * k + k + m * gap;                       // u of row 0
+        for (int i = slot; i < k; i += SLOTS) {
+            const int u = base - i;
+            dst[(long)i * N1] = win[u + u / k];
+        }
+        if (slot == 0) dst[(long)k * N1] = B[(long)m * gap + (long)(g0 + gl) * k];       // b row: no shift, never wraps
+    }
+}
+
 // ------------------------------------------------------------------------------------------------------------
 // plaintext quantisation: A = (int64)(float * double), |A| maximum, balanced base-256 digit planes
 // ------------------------------------------------------------------------------------------------------------
@@ -181,9 +215,23 @@ extern "C" int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* 
     GatherArgs a;
     a.rlwe = rlwe; a.mlwe = h->d_ptrs; a.primes = c->d_primes; a.N = c->N; a.N1 = h->N1; a.rank = h->rank; a.mlwe_num = mlwe_num;
     a.L = c->L; a.p_num = c->p_num;
-    long per = (long)(h->rank + 1) * h->N1;
-    dim3 grid((unsigned)((per + 255) / 256), l + 1, mlwe_num), block(256);
-    hipLaunchKernelGGL(rlwe_gather_kernel, grid, block, 0, c->stream, a);
+    const int k = h->rank;
+    const bool force_plain = getenv("CKKS_GATHER_PLAIN") != nullptr;              // test hook: the one-lane-per-word kernel
+    // 16-word row segments (one 128-byte line) when the window fits the LDS a workgroup may ask for, else 8-word segments
+    static const bool big_lds = hipFuncSetAttribute(reinterpret_cast<const void*>(rlwe_gather_tiled_kernel<16>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess;
+    const size_t lds_cap = big_lds ? 96 * 1024 : 64 * 1024;
+    const int G = (h->N1 % 16 == 0 && (size_t)17 * (k + 1) * 8 <= lds_cap) ? 16 : 8;
+    if (!force_plain && h->N1 % G == 0 && k % mlwe_num == 0 && (size_t)(G + 1) * (k + 1) * 8 <= (G == 16 ? lds_cap : 64 * 1024)) {
+        dim3 grid(h->N1 / G, l + 1, (mlwe_num + GATHER_M_CHUNK - 1) / GATHER_M_CHUNK), block(256);
+        const size_t lds = (size_t)(G + 1) * (k + 1) * sizeof(u64);
+        if (G == 16) hipLaunchKernelGGL(rlwe_gather_tiled_kernel<16>, grid, block, lds, c->stream, a);
+        else hipLaunchKernelGGL(rlwe_gather_tiled_kernel<8>, grid, block, lds, c->stream, a);
+    } else {
+        long per = (long)(h->rank + 1) * h->N1;
+        dim3 grid((unsigned)((per + 255) / 256), l + 1, mlwe_num), block(256);
+        hipLaunchKernelGGL(rlwe_gather_kernel, grid, block, 0, c->stream, a);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     // the pointer table was copied asynchronously from the caller's host array: make sure it is consumed before returning
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));

@@ -21,8 +21,14 @@ def make(logN, N1, q_ctx, p_ctx, p_rp, q_rp):
     return pair, dev, orc, rank
 
 
-@pytest.mark.parametrize("logN,N1,mlwe_num", [(10, 128, 8), (10, 128, 2), (12, 256, 16), (10, 64, 1)])
-def test_rlwe_decompose(logN, N1, mlwe_num):
+@pytest.mark.parametrize("plain", [False, True])
+@pytest.mark.parametrize("logN,N1,mlwe_num", [(10, 128, 8), (10, 128, 2), (12, 256, 16), (10, 64, 1), (14, 32, 512), (14, 32, 64),
+                                              (12, 8, 512), (10, 4, 256)])
+def test_rlwe_decompose(logN, N1, mlwe_num, plain, monkeypatch):
+    """Both gather kernels (LDS-tiled with 16- or 8-word row segments, and one lane per word - forced through the launcher's
+    test hook, and taken anyway when N1 is not a multiple of 8) against the oracle."""
+    if plain:
+        monkeypatch.setenv("CKKS_GATHER_PLAIN", "1")
     q = CFG2_Q[:3]
     pair, dev, orc, rank = make(logN, N1, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
     N, L = pair.N, len(q) - 1
