@@ -25,10 +25,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes moved by ONE pass launch of the default workload (1536 limbs), from the rocprofv3 counters FETCH_SIZE and
-# WRITE_SIZE of that launch, each scaled by what the same counter reads for a device-to-device copy of known size in the
-# same run (FETCH_SIZE reads 0.502 of the bytes copied, WRITE_SIZE 1.000): 768 MiB read + 12 MiB twiddles, 768 MiB written.
-NTT_PASS_TRAFFIC_BYTES_1536_LIMBS = 1.623e9
+# HBM bytes moved by ONE forward row-pass launch of the default workload (1536 limbs), from the rocprofv3 counters FETCH_SIZE
+# and WRITE_SIZE of that launch, each scaled by what the same counter reads for a device-to-device copy of known size in the
+# same run (FETCH_SIZE reads 0.500 of the bytes copied, WRITE_SIZE 1.000): 480 MiB of 5-byte inter-pass values + 12 MiB of
+# twiddles read, 768 MiB written.  (The strided pass of the same transform moves 1.309e9: 768 MiB read, 480 MiB written.)
+NTT_PASS_TRAFFIC_BYTES_1536_LIMBS = 1.321e9
 MFMA_I8_PEAK_TMACS = 2516.6          # 5.033 POP/s dense int8 = 2.5166e15 MAC/s
 
 
