@@ -1,0 +1,90 @@
+"""GPU end-to-end check of the ring-packed PCMM pipeline through the C ABI, the way the reference's test_rlwe_decomp.cu runs it
+(encrypt, rlweCipherDecompose, PPMM, mlweCipherPacking, decrypt, compare with the plaintext product, :92-98,195): the decrypted
+coefficients must be the matrix product of W with the coefficient-packed message, up to the scheme's rounding and noise.
+Key generation, encryption and decryption are plain host arithmetic here (they are not on the GPU path)."""
+import numpy as np
+import pytest
+
+from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
+from tests.helpers import negacyclic_mul
+from tests.params import CFG2_Q, CFG3_P
+
+pytestmark = pytest.mark.gpu
+
+
+def centred(v, q):
+    v %= q
+    return v - q if v > q // 2 else v
+
+
+@pytest.mark.parametrize("mlwe_num", [16, 4])
+def test_encrypt_decompose_ppmm_pack_decrypt(mlwe_num):
+    logN, N, N1, k = 10, 1024, 64, 16
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    gap = k // mlwe_num
+    ctx = Context_23(logN, [P0], [Q0, Q1])
+    sch = PCMM_Scheme(PCMM_Context(N1, k, [P0], [Q0, Q1], ctx))
+    rng = np.random.default_rng(7 + mlwe_num)
+    s = [int(v) for v in rng.integers(-1, 2, N)]
+    mu = [int(v) for v in rng.integers(-(1 << 30), 1 << 30, N)]
+    # ---- encrypt at level 1 (primes Q0, Q1), decryption convention mu = a*s + b (Scheme_23.cuh:125-126) ----
+    ct = np.zeros((2, 2, N), dtype=np.uint64)
+    e = [int(v) for v in rng.integers(-3, 4, N)]                            # one noise polynomial, reduced modulo every prime
+    for j, q in enumerate((Q0, Q1)):
+        a = [int(v) for v in rng.integers(0, q, N)]
+        a_s = negacyclic_mul(a, [v % q for v in s], q)
+        ct[0, j] = a
+        ct[1, j] = [(m + ee - x) % q for m, ee, x in zip(mu, e, a_s)]
+    d_ct = DeviceBuffer.from_numpy(ct)
+    ctx.ToNTTInplace(d_ct, 0, 1, 2, 2, 2)                                   # primes 1, 2 of [P0 | Q0 Q1]
+    # ---- repacking keys over [P0 | Q0]: key_i = (a_i, -a_i*s + P0*iota(s_i) + e_i), s_i[n] = s[i + n*k] (PCMM_Scheme.cuh:128-224) ----
+    keys = np.zeros((k, 2, 2, N), dtype=np.uint64)
+    for i in range(k):
+        iota = [0] * N
+        for n in range(N1):
+            iota[n * k] = s[i + n * k]
+        ek = [int(v) for v in rng.integers(-3, 4, N)]
+        for j, q in enumerate((P0, Q0)):
+            ai = [int(v) for v in rng.integers(0, q, N)]
+            ais = negacyclic_mul(ai, [v % q for v in s], q)
+            keys[i, 0, j] = ai
+            keys[i, 1, j] = [(-x + P0 * t + ee) % q for x, t, ee in zip(ais, iota, ek)]
+    d_keys = DeviceBuffer.from_numpy(keys)
+    ctx.ToNTTInplace(d_keys, 0, 0, 2 * k, 2, 2)                             # primes 0, 1
+    # ---- GPU pipeline ----
+    C = (k + 1) * N1
+    samples = [DeviceBuffer(8 * 2 * C) for _ in range(mlwe_num)]
+    sch.rlweCipherDecompose(d_ct, samples, mlwe_num, 0, 1)
+    M = Kin = mlwe_num
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    scaler = float(1 << 26)
+    d_out = DeviceBuffer(8 * M * 2 * C)
+    sch.PPMM(DeviceBuffer.from_numpy(W), samples, d_out, M, Kin, N1, Kin, 2, scaler)
+    assert sch.pcmm_context.info("last_path") == 1                           # the MFMA kernel ran
+    rows = [DeviceBuffer(8 * C) for _ in range(M)]                           # row m, first modulus (PPMM_kernel.cuh:345-348)
+    for m in range(M):
+        rows[m].L_.ckks_memcpy_d2d(rows[m].ptr, d_out.ptr + 8 * m * 2 * C, 8 * C)
+    d_res = DeviceBuffer(8 * 2 * 2 * N)
+    d_res.zero()
+    embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    sch.mlweCipherPacking(d_res, rows, M, 0, d_keys, embed, mult)
+    ctx.FromNTTInplace(d_res, 0, 1, 2, 1, 2)                                 # limb 0 (prime Q0) of both polynomials
+    res = d_res.download(np.uint64).reshape(2, 2, N)
+    # ---- decrypt and compare with the plaintext product ----
+    a2, b2 = [int(v) for v in res[0, 0]], [int(v) for v in res[1, 0]]
+    dec = [centred(x + y, Q0) for x, y in zip(negacyclic_mul(a2, [v % Q0 for v in s], Q0), b2)]
+    A = [[int(np.float64(W[m, n]) * scaler) for n in range(Kin)] for m in range(M)]     # the reference's quantisation (:148)
+    worst, biggest = 0, 0
+    for g in range(N1):
+        for m in range(M):
+            exact = sum(A[m][n] * mu[n * gap + g * k] for n in range(Kin))             # sample n holds mu[n*gap + g*k]
+            want = exact // Q1                                                            # fused rescale by the last prime
+            pos = g * k + m * gap
+            worst = max(worst, abs(dec[pos] - want))
+            biggest = max(biggest, abs(want))
+    # positions that no packed sample covers decrypt to rounding noise only
+    if gap > 1:
+        assert max(abs(dec[p]) for p in range(N) if (p % k) % gap) <= 16 * N
+    assert biggest > 1 << 15                                                  # the check is not vacuous
+    # rescale and ModDown rounding are O(N); the key noise contributes sum_i a_i * e_i / P0, about sqrt(k * N) * Q0 / P0 * 3
+    assert worst <= 16 * N, (worst, biggest)
