@@ -30,7 +30,7 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // loads complete in order: extra loads in flight can only make one of its waits longer, never shorter.
 __device__ __forceinline__ void async_copy16(const void* g, void* lds_base) {
     const unsigned l = (unsigned)(size_t)(lptr_t)lds_base;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory", "m0");
 }
 
 __device__ __forceinline__ double mulmod_f64(double a, double w, double q, double qinv) {
