@@ -103,19 +103,32 @@ __global__ __launch_bounds__(256) void rlwe_gather_tiled_kernel(GatherArgs a) {
 // ------------------------------------------------------------------------------------------------------------
 // plaintext quantisation: A = (int64)(float * double), |A| maximum, balanced base-256 digit planes
 // ------------------------------------------------------------------------------------------------------------
+constexpr int QUANT_PER_LANE = 8;
 __global__ __launch_bounds__(256) void quantise_kernel(const float* W, long long* A, unsigned long long* absmax, long count, double scaler) {
-    long i = (long)blockIdx.x * 256 + threadIdx.x;
+    __shared__ unsigned long long wave_max[4];
     unsigned long long m = 0;
-    if (i < count) {
-        long long v = (long long)((double)W[i] * scaler);
-        A[i] = v;
-        m = (unsigned long long)(v < 0 ? -v : v);
+    const long base = (long)blockIdx.x * 256 * QUANT_PER_LANE + threadIdx.x;
+#pragma unroll
+    for (int t = 0; t < QUANT_PER_LANE; t++) {
+        const long i = base + t * 256;
+        if (i < count) {
+            long long v = (long long)((double)W[i] * scaler);
+            A[i] = v;
+            const unsigned long long av = (unsigned long long)(v < 0 ? -v : v);
+            m = av > m ? av : m;
+        }
     }
     for (int off = 32; off > 0; off >>= 1) {
         unsigned long long o = __shfl_down(m, off);
         m = o > m ? o : m;
     }
-    if ((threadIdx.x & 63) == 0 && m) atomicMax(absmax, m);
+    // one atomic per workgroup: thousands of atomics on one word were most of this kernel's time
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) m = wave_max[w] > m ? wave_max[w] : m;
+        if (m) atomicMax(absmax, m);
+    }
 }
 // digit d of A (balanced, in [-128, 127]): byte d of (A + 0x80..80) xor 0x80
 __global__ __launch_bounds__(256) void digits_kernel(const long long* A, int8_t* dig, int M, int Kin, int Mpad, int Kpad, int DW) {
@@ -418,7 +431,8 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
     CKKS_HIP_TRY(hipMemcpyAsync(d_cst, cst.data(), PPMM_CONST_WORDS * sizeof(uint64_t), hipMemcpyHostToDevice, c->stream));
     long count = (long)M * Kin;
-    hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, c->stream, W, h->d_A, h->d_absmax, count, scaler);
+    hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 256 * QUANT_PER_LANE - 1) / (256 * QUANT_PER_LANE))), dim3(256), 0, c->stream, W, h->d_A,
+                       h->d_absmax, count, scaler);
     unsigned long long absmax = 0;
     CKKS_HIP_TRY(hipMemcpyAsync(&absmax, h->d_absmax, sizeof(absmax), hipMemcpyDeviceToHost, c->stream));
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
