@@ -52,6 +52,7 @@ def _declare(L):
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_rlwe_decompose_ntt": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_mlwe_pack": (i, [vp, vp, C.POINTER(vp), i, vp, vp, vp]),
+        "pcmm_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "pcmm_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
     }

@@ -224,6 +224,13 @@ class PCMM_Context:
         _check(self.L_.pcmm_info(self.h, name.encode(), C.byref(v)), "pcmm_info")
         return v.value
 
+    # -- PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
+    def ToNTTInplace(self, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size):
+        _check(self.L_.pcmm_ntt_fwd(self.h, _addr(data), poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "pcmm_ntt_fwd")
+
+    def FromNTTInplace(self, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size):
+        _check(self.L_.pcmm_ntt_inv(self.h, _addr(data), poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "pcmm_ntt_inv")
+
     def __del__(self):
         try:
             if self.h:

@@ -203,6 +203,7 @@ extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     (void)hipDeviceSynchronize();
     void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig};
     for (void* p : ptrs) if (p) (void)hipFree(p);
+    if (h->small) ckks_ctx_destroy(h->small);
     delete h;
     return CKKS_OK;
 }
@@ -374,6 +375,41 @@ extern "C" int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* c
     return CKKS_OK;
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// size-N1 transforms over the ring-pack primes: PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273,
+// kernels smallntt_60bit.cuh:7-152).  Same negacyclic transform, root rule and table convention as the big ring, so the big
+// ring's kernels run it from a table set built for N1; the reference's layout [batch][mod][poly][N1] is one launch per
+// (batch, modulus) with poly_mod_len = 1.  The reference runs N1 = 256 only; this runs every N1 >= 256.
+// ------------------------------------------------------------------------------------------------------------
+static int pcmm_small_ntt(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, bool inverse) {
+    if (!h || !data) return CKKS_E_INVALID;
+    if (poly_num <= 0 || mod_num <= 0 || mod_batch_size <= 0) return CKKS_OK;
+    if (start_mod_idx < 0 || start_mod_idx + mod_num > h->np + h->nq) { set_error("PCMM NTT: modulus range outside the ring-pack primes"); return CKKS_E_INVALID; }
+    int logN1 = 0;
+    while ((1 << logN1) < h->N1) logN1++;
+    if ((1 << logN1) != h->N1 || logN1 < 8) { set_error("PCMM NTT: N1 must be a power of two, at least 256"); return CKKS_E_INVALID; }
+    if (!h->small) {
+        int rc = ckks_ctx_create(&h->small, logN1, nullptr, 0, h->pq.data(), h->np + h->nq, nullptr, 0, 0);
+        if (rc) return rc;
+    }
+    h->small->stream = h->ctx->stream;
+    for (int z = 0; z < mod_batch_size; z++)
+        for (int j = 0; j < mod_num; j++) {
+            uint64_t* base = data + ((size_t)z * mod_num + j) * poly_num * h->N1;
+            int rc = launch_ntt(h->small, base, 0, start_mod_idx + j, poly_num, 1, 1, 0, 1, inverse);
+            if (rc) return rc;
+        }
+    return CKKS_OK;
+}
+extern "C" int pcmm_ntt_fwd(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
+    (void)start_poly_idx;                  // carried for the reference's signature; its kernels do not use it (smallntt_60bit.cuh:27-29)
+    return pcmm_small_ntt(h, data, poly_num, mod_num, start_mod_idx, mod_batch_size, false);
+}
+extern "C" int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
+    (void)start_poly_idx;
+    return pcmm_small_ntt(h, data, poly_num, mod_num, start_mod_idx, mod_batch_size, true);
+}
 
 static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
                        int M, int Kin, int mod_num, double scaler) {

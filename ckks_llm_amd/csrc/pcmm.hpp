@@ -21,6 +21,7 @@ struct pcmm_ctx {
     size_t zero_cap = 0;
     int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
     unsigned long long last_absmax = 0;
+    ckks_ctx* small = nullptr;               // tables of the size-N1 transform over the ring-pack primes, built on first use
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
 };
 

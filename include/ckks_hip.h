@@ -130,6 +130,12 @@ int ckks_hybrid_keyswitch(ckks_ctx* ctx, uint64_t* out, uint64_t* in_ntt, const 
 int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,
                     const uint64_t* q_ringpack, int q_count);
 int pcmm_ctx_destroy(pcmm_ctx* h);
+/* PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273; kernels smallntt_60bit.cuh:7-152): negacyclic transforms
+ * of size N1 over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1], limb (z, j, y) modulo
+ * pq_ringpack[start_mod_idx + j].  start_poly_idx is carried for the signature only (the reference's kernels ignore it).
+ * The reference runs N1 = 256 only and silently does nothing otherwise; here N1 >= 256, smaller rings return CKKS_E_INVALID. */
+int pcmm_ntt_fwd(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
+int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
 /* "N1", "mlwe_rank", and facts about the last PPMM call: "last_path" (1 = int8 MFMA kernel, 0 = generic 128-bit kernel),
  * "last_DW" / "last_DC" (base-256 digits of the plaintext matrix / of the residues), "last_absmax" (max |A|). */
 int pcmm_info(const pcmm_ctx* h, const char* name, long* value);

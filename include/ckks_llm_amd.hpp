@@ -205,6 +205,13 @@ public:
         check(pcmm_info(handle, name, &v), "pcmm_info");
         return v;
     }
+    // PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
+    void ToNTTInplace(uint64_tt* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
+        check(pcmm_ntt_fwd(handle, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "PCMM_Context::ToNTTInplace");
+    }
+    void FromNTTInplace(uint64_tt* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
+        check(pcmm_ntt_inv(handle, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "PCMM_Context::FromNTTInplace");
+    }
 };
 
 // The rlweCipherDecompose / PPMM members of PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48).

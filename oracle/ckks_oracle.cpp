@@ -883,6 +883,30 @@ int orc_mlwe_pack(const orc_pcmm* h, u64* rlwe_out, const u64* const* mlwe, int 
     return 0;
 }
 
+// PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273) with NTT256_kernel / INTT256_kernel
+// (smallntt_60bit.cuh:7-152): the negacyclic transform of size N1 over the ring-pack primes, root findMthRootOfUnity(2*N1, q)
+// (PCMM_Context.cuh:31), tables as fillTablePsi128_special (:73-77).  Layout [batch][mod][poly][N1]; prime of limb (z, j, y) is
+// pq_ringpack[start_mod_idx + j]; the kernels ignore start_poly_idx (:27-29).  The reference runs N1 = 256 only (:256,271).
+int orc_pcmm_ntt(const orc_pcmm* h, u64* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, int inverse) {
+    const uint32_t n1 = (uint32_t)h->N1;
+    if (poly_num < 0 || mod_num < 0 || start_mod_idx < 0 || start_mod_idx + mod_num > h->np + h->nq || (n1 & (n1 - 1)) || n1 < 2) return -1;
+    for (int j = 0; j < mod_num; j++) {
+        const u64 q = h->pq[start_mod_idx + j];
+        if ((q - 1) % (2 * (u64)n1)) return -1;
+        const u64 psi = orc_find_mth_root(2 * (u64)n1, q);
+        std::vector<u64> tab(n1), itab(n1);
+        orc_fill_psi_tables(psi, q, n1, tab.data(), itab.data(), nullptr, nullptr);
+        const u64 ninv = orc_invmod(n1 % q, q);
+        for (int z = 0; z < mod_batch_size; z++)
+            for (int y = 0; y < poly_num; y++) {
+                u64* limb = data + (((size_t)z * mod_num + j) * poly_num + y) * n1;
+                if (inverse) orc_intt_limb(limb, n1, q, itab.data(), ninv);
+                else orc_ntt_limb(limb, n1, q, tab.data());
+            }
+    }
+    return 0;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

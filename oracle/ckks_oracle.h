@@ -112,6 +112,10 @@ int orc_ppmm(const orc_pcmm*, const float* W, const uint64_t* const* mlwe, uint6
  * (key i at keys + i*N*mod_num*2 = [a | b], mod_num = np+nq-1 limbs, NTT domain).  One special prime, two ring-pack moduli. */
 int orc_mlwe_pack(const orc_pcmm*, uint64_t* rlwe_out, const uint64_t* const* mlwe, int mlwe_num, const uint64_t* keys);
 
+/* PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273): size-N1 transforms over the ring-pack primes,
+ * layout [mod_batch_size][mod_num][poly_num][N1], prime pq_ringpack[start_mod_idx + j]. */
+int orc_pcmm_ntt(const orc_pcmm*, uint64_t* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, int inverse);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

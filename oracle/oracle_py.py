@@ -60,6 +60,7 @@ def lib():
             "orc_rlwe_decompose": (i, [vp, P64, C.POINTER(P64), i, i]),
             "orc_ppmm": (i, [vp, C.POINTER(C.c_float), C.POINTER(P64), P64, i, i, i, d, l, l]),
             "orc_mlwe_pack": (i, [vp, P64, C.POINTER(P64), i, P64]),
+            "orc_pcmm_ntt": (i, [vp, P64, i, i, i, i, i]),
             "orc_max_threads": (i, []),
         }
         for name, (res, args) in sig.items():
@@ -180,6 +181,15 @@ class OraclePCMM:
         rc = self.L_.orc_rlwe_decompose(self.h, _ptr(rlwe_coeff), self._ptrs(mlwe), len(mlwe), l)
         if rc:
             raise ValueError("orc_rlwe_decompose: %d" % rc)
+
+    def ToNTTInplace(self, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size):
+        """PCMM_Context.cuh:243-258 on a host array [mod_batch_size][mod_num][poly_num][N1]."""
+        if self.L_.orc_pcmm_ntt(self.h, _ptr(data), poly_num, mod_num, start_mod_idx, mod_batch_size, 0):
+            raise ValueError("orc_pcmm_ntt")
+
+    def FromNTTInplace(self, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size):
+        if self.L_.orc_pcmm_ntt(self.h, _ptr(data), poly_num, mod_num, start_mod_idx, mod_batch_size, 1):
+            raise ValueError("orc_pcmm_ntt")
 
     def mlweCipherPacking(self, rlwe_out, mlwe, keys):
         """PCMM_Scheme.cuh:361-425 on host arrays: mlwe list of [(nq-1)][(rank+1)][N1] coefficient-domain arrays, keys

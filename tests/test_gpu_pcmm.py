@@ -153,3 +153,30 @@ def test_mlwe_packing_errors():
     pair, dev, orc, rank = make(10, 64, q[:2], CFG3_P[:1], [CFG3_P[0]], q[:2])
     with pytest.raises(CkksError):
         dev.mlweCipherPacking(big, [b] * 3, 3, 0, big, big, big)                  # 3 does not divide the rank
+
+
+@pytest.mark.parametrize("N1", [256, 1024])
+def test_small_ring_ntt(N1):
+    """PCMM_Context::ToNTTInplace / FromNTTInplace: size-N1 transforms over the ring-pack primes in the reference's
+    [batch][mod][poly][N1] layout against the oracle, and the error for rings the transform does not cover."""
+    from ckks_llm_amd import CkksError
+    q = CFG2_Q[:3]
+    pair, dev, orc, rank = make(12, N1, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
+    pq = [CFG3_P[0]] + q[:2]
+    rng = np.random.default_rng(N1)
+    batch, mod_num, polys = 2, 2, 5
+    data = np.empty((batch, mod_num, polys, N1), dtype=np.uint64)
+    for j in range(mod_num):
+        data[:, j] = rng.integers(0, pq[1 + j], (batch, polys, N1), dtype=np.uint64)
+    want = data.copy()
+    orc.ToNTTInplace(want.reshape(-1), polys, mod_num, 0, 1, batch)
+    d = to_dev(data)
+    dev.pcmm_context.ToNTTInplace(d, polys, mod_num, 0, 1, batch)
+    assert np.array_equal(from_dev(d, data.shape), want)
+    dev.pcmm_context.FromNTTInplace(d, polys, mod_num, 0, 1, batch)
+    assert np.array_equal(from_dev(d, data.shape), data)
+    with pytest.raises(CkksError):
+        dev.pcmm_context.ToNTTInplace(d, polys, 3, 0, 1, batch)              # moduli 1..3 of three
+    pair2, dev2, orc2, rank2 = make(12, 128, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
+    with pytest.raises(CkksError):
+        dev2.pcmm_context.ToNTTInplace(d, 1, 1, 0, 0, 1)                     # N1 = 128: below the smallest transform

@@ -184,3 +184,39 @@ def test_packing_rejects_what_the_reference_cannot_do():
     pc = O.OraclePCMM(ctx, 16, 16, [CFG2_Q[5]], CFG2_Q[:3])               # two remaining moduli: the reference's embedding overlaps
     with pytest.raises(ValueError):
         pc.mlweCipherPacking(np.zeros(2 * 3 * 256, dtype=np.uint64), [np.zeros(2 * 17 * 16, dtype=np.uint64)], np.zeros(16 * 2 * 3 * 256, dtype=np.uint64))
+
+
+def test_small_ring_ntt_is_the_negacyclic_transform():
+    """PCMM_Context::ToNTTInplace / FromNTTInplace (size N1 over the ring-pack primes): round trip, the convolution theorem
+    against the schoolbook negacyclic product, the closed form for a monomial, and the [batch][mod][poly][N1] layout."""
+    N1, k = 256, 4
+    qs = CFG2_Q[:3]
+    ctx = O.OracleContext(10, [], qs)
+    pc = O.OraclePCMM(ctx, N1, k, qs[:1], qs[1:])
+    rng = np.random.default_rng(11)
+    batch, mod_num, polys = 2, 2, 3
+    data = np.empty((batch, mod_num, polys, N1), dtype=np.uint64)
+    for j in range(mod_num):
+        data[:, j] = rng.integers(0, qs[1 + j], (batch, polys, N1), dtype=np.uint64)
+    work = data.copy()
+    pc.ToNTTInplace(work.reshape(-1), polys, mod_num, 0, 1, batch)          # primes pq[1], pq[2]
+    for j in range(mod_num):
+        q = qs[1 + j]
+        a, b = [int(v) for v in data[0, j, 0]], [int(v) for v in data[1, j, 2]]
+        prod = [(int(x) * int(y)) % q for x, y in zip(work[0, j, 0], work[1, j, 2])]
+        arr = np.array(prod, dtype=np.uint64).reshape(1, 1, 1, N1).copy()
+        # inverse of the pointwise product = negacyclic product (one limb of prime j: start_mod_idx 1 + j)
+        pc.FromNTTInplace(arr.reshape(-1), 1, 1, 0, 1 + j, 1)
+        assert [int(v) for v in arr.reshape(-1)] == negacyclic_mul(a, b, q)
+    back = work.copy()
+    pc.FromNTTInplace(back.reshape(-1), polys, mod_num, 0, 1, batch)
+    assert np.array_equal(back, data)
+    # monomial X^5 modulo pq[0]: position bitrev(i) holds psi^(5 * (2 i + 1)), psi the 2*N1-th root the reference's search finds
+    q = qs[0]
+    mono = np.zeros(N1, dtype=np.uint64); mono[5] = 1
+    pc.ToNTTInplace(mono, 1, 1, 0, 0, 1)
+    psi = O.lib().orc_find_mth_root(2 * N1, q)
+    assert pow(psi, N1, q) == q - 1
+    from tests.helpers import bitrev
+    for i in (0, 1, 7, 100, 255):
+        assert int(mono[bitrev(i, 8)]) == pow(psi, 5 * (2 * i + 1), q)
