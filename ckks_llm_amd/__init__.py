@@ -6,4 +6,5 @@ ckks_llm_amd/lib/libckks_hip.so).  This package is the thin host-side mirror of 
 Context_23 / PCMM_Context / PCMM_Scheme interface for that path; it has no CPU fallback.
 """
 from ._lib import load_library, LibraryMissing  # noqa: F401
-from .api import Context_23, PCMM_Context, PCMM_Scheme, DeviceBuffer, CkksError  # noqa: F401
+from .api import (Context_23, PCMM_Context, PCMM_Scheme, DeviceBuffer, CkksError, Scheme_23, SecretKey, Key,  # noqa: F401
+                  Plaintext, Ciphertext)

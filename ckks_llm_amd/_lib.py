@@ -47,6 +47,14 @@ def _declare(L):
         "ckks_keyswitch_23": (i, [vp, vp, vp, vp, i, vp, vp, vp]),
         "ckks_hybrid_modup": (i, [vp, vp, vp, i]), "ckks_hybrid_inner_product": (i, [vp, vp, vp, vp, i]),
         "ckks_hybrid_moddown": (i, [vp, vp, vp, i]), "ckks_hybrid_keyswitch": (i, [vp, vp, vp, vp, i, vp]),
+        "ckks_random_bytes": (i, [vp, vp, sz, C.c_char_p, C.c_uint64]),
+        "ckks_sample_uniform": (i, [vp, vp, vp, i, i, i]), "ckks_sample_gaussian": (i, [vp, vp, vp, i, i, i]),
+        "ckks_sample_zo": (i, [vp, vp, vp, d, i, i, i]), "ckks_sample_hwt": (i, [vp, vp, vp, i, i, i, i]),
+        "ckks_poly_mul": (i, [vp, vp, vp, vp, i, i, i, i, i]), "ckks_poly_add": (i, [vp, vp, vp, vp, i, i, i, i, i]),
+        "ckks_poly_sub": (i, [vp, vp, vp, vp, i, i, i, i, i]),
+        "ckks_keygen_secret": (i, [vp, vp, vp, i]), "ckks_keygen_public": (i, [vp, vp, vp, vp, vp]),
+        "ckks_encrypt": (i, [vp, vp, vp, vp, vp, vp, i]), "ckks_decrypt": (i, [vp, vp, vp, vp, i]),
+        "ckks_encode_coeffs": (i, [vp, vp, vp, l, i]), "ckks_decode_coeffs": (i, [vp, vp, vp, vp, d, i, i, i]),
         "pcmm_ctx_create": (i, [C.POINTER(vp), vp, i, i, u64p, i, u64p, i]), "pcmm_ctx_destroy": (i, [vp]),
         "pcmm_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),

@@ -206,6 +206,149 @@ class Context_23:
         _check(self.L_.ckks_hybrid_keyswitch(self.h, _addr(out), _addr(in_ntt), _addr(evk), l, _addr(scratch)), "ckks_hybrid_keyswitch")
 
 
+    # -- RNG::generateRandom_device (RNG.cuh:18), Sampler (Sampler.cuh:17-41), pointwise arithmetic (poly_arithmetic.cuh)
+    def generateRandom_device(self, a, n, key, nonce):
+        """n bytes of the Salsa20/20 stream of (32-byte key, 64-bit nonce).  The reference draws key and nonce from rand();
+        here the caller names them, so a run can be repeated."""
+        key = bytes(key)
+        if len(key) != 32:
+            raise ValueError("generateRandom_device: the key has 32 bytes")
+        _check(self.L_.ckks_random_bytes(self.h, _addr(a), n, key, nonce), "ckks_random_bytes")
+
+    def uniformSampler_xq(self, random, out, idx_out, idx_mod, mod_num):
+        _check(self.L_.ckks_sample_uniform(self.h, _addr(random), _addr(out), idx_out, idx_mod, mod_num), "ckks_sample_uniform")
+
+    def gaussianSampler_xq(self, random, out, idx_out, idx_mod, mod_num):
+        _check(self.L_.ckks_sample_gaussian(self.h, _addr(random), _addr(out), idx_out, idx_mod, mod_num), "ckks_sample_gaussian")
+
+    def ZOSampler(self, random, out, probability, idx_out, idx_mod, mod_num):
+        _check(self.L_.ckks_sample_zo(self.h, _addr(random), _addr(out), probability, idx_out, idx_mod, mod_num), "ckks_sample_zo")
+
+    def HWTSampler(self, random, out, h, idx_out, idx_mod, mod_num):
+        _check(self.L_.ckks_sample_hwt(self.h, _addr(random), _addr(out), h, idx_out, idx_mod, mod_num), "ckks_sample_hwt")
+
+    def barrett_batch_3param_device(self, c, a, b, idx_c, idx_a, idx_b, idx_mod, mod_num):
+        _check(self.L_.ckks_poly_mul(self.h, _addr(c), _addr(a), _addr(b), idx_c, idx_a, idx_b, idx_mod, mod_num), "ckks_poly_mul")
+
+    def poly_add_3param_batch_device(self, c, a, b, idx_c, idx_a, idx_b, idx_mod, mod_num):
+        _check(self.L_.ckks_poly_add(self.h, _addr(c), _addr(a), _addr(b), idx_c, idx_a, idx_b, idx_mod, mod_num), "ckks_poly_add")
+
+    def poly_sub_3param_batch_device(self, c, a, b, idx_c, idx_a, idx_b, idx_mod, mod_num):
+        _check(self.L_.ckks_poly_sub(self.h, _addr(c), _addr(a), _addr(b), idx_c, idx_a, idx_b, idx_mod, mod_num), "ckks_poly_sub")
+
+    # -- Context_23::encode_coeffs / decode_coeffs (Encoder.cuh:83-96, 113-186)
+    def encode_coeffs(self, vals, msg):
+        """vals: N device doubles; msg: Plaintext (level msg.l, integer scale msg.scale)."""
+        _check(self.L_.ckks_encode_coeffs(self.h, _addr(msg.mx_device), _addr(vals), int(msg.scale), msg.l), "ckks_encode_coeffs")
+
+    def decode_coeffs(self, msg, vals, is_bitRev=False):
+        """vals: N device doubles (written)."""
+        scratch = DeviceBuffer(8 * self.N * (msg.l + 1))
+        _check(self.L_.ckks_decode_coeffs(self.h, _addr(vals), _addr(msg.mx_device), scratch.ptr, float(msg.scale), msg.slots,
+                                          1 if is_bitRev else 0, msg.l), "ckks_decode_coeffs")
+        scratch.free()
+
+
+class Plaintext:
+    """Plaintext (Plaintext.cuh:6-76): one device buffer of L+1 limbs, level l, slots, scale."""
+
+    def __init__(self, N, L, l, slots, scale):
+        if l > L:
+            raise ValueError("new Plaintext error!")
+        self.N, self.L, self.l, self.slots, self.scale = N, L, l, slots, scale
+        self.mx_device = DeviceBuffer(8 * N * (L + 1))
+
+
+class Ciphertext:
+    """Ciphertext (Ciphertext.cuh:6-99): one device buffer [a: L+1 limbs | b: L+1 limbs]."""
+
+    def __init__(self, N, L, l, slots, scale):
+        self.N, self.L, self.l, self.slots, self.scale = N, L, l, slots, scale
+        self.cipher_device = DeviceBuffer(8 * N * (L + 1) * 2)
+        self.ax_device = self.cipher_device.ptr
+        self.bx_device = self.cipher_device.ptr + 8 * N * (L + 1)
+
+
+class SecretKey:
+    """SecretKey (SecretKey.cuh:9-31): sparse ternary secret of Hamming weight <= h over [P | Q], NTT domain, sampled from
+    5*h bytes of the context's stream under (key, nonce)."""
+
+    def __init__(self, context, h=64, key=bytes(32), nonce=0):
+        self.N, self.L, self.K = context.N, context.L, context.K
+        self.sx_device = DeviceBuffer(8 * self.N * (self.K + self.L + 1))
+        rnd = DeviceBuffer(5 * h + 64)
+        context.generateRandom_device(rnd, 5 * h, key, nonce)
+        _check(context.L_.ckks_keygen_secret(context.h, self.sx_device.ptr, rnd.ptr, h), "ckks_keygen_secret")
+        rnd.free()
+
+
+class Key:
+    """Key (Key.cuh:5-24): [a | b], (L+1+K)*dnum limbs each."""
+
+    def __init__(self, N, L, K, dnum):
+        self.N, self.L, self.K, self.dnum = N, L, K, dnum
+        self.cipher_device = DeviceBuffer(8 * N * (L + 1 + K) * dnum * 2)
+        self.ax_device = self.cipher_device.ptr
+        self.bx_device = self.cipher_device.ptr + 8 * N * (L + 1 + K) * dnum
+
+
+class Scheme_23:
+    """The members of Scheme_23 on this path (Scheme_23.h:113-182): addEncKey, encryptZero, encryptMsg, decryptMsg,
+    rescaleAndEqual.  Randomness is the context's Salsa20 stream under this object's key with a nonce that counts calls."""
+
+    def __init__(self, context, key=bytes(32)):
+        self.context = context
+        self.key = bytes(key)
+        self.nonce = 1
+        N, L = context.N, context.L
+        self.publicKey = None
+        self.in_enc = DeviceBuffer(9 * N)                                   # Scheme_23.cuh:38-39
+        self.vx_enc = DeviceBuffer(8 * N * (L + 1))
+        self.rescale_buffer = DeviceBuffer(8 * N * (L + 1) * 2)
+
+    def _next_nonce(self):
+        self.nonce += 1
+        return self.nonce
+
+    def addEncKey(self, secretKey):
+        c = self.context
+        N, L = c.N, c.L
+        self.publicKey = Key(N, L, 0, 1)
+        rnd = DeviceBuffer(8 * N * (L + 1) + 4 * N)
+        c.generateRandom_device(rnd, rnd.nbytes, self.key, self._next_nonce())
+        _check(c.L_.ckks_keygen_public(c.h, self.publicKey.cipher_device.ptr, secretKey.sx_device.ptr, rnd.ptr,
+                                       rnd.ptr + 8 * N * (L + 1)), "ckks_keygen_public")
+        rnd.free()
+
+    def _encrypt(self, cipher, mx, l):
+        if self.publicKey is None:
+            raise ValueError("encryptMsg: no encryption key (addEncKey)")
+        c = self.context
+        c.generateRandom_device(self.in_enc, 9 * c.N, self.key, self._next_nonce())
+        _check(c.L_.ckks_encrypt(c.h, cipher.cipher_device.ptr, mx, self.publicKey.cipher_device.ptr, self.in_enc.ptr,
+                                 self.vx_enc.ptr, l), "ckks_encrypt")
+
+    def encryptZero(self, cipher, l, slots):
+        cipher.l, cipher.slots = l, slots
+        self._encrypt(cipher, None, l)
+
+    def encryptMsg(self, cipher, message):
+        cipher.l, cipher.scale, cipher.slots = message.l, message.scale, message.slots
+        self._encrypt(cipher, message.mx_device.ptr, message.l)
+
+    def decryptMsg(self, plain, secretKey, cipher):
+        c = self.context
+        plain.l, plain.scale, plain.slots = cipher.l, cipher.scale, cipher.slots
+        _check(c.L_.ckks_decrypt(c.h, plain.mx_device.ptr, cipher.cipher_device.ptr, secretKey.sx_device.ptr, cipher.l), "ckks_decrypt")
+
+    def rescaleAndEqual(self, cipher):
+        """Scheme_23.cuh:369-385: divides by q_l, level l -> l-1, scale /= q_l."""
+        c = self.context
+        c.rescaleAndEqual(cipher.cipher_device, self.rescale_buffer, cipher.l)
+        cipher.scale = cipher.scale / c.qVec[cipher.l]
+        cipher.l -= 1
+
+
 class PCMM_Context:
     """PCMM_Context (pcmm/PCMM_Context.h:14-90)."""
 

@@ -341,6 +341,7 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     void* ptrs[] = {c->d_primes, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
                     c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_sched, c->d_ntt_mid};
     for (void* p : ptrs) if (p) (void)hipFree(p);
+    for (auto& e : c->decode_tabs) (void)hipFree(e.dev);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->ev_mid) (void)hipEventDestroy(c->ev_mid);

@@ -86,6 +86,8 @@ struct ckks_ctx {
     int cu_count = 256;
     void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
     size_t ntt_mid_cap = 0;
+    struct DecodeTab { int level, words; void* dev; };
+    std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     void* d_ntt_sched = nullptr;          // scheduler words of the fused NTT kernel (zero between launches)
 };
 

@@ -125,6 +125,49 @@ int ckks_hybrid_moddown(ckks_ctx* ctx, uint64_t* out, const uint64_t* in_pq_coef
  * scratch: (ceil((l+1)/p_num) + 2) * (p_num+q_num) * N words. */
 int ckks_hybrid_keyswitch(ckks_ctx* ctx, uint64_t* out, uint64_t* in_ntt, const uint64_t* evk, int l, uint64_t* scratch);
 
+/* ---- randomness, samplers, pointwise arithmetic, keys, encryption, coefficient encoding (the client side of the path) ---- */
+/* RNG::generateRandom_device (RNG.cuh:18-56; kernel VecCrypt, RNG_impl.cuh:72-176): n_bytes of the Salsa20/20 key stream of
+ * (32-byte key, 64-bit nonce), block counter from 0, written to dev.  The reference draws key and nonce from rand() and leaves
+ * the cipher's four diagonal words at zero (RNG_impl.cuh:37 is never written); here they are Salsa20's constants, so the output
+ * is the published cipher's stream.  A trailing partial block is truncated (the reference stops at floor(n/64) blocks). */
+int ckks_random_bytes(ckks_ctx* ctx, uint8_t* dev, size_t n_bytes, const uint8_t* key32, uint64_t nonce);
+/* Sampler::uniformSampler_xq / gaussianSampler_xq / ZOSampler / HWTSampler (Sampler.cuh:17-41; conversions Sampler_impl.cuh:13-113).
+ * random: device bytes (8 per value and limb for uniform; 4 per coefficient for gaussian; 1 per coefficient for ZO; 4*h + h for
+ * HWT), out: limbs idx_out.. of a device polynomial, primes idx_mod.. in pqt order.  Uniform, ZO and HWT give the reference's
+ * values for the same bytes; HWT zeroes the limbs first, lets the later word win when two name one position (a race in the
+ * reference), and keeps the reference's output offset idx_out + idx_mod.  The Gaussian (sigma 3.2, |value| <= 19) is the
+ * reference's step function of the 32-bit word with the steps placed by integer thresholds instead of float arithmetic. */
+int ckks_sample_uniform(ckks_ctx* ctx, const uint8_t* random, uint64_t* out, int idx_out, int idx_mod, int mod_num);
+int ckks_sample_gaussian(ckks_ctx* ctx, const uint8_t* random, uint64_t* out, int idx_out, int idx_mod, int mod_num);
+int ckks_sample_zo(ckks_ctx* ctx, const uint8_t* random, uint64_t* out, double probability, int idx_out, int idx_mod, int mod_num);
+int ckks_sample_hwt(ckks_ctx* ctx, const uint8_t* random, uint64_t* out, int h, int idx_out, int idx_mod, int mod_num);
+/* barrett_batch_3param_device, poly_add_3param_batch_device, poly_sub_3param_batch_device (poly_arithmetic.cuh:101-105, 423-427,
+ * 481-485): c[idx_c + t] = a[idx_a + t] (*, +, -) b[idx_b + t] modulo prime idx_mod + t, t < mod_num; c may alias a or b
+ * (which gives barrett_batch_device, poly_add_batch_device, poly_sub_batch_device and poly_sub2_batch_device, :37-41, 395-399, 467-478). */
+int ckks_poly_mul(ckks_ctx* ctx, uint64_t* c, const uint64_t* a, const uint64_t* b, int idx_c, int idx_a, int idx_b, int idx_mod, int mod_num);
+int ckks_poly_add(ckks_ctx* ctx, uint64_t* c, const uint64_t* a, const uint64_t* b, int idx_c, int idx_a, int idx_b, int idx_mod, int mod_num);
+int ckks_poly_sub(ckks_ctx* ctx, uint64_t* c, const uint64_t* a, const uint64_t* b, int idx_c, int idx_a, int idx_b, int idx_mod, int mod_num);
+/* SecretKey::SecretKey (SecretKey.cuh:18-31): sx = K+L+1 limbs over [P | Q], NTT domain, from 5*h random bytes */
+int ckks_keygen_secret(ckks_ctx* ctx, uint64_t* sx, const uint8_t* random, int h);
+/* Scheme_23::addEncKey (Scheme_23.cuh:54-80): pk = [a: L+1 limbs | b: L+1 limbs] = (a, e - a*s) over Q, NTT domain;
+ * random_a: 8*N*(L+1) bytes, random_e: 4*N bytes */
+int ckks_keygen_public(ckks_ctx* ctx, uint64_t* pk, const uint64_t* sx, const uint8_t* random_a, const uint8_t* random_e);
+/* Scheme_23::encryptZero + encryptMsg (Scheme_23.cuh:82-112): cipher = [a: L+1 limbs | b: L+1 limbs], limbs 0..l written:
+ * a = v*pk.a + e0, b = v*pk.b + e1 + m.  random: 9*N bytes = N (v) | 4*N (e0) | 4*N (e1), the reference's in_enc layout;
+ * mx: plaintext limbs in the NTT domain, or NULL for encryptZero; scratch: (l+1)*N words (Scheme_23::vx_enc). */
+int ckks_encrypt(ckks_ctx* ctx, uint64_t* cipher, const uint64_t* mx, const uint64_t* pk, const uint8_t* random, uint64_t* scratch, int l);
+/* Scheme_23::decryptMsg (Scheme_23.cuh:114-127): mx = a*s + b on limbs 0..l, limbs l+1..L zeroed */
+int ckks_decrypt(ckks_ctx* ctx, uint64_t* mx, const uint64_t* cipher, const uint64_t* sx, int l);
+/* Context_23::encode_coeffs (Encoder.cuh:67-96): coefficient i = (long)(vals[i] * scale) modulo q_0..q_l, then NTT; vals: N device
+ * doubles.  The reference stores q + data for negative data, which is the residue whenever |data| < q; the residue is taken here. */
+int ckks_encode_coeffs(ckks_ctx* ctx, uint64_t* mx, const double* vals, long scale, int l);
+/* Context_23::decode_coeffs (Encoder.cuh:113-186): iNTT of limbs 0..l (on a copy in scratch, (l+1)*N words), CRT of every
+ * coefficient j*gap and N/2 + j*gap (gap = N/2/slots, j < slots) to the centred integer modulo q_0..q_l, as a double divided by
+ * scale; other coefficients 0; is_bitrev writes to the bit-reversed index and multiplies by 256 (:171-173).  The reference does
+ * the CRT on the host with NTL::ZZ; here it runs on the device (mixed-radix digits, multi-word Horner, correctly rounded
+ * conversion), vals: N device doubles. */
+int ckks_decode_coeffs(ckks_ctx* ctx, double* vals, const uint64_t* mx, uint64_t* scratch, double scale, int slots, int is_bitrev, int l);
+
 /* ---- ring-packed PCMM ---- */
 /* PCMM_Context::PCMM_Context (PCMM_Context.cuh:7-57) */
 int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,

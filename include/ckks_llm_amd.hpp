@@ -102,6 +102,97 @@ public:
     void external_product_T(uint64_tt* output, const uint64_tt* cipher_modUp_QjtoT, const uint64_tt* swk_modUp_RitoT, int l) {
         check(ckks_external_product_t(handle, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l), "external_product_T");
     }
+
+    // RNG::generateRandom_device (RNG.cuh:18-56).  The reference draws a fresh key and nonce from rand() per call; here the
+    // context holds a key (settable) and a nonce that counts the calls, so a run can be repeated.
+    uint8_t rng_key[32] = {0};
+    uint64_t rng_nonce = 0;
+    void generateRandom_device(uint8_t* a, uint64_tt n) {
+        check(ckks_random_bytes(handle, a, (size_t)n, rng_key, ++rng_nonce), "generateRandom_device");
+    }
+    // Context_23::encode_coeffs / decode_coeffs (Encoder.cuh:83-96, 113-186); vals: N device doubles
+    template <class PlaintextT>
+    void encode_coeffs(const double* vals, PlaintextT& msg) {
+        check(ckks_encode_coeffs(handle, msg.mx_device, vals, (long)msg.scale, msg.l), "encode_coeffs");
+    }
+    template <class PlaintextT>
+    void decode_coeffs(PlaintextT& msg, double* vals, bool is_bitRev = false) {
+        uint64_tt* scratch = device_alloc_words((size_t)N * (msg.l + 1));
+        int rc = ckks_decode_coeffs(handle, vals, msg.mx_device, scratch, (double)msg.scale, msg.slots, is_bitRev ? 1 : 0, msg.l);
+        device_release(scratch);
+        check(rc, "decode_coeffs");
+    }
+};
+
+// Sampler (Sampler.cuh:12-54): conversions of random device bytes into limbs
+class Sampler {
+public:
+    static void uniformSampler_xq(Context_23& c, const uint8_t* in, uint64_tt* out, int idx_out, int idx_mod, int mod_num) {
+        check(ckks_sample_uniform(c.handle, in, out, idx_out, idx_mod, mod_num), "uniformSampler_xq");
+    }
+    static void gaussianSampler_xq(Context_23& c, const uint8_t* in, uint64_tt* out, int idx_out, int idx_mod, int mod_num) {
+        check(ckks_sample_gaussian(c.handle, in, out, idx_out, idx_mod, mod_num), "gaussianSampler_xq");
+    }
+    static void HWTSampler(Context_23& c, const uint8_t* in, uint64_tt* out, int h, int idx_out, int idx_mod, int mod_num) {
+        check(ckks_sample_hwt(c.handle, in, out, h, idx_out, idx_mod, mod_num), "HWTSampler");
+    }
+    static void ZOSampler(Context_23& c, const uint8_t* in, uint64_tt* out, double probability, int idx_out, int idx_mod, int mod_num) {
+        check(ckks_sample_zo(c.handle, in, out, probability, idx_out, idx_mod, mod_num), "ZOSampler");
+    }
+};
+
+// Plaintext (Plaintext.cuh:6-76): L+1 limbs, NTT domain
+class Plaintext {
+public:
+    uint64_tt* mx_device = nullptr;
+    int N = 0, l = 0, L = 0, slots = 0;
+    long double scale = 0;
+
+    Plaintext() {}
+    Plaintext(int N, int L, int l, int slots, long double scale) : N(N), l(l), L(L), slots(slots), scale(scale) {
+        if (l > L) std::cout << "new Plaintext error!" << std::endl;            // Plaintext.cuh:11
+        mx_device = device_alloc_words((size_t)N * (L + 1));
+    }
+    Plaintext(const Plaintext&) = delete;
+    Plaintext& operator=(const Plaintext&) = delete;
+    virtual ~Plaintext() { device_release(mx_device); }
+};
+
+// SecretKey (SecretKey.cuh:9-57): sparse ternary secret of Hamming weight <= h over [P | Q], NTT domain
+class SecretKey {
+public:
+    uint64_tt* sx_device = nullptr;
+    int N, L, K;
+
+    explicit SecretKey(Context_23& context, int h = 64) : N((int)context.N), L(context.L), K(context.K) {
+        sx_device = device_alloc_words((size_t)N * (K + L + 1));
+        uint64_tt* rnd = device_alloc_words((size_t)(5 * h + 7) / 8 + 8);
+        context.generateRandom_device(reinterpret_cast<uint8_t*>(rnd), (uint64_tt)5 * h);
+        int rc = ckks_keygen_secret(context.handle, sx_device, reinterpret_cast<uint8_t*>(rnd), h);
+        device_release(rnd);
+        check(rc, "SecretKey");
+    }
+    SecretKey(const SecretKey&) = delete;
+    SecretKey& operator=(const SecretKey&) = delete;
+    virtual ~SecretKey() { device_release(sx_device); }
+};
+
+// Key (Key.cuh:5-24): [a | b], (L+1+K)*dnum limbs each
+class Key {
+public:
+    uint64_tt* ax_device = nullptr;
+    uint64_tt* bx_device = nullptr;
+    uint64_tt* cipher_device = nullptr;
+    int N = 0, L = 0, K = 0, dnum = 0;
+
+    Key(int N, int L, int K, int dnum) : N(N), L(L), K(K), dnum(dnum) {
+        cipher_device = device_alloc_words((size_t)N * (L + 1 + K) * dnum * 2);
+        ax_device = cipher_device;
+        bx_device = cipher_device + (size_t)N * (L + 1 + K) * dnum;
+    }
+    Key(const Key&) = delete;
+    Key& operator=(const Key&) = delete;
+    virtual ~Key() { device_release(cipher_device); }
 };
 
 // Ciphertext (Ciphertext.cuh:5-99): one device buffer [a: L+1 limbs | b: L+1 limbs].
@@ -142,10 +233,15 @@ public:
     virtual ~MLWECiphertext() { device_release(cipher_device); }
 };
 
-// The members of Scheme_23 on the path (Scheme_23.h:113-182): rescale and the key-switch chain of mult_23.
+// The members of Scheme_23 on the path (Scheme_23.h:113-182): public-key encryption, decryption, rescale and the key-switch
+// chain of mult_23.
 class Scheme_23 {
 public:
     Context_23& context;
+    Key* publicKey = nullptr;
+    uint64_tt* vx_enc = nullptr;
+    uint8_t* in_enc = nullptr;
+    long random_len_for_enc = 0;
     // Scheme_23::mallocMemory (Scheme_23.cuh:7-51): scratch owned by the scheme
     uint64_tt* rescale_buffer = nullptr;
     uint64_tt* modUp_QjtoT_temp = nullptr;
@@ -155,6 +251,9 @@ public:
     explicit Scheme_23(Context_23& context) : context(context) {
         const size_t N = (size_t)context.N;
         rescale_buffer = device_alloc_words(2 * N * (context.L + 1));
+        vx_enc = device_alloc_words(N * (context.L + 1));
+        random_len_for_enc = (long)(N + 4 * N + 4 * N);                          // Scheme_23.cuh:38
+        in_enc = reinterpret_cast<uint8_t*>(device_alloc_words((size_t)random_len_for_enc / 8));
         if (context.t_num > 0) {
             modUp_QjtoT_temp = device_alloc_words(N * context.t_num * context.Qj_blockNum);
             exProduct_T_temp = device_alloc_words(N * context.t_num * context.Ri_blockNum * 2);
@@ -163,10 +262,46 @@ public:
     }
     Scheme_23(const Scheme_23&) = delete;
     ~Scheme_23() {
+        delete publicKey;
+        device_release(vx_enc);
+        uint64_tt* r = reinterpret_cast<uint64_tt*>(in_enc);
+        device_release(r);
         device_release(rescale_buffer);
         device_release(modUp_QjtoT_temp);
         device_release(exProduct_T_temp);
         device_release(modUp_TtoQj_buffer);
+    }
+
+    // Scheme_23::addEncKey (Scheme_23.cuh:54-80): pk = (a, e - a*s)
+    void addEncKey(SecretKey& secretKey) {
+        const size_t N = (size_t)context.N, L1 = (size_t)context.L + 1;
+        delete publicKey;
+        publicKey = new Key((int)N, context.L, 0, 1);
+        uint64_tt* rnd = device_alloc_words(N * L1 + N / 2);
+        uint8_t* r8 = reinterpret_cast<uint8_t*>(rnd);
+        context.generateRandom_device(r8, 8 * N * L1 + 4 * N);
+        int rc = ckks_keygen_public(context.handle, publicKey->cipher_device, secretKey.sx_device, r8, r8 + 8 * N * L1);
+        device_release(rnd);
+        check(rc, "addEncKey");
+    }
+    // Scheme_23::encryptZero / encryptMsg (Scheme_23.cuh:82-112); a missing key throws std::invalid_argument
+    void encryptZero(Ciphertext& cipher, int l, int slots) {
+        cipher.l = l;
+        cipher.slots = slots;
+        encrypt(cipher, nullptr, l);
+    }
+    void encryptMsg(Ciphertext& cipher, Plaintext& message) {
+        cipher.l = message.l;
+        cipher.scale = message.scale;
+        cipher.slots = message.slots;
+        encrypt(cipher, message.mx_device, message.l);
+    }
+    // Scheme_23::decryptMsg (Scheme_23.cuh:114-127)
+    void decryptMsg(Plaintext& plain, SecretKey& secretKey, Ciphertext& cipher) {
+        plain.l = cipher.l;
+        plain.scale = cipher.scale;
+        plain.slots = cipher.slots;
+        check(ckks_decrypt(context.handle, plain.mx_device, cipher.cipher_device, secretKey.sx_device, cipher.l), "decryptMsg");
     }
 
     // Scheme_23::rescaleAndEqual (Scheme_23.cuh:369-385); throws std::invalid_argument on level 0 (:192-194 style)
@@ -179,6 +314,13 @@ public:
     // A null key throws std::invalid_argument as the missing rotation / relinearisation key does (:198-201).
     void keySwitch_23(uint64_tt* out, uint64_tt* d2, const uint64_tt* swk, int l) {
         check(ckks_keyswitch_23(context.handle, out, d2, swk, l, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer), "keySwitch_23");
+    }
+
+private:
+    void encrypt(Ciphertext& cipher, const uint64_tt* mx, int l) {
+        if (!publicKey) throw std::invalid_argument("encryptMsg: no encryption key (addEncKey)");
+        context.generateRandom_device(in_enc, (uint64_tt)random_len_for_enc);
+        check(ckks_encrypt(context.handle, cipher.cipher_device, mx, publicKey->cipher_device, in_enc, vx_enc, l), "encryptMsg");
     }
 };
 

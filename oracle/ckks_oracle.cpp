@@ -907,6 +907,215 @@ int orc_pcmm_ntt(const orc_pcmm* h, u64* data, int poly_num, int mod_num, int st
     return 0;
 }
 
+// ------------------------------------------------------------------------------------------------
+// randomness, samplers, pointwise arithmetic, keys, encryption, coefficient encoding
+// ------------------------------------------------------------------------------------------------
+static inline uint32_t rotl32(uint32_t u, int c) { return (u << c) | (u >> (32 - c)); }
+static inline uint32_t le32(const uint8_t* x) { return (uint32_t)x[0] | ((uint32_t)x[1] << 8) | ((uint32_t)x[2] << 16) | ((uint32_t)x[3] << 24); }
+
+// RNG::generateRandom_device (RNG.cuh:18-56) + VecCrypt (RNG_impl.cuh:72-176): the buffer is zeroed and the Salsa20/20 key stream
+// of (key, 64-bit nonce) is XORed in, 64-byte block b at offset 64*b with block counter b.  The reference never initialises its
+// `sigma` constant (RNG_impl.cuh:37), i.e. runs with zero diagonal words; here the diagonal is Salsa20's "expand 32-byte k",
+// which makes the stream the published cipher's (pinned by the ECRYPT vectors).  A trailing partial block is truncated (the
+// reference stops at floor(n/64) blocks).
+void orc_salsa20_stream(uint8_t* out, size_t n, const uint8_t key[32], uint64_t nonce) {
+    static const uint8_t sigma[17] = "expand 32-byte k";
+    const size_t blocks = (n + 63) / 64;
+    for (size_t b = 0; b < blocks; b++) {
+        uint32_t j[16], x[16];
+        j[0] = le32(sigma); j[5] = le32(sigma + 4); j[10] = le32(sigma + 8); j[15] = le32(sigma + 12);
+        for (int i = 0; i < 4; i++) { j[1 + i] = le32(key + 4 * i); j[11 + i] = le32(key + 16 + 4 * i); }
+        j[6] = (uint32_t)nonce; j[7] = (uint32_t)(nonce >> 32);
+        j[8] = (uint32_t)b; j[9] = (uint32_t)((uint64_t)b >> 32);
+        memcpy(x, j, sizeof(x));
+        for (int r = 0; r < 20; r += 2) {
+#define ORC_QR(a, b_, c, d) x[b_] ^= rotl32(x[a] + x[d], 7); x[c] ^= rotl32(x[b_] + x[a], 9); x[d] ^= rotl32(x[c] + x[b_], 13); x[a] ^= rotl32(x[d] + x[c], 18);
+            ORC_QR(0, 4, 8, 12) ORC_QR(5, 9, 13, 1) ORC_QR(10, 14, 2, 6) ORC_QR(15, 3, 7, 11)     // columns
+            ORC_QR(0, 1, 2, 3) ORC_QR(5, 6, 7, 4) ORC_QR(10, 11, 8, 9) ORC_QR(15, 12, 13, 14)      // rows
+#undef ORC_QR
+        }
+        uint8_t blk[64];
+        for (int i = 0; i < 16; i++) {
+            uint32_t v = x[i] + j[i];
+            blk[4 * i] = (uint8_t)v; blk[4 * i + 1] = (uint8_t)(v >> 8); blk[4 * i + 2] = (uint8_t)(v >> 16); blk[4 * i + 3] = (uint8_t)(v >> 24);
+        }
+        const size_t take = (n - 64 * b < 64) ? n - 64 * b : 64;
+        memcpy(out + 64 * b, blk, take);
+    }
+}
+
+// convert_gaussian_xq (Sampler_impl.cuh:27-70) maps a 32-bit word u to trunc(3.2 * Phi^-1(u / (2^32 - 1))) in float arithmetic,
+// clamped to +-19.2.  That is a non-decreasing step function of u.  The oracle states it by its steps with the probability
+// taken at the middle of the word's cell, p = (u + 0.5) / 2^32:  value >= k  <=>  p >= Phi(k / 3.2)  <=>  u >= thr[k-1],
+// thr[k-1] = 2^32 - floor(2^32 * Q(k / 3.2) + 0.5), Q the upper tail 0.5 * erfc(x / sqrt 2), k = 1..19; negative side by the
+// symmetry u -> 2^32 - 1 - u.  It differs from the float pipeline only for words within float rounding of a step
+// (distribution-level agreement; the exact stream of the reference is not reproducible anyway: its key and nonce are rand()).
+void orc_gauss_thresholds(uint32_t thr[19]) {
+    for (int k = 1; k <= 19; k++) {
+        const double tail = 0.5 * erfc(((double)k / 3.2) / sqrt(2.0));
+        thr[k - 1] = (uint32_t)(4294967296.0 - floor(4294967296.0 * tail + 0.5));
+    }
+}
+static int gauss_value(uint32_t u, const uint32_t thr[19]) {
+    int v = 0;
+    for (int k = 0; k < 19; k++) { v += (u >= thr[k]); v -= ((uint32_t)~u >= thr[k]); }
+    return v;
+}
+
+// Sampler::uniformSampler_xq / convert_uniform_xq (Sampler.cuh:17-22, Sampler_impl.cuh:13-24): word i of mod_num*N 64-bit words
+// -> (u64)((double)w / 2^64 * (double)(q - 1)), q = prime idx_mod + i / N, written at out[i + idx_out * N]
+int orc_sample_uniform(const orc_ctx* c, const uint8_t* random, u64* out, int idx_out, int idx_mod, int mod_num) {
+    if (idx_mod < 0 || mod_num < 0 || idx_mod + mod_num > (int)c->pqt.size()) return -1;
+    const size_t N = (size_t)c->N;
+    for (size_t i = 0; i < N * (size_t)mod_num; i++) {
+        u64 w; memcpy(&w, random + 8 * i, 8);
+        double d = (double)w;
+        d /= 18446744073709551616.0;                        // (double)UINT64_MAX rounds to 2^64
+        d *= (double)(c->pqt[idx_mod + i / N] - 1);
+        out[i + (size_t)idx_out * N] = (u64)d;
+    }
+    return 0;
+}
+// Sampler::gaussianSampler_xq / convert_gaussian_xq (Sampler.cuh:24-29, Sampler_impl.cuh:27-70): N 32-bit words, one noise
+// coefficient each, written to mod_num limbs as its residue
+int orc_sample_gaussian(const orc_ctx* c, const uint8_t* random, u64* out, int idx_out, int idx_mod, int mod_num) {
+    if (idx_mod < 0 || mod_num < 0 || idx_mod + mod_num > (int)c->pqt.size()) return -1;
+    uint32_t thr[19];
+    orc_gauss_thresholds(thr);
+    const size_t N = (size_t)c->N;
+    for (size_t i = 0; i < N; i++) {
+        uint32_t u; memcpy(&u, random + 4 * i, 4);
+        const int dd = gauss_value(u, thr);
+        for (int t = 0; t < mod_num; t++)
+            out[i + ((size_t)idx_out + t) * N] = dd < 0 ? c->pqt[idx_mod + t] + (long long)dd : (u64)dd;
+    }
+    return 0;
+}
+// Sampler::ZOSampler / convert_ZO (Sampler.cuh:36-41, Sampler_impl.cuh:96-113): byte d -> 0 if d < 256*prob, 1 if d < 256*(1+prob)/2,
+// else q - 1
+int orc_sample_zo(const orc_ctx* c, const uint8_t* random, u64* out, double probability, int idx_out, int idx_mod, int mod_num) {
+    if (idx_mod < 0 || mod_num < 0 || idx_mod + mod_num > (int)c->pqt.size()) return -1;
+    const size_t N = (size_t)c->N;
+    for (size_t i = 0; i < N; i++) {
+        const float d = (float)random[i];
+        for (int t = 0; t < mod_num; t++) {
+            const u64 q = c->pqt[idx_mod + t];
+            u64 v;
+            if (d < 256.0f * probability) v = 0;
+            else if (d < 256.0f * (1 + probability) / 2) v = 1;
+            else v = q - 1;
+            out[i + ((size_t)idx_out + t) * N] = v;
+        }
+    }
+    return 0;
+}
+// Sampler::HWTSampler / convert_HWT (Sampler.cuh:31-34, Sampler_impl.cuh:74-93): h 32-bit words give positions (low logN bits), h
+// bytes after them give signs (byte >= 128 -> 1, else q - 1); output limb of prime t is idx_out + idx_mod + t (the reference adds
+// idx_mod to the output offset).  The limbs are zeroed first (the reference writes into fresh cudaMalloc memory,
+// SecretKey.cuh:27-29); when two words give the same position the later one wins (the reference leaves that to a race).
+int orc_sample_hwt(const orc_ctx* c, const uint8_t* random, u64* out, int h, int idx_out, int idx_mod, int mod_num) {
+    if (idx_mod < 0 || mod_num < 0 || idx_mod + mod_num > (int)c->pqt.size() || h < 0) return -1;
+    const size_t N = (size_t)c->N;
+    for (int t = 0; t < mod_num; t++) {
+        u64* limb = out + ((size_t)idx_out + idx_mod + t) * N;
+        const u64 q = c->pqt[idx_mod + t];
+        memset(limb, 0, 8 * N);
+        for (int k = 0; k < h; k++) {
+            uint32_t w; memcpy(&w, random + 4 * k, 4);
+            float d = (float)random[4 * (size_t)h + k];
+            d /= (256.0f / 2);
+            limb[w & (N - 1)] = d >= 1 ? 1 : q - 1;
+        }
+    }
+    return 0;
+}
+
+// barrett_batch_3param_device, poly_add_3param_batch_device, poly_sub_3param_batch_device (poly_arithmetic.cuh:101-105, 423-427,
+// 481-485): c[idx_c + t] = a[idx_a + t] (op) b[idx_b + t] mod prime idx_mod + t, t < mod_num; op 0 mul, 1 add, 2 sub
+int orc_poly_op(const orc_ctx* c, int op, u64* out, const u64* a, const u64* b, int idx_c, int idx_a, int idx_b, int idx_mod, int mod_num) {
+    if (idx_mod < 0 || mod_num < 0 || idx_mod + mod_num > (int)c->pqt.size() || op < 0 || op > 2) return -1;
+    const size_t N = (size_t)c->N;
+    for (int t = 0; t < mod_num; t++) {
+        const u64 q = c->pqt[idx_mod + t];
+        for (size_t i = 0; i < N; i++) {
+            const u64 x = a[((size_t)idx_a + t) * N + i], y = b[((size_t)idx_b + t) * N + i];
+            u64 r;
+            if (op == 0) r = orc_barrett128((u64)(((u128)x * y) >> 64), x * y, q, c->mu_hi[idx_mod + t], c->mu_lo[idx_mod + t]);
+            else if (op == 1) r = csub_q(x + y, q);
+            else r = csub_q(q + x - y, q);
+            out[((size_t)idx_c + t) * N + i] = r;
+        }
+    }
+    return 0;
+}
+
+// SecretKey::SecretKey (SecretKey.cuh:18-31): sparse ternary secret over all of [P | Q] from h words + h bytes, then NTT
+int orc_keygen_secret(const orc_ctx* c, u64* sx, const uint8_t* random, int h) {
+    const int KL = c->K + c->L + 1;
+    if (orc_sample_hwt(c, random, sx, h, 0, 0, KL)) return -1;
+    return orc_ntt_fwd(c, sx, 0, 0, 1, KL, KL);
+}
+// Scheme_23::addEncKey (Scheme_23.cuh:54-80): pk = (a, e - a*s) over Q, NTT domain; a from 8*N*(L+1) random bytes, e from 4*N
+int orc_keygen_public(const orc_ctx* c, u64* pk, const u64* sx, const uint8_t* random_a, const uint8_t* random_e) {
+    const int K = c->K, L1 = c->L + 1;
+    const size_t N = (size_t)c->N;
+    u64* ax = pk; u64* bx = pk + N * L1;
+    std::vector<u64> ex(N * L1);
+    if (orc_sample_uniform(c, random_a, ax, 0, K, L1)) return -1;
+    orc_sample_gaussian(c, random_e, ex.data(), 0, K, L1);
+    orc_ntt_fwd(c, ex.data(), 0, K, 1, L1, L1);
+    orc_poly_op(c, 0, bx, ax, sx, 0, 0, K, K, L1);
+    orc_poly_op(c, 2, bx, ex.data(), bx, 0, 0, 0, K, L1);               // poly_sub2: b = e - b
+    return 0;
+}
+// Scheme_23::encryptZero + encryptMsg (Scheme_23.cuh:82-112): random = N bytes (v) | N words (e0) | N words (e1);
+// a = v*pk.a + e0, b = v*pk.b + e1 (+ m), limbs 0..l of a ciphertext [a: L+1 | b: L+1]; mx may be null
+int orc_encrypt(const orc_ctx* c, u64* cipher, const u64* mx, const u64* pk, const uint8_t* random, int l) {
+    const int K = c->K, L1 = c->L + 1;
+    if (l < 0 || l > c->L) return -1;
+    const size_t N = (size_t)c->N;
+    u64* ax = cipher; u64* bx = cipher + N * L1;
+    std::vector<u64> vx(N * L1), ex(N * L1);
+    orc_sample_zo(c, random, vx.data(), 0.5, 0, K, l + 1);
+    orc_ntt_fwd(c, vx.data(), 0, K, 1, l + 1, L1);
+    orc_poly_op(c, 0, ax, vx.data(), pk, 0, 0, 0, K, l + 1);
+    orc_sample_gaussian(c, random + N, ex.data(), 0, K, l + 1);
+    orc_ntt_fwd(c, ex.data(), 0, K, 1, l + 1, L1);
+    orc_poly_op(c, 1, ax, ax, ex.data(), 0, 0, 0, K, l + 1);
+    orc_poly_op(c, 0, bx, vx.data(), pk + N * L1, 0, 0, 0, K, l + 1);
+    orc_sample_gaussian(c, random + N + 4 * N, ex.data(), 0, K, l + 1);
+    orc_ntt_fwd(c, ex.data(), 0, K, 1, l + 1, L1);
+    orc_poly_op(c, 1, bx, bx, ex.data(), 0, 0, 0, K, l + 1);
+    if (mx) orc_poly_op(c, 1, bx, bx, mx, 0, 0, 0, K, l + 1);
+    return 0;
+}
+// Scheme_23::decryptMsg (Scheme_23.cuh:114-127): m = a*s + b on limbs 0..l, limbs above zeroed
+int orc_decrypt(const orc_ctx* c, u64* mx, const u64* cipher, const u64* sx, int l) {
+    const int K = c->K, L1 = c->L + 1;
+    if (l < 0 || l > c->L) return -1;
+    const size_t N = (size_t)c->N;
+    memset(mx + (size_t)(l + 1) * N, 0, 8 * N * (size_t)(c->L - l));
+    orc_poly_op(c, 0, mx, cipher, sx, 0, 0, K, K, l + 1);
+    orc_poly_op(c, 1, mx, mx, cipher + N * L1, 0, 0, 0, K, l + 1);
+    return 0;
+}
+// Context_23::encode_coeffs (Encoder.cuh:67-96): coefficient i = (long)(vals[i] * scale) reduced modulo each q_j, then NTT.
+// The reference stores q + data for negative data, which is the residue whenever |data| < q; the true residue is taken here.
+int orc_encode_coeffs(const orc_ctx* c, u64* mx, const double* vals, long scale, int l) {
+    const int K = c->K, L1 = c->L + 1;
+    if (l < 0 || l > c->L) return -1;
+    const size_t N = (size_t)c->N;
+    for (int j = 0; j <= l; j++) {
+        const u64 q = c->pqt[K + j];
+        for (size_t i = 0; i < N; i++) {
+            const long data = (long)(vals[i] * scale);
+            const long r = data % (long)q;
+            mx[(size_t)j * N + i] = r < 0 ? (u64)(r + (long)q) : (u64)r;
+        }
+    }
+    return orc_ntt_fwd(c, mx, 0, K, 1, l + 1, L1);
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -25,6 +25,12 @@
  *                                  algebra in Python                            (tests/test_oracle_pcmm.py)
  *   PPMM                           Python big-int brute force + fused-rescale
  *                                  closed form                                  (tests/test_oracle_pcmm.py)
+ *   Salsa20 stream                 ECRYPT known-answer vectors                  (tests/test_oracle_scheme.py)
+ *   samplers                       scipy's normal tail for the Gaussian steps,
+ *                                  exact probabilities, hand-worked words       (tests/test_oracle_scheme.py)
+ *   keys, encryption, decryption   decrypt identities with Python negacyclic
+ *                                  algebra (a*s + b = m + small noise)          (tests/test_oracle_scheme.py)
+ *   coefficient encode / decode    Python big-integer CRT and exact rationals   (tests/test_oracle_scheme.py)
  */
 #pragma once
 #include <stdint.h>
@@ -115,6 +121,21 @@ int orc_mlwe_pack(const orc_pcmm*, uint64_t* rlwe_out, const uint64_t* const* ml
 /* PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273): size-N1 transforms over the ring-pack primes,
  * layout [mod_batch_size][mod_num][poly_num][N1], prime pq_ringpack[start_mod_idx + j]. */
 int orc_pcmm_ntt(const orc_pcmm*, uint64_t* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, int inverse);
+
+/* ---- randomness, samplers, pointwise arithmetic, keys, encryption, coefficient encoding ---- */
+void orc_salsa20_stream(uint8_t* out, size_t n, const uint8_t key[32], uint64_t nonce);
+void orc_gauss_thresholds(uint32_t thr[19]);
+int orc_sample_uniform(const orc_ctx*, const uint8_t* random, uint64_t* out, int idx_out, int idx_mod, int mod_num);
+int orc_sample_gaussian(const orc_ctx*, const uint8_t* random, uint64_t* out, int idx_out, int idx_mod, int mod_num);
+int orc_sample_zo(const orc_ctx*, const uint8_t* random, uint64_t* out, double probability, int idx_out, int idx_mod, int mod_num);
+int orc_sample_hwt(const orc_ctx*, const uint8_t* random, uint64_t* out, int h, int idx_out, int idx_mod, int mod_num);
+int orc_poly_op(const orc_ctx*, int op, uint64_t* c, const uint64_t* a, const uint64_t* b, int idx_c, int idx_a, int idx_b,
+                int idx_mod, int mod_num);
+int orc_keygen_secret(const orc_ctx*, uint64_t* sx, const uint8_t* random, int h);
+int orc_keygen_public(const orc_ctx*, uint64_t* pk, const uint64_t* sx, const uint8_t* random_a, const uint8_t* random_e);
+int orc_encrypt(const orc_ctx*, uint64_t* cipher, const uint64_t* mx, const uint64_t* pk, const uint8_t* random, int l);
+int orc_decrypt(const orc_ctx*, uint64_t* mx, const uint64_t* cipher, const uint64_t* sx, int l);
+int orc_encode_coeffs(const orc_ctx*, uint64_t* mx, const double* vals, long scale, int l);
 
 int orc_max_threads(void);
 

@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libckks_oracle.so")
 u64 = C.c_uint64
 P64 = C.POINTER(C.c_uint64)
+P8 = C.POINTER(C.c_uint8)
 
 
 def build(force=False):
@@ -22,6 +23,26 @@ def build(force=False):
 def _ptr(a):
     assert a.dtype == np.uint64 and a.flags["C_CONTIGUOUS"]
     return a.ctypes.data_as(P64)
+
+
+def _bytes(a):
+    assert a.dtype == np.uint8 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(P8)
+
+
+def salsa20_stream(n, key, nonce):
+    """n bytes of the Salsa20/20 key stream of (32-byte key, 64-bit nonce), block counter from 0 (RNG.cuh:18-56)."""
+    out = np.zeros(n, dtype=np.uint8)
+    k = np.frombuffer(bytes(key), dtype=np.uint8).copy()
+    assert k.size == 32
+    lib().orc_salsa20_stream(_bytes(out), n, _bytes(k), nonce)
+    return out
+
+
+def gauss_thresholds():
+    out = np.zeros(19, dtype=np.uint32)
+    lib().orc_gauss_thresholds(out.ctypes.data_as(C.POINTER(C.c_uint32)))
+    return out
 
 
 _lib = None
@@ -61,6 +82,14 @@ def lib():
             "orc_ppmm": (i, [vp, C.POINTER(C.c_float), C.POINTER(P64), P64, i, i, i, d, l, l]),
             "orc_mlwe_pack": (i, [vp, P64, C.POINTER(P64), i, P64]),
             "orc_pcmm_ntt": (i, [vp, P64, i, i, i, i, i]),
+            "orc_salsa20_stream": (None, [P8, C.c_size_t, P8, u64]),
+            "orc_gauss_thresholds": (None, [C.POINTER(C.c_uint32)]),
+            "orc_sample_uniform": (i, [vp, P8, P64, i, i, i]), "orc_sample_gaussian": (i, [vp, P8, P64, i, i, i]),
+            "orc_sample_zo": (i, [vp, P8, P64, d, i, i, i]), "orc_sample_hwt": (i, [vp, P8, P64, i, i, i, i]),
+            "orc_poly_op": (i, [vp, i, P64, P64, P64, i, i, i, i, i]),
+            "orc_keygen_secret": (i, [vp, P64, P8, i]), "orc_keygen_public": (i, [vp, P64, P64, P8, P8]),
+            "orc_encrypt": (i, [vp, P64, P64, P64, P8, i]), "orc_decrypt": (i, [vp, P64, P64, P64, i]),
+            "orc_encode_coeffs": (i, [vp, P64, C.POINTER(C.c_double), l, i]),
             "orc_max_threads": (i, []),
         }
         for name, (res, args) in sig.items():
@@ -155,6 +184,69 @@ class OracleContext:
 
     def hybrid_keyswitch(self, out, in_ntt, evk, l):
         self._ck(self.L_.orc_hybrid_keyswitch(self.h, _ptr(out), _ptr(in_ntt), _ptr(evk), l))
+
+    # ---- samplers (Sampler.cuh:17-54), pointwise arithmetic (poly_arithmetic.cuh), keys and encryption (Scheme_23.cuh:54-127) ----
+    def uniformSampler_xq(self, random, out, idx_out, idx_mod, mod_num):
+        self._ck(self.L_.orc_sample_uniform(self.h, _bytes(random), _ptr(out), idx_out, idx_mod, mod_num))
+
+    def gaussianSampler_xq(self, random, out, idx_out, idx_mod, mod_num):
+        self._ck(self.L_.orc_sample_gaussian(self.h, _bytes(random), _ptr(out), idx_out, idx_mod, mod_num))
+
+    def ZOSampler(self, random, out, probability, idx_out, idx_mod, mod_num):
+        self._ck(self.L_.orc_sample_zo(self.h, _bytes(random), _ptr(out), probability, idx_out, idx_mod, mod_num))
+
+    def HWTSampler(self, random, out, h, idx_out, idx_mod, mod_num):
+        self._ck(self.L_.orc_sample_hwt(self.h, _bytes(random), _ptr(out), h, idx_out, idx_mod, mod_num))
+
+    def poly_op(self, op, c, a, b, idx_c, idx_a, idx_b, idx_mod, mod_num):
+        """op 0: c = a*b (barrett_batch_3param_device), 1: c = a+b (poly_add_3param_batch_device), 2: c = a-b."""
+        self._ck(self.L_.orc_poly_op(self.h, op, _ptr(c), _ptr(a), _ptr(b), idx_c, idx_a, idx_b, idx_mod, mod_num))
+
+    def keygen_secret(self, sx, random, h):
+        self._ck(self.L_.orc_keygen_secret(self.h, _ptr(sx), _bytes(random), h))
+
+    def keygen_public(self, pk, sx, random_a, random_e):
+        self._ck(self.L_.orc_keygen_public(self.h, _ptr(pk), _ptr(sx), _bytes(random_a), _bytes(random_e)))
+
+    def encrypt(self, cipher, mx, pk, random, l):
+        self._ck(self.L_.orc_encrypt(self.h, _ptr(cipher), None if mx is None else _ptr(mx), _ptr(pk), _bytes(random), l))
+
+    def decrypt(self, mx, cipher, sx, l):
+        self._ck(self.L_.orc_decrypt(self.h, _ptr(mx), _ptr(cipher), _ptr(sx), l))
+
+    def encode_coeffs(self, mx, vals, scale, l):
+        assert vals.dtype == np.float64 and vals.size == self.N
+        self._ck(self.L_.orc_encode_coeffs(self.h, _ptr(mx), vals.ctypes.data_as(C.POINTER(C.c_double)), int(scale), l))
+
+    def decode_coeffs(self, mx, scale, slots, l, is_bitrev=False):
+        """Context_23::decode_coeffs (Encoder.cuh:113-186): iNTT of limbs 0..l, CRT to the centred integer modulo q_0..q_l
+        (Python integers for NTL::ZZ), divided by the scale; only coefficients j*gap and N/2 + j*gap, j < slots, are
+        produced (the rest stay 0); with is_bitrev the value goes to the bit-reversed index times 256 (:171-173)."""
+        from fractions import Fraction
+        N, K = self.N, self.K
+        buf = np.array(mx[: (l + 1) * N], dtype=np.uint64, copy=True)
+        full = np.zeros((self.L + 1) * N, dtype=np.uint64)
+        full[: (l + 1) * N] = buf
+        self.FromNTTInplace(full, 0, K, 1, l + 1, self.L + 1)
+        qs = [int(v) for v in self.q[: l + 1]]
+        Q = 1
+        for q in qs:
+            Q *= q
+        rec = [(Q // q) * pow(Q // q, -1, q) for q in qs]
+        out = np.zeros(N, dtype=np.float64)
+        gap = (N // 2) // slots
+        sc = Fraction(scale)
+        logN = self.logN
+        for j in range(slots):
+            for idx in (j * gap, N // 2 + j * gap):
+                x = sum(int(full[k * N + idx]) * rec[k] for k in range(l + 1)) % Q
+                c = x if x <= Q // 2 else x - Q
+                v = float(Fraction(c) / sc)
+                if is_bitrev:
+                    out[int(format(idx, "0%db" % logN)[::-1], 2)] = v * 256
+                else:
+                    out[idx] = v
+        return out
 
 
 class OraclePCMM:

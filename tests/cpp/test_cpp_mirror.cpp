@@ -3,7 +3,9 @@
 // oracle, bit for bit, and with assertions instead of prints.  Needs a GPU.  Exit code 0 = all checks passed.
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
+#include <algorithm>
 #include <unistd.h>
 #include <random>
 #include <vector>
@@ -125,6 +127,55 @@ static int run() {
     threw = false;
     try { pcmm_scheme.mlweCipherPacking(rlwe, mlwe, mlwe_num, 0); } catch (const std::invalid_argument&) { threw = true; }
     EXPECT(threw, "mlweCipherPacking without keys throws std::invalid_argument");
+
+    // ---- SecretKey, addEncKey, encode_coeffs, encryptMsg, decryptMsg, decode_coeffs: the context's stream is Salsa20 under its
+    //      key (zero here) with nonces 1, 2, 3 for the three draws, so the oracle can follow word for word ----
+    {
+        const int h = 64, L1 = context.L + 1;
+        const uint8_t zero_key[32] = {0};
+        context.rng_nonce = 0;
+        SecretKey sk(context, h);
+        std::vector<uint8_t> r1(5 * h), r2(8 * N * L1 + 4 * N), r3(9 * N);
+        orc_salsa20_stream(r1.data(), r1.size(), zero_key, 1);
+        orc_salsa20_stream(r2.data(), r2.size(), zero_key, 2);
+        orc_salsa20_stream(r3.data(), r3.size(), zero_key, 3);
+        std::vector<uint64_tt> o_sx((size_t)N * L1), o_pk((size_t)2 * N * L1), o_mx((size_t)N * L1), o_ct((size_t)2 * N * L1, 0), o_dec((size_t)N * L1);
+        orc_keygen_secret(orc, o_sx.data(), r1.data(), h);
+        EXPECT(download(sk.sx_device, o_sx.size()) == o_sx, "SecretKey == oracle");
+        scheme.addEncKey(sk);
+        orc_keygen_public(orc, o_pk.data(), o_sx.data(), r2.data(), r2.data() + 8 * N * L1);
+        EXPECT(download(scheme.publicKey->cipher_device, o_pk.size()) == o_pk, "addEncKey == oracle");
+        std::vector<double> vals(N);
+        std::uniform_real_distribution<double> ud(-3.0, 3.0);
+        for (double& v : vals) v = ud(rng);
+        void* vd = nullptr;
+        check(ckks_malloc(&vd, N * 8), "malloc vals");
+        check(ckks_memcpy_h2d(vd, vals.data(), N * 8), "h2d vals");
+        Plaintext msg((int)N, context.L, 2, (int)(N / 2), (long double)(1ll << 40));
+        context.encode_coeffs((const double*)vd, msg);
+        orc_encode_coeffs(orc, o_mx.data(), vals.data(), 1l << 40, 2);
+        EXPECT(download(msg.mx_device, (size_t)3 * N) == std::vector<uint64_tt>(o_mx.begin(), o_mx.begin() + 3 * N), "encode_coeffs == oracle");
+        Ciphertext enc((int)N, context.L, context.L, (int)(N / 2), 1.0L);
+        check(ckks_memset(enc.cipher_device, 0, o_ct.size() * 8), "memset");
+        scheme.encryptMsg(enc, msg);
+        orc_encrypt(orc, o_ct.data(), o_mx.data(), o_pk.data(), r3.data(), 2);
+        EXPECT(download(enc.cipher_device, o_ct.size()) == o_ct && enc.l == 2 && enc.scale == msg.scale, "encryptMsg == oracle, level and scale follow");
+        Plaintext dec((int)N, context.L, context.L, 1, 1.0L);
+        scheme.decryptMsg(dec, sk, enc);
+        orc_decrypt(orc, o_dec.data(), o_ct.data(), o_sx.data(), 2);
+        EXPECT(download(dec.mx_device, o_dec.size()) == o_dec && dec.l == 2 && dec.slots == (int)(N / 2), "decryptMsg == oracle");
+        context.decode_coeffs(dec, (double*)vd);
+        std::vector<double> back(N);
+        check(ckks_memcpy_d2h(back.data(), vd, N * 8), "d2h vals");
+        double worst = 0;
+        for (long i = 0; i < N; i++) worst = std::max(worst, std::fabs(back[i] - vals[i]));
+        EXPECT(worst > 0 && worst <= 19.0 * (N + h + 2) / (double)(1ll << 40), "decode_coeffs(decrypt(encrypt(encode(x)))) = x up to the encryption noise");
+        Scheme_23 bare(context);
+        threw = false;
+        try { bare.encryptZero(enc, 1, 1); } catch (const std::invalid_argument&) { threw = true; }
+        EXPECT(threw, "encryptZero without a public key throws std::invalid_argument");
+        ckks_free(vd);
+    }
 
     for (MLWECiphertext* m : mlwe) delete m;
     ckks_free(Wd);
