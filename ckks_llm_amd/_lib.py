@@ -55,6 +55,12 @@ def _declare(L):
         "ckks_keygen_secret": (i, [vp, vp, vp, i]), "ckks_keygen_public": (i, [vp, vp, vp, vp, vp]),
         "ckks_encrypt": (i, [vp, vp, vp, vp, vp, vp, i]), "ckks_decrypt": (i, [vp, vp, vp, vp, i]),
         "ckks_encode_coeffs": (i, [vp, vp, vp, l, i]), "ckks_decode_coeffs": (i, [vp, vp, vp, vp, d, i, i, i]),
+        "ckks_rot_group": (i, [vp, l, u64p]),
+        "ckks_poly_automorph_ntt": (i, [vp, vp, vp, C.c_uint64, i, i, i]), "ckks_poly_conjugate_ntt": (i, [vp, vp, vp, i, i, i]),
+        "ckks_keygen_switch_23": (i, [vp, vp, vp, vp, vp, vp, vp]),
+        "ckks_mult_23": (i, [vp, vp, vp, vp, vp, i, vp, vp, vp, vp]),
+        "ckks_rotate_23": (i, [vp, vp, vp, vp, l, i, vp, vp, vp, vp]),
+        "ckks_conjugate_23": (i, [vp, vp, vp, vp, i, vp, vp, vp, vp]),
         "pcmm_ctx_create": (i, [C.POINTER(vp), vp, i, i, u64p, i, u64p, i]), "pcmm_ctx_destroy": (i, [vp]),
         "pcmm_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),

@@ -236,6 +236,25 @@ class Context_23:
     def poly_sub_3param_batch_device(self, c, a, b, idx_c, idx_a, idx_b, idx_mod, mod_num):
         _check(self.L_.ckks_poly_sub(self.h, _addr(c), _addr(a), _addr(b), idx_c, idx_a, idx_b, idx_mod, mod_num), "ckks_poly_sub")
 
+    # -- rotGroups (Context_23.cuh:648-659) and the NTT-domain permutations (poly_arithmetic.cuh:581-680)
+    def rotGroups(self, idx):
+        v = C.c_uint64()
+        _check(self.L_.ckks_rot_group(self.h, idx, C.byref(v)), "ckks_rot_group")
+        return v.value
+
+    def sk_and_poly_LeftRot_ntt(self, device_a, device_b, rot_num, idx_a, idx_b, mod_num):
+        """a[perm(i)] = b[i] with the exponent rotGroups[N/2 - rot_num] (poly_arithmetic.cuh:581-596): X -> X^(5^rot_num)."""
+        _check(self.L_.ckks_poly_automorph_ntt(self.h, _addr(device_a), _addr(device_b), self.rotGroups(self.N // 2 - rot_num),
+                                               idx_a, idx_b, mod_num), "ckks_poly_automorph_ntt")
+
+    def sk_and_poly_LeftRot_inv(self, device_a, device_b, rot_num, idx_a, idx_b, mod_num):
+        """The same with the exponent rotGroups[rot_num] (poly_arithmetic.cuh:639-660): X -> X^(5^-rot_num)."""
+        _check(self.L_.ckks_poly_automorph_ntt(self.h, _addr(device_a), _addr(device_b), self.rotGroups(rot_num), idx_a, idx_b, mod_num),
+               "ckks_poly_automorph_ntt")
+
+    def sk_and_poly_conjugate(self, device_a, device_b, idx_a, idx_b, mod_num):
+        _check(self.L_.ckks_poly_conjugate_ntt(self.h, _addr(device_a), _addr(device_b), idx_a, idx_b, mod_num), "ckks_poly_conjugate_ntt")
+
     # -- Context_23::encode_coeffs / decode_coeffs (Encoder.cuh:83-96, 113-186)
     def encode_coeffs(self, vals, msg):
         """vals: N device doubles; msg: Plaintext (level msg.l, integer scale msg.scale)."""
@@ -292,9 +311,20 @@ class Key:
         self.bx_device = self.cipher_device.ptr + 8 * N * (L + 1 + K) * dnum
 
 
+class Key_decomp:
+    """Key_decomp (Key_decomp.cuh:5-24): a switching key in the T basis, [a | b] with dnum * Ri_blockNum * t_num limbs each."""
+
+    def __init__(self, N, dnum, t_num, Ri_blockNum):
+        self.N, self.dnum, self.t_num, self.Ri_blockNum = N, dnum, t_num, Ri_blockNum
+        self.cipher_device = DeviceBuffer(8 * N * dnum * t_num * Ri_blockNum * 2)
+        self.ax_device = self.cipher_device.ptr
+        self.bx_device = self.cipher_device.ptr + 8 * N * dnum * t_num * Ri_blockNum
+
+
 class Scheme_23:
     """The members of Scheme_23 on this path (Scheme_23.h:113-182): addEncKey, encryptZero, encryptMsg, decryptMsg,
-    rescaleAndEqual.  Randomness is the context's Salsa20 stream under this object's key with a nonce that counts calls."""
+    rescaleAndEqual, addMultKey_23, addConjKey_23, addLeftRotKey_23, mult_23, leftRotate_23, conjugate_23.
+    Randomness is the context's Salsa20 stream under this object's key with a nonce that counts calls."""
 
     def __init__(self, context, key=bytes(32)):
         self.context = context
@@ -305,6 +335,85 @@ class Scheme_23:
         self.in_enc = DeviceBuffer(9 * N)                                   # Scheme_23.cuh:38-39
         self.vx_enc = DeviceBuffer(8 * N * (L + 1))
         self.rescale_buffer = DeviceBuffer(8 * N * (L + 1) * 2)
+        self.rlk_23 = None
+        self.ConjKey_23 = None
+        self.rotKey_vec_23 = {}
+        if context.t_num:                                                   # Scheme_23::mallocMemory (Scheme_23.cuh:7-51)
+            T, RB, K = context.t_num, context.Ri_blockNum, context.K
+            self.sxsx = DeviceBuffer(8 * N * (K + L + 1))
+            self.temp_mul = DeviceBuffer(8 * N * (K + L + 1))
+            self.mul_work = DeviceBuffer(8 * N * (L + 1) * 3)               # axbx1_mul, axax_mul, bxbx_mul
+            self.modUp_QjtoT_temp = DeviceBuffer(8 * N * T * context.Qj_blockNum)
+            self.exProduct_T_temp = DeviceBuffer(8 * N * T * RB * 2)
+            self.modUp_TtoQj_buffer = DeviceBuffer(8 * N * T * RB * 2)
+
+    def _switch_key(self, s_to, s_from):
+        c = self.context
+        N, KL = c.N, c.K + c.L + 1
+        key = Key_decomp(N, c.dnum, c.t_num, c.Ri_blockNum)
+        na, ne = c.dnum * 8 * N * KL, c.dnum * 4 * N
+        rnd = DeviceBuffer(na + ne)                                         # KeySwitch_23.cuh:36-37
+        c.generateRandom_device(rnd, na + ne, self.key, self._next_nonce())
+        _check(c.L_.ckks_keygen_switch_23(c.h, key.cipher_device.ptr, _addr(s_to), _addr(s_from), rnd.ptr, rnd.ptr + na,
+                                          self.temp_mul.ptr), "ckks_keygen_switch_23")
+        rnd.free()
+        return key
+
+    def addMultKey_23(self, secretKey):
+        """KeySwitch_23.cuh:21-65: the key that switches s^2 to s."""
+        if self.rlk_23 is not None:
+            return
+        c = self.context
+        c.barrett_batch_3param_device(self.sxsx, secretKey.sx_device, secretKey.sx_device, 0, c.K, c.K, c.K, c.L + 1)
+        self.rlk_23 = self._switch_key(secretKey.sx_device, self.sxsx)
+
+    def addConjKey_23(self, secretKey):
+        """KeySwitch_23.cuh:69-114: the key that switches the reversed secret to s."""
+        if self.ConjKey_23 is not None:
+            return
+        c = self.context
+        c.sk_and_poly_conjugate(self.sxsx, secretKey.sx_device, 0, c.K, c.L + 1)
+        self.ConjKey_23 = self._switch_key(secretKey.sx_device, self.sxsx)
+
+    def addLeftRotKey_23(self, secretKey, rot_num):
+        """KeySwitch_23.cuh:119-165: the key that switches s to s(X^(5^-rot_num))."""
+        if rot_num in self.rotKey_vec_23:
+            return
+        c = self.context
+        c.sk_and_poly_LeftRot_inv(self.sxsx, secretKey.sx_device, rot_num, 0, 0, c.K + c.L + 1)
+        self.rotKey_vec_23[rot_num] = self._switch_key(self.sxsx, secretKey.sx_device.ptr + 8 * c.N * c.K)
+
+    def _ks_buffers(self):
+        return self.mul_work.ptr, self.modUp_QjtoT_temp.ptr, self.exProduct_T_temp.ptr, self.modUp_TtoQj_buffer.ptr
+
+    def mult_23(self, cipher_res, cipher1, cipher2):
+        """KeySwitch_23.cuh:192-236; level 0 or a missing key raise ValueError (std::invalid_argument there)."""
+        c = self.context
+        l = min(cipher1.l, cipher2.l)
+        key = self.rlk_23.cipher_device.ptr if self.rlk_23 is not None else None
+        if l != 0 and key is None:
+            raise ValueError("rotKey_23 not exists")
+        _check(c.L_.ckks_mult_23(c.h, cipher_res.cipher_device.ptr, cipher1.cipher_device.ptr, cipher2.cipher_device.ptr, key, l,
+                                 *self._ks_buffers()), "ckks_mult_23")
+        cipher_res.l, cipher_res.scale = l, cipher1.scale * cipher2.scale
+
+    def leftRotate_23(self, cipher_res, cipher, rotSlots):
+        """KeySwitch_23.cuh:556-586."""
+        c = self.context
+        if rotSlots not in self.rotKey_vec_23:
+            raise ValueError("rotKey_23 not exists")
+        _check(c.L_.ckks_rotate_23(c.h, cipher_res.cipher_device.ptr, cipher.cipher_device.ptr,
+                                   self.rotKey_vec_23[rotSlots].cipher_device.ptr, rotSlots, cipher.l, *self._ks_buffers()), "ckks_rotate_23")
+        cipher_res.l, cipher_res.scale, cipher_res.slots = cipher.l, cipher.scale, cipher.slots
+
+    def conjugate_23(self, cipher_res, cipher):
+        """KeySwitch_23.cuh:433-468."""
+        c = self.context
+        if self.ConjKey_23 is None:
+            raise ValueError("conjKey_23 not exists")
+        _check(c.L_.ckks_conjugate_23(c.h, cipher_res.cipher_device.ptr, cipher.cipher_device.ptr, self.ConjKey_23.cipher_device.ptr,
+                                      cipher.l, *self._ks_buffers()), "ckks_conjugate_23")
+        cipher_res.l, cipher_res.scale, cipher_res.slots = cipher.l, cipher.scale, cipher.slots
 
     def _next_nonce(self):
         self.nonce += 1

@@ -168,6 +168,35 @@ int ckks_encode_coeffs(ckks_ctx* ctx, uint64_t* mx, const double* vals, long sca
  * conversion), vals: N device doubles. */
 int ckks_decode_coeffs(ckks_ctx* ctx, double* vals, const uint64_t* mx, uint64_t* scratch, double scale, int slots, int is_bitrev, int l);
 
+/* ---- switching keys in the T basis and the operations built on the key switch ---- */
+/* Context_23::rotGroups (Context_23.cuh:648-659): 5^idx mod 2N */
+int ckks_rot_group(const ckks_ctx* ctx, long idx, uint64_t* value);
+/* sk_and_poly_LeftRot_ntt_double / sk_and_poly_LeftRot_inv (poly_arithmetic.cuh:581-660): the NTT-domain slot permutation
+ * out[j] = in[i] with 2*bitrev(j)+1 = pow * (2*bitrev(i)+1) mod 2N (the reference passes pow = rotGroups[N/2 - rot] or
+ * rotGroups[rot]), on limbs idx_in.. -> idx_out..; in the coefficient domain this is X -> X^(pow^-1).  Not in place. */
+int ckks_poly_automorph_ntt(ckks_ctx* ctx, uint64_t* out, const uint64_t* in, uint64_t pow, int idx_out, int idx_in, int mod_num);
+/* sk_and_poly_conjugate (poly_arithmetic.cuh:666-680): out[i] = in[N-1-i], i.e. X -> X^-1.  Not in place. */
+int ckks_poly_conjugate_ntt(ckks_ctx* ctx, uint64_t* out, const uint64_t* in, int idx_out, int idx_in, int mod_num);
+/* the body shared by Scheme_23::addMultKey_23 / addConjKey_23 / addLeftRotKey_23 (KeySwitch_23.cuh:36-64, 85-113, 136-165):
+ * swk (Key_decomp layout, [2][dnum][Ri_blockNum * t_num] limbs, NTT domain over T) switches from the secret s_from to the secret
+ * s_to.  s_to: K+L+1 limbs over [P | Q]; s_from: L+1 limbs over Q (s^2 for the multiplication key, the reversed s for the
+ * conjugation key, s itself for a rotation key whose s_to is the permuted s); both NTT domain.
+ * random_a: dnum * 8*N*(K+L+1) bytes, random_e: dnum * 4*N bytes; scratch: (K+L+1)*N words. */
+int ckks_keygen_switch_23(ckks_ctx* ctx, uint64_t* swk, const uint64_t* s_to, const uint64_t* s_from, const uint8_t* random_a,
+                          const uint8_t* random_e, uint64_t* scratch);
+/* Scheme_23::mult_23 (KeySwitch_23.cuh:192-236): out = c1 * c2 relinearised with rlk, limbs 0..l of [a: L+1 | b: L+1].
+ * work: 3*(L+1)*N words (the reference's axbx1_mul, axax_mul, bxbx_mul); the other three as in ckks_keyswitch_23.
+ * Level 0 or a null key: CKKS_E_STATE (std::invalid_argument in the reference, :194-201). */
+int ckks_mult_23(ckks_ctx* ctx, uint64_t* out, const uint64_t* c1, const uint64_t* c2, const uint64_t* rlk, int l, uint64_t* work,
+                 uint64_t* modUp_QjtoT_temp, uint64_t* exProduct_T_temp, uint64_t* modUp_TtoQj_buffer);
+/* Scheme_23::leftRotate_23 (KeySwitch_23.cuh:556-586): out = cipher rotated left by rot slots (decrypts to m(X^(5^rot))).
+ * work: 3*(L+1)*N words (a copy of a, and the reference's cipher_temp_pool).  out != cipher. */
+int ckks_rotate_23(ckks_ctx* ctx, uint64_t* out, const uint64_t* cipher, const uint64_t* rotkey, long rot, int l, uint64_t* work,
+                   uint64_t* modUp_QjtoT_temp, uint64_t* exProduct_T_temp, uint64_t* modUp_TtoQj_buffer);
+/* Scheme_23::conjugate_23 (KeySwitch_23.cuh:433-468): decrypts to m(X^-1).  work: (L+1)*N words.  out != cipher. */
+int ckks_conjugate_23(ckks_ctx* ctx, uint64_t* out, const uint64_t* cipher, const uint64_t* conjkey, int l, uint64_t* work,
+                      uint64_t* modUp_QjtoT_temp, uint64_t* exProduct_T_temp, uint64_t* modUp_TtoQj_buffer);
+
 /* ---- ring-packed PCMM ---- */
 /* PCMM_Context::PCMM_Context (PCMM_Context.cuh:7-57) */
 int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,

@@ -233,15 +233,39 @@ public:
     virtual ~MLWECiphertext() { device_release(cipher_device); }
 };
 
-// The members of Scheme_23 on the path (Scheme_23.h:113-182): public-key encryption, decryption, rescale and the key-switch
-// chain of mult_23.
+// Key_decomp (Key_decomp.cuh:5-24): a switching key in the T basis, [a | b] with dnum * Ri_blockNum * t_num limbs each
+class Key_decomp {
+public:
+    uint64_tt* ax_device = nullptr;
+    uint64_tt* bx_device = nullptr;
+    uint64_tt* cipher_device = nullptr;
+    int N = 0, dnum = 0, t_num = 0, Ri_blockNum = 0;
+
+    Key_decomp(int N, int dnum, int t_num, int Ri_blockNum) : N(N), dnum(dnum), t_num(t_num), Ri_blockNum(Ri_blockNum) {
+        cipher_device = device_alloc_words((size_t)N * dnum * t_num * Ri_blockNum * 2);
+        ax_device = cipher_device;
+        bx_device = cipher_device + (size_t)N * dnum * t_num * Ri_blockNum;
+    }
+    Key_decomp(const Key_decomp&) = delete;
+    Key_decomp& operator=(const Key_decomp&) = delete;
+    virtual ~Key_decomp() { device_release(cipher_device); }
+};
+
+// The members of Scheme_23 on the path (Scheme_23.h:113-182): public-key encryption, decryption, rescale, switching keys,
+// multiplication, rotation, conjugation.
 class Scheme_23 {
 public:
     Context_23& context;
     Key* publicKey = nullptr;
+    Key_decomp* rlk_23 = nullptr;
+    Key_decomp* ConjKey_23 = nullptr;
+    std::vector<Key_decomp*> rotKey_vec_23;
     uint64_tt* vx_enc = nullptr;
     uint8_t* in_enc = nullptr;
     long random_len_for_enc = 0;
+    uint64_tt* sxsx = nullptr;
+    uint64_tt* temp_mul = nullptr;
+    uint64_tt* mul_work = nullptr;            // axbx1_mul, axax_mul, bxbx_mul of the reference, contiguous
     // Scheme_23::mallocMemory (Scheme_23.cuh:7-51): scratch owned by the scheme
     uint64_tt* rescale_buffer = nullptr;
     uint64_tt* modUp_QjtoT_temp = nullptr;
@@ -254,7 +278,11 @@ public:
         vx_enc = device_alloc_words(N * (context.L + 1));
         random_len_for_enc = (long)(N + 4 * N + 4 * N);                          // Scheme_23.cuh:38
         in_enc = reinterpret_cast<uint8_t*>(device_alloc_words((size_t)random_len_for_enc / 8));
+        rotKey_vec_23.assign(N, nullptr);                                        // Scheme_23.cuh:41
         if (context.t_num > 0) {
+            sxsx = device_alloc_words(N * (context.K + context.L + 1));
+            temp_mul = device_alloc_words(N * (context.K + context.L + 1));
+            mul_work = device_alloc_words(3 * N * (context.L + 1));
             modUp_QjtoT_temp = device_alloc_words(N * context.t_num * context.Qj_blockNum);
             exProduct_T_temp = device_alloc_words(N * context.t_num * context.Ri_blockNum * 2);
             modUp_TtoQj_buffer = device_alloc_words(N * context.t_num * context.Ri_blockNum * 2);
@@ -263,6 +291,12 @@ public:
     Scheme_23(const Scheme_23&) = delete;
     ~Scheme_23() {
         delete publicKey;
+        delete rlk_23;
+        delete ConjKey_23;
+        for (Key_decomp* k : rotKey_vec_23) delete k;
+        device_release(sxsx);
+        device_release(temp_mul);
+        device_release(mul_work);
         device_release(vx_enc);
         uint64_tt* r = reinterpret_cast<uint64_tt*>(in_enc);
         device_release(r);
@@ -304,6 +338,51 @@ public:
         check(ckks_decrypt(context.handle, plain.mx_device, cipher.cipher_device, secretKey.sx_device, cipher.l), "decryptMsg");
     }
 
+    // Scheme_23::addMultKey_23 / addConjKey_23 / addLeftRotKey_23 (KeySwitch_23.cuh:21-165)
+    void addMultKey_23(SecretKey& secretKey) {
+        if (rlk_23) return;
+        const int K = context.K;
+        check(ckks_poly_mul(context.handle, sxsx, secretKey.sx_device, secretKey.sx_device, 0, K, K, K, context.L + 1), "addMultKey_23");
+        rlk_23 = switch_key(secretKey.sx_device, sxsx);
+    }
+    void addConjKey_23(SecretKey& secretKey) {
+        if (ConjKey_23) return;
+        check(ckks_poly_conjugate_ntt(context.handle, sxsx, secretKey.sx_device, 0, context.K, context.L + 1), "addConjKey_23");
+        ConjKey_23 = switch_key(secretKey.sx_device, sxsx);
+    }
+    void addLeftRotKey_23(SecretKey& secretKey, long rot_num) {
+        if (rotKey_vec_23.at((size_t)rot_num)) return;
+        uint64_tt pow = 0;
+        check(ckks_rot_group(context.handle, rot_num, &pow), "addLeftRotKey_23");
+        check(ckks_poly_automorph_ntt(context.handle, sxsx, secretKey.sx_device, pow, 0, 0, context.K + context.L + 1), "addLeftRotKey_23");
+        rotKey_vec_23[(size_t)rot_num] = switch_key(sxsx, secretKey.sx_device + (size_t)context.N * context.K);
+    }
+    // Scheme_23::mult_23 (KeySwitch_23.cuh:192-236); level 0 and a missing key throw std::invalid_argument
+    void mult_23(Ciphertext& cipher_res, Ciphertext& cipher1, Ciphertext& cipher2) {
+        const int l = cipher1.l < cipher2.l ? cipher1.l : cipher2.l;
+        check(ckks_mult_23(context.handle, cipher_res.cipher_device, cipher1.cipher_device, cipher2.cipher_device,
+                           rlk_23 ? rlk_23->cipher_device : nullptr, l, mul_work, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer), "mult_23");
+        cipher_res.l = l;
+        cipher_res.scale = cipher1.scale * cipher2.scale;
+    }
+    // Scheme_23::leftRotate_23 (KeySwitch_23.cuh:556-586)
+    void leftRotate_23(Ciphertext& cipher_res, Ciphertext& cipher, long rotSlots) {
+        Key_decomp* k = (rotSlots >= 0 && (size_t)rotSlots < rotKey_vec_23.size()) ? rotKey_vec_23[(size_t)rotSlots] : nullptr;
+        check(ckks_rotate_23(context.handle, cipher_res.cipher_device, cipher.cipher_device, k ? k->cipher_device : nullptr, rotSlots, cipher.l,
+                             mul_work, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer), "leftRotate_23");
+        cipher_res.l = cipher.l;
+        cipher_res.scale = cipher.scale;
+        cipher_res.slots = cipher.slots;
+    }
+    // Scheme_23::conjugate_23 (KeySwitch_23.cuh:433-468)
+    void conjugate_23(Ciphertext& cipher_res, Ciphertext& cipher) {
+        check(ckks_conjugate_23(context.handle, cipher_res.cipher_device, cipher.cipher_device, ConjKey_23 ? ConjKey_23->cipher_device : nullptr,
+                                cipher.l, mul_work, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer), "conjugate_23");
+        cipher_res.l = cipher.l;
+        cipher_res.scale = cipher.scale;
+        cipher_res.slots = cipher.slots;
+    }
+
     // Scheme_23::rescaleAndEqual (Scheme_23.cuh:369-385); throws std::invalid_argument on level 0 (:192-194 style)
     void rescaleAndEqual(Ciphertext& cipher) {
         check(ckks_rescale(context.handle, cipher.cipher_device, rescale_buffer, cipher.l), "rescaleAndEqual");
@@ -317,6 +396,19 @@ public:
     }
 
 private:
+    Key_decomp* switch_key(const uint64_tt* s_to, const uint64_tt* s_from) {
+        const size_t N = (size_t)context.N, KL = (size_t)context.K + context.L + 1;
+        const size_t na = (size_t)context.dnum * 8 * N * KL, ne = (size_t)context.dnum * 4 * N;      // KeySwitch_23.cuh:36
+        Key_decomp* key = new Key_decomp((int)N, context.dnum, context.t_num, context.Ri_blockNum);
+        uint64_tt* rnd = device_alloc_words((na + ne) / 8);
+        uint8_t* r8 = reinterpret_cast<uint8_t*>(rnd);
+        context.generateRandom_device(r8, na + ne);
+        int rc = ckks_keygen_switch_23(context.handle, key->cipher_device, s_to, s_from, r8, r8 + na, temp_mul);
+        device_release(rnd);
+        if (rc != CKKS_OK) delete key;
+        check(rc, "addSWKey_23");
+        return key;
+    }
     void encrypt(Ciphertext& cipher, const uint64_tt* mx, int l) {
         if (!publicKey) throw std::invalid_argument("encryptMsg: no encryption key (addEncKey)");
         context.generateRandom_device(in_enc, (uint64_tt)random_len_for_enc);

@@ -1116,6 +1116,126 @@ int orc_encode_coeffs(const orc_ctx* c, u64* mx, const double* vals, long scale,
     return orc_ntt_fwd(c, mx, 0, K, 1, l + 1, L1);
 }
 
+// ------------------------------------------------------------------------------------------------
+// automorphisms in the NTT domain, switching keys in the T basis, homomorphic multiply / rotate / conjugate
+// ------------------------------------------------------------------------------------------------
+// Context_23.cuh:648-659: rotGroups[i] = 5^i mod 2N
+u64 orc_rot_group(const orc_ctx* c, long idx) {
+    const u64 M = 2 * (u64)c->N;
+    u64 r = 1;
+    for (long i = 0; i < idx; i++) r = r * 5 % M;
+    return r;
+}
+// sk_and_poly_LeftRot_ntt_kernel / sk_and_poly_LeftRot_inv_kernel (poly_arithmetic.cuh:581-596, 639-653): NTT slot i holds the
+// evaluation at psi^(2*bitrev(i)+1); out[j] = in[i] with 2*bitrev(j)+1 = pow * (2*bitrev(i)+1) mod 2N, on mod_num limbs
+int orc_automorph_ntt(const orc_ctx* c, u64* out, const u64* in, u64 pow, int idx_out, int idx_in, int mod_num) {
+    const long N = c->N;
+    const u64 mask = 2 * (u64)N - 1;
+    for (int t = 0; t < mod_num; t++)
+        for (long i = 0; i < N; i++) {
+            u64 e = 2 * (u64)orc_bitrev((uint32_t)i, c->logN) + 1;
+            u64 j = (((pow * e) & mask) - 1) >> 1;
+            out[((long)idx_out + t) * N + orc_bitrev((uint32_t)j, c->logN)] = in[((long)idx_in + t) * N + i];
+        }
+    return 0;
+}
+// sk_and_poly_conjugate_kernel (poly_arithmetic.cuh:666-674): out[i] = in[N-1-i]
+int orc_conjugate_ntt(const orc_ctx* c, u64* out, const u64* in, int idx_out, int idx_in, int mod_num) {
+    const long N = c->N;
+    for (int t = 0; t < mod_num; t++)
+        for (long i = 0; i < N; i++) out[((long)idx_out + t) * N + i] = in[((long)idx_in + t) * N + N - 1 - i];
+    return 0;
+}
+
+// The body shared by Scheme_23::addMultKey_23 / addConjKey_23 / addLeftRotKey_23 (KeySwitch_23.cuh:36-64, 85-113, 136-165):
+// digit i of the key is (a_i, P * s_from restricted to the digit's primes + e_i - a_i * s_to) over [P | Q], taken to the
+// coefficient domain, lifted to the T basis block by block (modUpPQtoT_23) and transformed there.
+// s_to: K+L+1 limbs (pqt order), s_from: L+1 limbs over Q, both NTT domain; random_a: dnum * 8*N*(K+L+1) bytes,
+// random_e: dnum * 4*N bytes; swk: Key_decomp layout [2][dnum][Ri_blockNum * t_num] limbs.
+int orc_keygen_switch_23(const orc_ctx* c, u64* swk, const u64* s_to, const u64* s_from, const uint8_t* random_a, const uint8_t* random_e) {
+    const long N = c->N;
+    const int K = c->K, L = c->L, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum, KL = K + L + 1;
+    if (K <= 0 || T <= 0 || RB * T < KL) return -1;
+    const size_t digit = (size_t)N * T * RB;
+    u64* ax = swk; u64* bx = swk + digit * dnum;
+    std::vector<u64> temp((size_t)N * KL), ex((size_t)N * KL);
+    for (int i = 0; i < dnum; i++) {
+        std::fill(temp.begin(), temp.end(), 0);
+        for (int t = 0; t < K && i * K + t <= L; t++) {                            // sxsx_mul_P_3param (poly_arithmetic.cuh:526-541)
+            const int prime = K + i * K + t;
+            const u64 q = c->pqt[prime], Pq = c->PModqt[prime - K];
+            for (long x = 0; x < N; x++) {
+                const u64 a = s_from[((long)i * K + t) * N + x];
+                temp[(size_t)prime * N + x] = orc_barrett128((u64)(((u128)a * Pq) >> 64), a * Pq, q, c->mu_hi[prime], c->mu_lo[prime]);
+            }
+        }
+        orc_sample_gaussian(c, random_e + (size_t)i * N * 4, ex.data(), 0, 0, KL);
+        orc_ntt_fwd(c, ex.data(), 0, 0, 1, KL, KL);
+        orc_poly_op(c, 1, temp.data(), temp.data(), ex.data(), 0, 0, 0, 0, KL);
+        orc_sample_uniform(c, random_a + (size_t)i * N * KL * 8, ax + digit * i, 0, 0, KL);
+        orc_poly_op(c, 0, bx + digit * i, ax + digit * i, s_to, 0, 0, 0, 0, KL);
+        orc_poly_op(c, 2, bx + digit * i, temp.data(), bx + digit * i, 0, 0, 0, 0, KL);     // poly_sub2: b = temp - b
+    }
+    orc_ntt_inv(c, ax, 0, 0, dnum, KL, T * RB);
+    orc_ntt_inv(c, bx, 0, 0, dnum, KL, T * RB);
+    for (int i = 0; i < dnum; i++)
+        for (u64* part : {ax + digit * i, bx + digit * i}) {
+            std::copy(part, part + (size_t)N * KL, temp.begin());
+            if (orc_modup_pq_to_t(c, part, temp.data(), L, 1)) return -1;
+        }
+    return orc_ntt_fwd(c, swk, 0, KL, dnum * RB * 2, T, T);
+}
+
+// compute_c0c1c2_kernel (poly_arithmetic.cuh:787-818): a1*a2, b1*b2 and a1*b2 + a2*b1 through (a1+b1)(a2+b2) in 128 bits
+static void tensor_c0c1c2(const orc_ctx* c, u64* axbx, u64* axax, u64* bxbx, const u64* a1, const u64* a2, const u64* b1, const u64* b2, int limbs) {
+    const long N = c->N; const int K = c->K;
+    for (int t = 0; t < limbs; t++) {
+        const u64 q = c->pqt[K + t], mh = c->mu_hi[K + t], ml = c->mu_lo[K + t];
+        for (long x = 0; x < N; x++) {
+            const long o = (long)t * N + x;
+            const u128 t1 = (u128)a1[o] * a2[o], t2 = (u128)b1[o] * b2[o];
+            const u128 t3 = (u128)(a1[o] + b1[o]) * (a2[o] + b2[o]) - t1 - t2;
+            axax[o] = orc_barrett128((u64)(t1 >> 64), (u64)t1, q, mh, ml);
+            bxbx[o] = orc_barrett128((u64)(t2 >> 64), (u64)t2, q, mh, ml);
+            axbx[o] = orc_barrett128((u64)(t3 >> 64), (u64)t3, q, mh, ml);
+        }
+    }
+}
+// Scheme_23::mult_23 (KeySwitch_23.cuh:192-236): out = [a | b] with L+1 limbs each, limbs 0..l written
+int orc_mult_23(const orc_ctx* c, u64* out, const u64* c1, const u64* c2, const u64* rlk, int l) {
+    const long N = c->N; const int K = c->K, L1 = c->L + 1;
+    if (l < 1 || l > c->L) return -4;
+    std::vector<u64> axbx((size_t)N * L1, 0), axax((size_t)N * L1, 0), bxbx((size_t)N * L1, 0);
+    tensor_c0c1c2(c, axbx.data(), axax.data(), bxbx.data(), c1, c2, c1 + N * L1, c2 + N * L1, l + 1);
+    if (orc_keyswitch_23(c, out, axax.data(), rlk, l)) return -1;
+    orc_poly_op(c, 1, out, out, axbx.data(), 0, 0, 0, K, l + 1);                   // cipher_add_axbx_batch_device (:159-172)
+    orc_poly_op(c, 1, out + N * L1, out + N * L1, bxbx.data(), 0, 0, 0, K, l + 1);
+    return 0;
+}
+// Scheme_23::leftRotate_23 (KeySwitch_23.cuh:556-586): key switch of a, + b, then the slot permutation with 5^(N/2 - rot)
+int orc_rotate_23(const orc_ctx* c, u64* out, const u64* cipher, const u64* rotkey, long rot, int l) {
+    const long N = c->N; const int K = c->K, L1 = c->L + 1;
+    if (l < 0 || l > c->L || rot < 0 || rot > N / 2) return -1;
+    std::vector<u64> tmp((size_t)2 * N * L1, 0);
+    if (orc_keyswitch_23(c, tmp.data(), cipher, rotkey, l)) return -1;
+    orc_poly_op(c, 1, tmp.data() + N * L1, tmp.data() + N * L1, cipher + N * L1, 0, 0, 0, K, l + 1);
+    const u64 pow = orc_rot_group(c, N / 2 - rot);
+    orc_automorph_ntt(c, out, tmp.data(), pow, 0, 0, l + 1);
+    orc_automorph_ntt(c, out + N * L1, tmp.data() + N * L1, pow, 0, 0, l + 1);
+    return 0;
+}
+// Scheme_23::conjugate_23 (KeySwitch_23.cuh:433-468): reverse both polynomials, key switch of the reversed a, + reversed b
+int orc_conjugate_23(const orc_ctx* c, u64* out, const u64* cipher, const u64* conjkey, int l) {
+    const long N = c->N; const int K = c->K, L1 = c->L + 1;
+    if (l < 0 || l > c->L) return -1;
+    std::vector<u64> ar((size_t)N * L1, 0), br((size_t)N * L1, 0);
+    orc_conjugate_ntt(c, br.data(), cipher + N * L1, 0, 0, l + 1);
+    orc_conjugate_ntt(c, ar.data(), cipher, 0, 0, l + 1);
+    if (orc_keyswitch_23(c, out, ar.data(), conjkey, l)) return -1;
+    orc_poly_op(c, 1, out + N * L1, out + N * L1, br.data(), 0, 0, 0, K, l + 1);
+    return 0;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -31,6 +31,9 @@
  *   keys, encryption, decryption   decrypt identities with Python negacyclic
  *                                  algebra (a*s + b = m + small noise)          (tests/test_oracle_scheme.py)
  *   coefficient encode / decode    Python big-integer CRT and exact rationals   (tests/test_oracle_scheme.py)
+ *   NTT-domain automorphisms       coefficient-domain substitution X -> X^g     (tests/test_oracle_keys.py)
+ *   switching keys, mult / rotate  decrypt identities: product of messages,
+ *   / conjugate                    m(X^(5^r)), m(X^-1), within a noise bound   (tests/test_oracle_keys.py)
  */
 #pragma once
 #include <stdint.h>
@@ -136,6 +139,16 @@ int orc_keygen_public(const orc_ctx*, uint64_t* pk, const uint64_t* sx, const ui
 int orc_encrypt(const orc_ctx*, uint64_t* cipher, const uint64_t* mx, const uint64_t* pk, const uint8_t* random, int l);
 int orc_decrypt(const orc_ctx*, uint64_t* mx, const uint64_t* cipher, const uint64_t* sx, int l);
 int orc_encode_coeffs(const orc_ctx*, uint64_t* mx, const double* vals, long scale, int l);
+
+/* ---- automorphisms, switching keys in the T basis, homomorphic multiply / rotate / conjugate ---- */
+uint64_t orc_rot_group(const orc_ctx*, long idx);
+int orc_automorph_ntt(const orc_ctx*, uint64_t* out, const uint64_t* in, uint64_t pow, int idx_out, int idx_in, int mod_num);
+int orc_conjugate_ntt(const orc_ctx*, uint64_t* out, const uint64_t* in, int idx_out, int idx_in, int mod_num);
+int orc_keygen_switch_23(const orc_ctx*, uint64_t* swk, const uint64_t* s_to, const uint64_t* s_from, const uint8_t* random_a,
+                         const uint8_t* random_e);
+int orc_mult_23(const orc_ctx*, uint64_t* out, const uint64_t* c1, const uint64_t* c2, const uint64_t* rlk, int l);
+int orc_rotate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* rotkey, long rot, int l);
+int orc_conjugate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* conjkey, int l);
 
 int orc_max_threads(void);
 

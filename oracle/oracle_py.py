@@ -90,6 +90,11 @@ def lib():
             "orc_keygen_secret": (i, [vp, P64, P8, i]), "orc_keygen_public": (i, [vp, P64, P64, P8, P8]),
             "orc_encrypt": (i, [vp, P64, P64, P64, P8, i]), "orc_decrypt": (i, [vp, P64, P64, P64, i]),
             "orc_encode_coeffs": (i, [vp, P64, C.POINTER(C.c_double), l, i]),
+            "orc_rot_group": (u64, [vp, l]),
+            "orc_automorph_ntt": (i, [vp, P64, P64, u64, i, i, i]), "orc_conjugate_ntt": (i, [vp, P64, P64, i, i, i]),
+            "orc_keygen_switch_23": (i, [vp, P64, P64, P64, P8, P8]),
+            "orc_mult_23": (i, [vp, P64, P64, P64, P64, i]), "orc_rotate_23": (i, [vp, P64, P64, P64, l, i]),
+            "orc_conjugate_23": (i, [vp, P64, P64, P64, i]),
             "orc_max_threads": (i, []),
         }
         for name, (res, args) in sig.items():
@@ -217,6 +222,31 @@ class OracleContext:
     def encode_coeffs(self, mx, vals, scale, l):
         assert vals.dtype == np.float64 and vals.size == self.N
         self._ck(self.L_.orc_encode_coeffs(self.h, _ptr(mx), vals.ctypes.data_as(C.POINTER(C.c_double)), int(scale), l))
+
+    # ---- automorphisms, switching keys in the T basis, homomorphic multiply / rotate / conjugate (KeySwitch_23.cuh) ----
+    def rot_group(self, idx):
+        return int(self.L_.orc_rot_group(self.h, idx))
+
+    def automorph_ntt(self, out, inp, pow_, idx_out, idx_in, mod_num):
+        self._ck(self.L_.orc_automorph_ntt(self.h, _ptr(out), _ptr(inp), pow_, idx_out, idx_in, mod_num))
+
+    def conjugate_ntt(self, out, inp, idx_out, idx_in, mod_num):
+        self._ck(self.L_.orc_conjugate_ntt(self.h, _ptr(out), _ptr(inp), idx_out, idx_in, mod_num))
+
+    def keygen_switch_23(self, swk, s_to, s_from, random_a, random_e):
+        self._ck(self.L_.orc_keygen_switch_23(self.h, _ptr(swk), _ptr(s_to), _ptr(s_from), _bytes(random_a), _bytes(random_e)))
+
+    def mult_23(self, out, c1, c2, rlk, l):
+        rc = self.L_.orc_mult_23(self.h, _ptr(out), _ptr(c1), _ptr(c2), _ptr(rlk), l)
+        if rc == -4:
+            raise ValueError("Ciphertexts are on level 0")
+        self._ck(rc)
+
+    def leftRotate_23(self, out, cipher, rotkey, rot, l):
+        self._ck(self.L_.orc_rotate_23(self.h, _ptr(out), _ptr(cipher), _ptr(rotkey), rot, l))
+
+    def conjugate_23(self, out, cipher, conjkey, l):
+        self._ck(self.L_.orc_conjugate_23(self.h, _ptr(out), _ptr(cipher), _ptr(conjkey), l))
 
     def decode_coeffs(self, mx, scale, slots, l, is_bitrev=False):
         """Context_23::decode_coeffs (Encoder.cuh:113-186): iNTT of limbs 0..l, CRT to the centred integer modulo q_0..q_l

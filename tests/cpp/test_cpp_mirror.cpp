@@ -177,6 +177,79 @@ static int run() {
         ckks_free(vd);
     }
 
+    // ---- the reference's logN = 13 parameter set (5 q, 1 p, 3 t, gamma 3; Params.cuh) at N = 2^10: keys in the T basis,
+    //      mult_23, leftRotate_23, conjugate_23 against the oracle, word for word on the same stream ----
+    {
+        const std::vector<uint64_tt> q13 = {0x4001b00001ull, 0xfff9c0001ull, 0xfff8e0001ull, 0xfff840001ull, 0xfff700001ull};
+        const std::vector<uint64_tt> p13 = {0x10a19000001ull};
+        const std::vector<uint64_tt> t13 = {0xffffffffffc0001ull, 0xfffffffff840001ull, 0xfffffffff6a0001ull};
+        const int lg = 10, h = 64;
+        const long n = 1l << lg;
+        Context_23 c2(lg, p13, q13, t13, 3);
+        orc_ctx* o2 = orc_ctx_create(lg, p13.data(), 1, q13.data(), 5, t13.data(), 3, 3);
+        const int K = c2.K, L1 = c2.L + 1, KL = K + L1;
+        const size_t keyw = (size_t)2 * c2.dnum * c2.Ri_blockNum * c2.t_num * n;
+        const size_t na = (size_t)c2.dnum * 8 * n * KL, ne = (size_t)c2.dnum * 4 * n;
+        const uint8_t zero_key[32] = {0};
+        auto stream = [&](size_t bytes, uint64_t nonce) { std::vector<uint8_t> r(bytes); orc_salsa20_stream(r.data(), bytes, zero_key, nonce); return r; };
+        Scheme_23 s2(c2);
+        SecretKey sk(c2, h);                                   // nonce 1
+        s2.addEncKey(sk);                                      // nonce 2
+        s2.addMultKey_23(sk);                                  // nonce 3
+        s2.addConjKey_23(sk);                                  // nonce 4
+        s2.addLeftRotKey_23(sk, 7);                            // nonce 5
+        std::vector<uint64_tt> o_sx((size_t)n * KL), o_pk((size_t)2 * n * L1), o_ss((size_t)n * KL), o_key(keyw);
+        std::vector<uint8_t> r = stream(5 * h, 1);
+        orc_keygen_secret(o2, o_sx.data(), r.data(), h);
+        r = stream(8 * n * L1 + 4 * n, 2);
+        orc_keygen_public(o2, o_pk.data(), o_sx.data(), r.data(), r.data() + 8 * n * L1);
+        r = stream(na + ne, 3);
+        orc_poly_op(o2, 0, o_ss.data(), o_sx.data(), o_sx.data(), 0, K, K, K, L1);
+        orc_keygen_switch_23(o2, o_key.data(), o_sx.data(), o_ss.data(), r.data(), r.data() + na);
+        EXPECT(download(s2.rlk_23->cipher_device, keyw) == o_key, "addMultKey_23 == oracle");
+        std::vector<uint64_tt> o_rlk = o_key;
+        r = stream(na + ne, 4);
+        orc_conjugate_ntt(o2, o_ss.data(), o_sx.data(), 0, K, L1);
+        orc_keygen_switch_23(o2, o_key.data(), o_sx.data(), o_ss.data(), r.data(), r.data() + na);
+        EXPECT(download(s2.ConjKey_23->cipher_device, keyw) == o_key, "addConjKey_23 == oracle");
+        std::vector<uint64_tt> o_conj = o_key;
+        r = stream(na + ne, 5);
+        orc_automorph_ntt(o2, o_ss.data(), o_sx.data(), orc_rot_group(o2, 7), 0, 0, KL);
+        orc_keygen_switch_23(o2, o_key.data(), o_ss.data(), o_sx.data() + (size_t)n * K, r.data(), r.data() + na);
+        EXPECT(download(s2.rotKey_vec_23[7]->cipher_device, keyw) == o_key, "addLeftRotKey_23 == oracle");
+        // two ciphertexts (nonces 6, 7), then the three operations at the top level
+        Plaintext m1((int)n, c2.L, c2.L, (int)(n / 2), (long double)(1 << 20)), m2((int)n, c2.L, c2.L, (int)(n / 2), (long double)(1 << 20));
+        std::vector<uint64_tt> o_m1 = uniform_limbs(rng, q13, 1, n), o_m2 = uniform_limbs(rng, q13, 1, n);
+        upload(m1.mx_device, o_m1);
+        upload(m2.mx_device, o_m2);
+        Ciphertext e1((int)n, c2.L, c2.L, 1, 1.0L), e2((int)n, c2.L, c2.L, 1, 1.0L), res((int)n, c2.L, c2.L, 1, 1.0L);
+        s2.encryptMsg(e1, m1);
+        s2.encryptMsg(e2, m2);
+        std::vector<uint64_tt> o_c1((size_t)2 * n * L1), o_c2((size_t)2 * n * L1), o_res((size_t)2 * n * L1);
+        r = stream(9 * n, 6);
+        orc_encrypt(o2, o_c1.data(), o_m1.data(), o_pk.data(), r.data(), c2.L);
+        r = stream(9 * n, 7);
+        orc_encrypt(o2, o_c2.data(), o_m2.data(), o_pk.data(), r.data(), c2.L);
+        EXPECT(download(e1.cipher_device, o_c1.size()) == o_c1 && download(e2.cipher_device, o_c2.size()) == o_c2, "two encryptions == oracle");
+        s2.mult_23(res, e1, e2);
+        orc_mult_23(o2, o_res.data(), o_c1.data(), o_c2.data(), o_rlk.data(), c2.L);
+        EXPECT(download(res.cipher_device, o_res.size()) == o_res && res.scale == e1.scale * e2.scale, "mult_23 == oracle");
+        s2.leftRotate_23(res, e1, 7);
+        orc_rotate_23(o2, o_res.data(), o_c1.data(), o_key.data(), 7, c2.L);
+        EXPECT(download(res.cipher_device, o_res.size()) == o_res, "leftRotate_23 == oracle");
+        s2.conjugate_23(res, e1);
+        orc_conjugate_23(o2, o_res.data(), o_c1.data(), o_conj.data(), c2.L);
+        EXPECT(download(res.cipher_device, o_res.size()) == o_res, "conjugate_23 == oracle");
+        threw = false;
+        try { s2.leftRotate_23(res, e1, 8); } catch (const std::invalid_argument&) { threw = true; }
+        EXPECT(threw, "leftRotate_23 without its key throws std::invalid_argument");
+        Ciphertext lvl0((int)n, c2.L, 0, 1, 1.0L);
+        threw = false;
+        try { s2.mult_23(res, e1, lvl0); } catch (const std::invalid_argument&) { threw = true; }
+        EXPECT(threw, "mult_23 on level 0 throws std::invalid_argument");
+        orc_ctx_destroy(o2);
+    }
+
     for (MLWECiphertext* m : mlwe) delete m;
     ckks_free(Wd);
     orc_pcmm_destroy(orc_p);
