@@ -67,6 +67,10 @@ def _declare(L):
         "pcmm_rlwe_decompose_ntt": (i, [vp, vp, C.POINTER(vp), i, i]),
         "pcmm_mlwe_pack": (i, [vp, vp, C.POINTER(vp), i, vp, vp, vp]),
         "pcmm_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "pcmm_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
+        "pcmm_convert_mlwe_sk": (i, [vp, vp, vp]),
+        "pcmm_add_repacking_key": (i, [vp, vp, vp, vp, C.c_char_p, C.c_uint64, vp]),
+        "pcmm_mlwe_decrypt": (i, [vp, vp, vp, vp, i]),
+        "pcmm_decode_coeffs": (i, [vp, vp, vp, vp, C.c_longlong, i]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
     }

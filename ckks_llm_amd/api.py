@@ -465,6 +465,9 @@ class PCMM_Context:
         self.L_ = load_library()
         self.context, self.N1, self.mlwe_rank = context, N1, mlwe_rank
         self.p_ringpack, self.q_ringpack = list(p_ringpack), list(q_ringpack)
+        self.ringpack_p_count, self.ringpack_q_count = len(self.p_ringpack), len(self.q_ringpack)
+        self.ringpack_pq_count = self.ringpack_p_count + self.ringpack_q_count
+        self.pq_ringpack = self.p_ringpack + self.q_ringpack
         pa, qa = _arr(p_ringpack), _arr(q_ringpack)
         h = vp()
         _check(self.L_.pcmm_ctx_create(C.byref(h), context.h, N1, mlwe_rank, pa.ctypes.data_as(u64p), len(pa),
@@ -477,6 +480,12 @@ class PCMM_Context:
         return v.value
 
     # -- PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
+    def decodeCoeffs(self, msg, vals):
+        """PCMM_Context.cuh:165-178: vals = N1 device doubles."""
+        scratch = DeviceBuffer(8 * self.N1 * (msg.l + 1))
+        _check(self.L_.pcmm_decode_coeffs(self.h, _addr(vals), _addr(msg.mx_device), scratch.ptr, int(msg.scale), msg.l), "pcmm_decode_coeffs")
+        scratch.free()
+
     def ToNTTInplace(self, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size):
         _check(self.L_.pcmm_ntt_fwd(self.h, _addr(data), poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "pcmm_ntt_fwd")
 
@@ -492,12 +501,56 @@ class PCMM_Context:
             pass
 
 
-class PCMM_Scheme:
-    """The rlweCipherDecompose / PPMM members of PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48)."""
+class MLWESecretKey:
+    """MLWESecretKey (pcmm/MLWESecretKey.cuh:6-52): [L+1 moduli][k polynomials][N1]."""
 
-    def __init__(self, pcmm_context):
+    def __init__(self, N1, L, k):
+        self.N1, self.L, self.k = N1, L, k
+        self.sx_device = DeviceBuffer(8 * N1 * k * (L + 1))
+
+
+class MLWEPlaintext:
+    """MLWEPlaintext (pcmm/MLWEPlaintext.cuh:7-60): [L+1 moduli][N1]."""
+
+    def __init__(self, N1, L, l, scale):
+        self.N1, self.L, self.l, self.scale = N1, L, l, scale
+        self.mx_device = DeviceBuffer(8 * N1 * (L + 1))
+
+
+class PCMM_Scheme:
+    """PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48): convertMLWESKfromRLWESK, addRepakcingKey, rlweCipherDecompose, PPMM,
+    mlweCipherPacking, mlweDecrypt."""
+
+    def __init__(self, pcmm_context, key=bytes(32)):
         self.L_ = load_library()
         self.pcmm_context = pcmm_context
+        self.repackingKeys = None
+        self.key, self.nonce = bytes(key), 1 << 32
+
+    def convertMLWESKfromRLWESK(self, mlwe_sk, rlwe_sk):
+        """PCMM_Scheme.cuh:23-48."""
+        _check(self.L_.pcmm_convert_mlwe_sk(self.pcmm_context.h, _addr(mlwe_sk.sx_device), _addr(rlwe_sk.sx_device)), "pcmm_convert_mlwe_sk")
+
+    def addRepakcingKey(self, mlwe_sk, rlwe_sk):
+        """PCMM_Scheme.cuh:126-224; the keys stay in self.repackingKeys (one device buffer, key i at i*2*m*N words)."""
+        pc = self.pcmm_context
+        if self.repackingKeys is not None:
+            return                                                           # "repacking keys already generated!" (:152-155)
+        N = pc.context.N
+        m = pc.ringpack_p_count + pc.ringpack_q_count - 1
+        keys = DeviceBuffer(8 * N * m * 2 * pc.mlwe_rank)
+        scratch = DeviceBuffer(8 * N * (m + 1))
+        _check(self.L_.pcmm_add_repacking_key(pc.h, keys.ptr, _addr(mlwe_sk.sx_device), _addr(rlwe_sk.sx_device), self.key, self.nonce,
+                                              scratch.ptr), "pcmm_add_repacking_key")
+        self.nonce += pc.mlwe_rank
+        scratch.free()
+        self.repackingKeys = keys
+
+    def mlweDecrypt(self, mlwe_cipher, mlwe_sk, mlwe_plain, l):
+        """PCMM_Scheme.cuh:557-576; mlwe_cipher: device buffer of one sample."""
+        _check(self.L_.pcmm_mlwe_decrypt(self.pcmm_context.h, _addr(mlwe_plain.mx_device), _addr(mlwe_cipher), _addr(mlwe_sk.sx_device), l),
+               "pcmm_mlwe_decrypt")
+        mlwe_plain.l = l
 
     @staticmethod
     def _ptrs(bufs):

@@ -226,6 +226,27 @@ int pcmm_rlwe_decompose_ntt(pcmm_ctx* h, uint64_t* rlwe, uint64_t* const* mlwe_p
  * The reference's embedding is only meaningful for one special prime and two ring-pack moduli; other contexts get CKKS_E_INVALID. */
 int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* const* mlwe_ptrs_host, int mlwe_num,
                    const uint64_t* repacking_keys, uint64_t* embed_scratch, uint64_t* mult_scratch);
+/* PCMM_Scheme::convertMLWESKfromRLWESK (PCMM_Scheme.cuh:23-48; ringDown_kernel, ringSwitch.cuh:7-19): mlwe_sk =
+ * [p_count + q_count moduli][rank][N1], small polynomial i = the coefficients i + n*rank of the RLWE secret, NTT domain (size N1).
+ * rlwe_sk (K+L+1 limbs, NTT domain) is transformed back and forth in place as in the reference and ends unchanged.
+ * The two copies of the reference are kept as they are: RLWE limbs 0.. to key moduli 0.., then RLWE limbs K.. to key moduli
+ * p_count.. (so modulus slot 0 holds the secret modulo the FIRST special prime; nothing reads it).  Needs N1 >= 256. */
+int pcmm_convert_mlwe_sk(pcmm_ctx* h, uint64_t* mlwe_sk, uint64_t* rlwe_sk);
+/* PCMM_Scheme::addRepakcingKey (PCMM_Scheme.cuh:126-224): rank keys over the context primes [last p_count special primes |
+ * q_0 .. q_{q_count-2}], key i at keys + i*2*m*N = [a: m limbs | b: m limbs], m = p_count + q_count - 1, NTT domain,
+ * b = -a*s + p0 * iota(s_i) + e - the layout pcmm_mlwe_pack reads.  Randomness: key i draws 4*N bytes (e) then 8*N*m bytes (a)
+ * from the Salsa20 stream of (key32, nonce + i).  scratch: (m + 1)*N words.  mlwe_sk is taken to the coefficient domain and
+ * back on ALL its moduli (the reference brings back all but the last, :182).  b starts from zero (the reference writes the
+ * embedded secret into fresh cudaMalloc memory).  Needs N1 >= 256. */
+int pcmm_add_repacking_key(pcmm_ctx* h, uint64_t* keys, uint64_t* mlwe_sk, const uint64_t* rlwe_sk, const uint8_t* key32, uint64_t nonce,
+                           uint64_t* scratch);
+/* PCMM_Scheme::mlweDecrypt (PCMM_Scheme.cuh:531-576): plain[mod][n] = b + sum_i a_i * s_i for moduli 0..l of the sample, in the
+ * size-N1 NTT domain (where the reference leaves it); the sample is transformed in place and back.  Any rank (the reference
+ * instantiates 256 and 512).  Needs N1 >= 256. */
+int pcmm_mlwe_decrypt(pcmm_ctx* h, uint64_t* plain, uint64_t* mlwe_cipher, const uint64_t* mlwe_sk, int l);
+/* PCMM_Context::decodeCoeffs (PCMM_Context.cuh:149-178): inverse transform of a copy (scratch: (l+1)*N1 words), then the centred
+ * residue modulo the first ring-pack modulus divided by scaler; vals: N1 device doubles. */
+int pcmm_decode_coeffs(pcmm_ctx* h, double* vals, const uint64_t* plain, uint64_t* scratch, long long scaler, int l);
 /* PCMM_Scheme::PPMM device part (PPMM_kernel.cuh:93-252, launch :294-340):
  * out[m][mod][c] = fused-rescaled sum_n trunc(W[m][n]*scaler) * mlwe[n][mod][c] mod q_mod, for mod_num ring-pack
  * primes (the reference fixes mod_num = 2), c < (rank+1)*N1.  W: device fp32 row-major [M][Kin];

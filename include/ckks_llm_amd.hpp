@@ -416,6 +416,32 @@ private:
     }
 };
 
+// MLWESecretKey (pcmm/MLWESecretKey.cuh:6-52): [L+1 moduli][k polynomials][N1]
+class MLWESecretKey {
+public:
+    uint64_tt* sx_device = nullptr;
+    int N1 = 0, L = 0, k = 0;
+    MLWESecretKey(int N1, int L, int k) : N1(N1), L(L), k(k) { sx_device = device_alloc_words((size_t)N1 * k * (L + 1)); }
+    MLWESecretKey(const MLWESecretKey&) = delete;
+    MLWESecretKey& operator=(const MLWESecretKey&) = delete;
+    virtual ~MLWESecretKey() { device_release(sx_device); }
+};
+
+// MLWEPlaintext (pcmm/MLWEPlaintext.cuh:7-60): [L+1 moduli][N1]
+class MLWEPlaintext {
+public:
+    uint64_tt* mx_device = nullptr;
+    int N1 = 0, L = 0, l = 0;
+    long double scale = 0;
+    MLWEPlaintext(int N1, int L, int l, long double scale) : N1(N1), L(L), l(l), scale(scale) {
+        if (l > L) std::cout << "new MLWEPlaintext error!" << std::endl;
+        mx_device = device_alloc_words((size_t)N1 * (L + 1));
+    }
+    MLWEPlaintext(const MLWEPlaintext&) = delete;
+    MLWEPlaintext& operator=(const MLWEPlaintext&) = delete;
+    virtual ~MLWEPlaintext() { device_release(mx_device); }
+};
+
 // PCMM_Context (pcmm/PCMM_Context.h:14-90)
 class PCMM_Context {
 public:
@@ -446,6 +472,13 @@ public:
     void FromNTTInplace(uint64_tt* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
         check(pcmm_ntt_inv(handle, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "PCMM_Context::FromNTTInplace");
     }
+    // PCMM_Context::decodeCoeffs (PCMM_Context.cuh:165-178); vals: N1 device doubles
+    void decodeCoeffs(MLWEPlaintext& msg, double* vals) {
+        uint64_tt* scratch = device_alloc_words((size_t)N1 * (msg.l + 1));
+        int rc = pcmm_decode_coeffs(handle, vals, msg.mx_device, scratch, (long long)msg.scale, msg.l);
+        device_release(scratch);
+        check(rc, "decodeCoeffs");
+    }
 };
 
 // The rlweCipherDecompose / PPMM members of PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48).
@@ -459,6 +492,7 @@ public:
     uint64_tt* embeded_mlwe_buffer = nullptr;  // (rank+1) big polynomials over [p0 | q0] (PCMM_Scheme.cuh:12)
     uint64_tt* mult_key_output = nullptr;      // 4 limbs; the reference borrows scheme.modUp_TtoQj_buffer (PCMM_Scheme.cuh:394)
     uint64_tt* repackingKeys = nullptr;        // rank keys [a | b] over [p0 | q0], NTT domain, one buffer (PCMM_Scheme.cuh:166-176)
+    bool own_keys = false;
 
     PCMM_Scheme(PCMM_Context& pcmm_context, Scheme_23& scheme) : pcmm_context(pcmm_context), scheme(scheme) {
         const size_t N = (size_t)scheme.context.N;
@@ -470,10 +504,37 @@ public:
         device_release(ppmm_output);
         device_release(embeded_mlwe_buffer);
         device_release(mult_key_output);
+        if (own_keys) device_release(repackingKeys);
+    }
+
+    // PCMM_Scheme::convertMLWESKfromRLWESK (PCMM_Scheme.cuh:23-48)
+    void convertMLWESKfromRLWESK(MLWESecretKey& mlwe_sk, SecretKey& rlwe_sk) {
+        check(pcmm_convert_mlwe_sk(pcmm_context.handle, mlwe_sk.sx_device, rlwe_sk.sx_device), "convertMLWESKfromRLWESK");
+    }
+    // PCMM_Scheme::addRepakcingKey (PCMM_Scheme.cuh:126-224): the keys go to repackingKeys (owned), key i at i*2*m*N words;
+    // key i draws from the context's stream under the nonce rng_nonce + 1 + i
+    void addRepakcingKey(MLWESecretKey& mlwe_sk, SecretKey& rlwe_sk) {
+        if (repackingKeys) { std::cout << "repacking keys already generated!" << std::endl; return; }      // :152-155
+        Context_23& c = scheme.context;
+        const size_t N = (size_t)c.N, m = (size_t)pcmm_context.ringpack_pq_count - 1;
+        uint64_tt* keys = device_alloc_words(N * m * 2 * pcmm_context.mlwe_rank);
+        uint64_tt* scratch = device_alloc_words(N * (m + 1));
+        int rc = pcmm_add_repacking_key(pcmm_context.handle, keys, mlwe_sk.sx_device, rlwe_sk.sx_device, c.rng_key, c.rng_nonce + 1, scratch);
+        c.rng_nonce += (uint64_t)pcmm_context.mlwe_rank;
+        device_release(scratch);
+        if (rc != CKKS_OK) device_release(keys);
+        check(rc, "addRepakcingKey");
+        repackingKeys = keys;
+        own_keys = true;
+    }
+    // PCMM_Scheme::mlweDecrypt (PCMM_Scheme.cuh:557-576)
+    void mlweDecrypt(MLWECiphertext& mlwe_cipher, MLWESecretKey& mlwe_sk, MLWEPlaintext& mlwe_plain) {
+        mlwe_plain.l = mlwe_cipher.l;
+        check(pcmm_mlwe_decrypt(pcmm_context.handle, mlwe_plain.mx_device, mlwe_cipher.cipher_device, mlwe_sk.sx_device, mlwe_cipher.l), "mlweDecrypt");
     }
 
     // PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425): k MLWE samples -> 1 RLWE ciphertext with the repacking keys
-    // (the reference generates them in addRepakcingKey from the secret keys; here the caller installs them in repackingKeys).
+    // (from addRepakcingKey, or installed by the caller in repackingKeys).
     void mlweCipherPacking(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,
                            uint64_tt offset) {
         if (!repackingKeys) throw std::invalid_argument("mlweCipherPacking: repacking keys not exists");

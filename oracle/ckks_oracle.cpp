@@ -1236,6 +1236,101 @@ int orc_conjugate_23(const orc_ctx* c, u64* out, const u64* cipher, const u64* c
     return 0;
 }
 
+// ------------------------------------------------------------------------------------------------
+// MLWE secret key, repacking keys, MLWE decryption (the key side of the ring-packed PCMM)
+// ------------------------------------------------------------------------------------------------
+// PCMM_Scheme::convertMLWESKfromRLWESK (PCMM_Scheme.cuh:23-48) with ringDown_kernel (ringSwitch.cuh:7-19): the RLWE secret
+// (K+L+1 limbs, NTT domain, left unchanged) goes to the coefficient domain; small polynomial i takes the big coefficients
+// i + n*rank (n < N1).  The first launch copies RLWE limbs 0..nq-1 to key moduli 0..nq-1, the second RLWE limbs K..K+nq-1 to key
+// moduli np..np+nq-1 (overwriting where they overlap), exactly as the reference's two launches do; then every modulus is
+// transformed (size N1).  mlwe_sk: [np+nq moduli][rank][N1].
+int orc_pcmm_convert_mlwe_sk(const orc_pcmm* h, u64* mlwe_sk, const u64* rlwe_sk) {
+    const orc_ctx* c = h->ctx; const long N = c->N; const int N1 = h->N1, k = h->rank, np = h->np, nq = h->nq, K = c->K, KL = c->K + c->L + 1;
+    if ((long)N1 * k != N || nq > KL || K + nq > KL) return -1;
+    std::vector<u64> s(rlwe_sk, rlwe_sk + (size_t)KL * N);
+    orc_ntt_inv(c, s.data(), 0, 0, 1, KL, KL);
+    for (int pass = 0; pass < 2; pass++) {
+        const u64* big = s.data() + (pass ? (size_t)K * N : 0);
+        u64* small = mlwe_sk + (pass ? (size_t)np * N1 * k : 0);
+        for (int im = 0; im < nq; im++)
+            for (long g = 0; g < N; g++) small[(size_t)im * N + g] = big[(size_t)im * N + g / N1 + (g % N1) * k];
+    }
+    return orc_pcmm_ntt(h, mlwe_sk, k, np + nq, 0, 1, 0);
+}
+
+// PCMM_Scheme::addRepakcingKey (PCMM_Scheme.cuh:126-224) with EmbedMLWESKtoRLWESK (:126-149): key i over the context primes
+// [last np special primes | q_0 .. q_{nq-2}] is (a, -a*s + p0 * iota(s_i) + e), iota placing coefficient n of the small secret at
+// n*rank; layout key i at keys + i*2*mod_num*N = [a: mod_num limbs | b: mod_num limbs], mod_num = np+nq-1, NTT domain.
+// random: per key 4*N bytes (e) then 8*N*mod_num bytes (a), keys one after the other.  mlwe_sk (NTT domain) is not modified: the
+// reference transforms it back on np+nq-1 of its np+nq moduli only (:182), which leaves the last one in the coefficient domain.
+// b starts from zero here (the reference writes the embedded secret into fresh cudaMalloc memory).
+int orc_pcmm_add_repacking_key(const orc_pcmm* h, u64* keys, const u64* mlwe_sk, const u64* rlwe_sk, const uint8_t* random) {
+    const orc_ctx* c = h->ctx; const long N = c->N; const int N1 = h->N1, k = h->rank, np = h->np, nq = h->nq, K = c->K;
+    const int mod_num = np + nq - 1, first = K - np;
+    if ((long)N1 * k != N || K < np || (nq - 1) / np != 1) return -1;                       // "dnum not supported!" (:178-180)
+    for (int i = 0; i < mod_num; i++) if (c->pqt[first + i] != h->pq[i]) return -1;
+    std::vector<u64> sk(mlwe_sk, mlwe_sk + (size_t)(np + nq) * N);
+    orc_pcmm_ntt(h, sk.data(), k, np + nq, 0, 1, 1);
+    const u64 p0 = h->pq[0];
+    const size_t per_key = (size_t)4 * N + (size_t)8 * N * mod_num;
+    std::vector<u64> ex((size_t)mod_num * N), tmp((size_t)mod_num * N);
+    for (int i = 0; i < k; i++) {
+        u64* ax = keys + (size_t)i * 2 * mod_num * N;
+        u64* bx = ax + (size_t)mod_num * N;
+        std::fill(bx, bx + (size_t)mod_num * N, 0);
+        for (int im = 0; im < nq - 1; im++) {
+            const u64 qi = h->pq[np + im];
+            for (int n = 0; n < N1; n++) {
+                const u64 v = sk[(size_t)(np + im) * N + (size_t)i * N1 + n];
+                bx[(size_t)(np + im) * N + (size_t)n * k] = orc_barrett128((u64)(((u128)v * p0) >> 64), v * p0, qi, h->mu_hi[np + im], h->mu_lo[np + im]);
+            }
+        }
+        const uint8_t* r = random + per_key * i;
+        orc_sample_gaussian(c, r, ex.data(), 0, first, mod_num);
+        orc_sample_uniform(c, r + 4 * N, ax, 0, first, mod_num);
+        orc_poly_op(c, 1, bx, bx, ex.data(), 0, 0, 0, first, mod_num);
+        orc_ntt_fwd(c, bx, 0, first, 1, mod_num, mod_num);
+        orc_poly_op(c, 0, tmp.data(), rlwe_sk, ax, 0, first, 0, first, mod_num);
+        orc_poly_op(c, 2, bx, bx, tmp.data(), 0, 0, 0, first, mod_num);
+    }
+    return 0;
+}
+
+// PCMM_Scheme::mlweDecrypt (PCMM_Scheme.cuh:531-576): plain[mod][n] = b + sum_i a_i * s_i in the size-N1 NTT domain (128-bit
+// accumulation, one Barrett reduction), for moduli 0..l of the ciphertext = ring-pack primes np..np+l; the plaintext stays in
+// the NTT domain, the ciphertext (coefficient domain) is left unchanged.  mlwe_sk as convertMLWESKfromRLWESK leaves it.
+int orc_pcmm_mlwe_decrypt(const orc_pcmm* h, u64* plain, const u64* cipher, const u64* mlwe_sk, int l) {
+    const int N1 = h->N1, k = h->rank, np = h->np, nq = h->nq;
+    if (l < 0 || l + 1 > nq) return -1;
+    std::vector<u64> ct(cipher, cipher + (size_t)(l + 1) * (k + 1) * N1);
+    if (orc_pcmm_ntt(h, ct.data(), k + 1, l + 1, np, 1, 0)) return -1;
+    for (int im = 0; im <= l; im++) {
+        const u64 q = h->pq[np + im], mh = h->mu_hi[np + im], ml = h->mu_lo[np + im];
+        const u64* a = ct.data() + (size_t)im * (k + 1) * N1;
+        const u64* s = mlwe_sk + (size_t)(np + im) * k * N1;
+        for (int n = 0; n < N1; n++) {
+            u128 acc = a[(size_t)k * N1 + n];
+            for (int i = 0; i < k; i++) acc += (u128)a[(size_t)i * N1 + n] * s[(size_t)i * N1 + n];
+            plain[(size_t)im * N1 + n] = orc_barrett128((u64)(acc >> 64), (u64)acc, q, mh, ml);
+        }
+    }
+    return 0;
+}
+// PCMM_Context::decodeCoeffs (PCMM_Context.cuh:149-178): inverse transform of moduli 0..l, then the centred residue modulo the first
+// ring-pack modulus divided by the scale; N1 doubles
+int orc_pcmm_decode_coeffs(const orc_pcmm* h, double* vals, const u64* plain, long long scaler, int l) {
+    const int N1 = h->N1, np = h->np;
+    if (l < 0 || l + 1 > h->nq) return -1;
+    std::vector<u64> buf(plain, plain + (size_t)(l + 1) * N1);
+    if (orc_pcmm_ntt(h, buf.data(), 1, l + 1, np, 1, 1)) return -1;
+    const u64 mod = h->pq[np], mod2 = mod >> 1;
+    for (int n = 0; n < N1; n++) {
+        const long mi = (long)buf[n];
+        vals[n] = (u64)mi <= mod2 ? (double)mi / scaler : ((double)mi - (double)mod) / scaler;
+    }
+    return 0;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

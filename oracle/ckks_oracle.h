@@ -32,6 +32,9 @@
  *                                  algebra (a*s + b = m + small noise)          (tests/test_oracle_scheme.py)
  *   coefficient encode / decode    Python big-integer CRT and exact rationals   (tests/test_oracle_scheme.py)
  *   NTT-domain automorphisms       coefficient-domain substitution X -> X^g     (tests/test_oracle_keys.py)
+ *   MLWE secret, repacking keys,   s_i[n] = s[i + n*rank]; a*s + b = p0*iota(s_i) + small e; MLWE decryption of the
+ *   MLWE decryption                gather = the RLWE message at the gathered positions; whole pipeline decrypts to
+ *                                  W times the message with generated keys     (tests/test_oracle_pcmm.py)
  *   switching keys, mult / rotate  decrypt identities: product of messages,
  *   / conjugate                    m(X^(5^r)), m(X^-1), within a noise bound   (tests/test_oracle_keys.py)
  */
@@ -149,6 +152,12 @@ int orc_keygen_switch_23(const orc_ctx*, uint64_t* swk, const uint64_t* s_to, co
 int orc_mult_23(const orc_ctx*, uint64_t* out, const uint64_t* c1, const uint64_t* c2, const uint64_t* rlk, int l);
 int orc_rotate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* rotkey, long rot, int l);
 int orc_conjugate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* conjkey, int l);
+
+/* ---- MLWE secret key, repacking keys, MLWE decryption ---- */
+int orc_pcmm_convert_mlwe_sk(const orc_pcmm*, uint64_t* mlwe_sk, const uint64_t* rlwe_sk);
+int orc_pcmm_add_repacking_key(const orc_pcmm*, uint64_t* keys, const uint64_t* mlwe_sk, const uint64_t* rlwe_sk, const uint8_t* random);
+int orc_pcmm_mlwe_decrypt(const orc_pcmm*, uint64_t* plain, const uint64_t* cipher, const uint64_t* mlwe_sk, int l);
+int orc_pcmm_decode_coeffs(const orc_pcmm*, double* vals, const uint64_t* plain, long long scaler, int l);
 
 int orc_max_threads(void);
 

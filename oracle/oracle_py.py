@@ -95,6 +95,9 @@ def lib():
             "orc_keygen_switch_23": (i, [vp, P64, P64, P64, P8, P8]),
             "orc_mult_23": (i, [vp, P64, P64, P64, P64, i]), "orc_rotate_23": (i, [vp, P64, P64, P64, l, i]),
             "orc_conjugate_23": (i, [vp, P64, P64, P64, i]),
+            "orc_pcmm_convert_mlwe_sk": (i, [vp, P64, P64]), "orc_pcmm_add_repacking_key": (i, [vp, P64, P64, P64, P8]),
+            "orc_pcmm_mlwe_decrypt": (i, [vp, P64, P64, P64, i]),
+            "orc_pcmm_decode_coeffs": (i, [vp, C.POINTER(C.c_double), P64, C.c_longlong, i]),
             "orc_max_threads": (i, []),
         }
         for name, (res, args) in sig.items():
@@ -319,6 +322,20 @@ class OraclePCMM:
         rc = self.L_.orc_mlwe_pack(self.h, _ptr(rlwe_out), self._ptrs(mlwe), len(mlwe), _ptr(keys))
         if rc:
             raise ValueError("orc_mlwe_pack: %d" % rc)
+
+    def convertMLWESKfromRLWESK(self, mlwe_sk, rlwe_sk):
+        self.ctx._ck(self.L_.orc_pcmm_convert_mlwe_sk(self.h, _ptr(mlwe_sk), _ptr(rlwe_sk)))
+
+    def addRepakcingKey(self, keys, mlwe_sk, rlwe_sk, random):
+        self.ctx._ck(self.L_.orc_pcmm_add_repacking_key(self.h, _ptr(keys), _ptr(mlwe_sk), _ptr(rlwe_sk), _bytes(random)))
+
+    def mlweDecrypt(self, plain, cipher, mlwe_sk, l):
+        self.ctx._ck(self.L_.orc_pcmm_mlwe_decrypt(self.h, _ptr(plain), _ptr(cipher), _ptr(mlwe_sk), l))
+
+    def decodeCoeffs(self, plain, scaler, l):
+        out = np.zeros(self.N1, dtype=np.float64)
+        self.ctx._ck(self.L_.orc_pcmm_decode_coeffs(self.h, out.ctypes.data_as(C.POINTER(C.c_double)), _ptr(plain), int(scaler), l))
+        return out
 
     def PPMM(self, W, mlwe, out, M, Kin, mod_num, scaler, col_begin=0, col_count=None):
         C_ = (self.rank + 1) * self.N1

@@ -220,3 +220,111 @@ def test_small_ring_ntt_is_the_negacyclic_transform():
     from tests.helpers import bitrev
     for i in (0, 1, 7, 100, 255):
         assert int(mono[bitrev(i, 8)]) == pow(psi, 5 * (2 * i + 1), q)
+
+
+def test_mlwe_secret_repacking_keys_and_mlwe_decryption_with_generated_keys():
+    """convertMLWESKfromRLWESK, addRepakcingKey, mlweDecrypt and decodeCoeffs (PCMM_Scheme.cuh:23-48, 126-224, 531-576; PCMM_Context.cuh:149-178)
+    with keys from the oracle's own generators: the small secrets are the strided coefficients of the big one; every repacking key satisfies
+    a*s + b = p0*iota(s_i) + e with one small e for both primes; an MLWE sample of the gather decrypts to exactly the RLWE decryption at the
+    gathered positions; and gather -> PPMM -> packing with these keys decrypts to W times the message."""
+    from tests.params import CFG3_P
+    logN, N, N1, k, h = 8, 256, 16, 16, 32
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    pq = [P0, Q0, Q1]
+    ctx = O.OracleContext(logN, [P0], [Q0, Q1])
+    pc = O.OraclePCMM(ctx, N1, k, [P0], [Q0, Q1])
+    per_key = 4 * N + 8 * N * 2
+    stream = O.salsa20_stream(5 * h + 64 + 8 * N * 2 + 4 * N + 9 * N + k * per_key, bytes(range(32)), 77)
+    sx = np.zeros((3, N), dtype=np.uint64)
+    ctx.keygen_secret(sx.reshape(-1), np.ascontiguousarray(stream[:5 * h]), h)
+    sc = sx.copy()
+    ctx.FromNTTInplace(sc.reshape(-1), 0, 0, 1, 3, 3)
+    s = [int(v) if v <= 1 else -1 for v in sc[0]]
+    # ---- MLWE secret ----
+    msk = np.zeros((3, k, N1), dtype=np.uint64)
+    pc.convertMLWESKfromRLWESK(msk.reshape(-1), sx.reshape(-1))
+    small = msk.copy()
+    pc.FromNTTInplace(small.reshape(-1), k, 3, 0, 0, 1)
+    for j, q in enumerate(pq):
+        for i in range(k):
+            assert [int(v) for v in small[j, i]] == [s[i + n * k] % q for n in range(N1)]
+    # ---- repacking keys ----
+    o = 5 * h + 64
+    pk = np.zeros((2, 2, N), dtype=np.uint64)
+    ctx.keygen_public(pk.reshape(-1), sx.reshape(-1), np.ascontiguousarray(stream[o:o + 8 * N * 2]), np.ascontiguousarray(stream[o + 8 * N * 2:o + 8 * N * 2 + 4 * N]))
+    o += 8 * N * 2 + 4 * N
+    renc = np.ascontiguousarray(stream[o:o + 9 * N])
+    o += 9 * N
+    keys = np.zeros((k, 2, 2, N), dtype=np.uint64)
+    msk_before = msk.copy()
+    pc.addRepakcingKey(keys.reshape(-1), msk.reshape(-1), sx.reshape(-1), np.ascontiguousarray(stream[o:o + k * per_key]))
+    assert np.array_equal(msk, msk_before)
+    kc = keys.copy()
+    for i in range(k):
+        for y in range(2):
+            ctx.FromNTTInplace(kc[i, y].reshape(-1), 0, 0, 1, 2, 2)
+    seen = set()
+    for i in (0, 5, k - 1):
+        es = []
+        for j, q in enumerate((P0, Q0)):
+            a_s = negacyclic_mul([int(v) for v in kc[i, 0, j]], [v % q for v in s], q)
+            iota = [0] * N
+            for n in range(N1):
+                iota[n * k] = s[i + n * k]
+            e = [(x + int(b) - P0 * t) % q for x, b, t in zip(a_s, kc[i, 1, j], iota)]
+            es.append([v - q if v > q // 2 else v for v in e])
+        assert es[0] == es[1] and max(abs(v) for v in es[0]) <= 19 and any(es[0])
+        seen.add(tuple(es[0]))
+    assert len(seen) == 3                                                   # every key has its own noise
+    # ---- encrypt, gather, MLWE decryption = RLWE decryption at the gathered positions ----
+    rng = np.random.default_rng(3)
+    mu = [int(v) for v in rng.integers(-(1 << 32), 1 << 32, N)]
+    mx = np.zeros((2, N), dtype=np.uint64)
+    for j, q in enumerate((Q0, Q1)):
+        mx[j] = [v % q for v in mu]
+    ctx.ToNTTInplace(mx.reshape(-1), 0, 1, 1, 2, 2)
+    ct = np.zeros((2, 2, N), dtype=np.uint64)
+    ctx.encrypt(ct.reshape(-1), mx.reshape(-1), pk.reshape(-1), renc, 1)
+    dec = np.zeros((2, N), dtype=np.uint64)
+    ctx.decrypt(dec.reshape(-1), ct.reshape(-1), sx.reshape(-1), 1)
+    ctx.FromNTTInplace(dec.reshape(-1), 0, 1, 1, 2, 2)
+    ctc = ct.copy()
+    ctx.FromNTTInplace(ctc.reshape(-1), 0, 1, 2, 2, 2)
+    mlwe_num = 4
+    gap = k // mlwe_num
+    mlwe = [np.zeros((2, k + 1, N1), dtype=np.uint64) for _ in range(mlwe_num)]
+    pc.rlweCipherDecompose(ctc.reshape(-1), [m.reshape(-1) for m in mlwe], 1)
+    for j in range(mlwe_num):
+        before = mlwe[j].copy()
+        plain = np.zeros((2, N1), dtype=np.uint64)
+        pc.mlweDecrypt(plain.reshape(-1), mlwe[j].reshape(-1), msk.reshape(-1), 1)
+        assert np.array_equal(mlwe[j], before)
+        vals = pc.decodeCoeffs(plain.reshape(-1), 1 << 10, 1)
+        pcoef = plain.copy()
+        pc.FromNTTInplace(pcoef.reshape(-1), 1, 2, 0, 1, 1)
+        for im in range(2):
+            assert [int(v) for v in pcoef[im]] == [int(dec[im, j * gap + n * k]) for n in range(N1)]
+        want = [(int(v) if v <= Q0 // 2 else int(v) - Q0) / 1024.0 for v in pcoef[0]]
+        assert list(vals) == want
+    # ---- gather -> PPMM -> packing with the generated keys decrypts to W * mu ----
+    M = Kin = mlwe_num
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    scaler = float(1 << 26)
+    C = (k + 1) * N1
+    out = np.zeros((M, 2, C), dtype=np.uint64)
+    pc.PPMM(W, [m.reshape(-1) for m in mlwe], out.reshape(-1), M, Kin, 2, scaler)
+    rows = [np.ascontiguousarray(out[m, 0]) for m in range(M)]
+    res = np.zeros((2, 2, N), dtype=np.uint64)
+    pc.mlweCipherPacking(res.reshape(-1), rows, keys.reshape(-1))
+    d2 = np.zeros((2, N), dtype=np.uint64)
+    ctx.decrypt(d2.reshape(-1), res.reshape(-1), sx.reshape(-1), 0)
+    ctx.FromNTTInplace(d2.reshape(-1), 0, 1, 1, 1, 2)
+    got = [int(v) if v <= Q0 // 2 else int(v) - Q0 for v in d2[0]]
+    A = [[int(np.float64(W[m, n]) * scaler) for n in range(Kin)] for m in range(M)]
+    worst = biggest = 0
+    for g in range(N1):
+        for m in range(M):
+            want = sum(A[m][n] * mu[n * gap + g * k] for n in range(Kin)) // Q1
+            worst = max(worst, abs(got[g * k + m * gap] - want))
+            biggest = max(biggest, abs(want))
+    assert biggest > 1 << 16 and worst <= N, (worst, biggest)
