@@ -42,7 +42,7 @@ def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3):
     DW, DC, path = sch.pcmm_context.info("last_DW"), sch.pcmm_context.info("last_DC"), sch.pcmm_context.info("last_path")
     word_macs = float(M) * Kin * C * L
     macs = word_macs * DW * DC
-    res = {"workload": "configs[3]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (M, Kin, N1, L, C),
+    res = {"workload": "configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (3 if M == 768 else 4, M, Kin, N1, L, C),
            "ms": round(best, 3), "word_MAC_per_s": round(word_macs / (best * 1e-3), 1), "int8_MAC_per_s": round(macs / (best * 1e-3), 1),
            "D_w": DW, "D_c": DC, "kernel": "int8 MFMA" if path == 1 else "generic u128",
            "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
@@ -144,4 +144,5 @@ def bench_decompose(P, N1=128, L1=12, reps=5):
 
 
 def run(P):
-    return {"ppmm": bench_ppmm(P), "keyswitch": bench_keyswitch(P), "decompose": bench_decompose(P), "packing": bench_packing(P)}
+    return {"ppmm": bench_ppmm(P), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "keyswitch": bench_keyswitch(P),
+            "decompose": bench_decompose(P), "packing": bench_packing(P)}

@@ -130,14 +130,16 @@ __global__ __launch_bounds__(256) void quantise_kernel(const float* W, long long
         if (m) atomicMax(absmax, m);
     }
 }
-// digit d of A (balanced, in [-128, 127]): byte d of (A + 0x80..80) xor 0x80
+// digit d of A (balanced, in [-128, 127]): byte d of (A + 0x80..80) xor 0x80.  The planes are written in the order the MFMA kernel
+// stages them: [digit][16-row group][64-deep K step] slabs of 1 KiB, inside a slab [16-byte k chunk][row][16 k].
 __global__ __launch_bounds__(256) void digits_kernel(const long long* A, int8_t* dig, int M, int Kin, int Mpad, int Kpad, int DW) {
     long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= (long)Mpad * Kpad) return;
     int m = (int)(i / Kpad), n = (int)(i % Kpad);
     unsigned long long biased = 0x8080808080808080ull;
     if (m < M && n < Kin) biased += (unsigned long long)A[(long)m * Kin + n];
-    for (int d = 0; d < DW; d++) dig[(long)d * Mpad * Kpad + i] = (int8_t)(((biased >> (8 * d)) & 0xff) ^ 0x80);
+    const long pos = ((long)(m >> 4) * (Kpad >> 6) + (n >> 6)) * 1024 + ((n & 63) >> 4) * 256 + (m & 15) * 16 + (n & 15);
+    for (int d = 0; d < DW; d++) dig[(long)d * Mpad * Kpad + pos] = (int8_t)(((biased >> (8 * d)) & 0xff) ^ 0x80);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -477,7 +479,6 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
     a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
     a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np;
-
     // digit counts: DW digits cover |A| < 2^(8*DW-1); DC digits cover residues < 2^(8*DC-1)
     int DW = 1; while (DW < 8 && absmax >= (1ull << (8 * DW - 1))) DW++;
     int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;

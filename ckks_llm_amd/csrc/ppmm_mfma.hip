@@ -18,7 +18,7 @@ namespace ckks {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int MT = 128, CT = 64, KS = 64;        // workgroup tile and K step
+constexpr int CT = 64, KS = 64;                  // column tile and K step; the row tile is 16 rows per wave of the workgroup
 constexpr int DCMAX = 5;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -45,7 +45,8 @@ __device__ __forceinline__ double balance_f64(double x, double q, double qinv) {
 
 // ------------------------------------------------------------------------------------------------------------
 // Pass 1: residue digit planes.  Every residue is read ONCE, split into DC balanced base-256 digits and written in the
-// order the MFMA kernel stages it:  Bdig[prime][K step][digit][column][64 k]  (k contiguous, 64 B per column).
+// order the MFMA kernel stages it:  Bdig[prime][K step][64-column tile][digit][16-column slab] slabs of 1 KiB, inside a slab
+// [16-byte k chunk][column][16 k].
 // One workgroup (256 lanes) handles 64 k x 64 columns: coalesced 512 B row reads, a byte transpose in registers,
 // LDS to gather the 4 waves' quarter rows, then 16 B per lane coalesced writes.
 // ------------------------------------------------------------------------------------------------------------
@@ -81,8 +82,8 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
     int8_t* dst = bdig + (((long)im * gridDim.y + ks) * gridDim.x + blockIdx.x) * (long)(DC * CT * KS);
 #pragma unroll
     for (int t = 0; t < DC * CT * KS / (256 * 16); t++) {
-        const int flat = (t * 256 + tid) * 16;                  // byte offset in [digit][column][64]
-        const int jj = flat / (CT * KS), col = (flat / KS) % CT, chunk = (flat % KS) / 16;
+        const int flat = (t * 256 + tid) * 16;                  // byte offset in [digit][16-column slab][16-byte k chunk][column][16]
+        const int jj = flat / (CT * KS), col = ((flat >> 10) & 3) * 16 + ((flat >> 4) & 15), chunk = (flat >> 8) & 3;
         *reinterpret_cast<uint4*>(dst + flat) = *reinterpret_cast<const uint4*>(&tile[jj][col][16 * (chunk ^ ((col >> 1) & 3))]);
     }
 }
@@ -98,23 +99,34 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
 // ksteps is a multiple of 3), so that the compiler can tell that the asynchronous writes of a step never alias the
 // operands its MFMAs read; otherwise it waits for the loads before the first LDS read and the overlap is lost.
 // ------------------------------------------------------------------------------------------------------------
-constexpr int NWAVES = 8;
-
-template <int DW>
-__global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_tiles) {
-    constexpr int DC = DCMAX, ND = DW + DC - 1;
-    constexpr int A_SLABS = DW * 8, B_SLABS = DC * 4;            // 1 KiB slabs per step
+// The kernel is written for NWAVES waves (16 rows of the tile each) and a ring of RING slots; the launcher instantiates
+//   NWAVES = 8, RING = 3: 128 x 64 tile, one workgroup per CU (135 KiB of LDS), loads issued two steps ahead.
+// The other shape that fits the LDS (NWAVES = 4, RING = 2: 64 x 64 tile, 64 KiB, two workgroups per CU that drift out of phase)
+// was measured and is no faster (its single step of load lead time costs what the overlap of the two workgroups gains).
+template <int DW, int NWAVES, int RING>
+__global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_block) {
+    constexpr int DC = DCMAX, ND = DW + DC - 1, MT = 16 * NWAVES;
+    constexpr int A_SLABS = DW * (MT / 16), B_SLABS = DC * 4;    // 1 KiB slabs per step
     constexpr int A_PER_WAVE = (A_SLABS + NWAVES - 1) / NWAVES, B_PER_WAVE = (B_SLABS + NWAVES - 1) / NWAVES;
+    constexpr int AHEAD = RING - 1;                              // how many steps ahead of its use a slot is refilled
+    static_assert(RING == 2 || RING == 3, "ring depth");
     __shared__ __align__(16) int8_t lds_a0[DW][MT][KS];
     __shared__ __align__(16) int8_t lds_a1[DW][MT][KS];
-    __shared__ __align__(16) int8_t lds_a2[DW][MT][KS];
+    __shared__ __align__(16) int8_t lds_a2[RING == 3 ? DW : 1][RING == 3 ? MT : 1][KS];
     __shared__ __align__(16) int8_t lds_b0[DC][CT][KS];
     __shared__ __align__(16) int8_t lds_b1[DC][CT][KS];
-    __shared__ __align__(16) int8_t lds_b2[DC][CT][KS];
+    __shared__ __align__(16) int8_t lds_b2[RING == 3 ? DC : 1][RING == 3 ? CT : 1][KS];
 
-    // XCD-aware tile numbering: ids congruent mod 8 share an XCD; consecutive ones there share the column panel
+    // XCD-aware tile numbering: ids congruent mod 8 share an XCD and start in increasing order there, about 32 at a time (one per
+    // CU).  Those 32 should share operands inside the XCD's 4 MiB L2: consecutive ids form an m_block x (32 / m_block) patch of
+    // tiles (m_block row tiles that all read the same column panels), and the patches sweep the column panels before moving to the
+    // next m_block row tiles.  All workgroups of a patch advance through K at the same pace, so the L2 only has to hold a window of
+    // their plaintext and residue slabs.  (With every row tile in one patch, 32 row tiles at M = 4096 re-read the plaintext digit
+    // planes, which no longer fit the L2, for every column panel and prime: 40 times the algorithmic traffic.)
     const unsigned id = blockIdx.x, xcd = id & 7, j = id >> 3;
-    const unsigned m_tile = j % m_tiles, c_tile = (j / m_tiles) * 8 + xcd;
+    const unsigned c_per_xcd = ((unsigned)c_tiles + 7) / 8;
+    const unsigned ml = j % m_block, t = j / m_block;
+    const unsigned m_tile = (t / c_per_xcd) * m_block + ml, c_tile = (t % c_per_xcd) * 8 + xcd;
     if (c_tile >= (unsigned)c_tiles) return;
     const int m0 = m_tile * MT;
     const unsigned c0 = c_tile * CT;
@@ -123,26 +135,27 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);          // wave-uniform
     const int wm = wave >> 1, wc = wave & 1;
     const int lr = lane & 15, lg = lane >> 4;
-    const int frag_off = 16 * (lg ^ (((lr >> 1) + (lr >> 3)) & 3));                   // swizzled position of this lane's operand chunk
+    // A 1 KiB slab (16 rows or columns x 64 k) is stored [16-byte k chunk g][row r][16 k] in global memory and in LDS alike, so that
+    // lane lr + 16 lg, which needs chunk lg of row lr as its MFMA operand, reads byte 16 * lane of the slab, and the asynchronous load
+    // that fills it (lane l writes byte 16 l) fetches 1 KiB of contiguous global memory.  A ds_read_b128 whose lanes read consecutive
+    // 16-byte chunks runs at the full 256 B/clk of the LDS; every other assignment of the same 64 chunks to the 64 lanes measured
+    // 1.7 times slower on this part, whatever the swizzle.
+    const int frag_off = 16 * lane;
     const int ksteps = a.Kpad / KS;
     const long plane = (long)a.Mpad * a.Kpad;
-    // plaintext digits: slab (d, rr) = rows 16*rr..+15 of digit d, 64 B each; lane -> row lane/4, 16-byte chunk lane%4
-    // LDS position (lane & 3) of slab row r = lane/4 receives the 16-byte chunk (lane & 3) ^ swz(r), swz(r) = ((r >> 1) + (r >> 3)) & 3:
-    // lanes reading one chunk of consecutive rows (64 B apart) then hit distinct 16-byte bank groups both within every aligned
-    // 8 lanes (128 B of banks) and within every aligned 16 lanes (256 B of banks).
-    const int swz_ld = (((lane >> 2) >> 1) + ((lane >> 2) >> 3)) & 3;
-    const int8_t* a_lane = a.Adig + (long)(m0 + (lane >> 2)) * a.Kpad + 16 * ((lane & 3) ^ swz_ld);
-    // residue digits: [prime][K step][digit][column][64]; slab (jj, cc) = columns 16*cc..+15 of digit jj = 1 KiB contiguous
+    // plaintext digits: [digit][16-row group][K step] slabs
+    const int8_t* a_lane = a.Adig + (long)(m0 / 16) * ksteps * 1024 + 16 * lane;
+    // residue digits: [prime][K step][column tile][digit][16-column slab] slabs
     const long b_step = (long)c_tiles * (DC * CT * KS);                 // bytes per (prime, K step)
-    const int8_t* b_lane = bdig + (long)c_tile * (DC * CT * KS) + 16 * (lane ^ swz_ld);
+    const int8_t* b_lane = bdig + (long)c_tile * (DC * CT * KS) + 16 * lane;
 
     auto issue = [&](int ks, int im, int8_t (*adst)[MT][KS], int8_t (*bdst)[CT][KS]) {
 #pragma unroll
         for (int t = 0; t < A_PER_WAVE; t++) {
             int slab = wave + NWAVES * t;
             slab = slab < A_SLABS ? slab : A_SLABS - 1;                  // surplus lanes re-load the last slab (same bytes)
-            const int d = slab >> 3, rr = slab & 7;
-            async_copy16(a_lane + d * plane + (long)(rr * 16) * a.Kpad + ks * KS, &adst[d][rr * 16][0]);
+            const int d = slab / (MT / 16), rr = slab % (MT / 16);
+            async_copy16(a_lane + d * plane + ((long)rr * ksteps + ks) * 1024, &adst[d][rr * 16][0]);
         }
         const int8_t* bsrc = b_lane + ((long)im * ksteps + ks) * b_step;
 #pragma unroll
@@ -157,47 +170,57 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
         __syncthreads();                            // ... and so have everybody else's
     };
 
-    // (ks2, im2): K step and prime of global step s+2, advanced without divisions; past the end the loads re-fetch valid
+    // (ks2, im2): K step and prime of global step s+AHEAD, advanced without divisions; past the end the loads re-fetch valid
     // data into slots nobody reads again, so that a step has no branches.
     auto advance = [&](int& ks, int& im) { if (++ks == ksteps) { ks = 0; --im; } };
     int ks2 = 0, im2 = a.mod_num - 1;
     issue(ks2, im2, lds_a0, lds_b0);
     advance(ks2, im2);
-    issue(ks2, im2 < 0 ? 0 : im2, lds_a1, lds_b1);
-    advance(ks2, im2);
+    if (RING == 3) {
+        issue(ks2, im2 < 0 ? 0 : im2, lds_a1, lds_b1);
+        advance(ks2, im2);
+    }
     wait_loads();
 
     v4i acc[ND][2][2];
-    // one K step reading ring slot R (compile time), refilling slot (R + 2) % 3 for step s + 2
+    // one K step reading ring slot R (compile time), refilling the slot read one step ago for step s + AHEAD
     auto kstep = [&](auto slot) {
-        constexpr int R = decltype(slot)::value, W = (R + 2) % 3;
-        int8_t (*A_cur)[MT][KS] = R == 0 ? lds_a0 : R == 1 ? lds_a1 : lds_a2;
-        int8_t (*B_cur)[CT][KS] = R == 0 ? lds_b0 : R == 1 ? lds_b1 : lds_b2;
-        int8_t (*A_nxt)[MT][KS] = W == 0 ? lds_a0 : W == 1 ? lds_a1 : lds_a2;
-        int8_t (*B_nxt)[CT][KS] = W == 0 ? lds_b0 : W == 1 ? lds_b1 : lds_b2;
-        // The refill of slot W is issued before any operand read of this step: an LDS read placed behind an asynchronous
-        // load in program order makes the compiler wait for every load in flight.
-        issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
-        v4i bf[2][DC];
+        constexpr int R = decltype(slot)::value, W = (R + RING - 1) % RING;
+        typedef int8_t (*aslot_t)[MT][KS];
+        typedef int8_t (*bslot_t)[CT][KS];
+        aslot_t A_cur = R == 0 ? lds_a0 : R == 1 ? lds_a1 : reinterpret_cast<aslot_t>(lds_a2);
+        bslot_t B_cur = R == 0 ? lds_b0 : R == 1 ? lds_b1 : reinterpret_cast<bslot_t>(lds_b2);
+        aslot_t A_nxt = W == 0 ? lds_a0 : W == 1 ? lds_a1 : reinterpret_cast<aslot_t>(lds_a2);
+        bslot_t B_nxt = W == 0 ? lds_b0 : W == 1 ? lds_b1 : reinterpret_cast<bslot_t>(lds_b2);
+        // operand reads in the order the MFMAs consume them (LDS reads return in order, so the first MFMA waits for its own two
+        // operands only): plaintext chunks of the first 16 rows, residue chunks of the first 16 columns, then the rest
+        v4i bf[2][DC], af[2][DW];
+#pragma unroll
+        for (int d = 0; d < DW; d++) af[0][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32][0] + frag_off);
 #pragma unroll
         for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16 + lr][frag_off]);
+            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16][0] + frag_off);
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
-            v4i af[DW];
+        for (int d = 0; d < DW; d++) af[1][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + 16][0] + frag_off);
 #pragma unroll
-            for (int d = 0; d < DW; d++) af[d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + mt * 16 + lr][frag_off]);
+        for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
+            for (int nt = 0; nt < 2; nt++) {
 #pragma unroll
-                for (int d = 0; d < DW; d++)
+                for (int jj = 0; jj < DC; jj++)
 #pragma unroll
-                    for (int jj = 0; jj < DC; jj++)
-                        acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
-        }
-        // the loads issued one step ago (for step s+1) must have landed; the ones just issued may stay in flight
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (A_PER_WAVE + B_PER_WAVE));      // vmcnt(loads of one step)
+                    for (int d = 0; d < DW; d++)
+                        acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[mt][d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
+                // the refill of slot W (read one step ago, released by the barrier that ended that step) goes out behind the operand
+                // reads and the first quarter of the MFMAs, so that the matrix pipe starts as early as possible in a step; the loads
+                // are opaque assembly, the compiler adds no wait for them
+                if (mt == 0 && nt == 0) issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
+            }
+        // the loads for step s+1 must have landed: with three slots those were issued one step ago and the ones just issued may
+        // stay in flight; with two slots they are the ones just issued
+        if (RING == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (A_PER_WAVE + B_PER_WAVE));      // vmcnt(loads of one step)
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                                            // vmcnt(0)
         __syncthreads();
         advance(ks2, im2);
     };
@@ -205,61 +228,97 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
     // r_last (residues modulo the last prime, < 2^39) of this lane's 16 outputs, kept in registers for the fused rescale
     // of the other primes: low words, and the 7 high bits packed four to a word.
     unsigned rl_lo[2][4][2], rl_hi[2][2];
+    // constants of the prime in work, requested before its K loop so that the epilogue does not start with a round trip to memory
+    double q = 0, qinv = 0, c32 = 0, qli = 0;
     auto epilogue = [&](int im, auto last_c, auto full_c) {
         constexpr bool LAST = decltype(last_c)::value, FULL = decltype(full_c)::value;
         // The output addressing starts from a value the optimiser cannot hoist above the K loop (it would otherwise keep
         // the row pointers alive across the loop).
         long row_stride = (long)a.mod_num * a.C;
         asm volatile("" : "+s"(row_stride));
-        const PrimeConst& pr = a.pq[a.np + im];
-        const double q = pr.qd, qinv = pr.qinv_d;
-        const double c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
-        const double qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
         const int mrow = m0 + wm * 32 + 4 * lg;
         u64* obase = a.out + (long)im * a.C + c0 + wc * 32 + lr;
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) {
+            // rows of the M padding are clamped for addressing; their stores are skipped
+            u64* orow[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int row = mrow + mt * 16 + r;
-                // rows of the M padding are clamped for addressing; their stores are skipped
-                u64* orow = obase + (long)(FULL || row < a.M ? row : a.M - 1) * row_stride;
+                orow[r] = obase + (long)(FULL || row < a.M ? row : a.M - 1) * row_stride;
+            }
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++) {
-                    // Horner inside each group of four diagonals: y_g = sum_{i<4} 256^i S_{4g+i}; |S_e| <= DW * Kpad * 2^14 and the
-                    // launcher admits DW * Kpad < 2^15 only, so |y_g| < 2^53 and every step is exact
-                    double y0 = (double)acc[3][mt][nt][r], y1 = (double)acc[ND - 1][mt][nt][r];
+            for (int nt = 0; nt < 2; nt++) {
+                // The four outputs of a lane in one MFMA tile advance together, one operation at a time: every operation below is
+                // a chain link of one output, and four independent links in flight hide the FP64 pipeline latency.
+                // Horner inside each group of four diagonals: y_g = sum_{i<4} 256^i S_{4g+i}; |S_e| <= DW * Kpad * 2^14 and the
+                // launcher admits DW * Kpad < 2^15 only, so |y_g| < 2^53 and every step is exact
+                double y0[4], y1[4], t[4];
 #pragma unroll
-                    for (int e = 2; e >= 0; e--) y0 = __builtin_fma(y0, 256.0, (double)acc[e][mt][nt][r]);
+                for (int r = 0; r < 4; r++) { y0[r] = (double)acc[3][mt][nt][r]; y1[r] = (double)acc[ND - 1][mt][nt][r]; }
 #pragma unroll
-                    for (int e = ND - 2; e >= 4; e--) y1 = __builtin_fma(y1, 256.0, (double)acc[e][mt][nt][r]);
-                    // |y0 + (y1 * 2^32 mod q)| < 2^53 + 0.51 q: one exact addition, one reduction to (-0.51 q, 0.51 q)
-                    double t = balance_f64(y0 + mulmod_f64(y1, c32, q, qinv), q, qinv);
-                    double res;
-                    if (LAST) {
-                        res = t;
-                    } else {
-                        // (r_i + q_i - r_last) * q_last^-1 mod q_i ; r_last is used as an integer without reduction
-                        // modulo q_i, as in PPMM_kernel.cuh:243-247
+                for (int e = 2; e >= 0; e--)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y0[r] = __builtin_fma(y0[r], 256.0, (double)acc[e][mt][nt][r]);
+#pragma unroll
+                for (int e = ND - 2; e >= 4; e--)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y1[r] = __builtin_fma(y1[r], 256.0, (double)acc[e][mt][nt][r]);
+                // |y0 + (y1 * 2^32 mod q)| < 2^53 + 0.51 q: one exact addition, one reduction to (-0.51 q, 0.51 q)
+                {
+                    double h[4], l[4], c[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h[r] = y1[r] * c32;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) l[r] = __builtin_fma(y1[r], c32, -h[r]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) c[r] = __builtin_rint(h[r] * qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) t[r] = y0[r] + (__builtin_fma(-c[r], q, h[r]) + l[r]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) c[r] = __builtin_rint(t[r] * qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) t[r] = __builtin_fma(-c[r], q, t[r]);
+                }
+                if (!LAST) {
+                    // (r_i + q_i - r_last) * q_last^-1 mod q_i ; r_last is used as an integer without reduction modulo q_i, as in
+                    // PPMM_kernel.cuh:243-247
+                    double h[4], l[4], c[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
                         const unsigned hi = (rl_hi[mt][nt] >> (8 * r)) & 0xff;
-                        const double rlast = __builtin_fma((double)hi, 4294967296.0, (double)rl_lo[mt][r][nt]);
-                        res = mulmod_f64(t - rlast, qli, q, qinv);
+                        t[r] -= __builtin_fma((double)hi, 4294967296.0, (double)rl_lo[mt][r][nt]);
                     }
-                    res = res < 0.0 ? res + q : res;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h[r] = t[r] * qli;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) l[r] = __builtin_fma(t[r], qli, -h[r]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) c[r] = __builtin_rint(h[r] * qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) t[r] = __builtin_fma(-c[r], q, h[r]) + l[r];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const double res = t[r] < 0.0 ? t[r] + q : t[r];
                     // res is an integer in [0, q): adding 2^52 leaves it in the low mantissa bits
                     const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFull;
                     if (LAST) {
                         rl_lo[mt][r][nt] = (unsigned)ures;
                         rl_hi[mt][nt] = (r == 0 ? 0u : rl_hi[mt][nt]) | ((unsigned)(ures >> 32) << (8 * r));
                     }
-                    if (FULL) orow[nt * 16] = ures;
-                    else if (row < a.M) orow[nt * 16] = ures;
+                    if (FULL) orow[r][nt * 16] = ures;
+                    else if (mrow + mt * 16 + r < a.M) orow[r][nt * 16] = ures;
                 }
             }
         }
     };
 
     for (int im = a.mod_num - 1; im >= 0; im--) {
+        q = a.pq[a.np + im].qd;
+        qinv = a.pq[a.np + im].qinv_d;
+        c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
+        qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
 #pragma unroll
         for (int e = 0; e < ND; e++)
 #pragma unroll
@@ -267,10 +326,10 @@ __global__ __launch_bounds__(64 * NWAVES) void ppmm_mfma_kernel(PpmmArgs a, cons
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++) acc[e][mt][nt] = v4i{0, 0, 0, 0};
 
-        for (int ks = 0; ks < ksteps; ks += 3) {
+        for (int ks = 0; ks < ksteps; ks += RING) {
             kstep(std::integral_constant<int, 0>{});
             kstep(std::integral_constant<int, 1>{});
-            kstep(std::integral_constant<int, 2>{});
+            if constexpr (RING == 3) kstep(std::integral_constant<int, 2>{});
         }
 
         // ---- end of a prime: exact recombination, reduction mod q, fused rescale ----
@@ -286,10 +345,13 @@ size_t ppmm_bdig_bytes(const PpmmArgs& a) { return (size_t)a.mod_num * a.Kpad * 
 
 template <int DW>
 static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig) {
-    const int c_tiles = (int)(a.C / CT), m_tiles = a.Mpad / MT;
+    const int c_tiles = (int)(a.C / CT);
     hipLaunchKernelGGL(ppmm_pack_kernel, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
+    const int m_tiles = a.Mpad / 128;
+    int m_block = 1;                                   // row tiles per patch: the largest divisor of m_tiles up to 6
+    for (int d = 2; d <= 6; d++) if (m_tiles % d == 0) m_block = d;
     const unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
-    hipLaunchKernelGGL(ppmm_mfma_kernel<DW>, dim3(blocks), dim3(64 * NWAVES), 0, stream, a, (const int8_t*)bdig, c_tiles, m_tiles);
+    hipLaunchKernelGGL((ppmm_mfma_kernel<DW, 8, 3>), dim3(blocks), dim3(512), 0, stream, a, (const int8_t*)bdig, c_tiles, m_block);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }

@@ -180,3 +180,51 @@ def test_small_ring_ntt(N1):
     pair2, dev2, orc2, rank2 = make(12, 128, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
     with pytest.raises(CkksError):
         dev2.pcmm_context.ToNTTInplace(d, 1, 1, 0, 0, 1)                     # N1 = 128: below the smallest transform
+
+
+@pytest.mark.parametrize("M,Kin", [(768, 768), (4096, 4096)])
+def test_ppmm_full_size_sampled_against_oracle(M, Kin):
+    """BASELINE configs 4 and 5 at their real shape (N = 2^16, N1 = 128, rank 512, C = 65,664 columns, 12 primes below 2^36, W ~ N(0, 0.02)
+    at scale 2^26): the whole product runs on the device; 24 rows of W over three column panels (the first columns, a panel inside the a
+    part that straddles a 64-column tile edge, the last columns of the b part) are recomputed by the oracle with the full contraction length
+    and compared on every modulus.  Operands: 16 distinct seeded samples, repeated."""
+    L, N1 = 12, 128
+    primes = CFG2_Q[:L]
+    pair = Pair(16, [], primes)
+    rank = pair.N // N1
+    C = (rank + 1) * N1
+    dev = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, pair.dev))
+    orc = O.OraclePCMM(pair.orc, N1, rank, [], primes)
+    rng = np.random.default_rng(M)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    seeds, dseeds = [], []
+    for s in range(16):
+        a = np.empty((L, C), dtype=np.uint64)
+        for j, q in enumerate(primes):
+            a[j] = rng.integers(0, q, C, dtype=np.uint64)
+        seeds.append(a)
+        dseeds.append(to_dev(a))
+    per = 8 * L * C
+    bufs = []
+    for n in range(Kin):
+        b = DeviceBuffer(per)
+        b.L_.ckks_memcpy_d2d(b.ptr, dseeds[n % 16].ptr, per)
+        bufs.append(b)
+    dout = DeviceBuffer(8 * M * L * C)
+    scaler = float(2 ** 26)
+    dev.PPMM(DeviceBuffer.from_numpy(W), bufs, dout, M, Kin, N1, Kin, L, scaler)
+    assert dev.pcmm_context.info("last_path") == 1 and dev.pcmm_context.info("last_DW") == 3
+    rows = sorted(set([0, M - 1, 127, 128] + [int(v) for v in rng.integers(0, M, 20)]))
+    Wsub = np.ascontiguousarray(W[rows])
+    mlwe = [seeds[n % 16].reshape(-1) for n in range(Kin)]
+    want = np.zeros((len(rows), L, C), dtype=np.uint64)             # only the panel columns get touched
+    panels = [(0, 8), (60, 8), (C - 8, 8)]
+    for c0, cnt in panels:
+        orc.PPMM(Wsub, mlwe, want.reshape(-1), len(rows), Kin, L, scaler, c0, cnt)
+    for r, m in enumerate(rows):
+        for j in range(L):
+            for c0, cnt in panels:
+                got = dout.download(np.uint64, cnt, 8 * ((m * L + j) * C + c0))
+                assert np.array_equal(got, want[r, j, c0:c0 + cnt]), (m, j, c0)
+    for b in bufs + dseeds + [dout]:
+        b.free()
