@@ -143,6 +143,74 @@ def bench_decompose(P, N1=128, L1=12, reps=5):
                          "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
 
 
+def bench_pcmm_fused(P, M=768, N1=128, L=12, reps=5):
+    """configs[3] as a layer runs it: two RLWE ciphertexts -> 512 + 256 samples -> PPMM 768 x 768, with the gather writing the int8 digit
+    planes of the MFMA kernel directly (no 8-byte MLWE samples in between), next to the two-step path on the same ciphertexts."""
+    from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
+    primes = P.CFG2_Q[:L]
+    ctx = Context_23(16, [], primes)
+    N = 1 << 16
+    rank = N // N1
+    C = (rank + 1) * N1
+    sch = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, ctx))
+    rng = np.random.default_rng(6)
+    parts = [(512, 0), (256, 512)]
+    Kin = 768
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    dW = DeviceBuffer.from_numpy(W)
+    cts = []
+    for _ in parts:
+        a = np.empty((2, L, N), dtype=np.uint64)
+        for j, q in enumerate(primes):
+            a[:, j] = rng.integers(0, q, (2, N), dtype=np.uint64)
+        cts.append(DeviceBuffer.from_numpy(a))
+    out = DeviceBuffer(8 * M * L * C)
+    scaler = float(2 ** 26)
+
+    def fused():
+        sch.packed_begin(Kin, L)
+        for (n, off), ct in zip(parts, cts):
+            sch.rlweCipherDecompose_packed(ct, n, off, L - 1)
+        sch.PPMM_packed(dW, out, M, scaler)
+
+    bufs = [DeviceBuffer(8 * L * C) for _ in range(Kin)]
+
+    def two_step():
+        for (n, off), ct in zip(parts, cts):
+            sch.rlweCipherDecompose(ct, bufs[off:off + n], n, 0, L - 1)
+        sch.PPMM(dW, bufs, out, M, Kin, N1, Kin, L, scaler)
+
+    res = {}
+    for name, f in (("two_step", two_step), ("fused", fused)):
+        f()
+        ctx.sync()
+        best = 1e30
+        for _ in range(reps):
+            ctx.timer_start()
+            f()
+            best = min(best, ctx.timer_stop())
+        res[name + "_ms"] = round(best, 3)
+    sch.packed_begin(Kin, L)
+    for (n, off), ct in zip(parts, cts):
+        sch.rlweCipherDecompose_packed(ct, n, off, L - 1)
+    best = 1e30
+    for _ in range(reps):
+        ctx.timer_start()
+        sch.PPMM_packed(dW, out, M, scaler)
+        best = min(best, ctx.timer_stop())
+    DW = sch.pcmm_context.info("last_DW")
+    macs = float(M) * Kin * C * L * DW * 5
+    res.update({"workload": "configs[3] as a layer: 2 RLWE ciphertexts (N=2^16, 12 primes) -> 512 + 256 samples -> PPMM 768x768",
+                "ppmm_on_digit_planes_ms": round(best, 3),
+                "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
+                             "unit": "TMAC/s (int8)", "frac": round(macs / (best * 1e-3) / MFMA_I8_PEAK_MACS, 4)},
+                "layer_frac_of_mfma_peak": {"two_step": round(macs / (res["two_step_ms"] * 1e-3) / MFMA_I8_PEAK_MACS, 4),
+                                            "fused": round(macs / (res["fused_ms"] * 1e-3) / MFMA_I8_PEAK_MACS, 4)}})
+    for b in bufs + cts + [out, dW]:
+        b.free()
+    return res
+
+
 def run(P):
-    return {"ppmm": bench_ppmm(P), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "keyswitch": bench_keyswitch(P),
+    return {"ppmm": bench_ppmm(P), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P)}

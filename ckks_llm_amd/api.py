@@ -582,6 +582,18 @@ class PCMM_Scheme:
         _check(self.L_.pcmm_ppmm(self.pcmm_context.h, _addr(plain_mat), self._ptrs(mlwe_cipher_decomposed[:mlwe_num]), _addr(out),
                                  mat_M, mat_N, mod_num, float(scaler)), "pcmm_ppmm")
 
+    # -- the gather writing PPMM's operand directly (no counterpart in the reference: its layer runs rlweCipherDecompose and PPMM back
+    #    to back through 8-byte MLWE samples, Bert.cuh:411-424)
+    def packed_begin(self, mat_N, mod_num):
+        _check(self.L_.pcmm_packed_begin(self.pcmm_context.h, mat_N, mod_num), "pcmm_packed_begin")
+
+    def rlweCipherDecompose_packed(self, rlwe_cipher, mlwe_num, offset, l):
+        """Samples offset .. offset + mlwe_num - 1 of the opened operand from one RLWE ciphertext (NTT domain, level l)."""
+        _check(self.L_.pcmm_rlwe_decompose_packed(self.pcmm_context.h, _addr(rlwe_cipher), offset, mlwe_num, l), "pcmm_rlwe_decompose_packed")
+
+    def PPMM_packed(self, plain_mat, out, mat_M, scaler):
+        _check(self.L_.pcmm_ppmm_packed(self.pcmm_context.h, _addr(plain_mat), _addr(out), mat_M, float(scaler)), "pcmm_ppmm_packed")
+
     def PPMM_strided(self, plain_mat, mlwe_all, out, mat_M, mat_N, mod_num, scaler):
         _check(self.L_.pcmm_ppmm_strided(self.pcmm_context.h, _addr(plain_mat), _addr(mlwe_all), _addr(out), mat_M, mat_N,
                                          mod_num, float(scaler)), "pcmm_ppmm_strided")

@@ -100,6 +100,72 @@ __global__ __launch_bounds__(256) void rlwe_gather_tiled_kernel(GatherArgs a) {
     }
 }
 
+// The gather writing PPMM's operand directly: the same window in LDS, but instead of 8-byte words in the MLWE layout the five
+// balanced base-256 digits of every value go straight into the residue digit planes of the MFMA kernel
+// (Bdig[prime][K step][64-column tile][digit][16-column slab], slab = [16-byte k chunk][column][16 k]; sample = k index,
+// column = row i * N1 + g).  A workgroup owns 16 consecutive g of one prime and 64 consecutive samples; a wave takes a row i at
+// a time, lane (col, kc) = 16 samples of one column, so that a wave writes one whole 1 KiB slab per digit with one store.
+// The MLWE samples never exist as 8-byte words: 5 bytes are written per value instead of 8 written, 8 read and 5 written.
+struct GatherDigitsArgs {
+    const u64* rlwe;
+    int8_t* bdig;
+    const PrimeConst* primes;
+    long N;
+    int N1, rank, mlwe_num, L, p_num, kstep0, ksteps, c_tiles;
+};
+__global__ __launch_bounds__(256) void rlwe_gather_digits_kernel(GatherDigitsArgs a) {
+    extern __shared__ u64 win[];                                     // 17 * (k + 1) words
+    constexpr int G = 16;
+    const int k = a.rank, N1 = a.N1, im = blockIdx.y, g0 = blockIdx.x * G;
+    const int gap = k / a.mlwe_num;
+    const u64 q = a.primes[a.p_num + im].q;
+    const u64* A = a.rlwe + a.N * im;
+    const u64* B = a.rlwe + a.N * (a.L + 1 + im);
+    for (int u = threadIdx.x + 1; u < (G + 1) * k; u += 256) {
+        const long p = (long)g0 * k + u - k;
+        win[u + u / k] = p >= 0 ? A[p] : negate_mod(A[a.N + p], q);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, kc = lane >> 4;
+    const int m0 = blockIdx.z * 64 + 16 * kc;                        // first of this lane's 16 samples
+    int8_t* step_base = a.bdig + ((long)im * a.ksteps + a.kstep0 + blockIdx.z) * (long)a.c_tiles * (5 * 64 * 64) + kc * 256 + col * 16;
+    for (int i = wave; i <= k; i += 4) {
+        uint4 dig[5];
+        unsigned* dw = reinterpret_cast<unsigned*>(dig);
+#pragma unroll
+        for (int grp = 0; grp < 4; grp++) {
+            u64 y[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int m = m0 + 4 * grp + t;
+                u64 x;
+                if (i < k) {
+                    const int d = m * gap - i;                       // in (-k, k)
+                    x = win[(col + 1) * k + d + col + 1 - (d < 0)];
+                } else {
+                    x = B[(long)m * gap + (long)(g0 + col) * k];     // b row: no shift, never wraps
+                }
+                y[t] = x + 0x8080808080ull;                          // bytes = digit + 128
+            }
+            const unsigned x0 = (unsigned)y[0], x1 = (unsigned)y[1], x2 = (unsigned)y[2], x3 = (unsigned)y[3];
+            const unsigned t0 = __byte_perm(x0, x1, 0x5140), t1 = __byte_perm(x0, x1, 0x7362);
+            const unsigned t2 = __byte_perm(x2, x3, 0x5140), t3 = __byte_perm(x2, x3, 0x7362);
+            dw[0 * 4 + grp] = __byte_perm(t0, t2, 0x5410) ^ 0x80808080u;
+            dw[1 * 4 + grp] = __byte_perm(t0, t2, 0x7632) ^ 0x80808080u;
+            dw[2 * 4 + grp] = __byte_perm(t1, t3, 0x5410) ^ 0x80808080u;
+            dw[3 * 4 + grp] = __byte_perm(t1, t3, 0x7632) ^ 0x80808080u;
+            const unsigned h01 = __byte_perm((unsigned)(y[0] >> 32), (unsigned)(y[1] >> 32), 0x0040);
+            const unsigned h23 = __byte_perm((unsigned)(y[2] >> 32), (unsigned)(y[3] >> 32), 0x0040);
+            dw[4 * 4 + grp] = __byte_perm(h01, h23, 0x5410) ^ 0x80808080u;
+        }
+        const long c = (long)i * N1 + g0;                            // first column of this wave's slab
+        int8_t* dst = step_base + (c / 64) * (5 * 64 * 64) + ((c % 64) / 16) * 1024;
+#pragma unroll
+        for (int jj = 0; jj < 5; jj++) *reinterpret_cast<uint4*>(dst + jj * 4096) = dig[jj];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------------------
 // plaintext quantisation: A = (int64)(float * double), |A| maximum, balanced base-256 digit planes
 // ------------------------------------------------------------------------------------------------------------
@@ -414,8 +480,8 @@ extern "C" int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_n
 }
 
 static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
-                       int M, int Kin, int mod_num, double scaler) {
-    if (!h || !W || !out || (!ptrs_host && !strided)) return CKKS_E_INVALID;
+                       int M, int Kin, int mod_num, double scaler, bool packed = false) {
+    if (!h || !W || !out || (!ptrs_host && !strided && !packed)) return CKKS_E_INVALID;
     if (M <= 0 || Kin <= 0 || mod_num < 1 || mod_num > h->nq || mod_num > 64) { set_error("PPMM: bad shape or mod_num"); return CKKS_E_INVALID; }
     ckks_ctx* c = h->ctx;
     const long C = (long)(h->rank + 1) * h->N1;
@@ -424,19 +490,21 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     // kernel needs no bounds checks along K.  A contiguous operand goes through a generated table.
     const int Kpad_tab = (Kin + 191) / 192 * 192;
     size_t zero_words = (size_t)mod_num * C;
-    if (Kpad_tab > Kin && zero_words > h->zero_cap) {
+    if (!packed && Kpad_tab > Kin && zero_words > h->zero_cap) {
         if (h->d_zero) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_zero); h->d_zero = nullptr; }
         CKKS_HIP_TRY(hipMalloc((void**)&h->d_zero, zero_words * sizeof(uint64_t)));
         CKKS_HIP_TRY(hipMemset(h->d_zero, 0, zero_words * sizeof(uint64_t)));
         h->zero_cap = zero_words;
     }
-    std::vector<const uint64_t*> tab(Kpad_tab);
-    for (int n = 0; n < Kpad_tab; n++)
-        tab[n] = n >= Kin ? h->d_zero : (ptrs_host ? ptrs_host[n] : strided + (size_t)n * mod_num * C);
     bool aligned16 = true;
-    for (int n = 0; n < Kin; n++) aligned16 = aligned16 && (((uintptr_t)tab[n]) & 15) == 0;
-    if ((rc = upload_ptrs(h, tab.data(), Kpad_tab))) return rc;
-    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
+    if (!packed) {
+        std::vector<const uint64_t*> tab(Kpad_tab);
+        for (int n = 0; n < Kpad_tab; n++)
+            tab[n] = n >= Kin ? h->d_zero : (ptrs_host ? ptrs_host[n] : strided + (size_t)n * mod_num * C);
+        for (int n = 0; n < Kin; n++) aligned16 = aligned16 && (((uintptr_t)tab[n]) & 15) == 0;
+        if ((rc = upload_ptrs(h, tab.data(), Kpad_tab))) return rc;
+        CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
+    }
     // workspace
     const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 191) / 192 * 192;   // K padded to a multiple of three 64-deep MFMA steps (LDS ring of three slots)
     size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
@@ -485,18 +553,21 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
     const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
                          (long)Kpad * (DW <= 3 ? 3 : 4) <= 16384 && absmax < qmin && qmin > (1ull << 25);
+    if (packed && !mfma_ok) { set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
         hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
         size_t need = ppmm_bdig_bytes(a);
+        if (packed && need > h->Bdig_cap) { set_error("PPMM on digit planes: planes not opened for this shape"); return CKKS_E_STATE; }
         if (need > h->Bdig_cap) {
             if (h->d_Bdig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Bdig); h->d_Bdig = nullptr; h->Bdig_cap = 0; }
             hipError_t e = hipMalloc((void**)&h->d_Bdig, need);
             if (e != hipSuccess) { set_error("PPMM: cannot allocate the residue digit planes"); return CKKS_E_NOMEM; }
             h->Bdig_cap = need;
         }
-        rc = launch_ppmm_mfma_impl(c->stream, a, DW, h->d_Bdig);
+        if (!packed) h->packed_K = h->packed_mods = 0;     // the planes now hold this call's operands
+        rc = launch_ppmm_mfma_impl(c->stream, a, DW, h->d_Bdig, !packed);
         if (rc) return rc;
     } else {
         dim3 grid((unsigned)((C + 255) / 256), M), block(256);
@@ -519,4 +590,65 @@ extern "C" int pcmm_ppmm(pcmm_ctx* h, const float* W, const uint64_t* const* mlw
 }
 extern "C" int pcmm_ppmm_strided(pcmm_ctx* h, const float* W, const uint64_t* mlwe, uint64_t* out, int M, int Kin, int mod_num, double scaler) {
     return ppmm_common(h, W, nullptr, mlwe, out, M, Kin, mod_num, scaler);
+}
+
+// ---- gather straight into the operand digit planes, and the contraction on them ----
+extern "C" int pcmm_packed_begin(pcmm_ctx* h, int Kin, int mod_num) {
+    if (!h) return CKKS_E_INVALID;
+    ckks_ctx* c = h->ctx;
+    const long C = (long)(h->rank + 1) * h->N1;
+    if (Kin <= 0 || Kin % 64 || mod_num < 1 || mod_num > h->nq || mod_num > 64 || C % 64 || h->N1 % 16) {
+        set_error("pcmm_packed_begin: Kin must be a positive multiple of 64, mod_num within the ring-pack moduli, N1 a multiple of 16");
+        return CKKS_E_INVALID;
+    }
+    for (int i = 0; i < mod_num; i++)
+        if (h->pq[h->np + i] >= (1ull << 39)) { set_error("pcmm_packed_begin: the digit planes hold primes below 2^39"); return CKKS_E_INVALID; }
+    const int Kpad = (Kin + 191) / 192 * 192;
+    const size_t need = (size_t)mod_num * Kpad * C * 5;
+    if (need > h->Bdig_cap) {
+        if (h->d_Bdig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Bdig); h->d_Bdig = nullptr; h->Bdig_cap = 0; }
+        hipError_t e = hipMalloc((void**)&h->d_Bdig, need);
+        if (e != hipSuccess) { set_error("pcmm_packed_begin: cannot allocate the residue digit planes"); return CKKS_E_NOMEM; }
+        h->Bdig_cap = need;
+    }
+    // K steps of the padding hold zero digits
+    if (Kpad > Kin) {
+        const size_t step = (size_t)C * 64 * 5;
+        for (int im = 0; im < mod_num; im++)
+            CKKS_HIP_TRY(hipMemsetAsync(h->d_Bdig + ((size_t)im * (Kpad / 64) + Kin / 64) * step, 0, (size_t)(Kpad - Kin) / 64 * step, c->stream));
+    }
+    h->packed_K = Kin; h->packed_mods = mod_num;
+    return CKKS_OK;
+}
+
+extern "C" int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int l) {
+    if (!h || !rlwe) return CKKS_E_INVALID;
+    ckks_ctx* c = h->ctx;
+    const int k = h->rank;
+    if (h->packed_K == 0) { set_error("rlweCipherDecompose to digit planes: planes not opened (pcmm_packed_begin)"); return CKKS_E_STATE; }
+    if (mlwe_num > k) { set_error("rlweCipherDecompose extract number must be <= mlwe_rank"); return CKKS_E_INVALID; }   // PCMM_Scheme.cuh:103-106
+    if (mlwe_num <= 0 || mlwe_num % 64 || k % mlwe_num || sample_offset < 0 || sample_offset % 64 || sample_offset + mlwe_num > h->packed_K ||
+        l < 0 || l > c->L || l + 1 != h->packed_mods || (long)h->N1 * k != c->N) {
+        set_error("rlweCipherDecompose to digit planes: samples come in multiples of 64 that divide the rank, inside the opened shape, at its level");
+        return CKKS_E_INVALID;
+    }
+    const size_t lds = (size_t)17 * (k + 1) * sizeof(u64);
+    static const bool big_lds = hipFuncSetAttribute(reinterpret_cast<const void*>(rlwe_gather_digits_kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess;
+    if (lds > (big_lds ? 96 * 1024 : 64 * 1024)) { set_error("rlweCipherDecompose to digit planes: rank too large for the LDS window"); return CKKS_E_INVALID; }
+    int rc;
+    const int K = c->K;
+    if ((rc = launch_ntt(c, rlwe, 0, K, 2, l + 1, c->L + 1, 0, 1, true))) return rc;              // PCMM_Scheme.cuh:113
+    GatherDigitsArgs a;
+    a.rlwe = rlwe; a.bdig = h->d_Bdig; a.primes = c->d_primes; a.N = c->N; a.N1 = h->N1; a.rank = k; a.mlwe_num = mlwe_num; a.L = c->L;
+    a.p_num = c->p_num; a.kstep0 = sample_offset / 64; a.ksteps = (h->packed_K + 191) / 192 * 3; a.c_tiles = (int)((long)(k + 1) * h->N1 / 64);
+    hipLaunchKernelGGL(rlwe_gather_digits_kernel, dim3(h->N1 / 16, l + 1, mlwe_num / 64), dim3(256), lds, c->stream, a);
+    CKKS_HIP_TRY(hipGetLastError());
+    return launch_ntt(c, rlwe, 0, K, 2, l + 1, c->L + 1, 0, 1, false);                            // :122
+}
+
+extern "C" int pcmm_ppmm_packed(pcmm_ctx* h, const float* W, uint64_t* out, int M, double scaler) {
+    if (!h) return CKKS_E_INVALID;
+    if (h->packed_K == 0) { set_error("PPMM on digit planes: planes not opened (pcmm_packed_begin)"); return CKKS_E_STATE; }
+    return ppmm_common(h, W, nullptr, nullptr, out, M, h->packed_K, h->packed_mods, scaler, true);
 }

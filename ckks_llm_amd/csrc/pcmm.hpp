@@ -19,6 +19,7 @@ struct pcmm_ctx {
     size_t Bdig_cap = 0;
     uint64_t* d_zero = nullptr;              // zero rows the K padding of the row-pointer table points to
     size_t zero_cap = 0;
+    int packed_K = 0, packed_mods = 0;       // shape the residue digit planes were opened for by pcmm_packed_begin (0: not open)
     int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
     unsigned long long last_absmax = 0;
     ckks_ctx* small = nullptr;               // tables of the size-N1 transform over the ring-pack primes, built on first use
@@ -48,6 +49,6 @@ struct PpmmArgs {
 };
 
 size_t ppmm_bdig_bytes(const PpmmArgs& a);
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig);
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig, bool pack);
 
 }  // namespace ckks

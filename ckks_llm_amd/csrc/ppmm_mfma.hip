@@ -344,9 +344,9 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
 size_t ppmm_bdig_bytes(const PpmmArgs& a) { return (size_t)a.mod_num * a.Kpad * a.C * DCMAX; }
 
 template <int DW>
-static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig) {
+static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool pack) {
     const int c_tiles = (int)(a.C / CT);
-    hipLaunchKernelGGL(ppmm_pack_kernel, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
+    if (pack) hipLaunchKernelGGL(ppmm_pack_kernel, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
     const int m_tiles = a.Mpad / 128;
     int m_block = 1;                                   // row tiles per patch: the largest divisor of m_tiles up to 6
     for (int d = 2; d <= 6; d++) if (m_tiles % d == 0) m_block = d;
@@ -356,9 +356,10 @@ static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig) {
     return CKKS_OK;
 }
 
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig) {
-    if (DW <= 3) return launch_dw<3>(stream, a, bdig);
-    return launch_dw<4>(stream, a, bdig);
+// pack = false: the digit planes were written by the caller (the gather that emits them directly)
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig, bool pack) {
+    if (DW <= 3) return launch_dw<3>(stream, a, bdig, pack);
+    return launch_dw<4>(stream, a, bdig, pack);
 }
 
 }  // namespace ckks

@@ -257,6 +257,19 @@ int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_
 int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev, uint64_t* out_dev, int M, int Kin,
                       int mod_num, double scaler);
 
+/* ---- the gather writing PPMM's operand directly.  No counterpart in the reference, where rlweCipherDecompose materialises every
+ * MLWE sample as 8-byte words that PPMM reads back (PCMM_Scheme.cuh:90-125, PPMM_kernel.cuh:254-349); in a layer the two always
+ * follow each other (Bert.cuh:411-424), so the samples can go straight into the int8 digit planes the MFMA kernel reads
+ * (5 bytes per residue).  Results are bit-identical to pcmm_rlwe_decompose_ntt followed by pcmm_ppmm.
+ *   pcmm_packed_begin(h, Kin, mod_num)      opens the planes for Kin samples (a multiple of 64) over mod_num moduli
+ *   pcmm_rlwe_decompose_packed(...)         samples sample_offset .. sample_offset + mlwe_num - 1 (multiples of 64; mlwe_num divides
+ *                                           the rank) from one RLWE ciphertext at level l = mod_num - 1 (NTT domain, restored)
+ *   pcmm_ppmm_packed(h, W, out, M, scaler)  the contraction over the Kin samples; out as pcmm_ppmm
+ * A call of pcmm_ppmm / pcmm_ppmm_strided reuses the same work space and closes the planes (CKKS_E_STATE afterwards). ---- */
+int pcmm_packed_begin(pcmm_ctx* h, int Kin, int mod_num);
+int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int l);
+int pcmm_ppmm_packed(pcmm_ctx* h, const float* W_dev, uint64_t* out_dev, int M, double scaler);
+
 #ifdef __cplusplus
 }
 #endif

@@ -589,6 +589,40 @@ public:
         }
     }
     long last_scaler = 0;
+
+    // The same layer step without 8-byte MLWE samples in between (no counterpart in the reference, where rlweCipherDecompose and PPMM
+    // run back to back, Bert.cuh:411-424): the gather writes the operand digit planes of the MFMA kernel directly.
+    //   packedBegin(mat_N)                                   opens the planes for mat_N samples (a multiple of 64)
+    //   rlweCipherDecomposePacked(cipher, mlwe_num, offset)  samples offset .. offset + mlwe_num - 1 from one ciphertext
+    //   PPMMPacked(plain_mat, rows, mat_M)                   the product; row i (first modulus) lands in rows[i] as PPMM leaves it
+    void packedBegin(int mat_N) {
+        packed_N = mat_N;
+        check(pcmm_packed_begin(pcmm_context.handle, mat_N, pcmm_context.ringpack_q_count), "packedBegin");
+    }
+    void rlweCipherDecomposePacked(Ciphertext& rlwe_cipher, uint64_tt mlwe_num, uint64_tt offset) {
+        packed_scale = rlwe_cipher.scale;
+        check(pcmm_rlwe_decompose_packed(pcmm_context.handle, rlwe_cipher.cipher_device, (int)offset, (int)mlwe_num, rlwe_cipher.l), "rlweCipherDecomposePacked");
+    }
+    void PPMMPacked(float* plain_mat, std::vector<MLWECiphertext*>& rows, int mat_M) {
+        const int mod_num = pcmm_context.ringpack_q_count;
+        const size_t C = (size_t)pcmm_context.N1 * (pcmm_context.mlwe_rank + 1);
+        const size_t need = (size_t)mat_M * mod_num * C;
+        if (need > ppmm_output_words) {
+            device_release(ppmm_output);
+            ppmm_output = device_alloc_words(need);
+            ppmm_output_words = need;
+        }
+        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * (long double)(1ll << 49) / packed_scale);      // PPMM_kernel.cuh:283-284
+        last_scaler = scaler;
+        check(pcmm_ppmm_packed(pcmm_context.handle, plain_mat, ppmm_output, mat_M, (double)scaler), "PPMMPacked");
+        const size_t n = rows.size() < (size_t)mat_M ? rows.size() : (size_t)mat_M;
+        for (size_t i = 0; i < n; i++) {
+            rows[i]->scale = packed_scale * scaler / (long double)pcmm_context.q_ringpack[1];
+            check(ckks_memcpy_d2d(rows[i]->cipher_device, ppmm_output + i * C * mod_num, sizeof(uint64_tt) * C), "PPMMPacked copy back");
+        }
+    }
+    int packed_N = 0;
+    long double packed_scale = 0;
 };
 
 }  // namespace ckks_llm_amd

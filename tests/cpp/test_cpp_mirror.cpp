@@ -250,6 +250,45 @@ static int run() {
         orc_ctx_destroy(o2);
     }
 
+    // ---- the layer step without 8-byte samples in between: packedBegin + rlweCipherDecomposePacked + PPMMPacked must leave what
+    //      rlweCipherDecompose + PPMM leave (N = 2^13, N1 = 128, rank 64, two 36-bit ring-pack primes, 64 samples) ----
+    {
+        const std::vector<uint64_tt> q2 = {0xffff00001ull, 0xfff9c0001ull};
+        const int lg = 13, n1 = 128;
+        const long n = 1l << lg;
+        const int rk = (int)(n / n1), rows_m = 32;
+        Context_23 c3(lg, {}, q2);
+        Scheme_23 s3(c3);
+        PCMM_Context pc3(n1, rk, {}, q2, c3);
+        PCMM_Scheme ps3(pc3, s3);
+        Ciphertext ct3((int)n, c3.L, c3.L, 1, (long double)(1ll << 59));   // PPMM scaler = q1 * 2^49 / scale = about 2^26
+        upload(ct3.cipher_device, uniform_limbs(rng, q2, 2, n));
+        std::vector<float> W3((size_t)rows_m * rk);
+        std::normal_distribution<float> nd3(0.f, 0.02f);
+        for (float& w : W3) w = nd3(rng);
+        void* W3d = nullptr;
+        check(ckks_malloc(&W3d, W3.size() * 4), "malloc W3");
+        check(ckks_memcpy_h2d(W3d, W3.data(), W3.size() * 4), "h2d W3");
+        std::vector<MLWECiphertext*> smp;
+        for (int i = 0; i < rk; i++) smp.push_back(new MLWECiphertext(n1, 1, 1, rk, ct3.scale));
+        ps3.rlweCipherDecompose(ct3, smp, rk, 0);
+        ps3.PPMM((float*)W3d, smp, rows_m, rk, n1, rk);
+        const size_t words = (size_t)rows_m * 2 * (size_t)n1 * (rk + 1);
+        std::vector<uint64_tt> two_step = download(ps3.ppmm_output, words);
+        const long double scale_after = smp[0]->scale;
+        std::vector<MLWECiphertext*> rows3;
+        for (int i = 0; i < rows_m; i++) rows3.push_back(new MLWECiphertext(n1, 1, 1, rk, 1.0L));
+        ps3.packedBegin(rk);
+        ps3.rlweCipherDecomposePacked(ct3, rk, 0);
+        ps3.PPMMPacked((float*)W3d, rows3, rows_m);
+        EXPECT(download(ps3.ppmm_output, words) == two_step && pc3.info("last_path") == 1, "packed gather + PPMMPacked == rlweCipherDecompose + PPMM (MFMA kernel)");
+        EXPECT(download(rows3[5]->cipher_device, (size_t)n1 * (rk + 1)) == download(smp[5]->cipher_device, (size_t)n1 * (rk + 1)) && rows3[5]->scale == scale_after,
+               "PPMMPacked leaves the rows and the scale as PPMM does");
+        for (MLWECiphertext* m : smp) delete m;
+        for (MLWECiphertext* m : rows3) delete m;
+        ckks_free(W3d);
+    }
+
     for (MLWECiphertext* m : mlwe) delete m;
     ckks_free(Wd);
     orc_pcmm_destroy(orc_p);

@@ -228,3 +228,53 @@ def test_ppmm_full_size_sampled_against_oracle(M, Kin):
                 assert np.array_equal(got, want[r, j, c0:c0 + cnt]), (m, j, c0)
     for b in bufs + dseeds + [dout]:
         b.free()
+
+
+@pytest.mark.parametrize("logN,N1,L,parts", [(13, 128, 2, [(64, 0)]), (14, 64, 3, [(256, 0), (128, 256), (64, 384)]), (16, 128, 12, [(512, 0), (256, 512)])])
+def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
+    """pcmm_packed_begin / pcmm_rlwe_decompose_packed / pcmm_ppmm_packed against the two-step path on the same ciphertexts (and through it against
+    the oracle, which pins that path): bit-identical outputs; the last shape is BASELINE config 4 (768 samples from two ciphertexts, the second
+    with every other sample)."""
+    from ckks_llm_amd import CkksError
+    primes = CFG2_Q[:L]
+    pair = Pair(logN, [], primes)
+    N = pair.N
+    rank = N // N1
+    C = (rank + 1) * N1
+    dev = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, pair.dev))
+    Kin = sum(n for n, _ in parts)
+    M = 96 if logN < 16 else 768
+    rng = np.random.default_rng(logN)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    dW = DeviceBuffer.from_numpy(W)
+    cts = [to_dev(limbs_uniform(100 + i, primes, 2, N)) for i in range(len(parts))]
+    before = [from_dev(c, (2, L, N)) for c in cts]
+    scaler = float(2 ** 26)
+    # two-step path
+    bufs = []
+    for (n, off), ct in zip(parts, cts):
+        part = [DeviceBuffer(8 * L * C) for _ in range(n)]
+        dev.rlweCipherDecompose(ct, part, n, 0, L - 1)
+        bufs += part
+    want = DeviceBuffer(8 * M * L * C)
+    dev.PPMM(dW, bufs, want, M, Kin, N1, Kin, L, scaler)
+    assert dev.pcmm_context.info("last_path") == 1
+    with pytest.raises(ValueError):
+        dev.PPMM_packed(dW, want, M, scaler)                               # the planes are not open
+    want_host = want.download()
+    # fused path
+    got = DeviceBuffer(8 * M * L * C)
+    got.zero()
+    dev.packed_begin(Kin, L)
+    for (n, off), ct in zip(parts, cts):
+        dev.rlweCipherDecompose_packed(ct, n, off, L - 1)
+    dev.PPMM_packed(dW, got, M, scaler)
+    assert np.array_equal(got.download(), want_host)
+    for c, b in zip(cts, before):
+        assert np.array_equal(from_dev(c, b.shape), b)                     # the ciphertexts are back in the NTT domain, unchanged
+    with pytest.raises(CkksError):
+        dev.rlweCipherDecompose_packed(cts[0], 48, 0, L - 1)               # not a multiple of 64
+    with pytest.raises(CkksError):
+        dev.rlweCipherDecompose_packed(cts[0], parts[0][0], Kin, L - 1)    # beyond the opened shape
+    for b in bufs + cts + [want, got, dW]:
+        b.free()
