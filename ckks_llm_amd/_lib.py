@@ -71,7 +71,7 @@ def _declare(L):
         "pcmm_add_repacking_key": (i, [vp, vp, vp, vp, C.c_char_p, C.c_uint64, vp]),
         "pcmm_mlwe_decrypt": (i, [vp, vp, vp, vp, i]),
         "pcmm_decode_coeffs": (i, [vp, vp, vp, vp, C.c_longlong, i]),
-        "pcmm_packed_begin": (i, [vp, i, i]), "pcmm_rlwe_decompose_packed": (i, [vp, vp, i, i, i]),
+        "pcmm_packed_begin": (i, [vp, i, i]), "pcmm_rlwe_decompose_packed": (i, [vp, vp, i, i, i, i]),
         "pcmm_ppmm_packed": (i, [vp, vp, vp, i, d]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),

@@ -587,9 +587,11 @@ class PCMM_Scheme:
     def packed_begin(self, mat_N, mod_num):
         _check(self.L_.pcmm_packed_begin(self.pcmm_context.h, mat_N, mod_num), "pcmm_packed_begin")
 
-    def rlweCipherDecompose_packed(self, rlwe_cipher, mlwe_num, offset, l):
-        """Samples offset .. offset + mlwe_num - 1 of the opened operand from one RLWE ciphertext (NTT domain, level l)."""
-        _check(self.L_.pcmm_rlwe_decompose_packed(self.pcmm_context.h, _addr(rlwe_cipher), offset, mlwe_num, l), "pcmm_rlwe_decompose_packed")
+    def rlweCipherDecompose_packed(self, rlwe_cipher, mlwe_num, offset, l, take=None):
+        """The first `take` (default: all) of the mlwe_num samples of one RLWE ciphertext (NTT domain, level l) become samples
+        offset .. offset + take - 1 of the opened operand."""
+        _check(self.L_.pcmm_rlwe_decompose_packed(self.pcmm_context.h, _addr(rlwe_cipher), offset, mlwe_num, mlwe_num if take is None else take, l),
+               "pcmm_rlwe_decompose_packed")
 
     def PPMM_packed(self, plain_mat, out, mat_M, scaler):
         _check(self.L_.pcmm_ppmm_packed(self.pcmm_context.h, _addr(plain_mat), _addr(out), mat_M, float(scaler)), "pcmm_ppmm_packed")

@@ -269,7 +269,7 @@ extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, 
 extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     if (!h) return CKKS_OK;
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig};
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     if (h->small) ckks_ctx_destroy(h->small);
     delete h;
@@ -446,17 +446,106 @@ extern "C" int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* c
 
 // ------------------------------------------------------------------------------------------------------------
 // size-N1 transforms over the ring-pack primes: PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273,
-// kernels smallntt_60bit.cuh:7-152).  Same negacyclic transform, root rule and table convention as the big ring, so the big
-// ring's kernels run it from a table set built for N1; the reference's layout [batch][mod][poly][N1] is one launch per
-// (batch, modulus) with poly_mod_len = 1.  The reference runs N1 = 256 only; this runs every N1 >= 256.
+// kernels smallntt_60bit.cuh:7-152).  Same negacyclic transform, root rule and table convention as the big ring.  For
+// N1 >= 256 the big ring's kernels run it from a table set built for N1; the reference's layout [batch][mod][poly][N1] is
+// one launch per (batch, modulus) with poly_mod_len = 1.  For N1 < 256 (the BERT layer runs N1 = 128 = token count) a
+// wave per polynomial runs all stages in LDS.  The reference runs N1 = 256 only and returns without work otherwise (:256,271).
 // ------------------------------------------------------------------------------------------------------------
+struct SmallRingArgs {
+    u64* data;
+    const u64* tw;                // [ring-pack prime][forward | inverse][N1]: psi_table / psiinv_table of the size-N1 ring
+    const PrimeConst* pq;
+    long polys;                   // batch * mod_num * poly_num
+    int N1, poly_num, mod_num, start_mod, inverse;
+    u64 n_inv[8];
+};
+__device__ __forceinline__ u64 small_mulmod(u64 a, u64 b, const PrimeConst& p) {
+    u128w acc{0, 0};
+    mac128(acc, a, b);
+    return barrett128(acc, p.q, p.mu_hi, p.mu_lo);
+}
+__global__ __launch_bounds__(256) void small_ring_ntt_kernel(SmallRingArgs a) {
+    __shared__ u64 buf[4][128];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long poly = (long)blockIdx.x * 4 + wave;
+    const bool live = poly < a.polys;
+    const int n = a.N1, half = n >> 1;
+    const int j = live ? (int)((poly / a.poly_num) % a.mod_num) : 0;
+    const PrimeConst p = a.pq[a.start_mod + j];
+    const u64* tw = a.tw + ((size_t)(a.start_mod + j) * 2 + (a.inverse ? 1 : 0)) * n;
+    u64* x = a.data + (live ? poly : 0) * n;
+    u64* b = buf[wave];
+    if (live)
+        for (int i = lane; i < n; i += 64) b[i] = x[i];
+    __syncthreads();
+    const bool work = live && lane < half;
+    if (!a.inverse) {
+        for (int m = 1, t = half; m < n; m <<= 1, t >>= 1) {
+            if (work) {
+                const int i = lane / t, lo = 2 * i * t + lane % t;
+                const u64 U = b[lo], V = small_mulmod(b[lo + t], tw[m + i], p);
+                b[lo] = csub(U + V, p.q);
+                b[lo + t] = csub(U + p.q - V, p.q);
+            }
+            __syncthreads();
+        }
+    } else {
+        for (int h = half, t = 1; h >= 1; h >>= 1, t <<= 1) {
+            if (work) {
+                const int i = lane / t, lo = 2 * i * t + lane % t;
+                const u64 U = b[lo], V = b[lo + t];
+                const u64 s = csub(U + V, p.q), d = csub(U + p.q - V, p.q);
+                b[lo] = h == 1 ? small_mulmod(s, a.n_inv[a.start_mod + j], p) : s;
+                b[lo + t] = small_mulmod(d, tw[h + i], p);            // the table's entry 1 already carries N1^-1 (Utils.cuh:200)
+            }
+            __syncthreads();
+        }
+    }
+    if (live)
+        for (int i = lane; i < n; i += 64) x[i] = b[i];
+}
+
+static int pcmm_tiny_ntt(pcmm_ctx* h, int logN1, uint64_t* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, bool inverse) {
+    const int n = h->N1, tot = h->np + h->nq;
+    if (logN1 < 1 || tot > 8) { set_error("PCMM NTT: N1 must be at least 2 and at most 8 ring-pack primes"); return CKKS_E_INVALID; }
+    if (!h->d_small_tw) {
+        std::vector<u64> tab((size_t)tot * 2 * n);
+        for (int i = 0; i < tot; i++) {
+            const u64 q = h->pq[i];
+            if ((q - 1) % (2 * (u64)n)) { set_error("PCMM NTT: a ring-pack prime is not 1 modulo 2 * N1"); return CKKS_E_INVALID; }
+            const u64 psi = H::mth_root(2 * (u64)n, q), psiinv = H::invmod(psi, q);
+            u64 pw = 1, ipw = 1;
+            for (int k = 0; k < n; k++) {                                  // fillTablePsi128_special (Utils.cuh:190-201)
+                const uint32_t r = H::bitrev((uint32_t)k, logN1);
+                tab[((size_t)i * 2 + 0) * n + r] = pw;
+                tab[((size_t)i * 2 + 1) * n + r] = ipw;
+                pw = H::mulmod(pw, psi, q);
+                ipw = H::mulmod(ipw, psiinv, q);
+            }
+            h->small_n_inv[i] = H::invmod((u64)n % q, q);
+            tab[((size_t)i * 2 + 1) * n + 1] = H::mulmod(tab[((size_t)i * 2 + 1) * n + 1], h->small_n_inv[i], q);
+        }
+        CKKS_HIP_TRY(hipMalloc((void**)&h->d_small_tw, tab.size() * sizeof(u64)));
+        CKKS_HIP_TRY(hipMemcpy(h->d_small_tw, tab.data(), tab.size() * sizeof(u64), hipMemcpyHostToDevice));
+    }
+    SmallRingArgs a;
+    a.data = (u64*)data; a.tw = h->d_small_tw; a.pq = h->d_pq;
+    a.polys = (long)mod_batch_size * mod_num * poly_num;
+    a.N1 = n; a.poly_num = poly_num; a.mod_num = mod_num; a.start_mod = start_mod_idx; a.inverse = inverse ? 1 : 0;
+    for (int i = 0; i < 8; i++) a.n_inv[i] = i < tot ? h->small_n_inv[i] : 0;
+    hipLaunchKernelGGL(small_ring_ntt_kernel, dim3((unsigned)((a.polys + 3) / 4)), dim3(256), 0, h->ctx->stream, a);
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+
 static int pcmm_small_ntt(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_mod_idx, int mod_batch_size, bool inverse) {
     if (!h || !data) return CKKS_E_INVALID;
     if (poly_num <= 0 || mod_num <= 0 || mod_batch_size <= 0) return CKKS_OK;
     if (start_mod_idx < 0 || start_mod_idx + mod_num > h->np + h->nq) { set_error("PCMM NTT: modulus range outside the ring-pack primes"); return CKKS_E_INVALID; }
     int logN1 = 0;
     while ((1 << logN1) < h->N1) logN1++;
-    if ((1 << logN1) != h->N1 || logN1 < 8) { set_error("PCMM NTT: N1 must be a power of two, at least 256"); return CKKS_E_INVALID; }
+    if ((1 << logN1) != h->N1) { set_error("PCMM NTT: N1 must be a power of two"); return CKKS_E_INVALID; }
+    if (logN1 < 8) return pcmm_tiny_ntt(h, logN1, data, poly_num, mod_num, start_mod_idx, mod_batch_size, inverse);
     if (!h->small) {
         int rc = ckks_ctx_create(&h->small, logN1, nullptr, 0, h->pq.data(), h->np + h->nq, nullptr, 0, 0);
         if (rc) return rc;
@@ -621,14 +710,14 @@ extern "C" int pcmm_packed_begin(pcmm_ctx* h, int Kin, int mod_num) {
     return CKKS_OK;
 }
 
-extern "C" int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int l) {
+extern "C" int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int take, int l) {
     if (!h || !rlwe) return CKKS_E_INVALID;
     ckks_ctx* c = h->ctx;
     const int k = h->rank;
     if (h->packed_K == 0) { set_error("rlweCipherDecompose to digit planes: planes not opened (pcmm_packed_begin)"); return CKKS_E_STATE; }
     if (mlwe_num > k) { set_error("rlweCipherDecompose extract number must be <= mlwe_rank"); return CKKS_E_INVALID; }   // PCMM_Scheme.cuh:103-106
-    if (mlwe_num <= 0 || mlwe_num % 64 || k % mlwe_num || sample_offset < 0 || sample_offset % 64 || sample_offset + mlwe_num > h->packed_K ||
-        l < 0 || l > c->L || l + 1 != h->packed_mods || (long)h->N1 * k != c->N) {
+    if (mlwe_num <= 0 || k % mlwe_num || take <= 0 || take > mlwe_num || take % 64 || sample_offset < 0 || sample_offset % 64 ||
+        sample_offset + take > h->packed_K || l < 0 || l > c->L || l + 1 != h->packed_mods || (long)h->N1 * k != c->N) {
         set_error("rlweCipherDecompose to digit planes: samples come in multiples of 64 that divide the rank, inside the opened shape, at its level");
         return CKKS_E_INVALID;
     }
@@ -642,7 +731,7 @@ extern "C" int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sampl
     GatherDigitsArgs a;
     a.rlwe = rlwe; a.bdig = h->d_Bdig; a.primes = c->d_primes; a.N = c->N; a.N1 = h->N1; a.rank = k; a.mlwe_num = mlwe_num; a.L = c->L;
     a.p_num = c->p_num; a.kstep0 = sample_offset / 64; a.ksteps = (h->packed_K + 191) / 192 * 3; a.c_tiles = (int)((long)(k + 1) * h->N1 / 64);
-    hipLaunchKernelGGL(rlwe_gather_digits_kernel, dim3(h->N1 / 16, l + 1, mlwe_num / 64), dim3(256), lds, c->stream, a);
+    hipLaunchKernelGGL(rlwe_gather_digits_kernel, dim3(h->N1 / 16, l + 1, take / 64), dim3(256), lds, c->stream, a);
     CKKS_HIP_TRY(hipGetLastError());
     return launch_ntt(c, rlwe, 0, K, 2, l + 1, c->L + 1, 0, 1, false);                            // :122
 }

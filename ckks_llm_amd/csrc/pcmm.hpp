@@ -23,6 +23,8 @@ struct pcmm_ctx {
     int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
     unsigned long long last_absmax = 0;
     ckks_ctx* small = nullptr;               // tables of the size-N1 transform over the ring-pack primes, built on first use
+    uint64_t* d_small_tw = nullptr;          // tables of the size-N1 transform when N1 < 256: [prime][forward | inverse][N1]
+    uint64_t small_n_inv[8] = {};            // N1^-1 modulo each ring-pack prime (N1 < 256)
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
 };
 

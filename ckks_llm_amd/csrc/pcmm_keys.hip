@@ -6,8 +6,8 @@
 // PCMM_Context::decodeCoeffs (PCMM_Context.cuh:149-178).
 //
 // Per repacking key the reference runs nine launches; here a key is one random-stream launch, one fused sampling kernel (a, and
-// e + p0 * iota(s_i) in the coefficient domain), one transform and one combining kernel.  The size-N1 transforms go through the
-// library's own small-ring tables, so these entry points need N1 >= 256 like pcmm_ntt_fwd.
+// e + p0 * iota(s_i) in the coefficient domain), one transform and one combining kernel.  The size-N1 transforms are
+// pcmm_ntt_fwd / pcmm_ntt_inv, which run every power of two N1 (the reference's run N1 = 256 only).
 #include <hip/hip_runtime.h>
 #include <cmath>
 #include <string>
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(THREADS) void mlwe_decode_kernel(double* vals, cons
 int shape_ok(pcmm_ctx* h, const char* who) {
     if (!h || !h->ctx) { set_error(std::string(who) + ": null handle"); return CKKS_E_INVALID; }
     if ((long)h->N1 * h->rank != h->ctx->N) { set_error(std::string(who) + ": N1 * rank must be N"); return CKKS_E_INVALID; }
-    if (h->N1 < 256) { set_error(std::string(who) + ": needs the size-N1 transform, N1 >= 256"); return CKKS_E_INVALID; }
+    if (h->N1 % 64) { set_error(std::string(who) + ": N1 must be a multiple of 64"); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
 

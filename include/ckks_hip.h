@@ -205,7 +205,8 @@ int pcmm_ctx_destroy(pcmm_ctx* h);
 /* PCMM_Context::ToNTTInplace / FromNTTInplace (PCMM_Context.cuh:243-273; kernels smallntt_60bit.cuh:7-152): negacyclic transforms
  * of size N1 over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1], limb (z, j, y) modulo
  * pq_ringpack[start_mod_idx + j].  start_poly_idx is carried for the signature only (the reference's kernels ignore it).
- * The reference runs N1 = 256 only and silently does nothing otherwise; here N1 >= 256, smaller rings return CKKS_E_INVALID. */
+ * The reference runs N1 = 256 only and silently does nothing otherwise; here every power of two N1 >= 2
+ * runs (N1 < 256, such as the BERT layer's 128, through a wave-per-polynomial LDS kernel). */
 int pcmm_ntt_fwd(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
 int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
 /* "N1", "mlwe_rank", and facts about the last PPMM call: "last_path" (1 = int8 MFMA kernel, 0 = generic 128-bit kernel),
@@ -230,19 +231,19 @@ int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* const* mlwe_
  * [p_count + q_count moduli][rank][N1], small polynomial i = the coefficients i + n*rank of the RLWE secret, NTT domain (size N1).
  * rlwe_sk (K+L+1 limbs, NTT domain) is transformed back and forth in place as in the reference and ends unchanged.
  * The two copies of the reference are kept as they are: RLWE limbs 0.. to key moduli 0.., then RLWE limbs K.. to key moduli
- * p_count.. (so modulus slot 0 holds the secret modulo the FIRST special prime; nothing reads it).  Needs N1 >= 256. */
+ * p_count.. (so modulus slot 0 holds the secret modulo the FIRST special prime; nothing reads it).  N1 a multiple of 64. */
 int pcmm_convert_mlwe_sk(pcmm_ctx* h, uint64_t* mlwe_sk, uint64_t* rlwe_sk);
 /* PCMM_Scheme::addRepakcingKey (PCMM_Scheme.cuh:126-224): rank keys over the context primes [last p_count special primes |
  * q_0 .. q_{q_count-2}], key i at keys + i*2*m*N = [a: m limbs | b: m limbs], m = p_count + q_count - 1, NTT domain,
  * b = -a*s + p0 * iota(s_i) + e - the layout pcmm_mlwe_pack reads.  Randomness: key i draws 4*N bytes (e) then 8*N*m bytes (a)
  * from the Salsa20 stream of (key32, nonce + i).  scratch: (m + 1)*N words.  mlwe_sk is taken to the coefficient domain and
  * back on ALL its moduli (the reference brings back all but the last, :182).  b starts from zero (the reference writes the
- * embedded secret into fresh cudaMalloc memory).  Needs N1 >= 256. */
+ * embedded secret into fresh cudaMalloc memory).  N1 a multiple of 64. */
 int pcmm_add_repacking_key(pcmm_ctx* h, uint64_t* keys, uint64_t* mlwe_sk, const uint64_t* rlwe_sk, const uint8_t* key32, uint64_t nonce,
                            uint64_t* scratch);
 /* PCMM_Scheme::mlweDecrypt (PCMM_Scheme.cuh:531-576): plain[mod][n] = b + sum_i a_i * s_i for moduli 0..l of the sample, in the
  * size-N1 NTT domain (where the reference leaves it); the sample is transformed in place and back.  Any rank (the reference
- * instantiates 256 and 512).  Needs N1 >= 256. */
+ * instantiates 256 and 512).  N1 a multiple of 64. */
 int pcmm_mlwe_decrypt(pcmm_ctx* h, uint64_t* plain, uint64_t* mlwe_cipher, const uint64_t* mlwe_sk, int l);
 /* PCMM_Context::decodeCoeffs (PCMM_Context.cuh:149-178): inverse transform of a copy (scratch: (l+1)*N1 words), then the centred
  * residue modulo the first ring-pack modulus divided by scaler; vals: N1 device doubles. */
@@ -262,12 +263,13 @@ int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev,
  * follow each other (Bert.cuh:411-424), so the samples can go straight into the int8 digit planes the MFMA kernel reads
  * (5 bytes per residue).  Results are bit-identical to pcmm_rlwe_decompose_ntt followed by pcmm_ppmm.
  *   pcmm_packed_begin(h, Kin, mod_num)      opens the planes for Kin samples (a multiple of 64) over mod_num moduli
- *   pcmm_rlwe_decompose_packed(...)         samples sample_offset .. sample_offset + mlwe_num - 1 (multiples of 64; mlwe_num divides
- *                                           the rank) from one RLWE ciphertext at level l = mod_num - 1 (NTT domain, restored)
+ *   pcmm_rlwe_decompose_packed(...)         the first `take` of the mlwe_num samples that rlweCipherDecompose extracts from one RLWE
+ *                                           ciphertext (mlwe_num divides the rank; level l = mod_num - 1; NTT domain, restored) become
+ *                                           samples sample_offset .. sample_offset + take - 1 (take, sample_offset: multiples of 64)
  *   pcmm_ppmm_packed(h, W, out, M, scaler)  the contraction over the Kin samples; out as pcmm_ppmm
  * A call of pcmm_ppmm / pcmm_ppmm_strided reuses the same work space and closes the planes (CKKS_E_STATE afterwards). ---- */
 int pcmm_packed_begin(pcmm_ctx* h, int Kin, int mod_num);
-int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int l);
+int pcmm_rlwe_decompose_packed(pcmm_ctx* h, uint64_t* rlwe, int sample_offset, int mlwe_num, int take, int l);
 int pcmm_ppmm_packed(pcmm_ctx* h, const float* W_dev, uint64_t* out_dev, int M, double scaler);
 
 #ifdef __cplusplus

@@ -593,15 +593,16 @@ public:
     // The same layer step without 8-byte MLWE samples in between (no counterpart in the reference, where rlweCipherDecompose and PPMM
     // run back to back, Bert.cuh:411-424): the gather writes the operand digit planes of the MFMA kernel directly.
     //   packedBegin(mat_N)                                   opens the planes for mat_N samples (a multiple of 64)
-    //   rlweCipherDecomposePacked(cipher, mlwe_num, offset)  samples offset .. offset + mlwe_num - 1 from one ciphertext
+    //   rlweCipherDecomposePacked(cipher, mlwe_num, offset, take)  the first take (default all) of a ciphertext's mlwe_num samples -> samples offset ..
     //   PPMMPacked(plain_mat, rows, mat_M)                   the product; row i (first modulus) lands in rows[i] as PPMM leaves it
     void packedBegin(int mat_N) {
         packed_N = mat_N;
         check(pcmm_packed_begin(pcmm_context.handle, mat_N, pcmm_context.ringpack_q_count), "packedBegin");
     }
-    void rlweCipherDecomposePacked(Ciphertext& rlwe_cipher, uint64_tt mlwe_num, uint64_tt offset) {
+    void rlweCipherDecomposePacked(Ciphertext& rlwe_cipher, uint64_tt mlwe_num, uint64_tt offset, uint64_tt take = 0) {
         packed_scale = rlwe_cipher.scale;
-        check(pcmm_rlwe_decompose_packed(pcmm_context.handle, rlwe_cipher.cipher_device, (int)offset, (int)mlwe_num, rlwe_cipher.l), "rlweCipherDecomposePacked");
+        check(pcmm_rlwe_decompose_packed(pcmm_context.handle, rlwe_cipher.cipher_device, (int)offset, (int)mlwe_num, (int)(take ? take : mlwe_num),
+                                         rlwe_cipher.l), "rlweCipherDecomposePacked");
     }
     void PPMMPacked(float* plain_mat, std::vector<MLWECiphertext*>& rows, int mat_M) {
         const int mod_num = pcmm_context.ringpack_q_count;

@@ -155,10 +155,11 @@ def test_mlwe_packing_errors():
         dev.mlweCipherPacking(big, [b] * 3, 3, 0, big, big, big)                  # 3 does not divide the rank
 
 
-@pytest.mark.parametrize("N1", [256, 1024])
+@pytest.mark.parametrize("N1", [16, 64, 128, 256, 1024])
 def test_small_ring_ntt(N1):
     """PCMM_Context::ToNTTInplace / FromNTTInplace: size-N1 transforms over the ring-pack primes in the reference's
-    [batch][mod][poly][N1] layout against the oracle, and the error for rings the transform does not cover."""
+    [batch][mod][poly][N1] layout against the oracle (N1 < 256, the BERT layer's token-count ring among them, runs a kernel of its
+    own), and the error for a modulus range outside the ring-pack primes."""
     from ckks_llm_amd import CkksError
     q = CFG2_Q[:3]
     pair, dev, orc, rank = make(12, N1, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
@@ -177,9 +178,6 @@ def test_small_ring_ntt(N1):
     assert np.array_equal(from_dev(d, data.shape), data)
     with pytest.raises(CkksError):
         dev.pcmm_context.ToNTTInplace(d, polys, 3, 0, 1, batch)              # moduli 1..3 of three
-    pair2, dev2, orc2, rank2 = make(12, 128, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
-    with pytest.raises(CkksError):
-        dev2.pcmm_context.ToNTTInplace(d, 1, 1, 0, 0, 1)                     # N1 = 128: below the smallest transform
 
 
 @pytest.mark.parametrize("M,Kin", [(768, 768), (4096, 4096)])
@@ -230,11 +228,13 @@ def test_ppmm_full_size_sampled_against_oracle(M, Kin):
         b.free()
 
 
-@pytest.mark.parametrize("logN,N1,L,parts", [(13, 128, 2, [(64, 0)]), (14, 64, 3, [(256, 0), (128, 256), (64, 384)]), (16, 128, 12, [(512, 0), (256, 512)])])
+@pytest.mark.parametrize("logN,N1,L,parts", [(13, 128, 2, [(64, 0, 64)]), (14, 64, 3, [(256, 0, 256), (128, 256, 128), (256, 384, 64)]),
+                                             (16, 128, 12, [(512, 0, 512), (256, 512, 256)]), (16, 128, 2, [(512, 0, 512), (512, 512, 256)])])
 def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
     """pcmm_packed_begin / pcmm_rlwe_decompose_packed / pcmm_ppmm_packed against the two-step path on the same ciphertexts (and through it against
-    the oracle, which pins that path): bit-identical outputs; the last shape is BASELINE config 4 (768 samples from two ciphertexts, the second
-    with every other sample)."""
+    the oracle, which pins that path): bit-identical outputs.  parts = (samples extracted from a ciphertext, offset, how many of them are used);
+    the third shape is BASELINE config 4 (768 samples from two ciphertexts, the second with every other sample), the fourth the reference layer's
+    choice (Bert.cuh:411-412, 420: 512 + 512 extracted, the first 768 multiplied)."""
     from ckks_llm_amd import CkksError
     primes = CFG2_Q[:L]
     pair = Pair(logN, [], primes)
@@ -242,7 +242,7 @@ def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
     rank = N // N1
     C = (rank + 1) * N1
     dev = PCMM_Scheme(PCMM_Context(N1, rank, [], primes, pair.dev))
-    Kin = sum(n for n, _ in parts)
+    Kin = sum(t for _, _, t in parts)
     M = 96 if logN < 16 else 768
     rng = np.random.default_rng(logN)
     W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
@@ -252,10 +252,10 @@ def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
     scaler = float(2 ** 26)
     # two-step path
     bufs = []
-    for (n, off), ct in zip(parts, cts):
+    for (n, off, take), ct in zip(parts, cts):
         part = [DeviceBuffer(8 * L * C) for _ in range(n)]
         dev.rlweCipherDecompose(ct, part, n, 0, L - 1)
-        bufs += part
+        bufs += part[:take]
     want = DeviceBuffer(8 * M * L * C)
     dev.PPMM(dW, bufs, want, M, Kin, N1, Kin, L, scaler)
     assert dev.pcmm_context.info("last_path") == 1
@@ -266,8 +266,8 @@ def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
     got = DeviceBuffer(8 * M * L * C)
     got.zero()
     dev.packed_begin(Kin, L)
-    for (n, off), ct in zip(parts, cts):
-        dev.rlweCipherDecompose_packed(ct, n, off, L - 1)
+    for (n, off, take), ct in zip(parts, cts):
+        dev.rlweCipherDecompose_packed(ct, n, off, L - 1, take)
     dev.PPMM_packed(dW, got, M, scaler)
     assert np.array_equal(got.download(), want_host)
     for c, b in zip(cts, before):
@@ -275,6 +275,6 @@ def test_gather_to_digit_planes_equals_decompose_then_ppmm(logN, N1, L, parts):
     with pytest.raises(CkksError):
         dev.rlweCipherDecompose_packed(cts[0], 48, 0, L - 1)               # not a multiple of 64
     with pytest.raises(CkksError):
-        dev.rlweCipherDecompose_packed(cts[0], parts[0][0], Kin, L - 1)    # beyond the opened shape
+        dev.rlweCipherDecompose_packed(cts[0], parts[0][0], Kin, L - 1, 64)  # beyond the opened shape
     for b in bufs + cts + [want, got, dW]:
         b.free()

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 KEY = bytes(range(3, 35))
 
 
-@pytest.mark.parametrize("logN,N1", [(12, 256), (13, 512)])
+@pytest.mark.parametrize("logN,N1", [(12, 256), (13, 512), (12, 128), (11, 64)])
 def test_mlwe_keys_and_decryption_match_oracle(logN, N1):
     P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
     pair = Pair(logN, [P0], [Q0, Q1])
@@ -63,8 +63,8 @@ def test_mlwe_keys_and_decryption_match_oracle(logN, N1):
         assert L_.pcmm_decode_coeffs(dev_pc.h, d_vals.ptr, d_plain.ptr, scratch.ptr, 1 << 20, l) == 0
         assert np.array_equal(d_vals.download(np.float64), vals)
     assert L_.pcmm_mlwe_decrypt(dev_pc.h, d_plain.ptr, d_sample.ptr, d_msk.ptr, 2) != 0
-    small = PCMM_Context(128, N // 128, [P0], [Q0, Q1], pair.dev)
-    assert L_.pcmm_convert_mlwe_sk(small.h, d_msk.ptr, d_sx.ptr) != 0      # N1 = 128: below the smallest size-N1 transform
+    odd = PCMM_Context(32, N // 32, [P0], [Q0, Q1], pair.dev)
+    assert L_.pcmm_convert_mlwe_sk(odd.h, d_msk.ptr, d_sx.ptr) != 0        # N1 = 32: the key side needs a multiple of 64
 
 
 def test_reference_test_program_flow():

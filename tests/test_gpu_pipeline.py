@@ -88,3 +88,69 @@ def test_encrypt_decompose_ppmm_pack_decrypt(mlwe_num):
     assert biggest > 1 << 15                                                  # the check is not vacuous
     # rescale and ModDown rounding are O(N); the key noise contributes sum_i a_i * e_i / P0, about sqrt(k * N) * Q0 / P0 * 3
     assert worst <= 16 * N, (worst, biggest)
+
+
+def test_bert_base_layer_on_encrypted_activations():
+    """BASELINE config 4 end to end at its real ring: 128 tokens x 768 activations ~ N(0, 1), coefficient-packed into two RLWE ciphertexts at
+    N = 2^16 (ternary secret of weight 192, Gaussian error 3.2, public-key encryption), times W 768 x 768 ~ N(0, 0.02), out as three ring-packed
+    ciphertexts of 256 features each - the sequence of Bert::PCMM_Boot_768_768 between its slot/coefficient conversions (Bert.cuh:411-424, 473,
+    482, 491) - with every key generated on the device, the gather writing PPMM's operand planes directly, and the decrypted result compared with
+    the plaintext product as the reference's test program does (GetPrecisionStats, precision.cuh:104)."""
+    from ckks_llm_amd import Ciphertext, MLWESecretKey, Plaintext, Scheme_23, SecretKey
+    logN, N1 = 16, 128
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    ctx = Context_23(logN, [P0], [Q0, Q1])
+    N, L = ctx.N, ctx.L
+    k = N // N1
+    key = bytes(range(32))
+    scheme = Scheme_23(ctx, key=key)
+    sk = SecretKey(ctx, h=192, key=key, nonce=1)
+    pc = PCMM_Context(N1, k, [P0], [Q0, Q1], ctx)
+    ps = PCMM_Scheme(pc, key=key)
+    mlwe_sk = MLWESecretKey(N1, pc.ringpack_pq_count - 1, k)
+    ps.convertMLWESKfromRLWESK(mlwe_sk, sk)
+    scheme.addEncKey(sk)
+    ps.addRepakcingKey(mlwe_sk, sk)
+    rng = np.random.default_rng(4)
+    tokens, feat = N1, 768
+    X = rng.normal(0, 1, (tokens, feat))
+    W = rng.normal(0, 0.02, (feat, feat)).astype(np.float32)
+    want = X @ W.astype(np.float64).T                                      # [token][output feature]
+    x_scale = 1 << 33
+    cts = []
+    for lo, hi in ((0, 512), (512, 768)):
+        coeffs = np.zeros((tokens, k))
+        coeffs[:, : hi - lo] = X[:, lo:hi]                                  # coefficient n * k + m = X[n][lo + m]
+        msg = Plaintext(N, L, L, N // 2, x_scale)
+        ctx.encode_coeffs(DeviceBuffer.from_numpy(coeffs.reshape(-1)), msg)
+        ct = Ciphertext(N, L, L, N // 2, x_scale)
+        scheme.encryptMsg(ct, msg)
+        cts.append(ct)
+    C = (k + 1) * N1
+    scaler = float(1 << 29)
+    out = DeviceBuffer(8 * feat * 2 * C)
+    ps.packed_begin(feat, 2)
+    ps.rlweCipherDecompose_packed(cts[0].cipher_device, 512, 0, 1)
+    ps.rlweCipherDecompose_packed(cts[1].cipher_device, 512, 512, 1, take=256)
+    ps.PPMM_packed(DeviceBuffer.from_numpy(W), out, feat, scaler)
+    assert pc.info("last_path") == 1 and pc.info("last_DW") == 4
+    rows = [DeviceBuffer(8 * C) for _ in range(feat)]
+    for m in range(feat):
+        rows[m].L_.ckks_memcpy_d2d(rows[m].ptr, out.ptr + 8 * m * 2 * C, 8 * C)
+    out_scale = x_scale * scaler / Q1
+    embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    dec, d_vals = Plaintext(N, L, 0, N // 2, 1), DeviceBuffer(8 * N)
+    worst = []
+    for j in range(3):
+        res = Ciphertext(N, L, 0, N // 2, out_scale)
+        res.cipher_device.zero()
+        ps.mlweCipherPacking(res.cipher_device, rows[256 * j: 256 * (j + 1)], 256, 0, ps.repackingKeys, embed, mult)
+        res.l, res.scale = 0, out_scale
+        scheme.decryptMsg(dec, sk, res)
+        ctx.decode_coeffs(dec, d_vals)
+        got = d_vals.download(np.float64).reshape(tokens, k)                # coefficient n * k + 2 m = Y[n][256 j + m]
+        err = np.abs(got[:, 0:512:2] - want[:, 256 * j: 256 * (j + 1)])
+        worst.append(err.max())
+        assert np.abs(got[:, 1:512:2]).max() < 2.0 ** -9                    # the positions between the packed samples hold noise only
+        assert np.median(err) < 2.0 ** -13
+    assert np.abs(want).max() > 2.0 and max(worst) < 2.0 ** -10, worst
