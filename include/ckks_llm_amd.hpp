@@ -577,8 +577,7 @@ public:
         }
         std::vector<const uint64_tt*> ptrs(mlwe_num);
         for (int i = 0; i < mlwe_num; i++) ptrs[i] = mlwe_cipher_decomposed[i]->cipher_device;
-        const long double target_scale = (long double)(1ll << 49);
-        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * target_scale / mlwe_cipher_decomposed[0]->scale);
+        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * ppmm_target_scale / mlwe_cipher_decomposed[0]->scale);
         last_scaler = scaler;
         check(pcmm_ppmm(pcmm_context.handle, plain_mat, ptrs.data(), ppmm_output, mat_M, mat_N, mod_num, (double)scaler), "PPMM");
         const int rows = mat_M < mlwe_num ? mat_M : mlwe_num;
@@ -589,6 +588,9 @@ public:
         }
     }
     long last_scaler = 0;
+    // scale of the product rows; the reference fixes 2^49 (PPMM_kernel.cuh:283), which suits its 50- to 60-bit ring-pack primes; a
+    // caller with shorter primes lowers it so that the rows stay below q_ringpack[0] / 2
+    long double ppmm_target_scale = (long double)(1ll << 49);
 
     // The same layer step without 8-byte MLWE samples in between (no counterpart in the reference, where rlweCipherDecompose and PPMM
     // run back to back, Bert.cuh:411-424): the gather writes the operand digit planes of the MFMA kernel directly.
@@ -613,7 +615,7 @@ public:
             ppmm_output = device_alloc_words(need);
             ppmm_output_words = need;
         }
-        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * (long double)(1ll << 49) / packed_scale);      // PPMM_kernel.cuh:283-284
+        const long scaler = (long)((long double)pcmm_context.q_ringpack[1] * ppmm_target_scale / packed_scale);             // PPMM_kernel.cuh:283-284
         last_scaler = scaler;
         check(pcmm_ppmm_packed(pcmm_context.handle, plain_mat, ppmm_output, mat_M, (double)scaler), "PPMMPacked");
         const size_t n = rows.size() < (size_t)mat_M ? rows.size() : (size_t)mat_M;
