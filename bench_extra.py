@@ -211,6 +211,45 @@ def bench_pcmm_fused(P, M=768, N1=128, L=12, reps=5):
     return res
 
 
+def bench_hoisted_level(P, gs=16, bs=4, reps=3):
+    """The giant step of one level of the slot <-> coefficient transforms (EncodingMatrix::Giant_Rotate_And_Mult_PlaintT) on the
+    reference's logN = 16 parameter set at the top level: gs - 1 keyed rotations and the unrotated pair, each multiplied into bs
+    baby steps.  Algorithmic bytes: every key once, the digits, P * (a, b), every plaintext and the bs output pairs once."""
+    import ctypes as C
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    R = P.REF_PARAMS[16]
+    ctx = Context_23(16, R["p"], R["q"], R["t"], R["gamma"])
+    N, T, RB, dnum, l = ctx.N, ctx.t_num, ctx.Ri_blockNum, ctx.dnum, ctx.L
+    digits, blockNum = -(-(l + 1) // ctx.K), -(-(ctx.K + l + 1) // ctx.gamma)
+    rng = np.random.default_rng(8)
+    chunk = DeviceBuffer.from_numpy(rng.integers(0, min(R["t"]), size=8 * N, dtype=np.uint64))
+
+    def filled(limbs):
+        buf = DeviceBuffer(8 * N * limbs)
+        for i in range(0, limbs, 8):
+            n = min(8, limbs - i)
+            buf.L_.ckks_memcpy_d2d(buf.ptr + 8 * N * i, chunk.ptr, 8 * N * n)
+        return buf
+
+    keys = [None] + [filled(2 * dnum * RB * T) for _ in range(gs - 1)]
+    plains = [filled(T) for _ in range(bs * gs)]
+    up, pqT, out = filled(ctx.Qj_blockNum * T), filled(2 * RB * T), DeviceBuffer(8 * N * bs * 2 * RB * T)
+    tab = lambda bufs: (C.c_void_p * len(bufs))(*[(b.ptr if b is not None else None) for b in bufs])
+    ints = lambda v: (C.c_int * len(v))(*v)
+    args = (ctx.h, out.ptr, pqT.ptr, up.ptr, tab(keys), ints([-1] + list(range(1, gs))), tab(plains), ints([gs] * bs), bs, gs, l)
+    assert ctx.L_.ckks_giant_rotate_mult_plain_t(*args) == 0
+    ctx.timer_start()
+    for _ in range(reps):
+        ctx.L_.ckks_giant_rotate_mult_plain_t(*args)
+    ms = ctx.timer_stop() / reps
+    limbs = (gs - 1) * 2 * digits * blockNum * T + digits * T + 2 * blockNum * T + bs * gs * T + bs * 2 * blockNum * T
+    nbytes = limbs * 8 * N
+    return {"workload": "Giant_Rotate_And_Mult_PlaintT N=2^16, reference logN=16 primes (28 Q, 4 P, 8 T of 60 bits), level 27, gs=%d bs=%d" % (gs, bs),
+            "ms": round(ms, 3),
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(nbytes / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": nbytes}}
+
+
 def run(P):
     return {"ppmm": bench_ppmm(P), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P),
-            "decompose": bench_decompose(P), "packing": bench_packing(P)}
+            "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}

@@ -61,6 +61,11 @@ def _declare(L):
         "ckks_mult_23": (i, [vp, vp, vp, vp, vp, i, vp, vp, vp, vp]),
         "ckks_rotate_23": (i, [vp, vp, vp, vp, l, i, vp, vp, vp, vp]),
         "ckks_conjugate_23": (i, [vp, vp, vp, vp, i, vp, vp, vp, vp]),
+        "ckks_cipher_mul_p": (i, [vp, vp, vp, i]), "ckks_cipher_add_t": (i, [vp, vp, vp, i]), "ckks_rescale_coeff": (i, [vp, vp, i]),
+        "ckks_giant_rotate_mult_plain_t": (i, [vp, vp, vp, vp, C.POINTER(vp), C.POINTER(i), C.POINTER(vp), C.POINTER(i), i, i, i]),
+        "ckks_baby_rotate": (i, [vp, vp, vp, vp, i, C.POINTER(vp), C.POINTER(i), i]),
+        "ckks_bsgs_scratch_words": (i, [vp, i, C.POINTER(sz)]),
+        "ckks_bsgs_level_23": (i, [vp, vp, i, C.POINTER(vp), C.POINTER(i), C.POINTER(i), C.POINTER(vp), C.POINTER(i), C.POINTER(vp), i, i, vp]),
         "pcmm_ctx_create": (i, [C.POINTER(vp), vp, i, i, u64p, i, u64p, i]), "pcmm_ctx_destroy": (i, [vp]),
         "pcmm_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "pcmm_rlwe_decompose": (i, [vp, vp, C.POINTER(vp), i, i]),

@@ -406,6 +406,13 @@ class Scheme_23:
                                    self.rotKey_vec_23[rotSlots].cipher_device.ptr, rotSlots, cipher.l, *self._ks_buffers()), "ckks_rotate_23")
         cipher_res.l, cipher_res.scale, cipher_res.slots = cipher.l, cipher.scale, cipher.slots
 
+    def rescaleAndEqual_noNTT(self, cipher):
+        """Scheme_23.cuh:427-440: rescale of a coefficient-domain ciphertext."""
+        c = self.context
+        _check(c.L_.ckks_rescale_coeff(c.h, cipher.cipher_device.ptr, cipher.l), "ckks_rescale_coeff")
+        cipher.scale = cipher.scale / c.qVec[cipher.l]
+        cipher.l -= 1
+
     def conjugate_23(self, cipher_res, cipher):
         """KeySwitch_23.cuh:433-468."""
         c = self.context
@@ -499,6 +506,77 @@ class PCMM_Context:
                 self.h = None
         except Exception:
             pass
+
+
+class PlaintextT:
+    """PlaintextT (bootstrapping/Bootstrapping_encoding.h): a plaintext over the T primes, NTT domain, t_num limbs, as the slot <->
+    coefficient transforms multiply it into rotated ciphertexts."""
+
+    def __init__(self, N, t_num, scale=1.0):
+        self.N, self.t_num, self.scale = N, t_num, scale
+        self.mx_device = DeviceBuffer(8 * N * t_num)
+
+
+def _addr_or_null(x):
+    if x is None:
+        return None
+    return _addr(x.cipher_device if hasattr(x, "cipher_device") else x.mx_device if hasattr(x, "mx_device") else x)
+
+
+def _ptr_table(items):
+    T = C.c_void_p * max(len(items), 1)
+    return T(*[_addr_or_null(x) for x in items])
+
+
+def _int_table(vals):
+    T = C.c_int * max(len(vals), 1)
+    return T(*[int(v) for v in vals])
+
+
+class EncodingMatrix:
+    """The hoisted baby-step / giant-step part of EncodingMatrix (Bootstrapping_C2S_S2C_impl.cuh): Giant_Rotate_And_Mult_PlaintT,
+    Baby_Rotate, and one level of EvalCoeffsToSlots / EvalSlotsToCoeffs around them.  The plaintext diagonals and the rotation
+    tables of a level (A[s], rot_in[s], rot_out[s]) come from the caller; their generation belongs to the bootstrapping set-up and
+    is not part of this library."""
+
+    def __init__(self, scheme):
+        self.scheme = scheme
+        self._scratch = None
+
+    def Giant_Rotate_And_Mult_PlaintT(self, bs_cipher_T, PQ_to_T_temp, modUp_QjtoT_temp, rotKey_pointer, rotSlots_vec, plaintextT_pointer,
+                                      accNum_vec, bs, gs, l):
+        c = self.scheme.context
+        _check(c.L_.ckks_giant_rotate_mult_plain_t(c.h, _addr(bs_cipher_T), _addr(PQ_to_T_temp), _addr(modUp_QjtoT_temp), _ptr_table(rotKey_pointer),
+                                                   _int_table(rotSlots_vec), _ptr_table(plaintextT_pointer), _int_table(accNum_vec), bs, gs, l),
+               "Giant_Rotate_And_Mult_PlaintT")
+
+    def Baby_Rotate(self, output, modUp_QjtoT_temp, input, rotNum_here, rotKey_pointer, rotSlots_vec, l):
+        c = self.scheme.context
+        _check(c.L_.ckks_baby_rotate(c.h, _addr(output), _addr(modUp_QjtoT_temp), _addr(input), rotNum_here, _ptr_table(rotKey_pointer),
+                                     _int_table(rotSlots_vec), l), "Baby_Rotate")
+
+    def EvalLevel(self, A_s, cipher, rot_in, rot_out, b, g, numRotations, rescale=True):
+        """One pass of the level loop (Bootstrapping_C2S_S2C_impl.cuh:254-382): cipher is in the COEFFICIENT domain and stays there.
+        A_s[G + j] is the plaintext of baby step G / g and rotation j; index numRotations has none (:290-300).  Keys are taken from
+        scheme.rotKey_vec_23; a missing one raises ValueError as the reference's key switches do."""
+        sch, c = self.scheme, self.scheme.context
+        plain, acc = [None] * (b * g), [0] * b
+        for i in range(b):
+            for j in range(g):
+                if i * g + j != numRotations and i * g + j < len(A_s):
+                    plain[i * g + j] = A_s[i * g + j]
+                    acc[i] += 1
+        key = lambda r: sch.rotKey_vec_23.get(r) if r else None
+        words = C.c_size_t(0)
+        _check(c.L_.ckks_bsgs_scratch_words(c.h, b, C.byref(words)), "ckks_bsgs_scratch_words")
+        if self._scratch is None or self._scratch.nbytes < 8 * words.value:
+            self._scratch = DeviceBuffer(8 * words.value)
+        _check(c.L_.ckks_bsgs_level_23(c.h, _addr(cipher.cipher_device), cipher.l, _ptr_table(plain), _int_table(acc), _int_table(rot_in),
+                                       _ptr_table([key(r) for r in rot_in]), _int_table(rot_out), _ptr_table([key(r) for r in rot_out]), b, g,
+                                       self._scratch.ptr), "EvalLevel")
+        cipher.scale = cipher.scale * A_s[0].scale
+        if rescale:
+            self.scheme.rescaleAndEqual_noNTT(cipher)
 
 
 class MLWESecretKey:

@@ -197,6 +197,41 @@ int ckks_rotate_23(ckks_ctx* ctx, uint64_t* out, const uint64_t* cipher, const u
 int ckks_conjugate_23(ckks_ctx* ctx, uint64_t* out, const uint64_t* cipher, const uint64_t* conjkey, int l, uint64_t* work,
                       uint64_t* modUp_QjtoT_temp, uint64_t* exProduct_T_temp, uint64_t* modUp_TtoQj_buffer);
 
+/* ---- hoisted rotations of the slot <-> coefficient transforms (baby-step / giant-step in the T basis) ---- */
+/* cipher_mul_P_batch as the transforms call it (poly_arithmetic.cuh:863-887; Bootstrapping_C2S_S2C_impl.cuh:270): cipher is a pair of
+ * L+1 limbs (coefficient or NTT domain), out a pair of K+L+1 limbs over [P | Q]: special limbs zero, limb K+i = c_i * P mod q_i for
+ * i <= l, limbs above l untouched. */
+int ckks_cipher_mul_p(ckks_ctx* ctx, uint64_t* out, const uint64_t* cipher, int l);
+/* cipher_add_T_batch_device (poly_arithmetic.cuh:143-153, 409-413): a += b on `blocks` groups of t_num limbs modulo the T primes. */
+int ckks_cipher_add_t(ckks_ctx* ctx, uint64_t* a, const uint64_t* b, int blocks);
+/* Scheme_23::rescaleAndEqual_noNTT (Scheme_23.cuh:321-337, 427-440): rescale of a coefficient-domain pair from level l to l-1 in
+ * place; limb l is left as it is.  Level 0 is refused. */
+int ckks_rescale_coeff(ckks_ctx* ctx, uint64_t* cipher, int l);
+/* EncodingMatrix::Giant_Rotate_And_Mult_PlaintT (Bootstrapping_C2S_S2C_impl.cuh:7-152).  PQ_to_T = P * (a, b) in the T basis, NTT
+ * domain, [a | b][Ri_blockNum][t_num] limbs; modUp_QjtoT = the digits of a in T, NTT domain, [digit][t_num]; rotKeys_host[j], j < gs:
+ * device pointer to the rotation key of rotSlots_host[j] slots ([a | b][dnum][Ri_blockNum][t_num]) or NULL for "no rotation";
+ * plaintextT_host[i * gs + j]: device pointer to t_num limbs of the plaintext (T basis, NTT domain) of baby step i < bs and
+ * rotation j, read for j < accNum_host[i].  bs_cipher_T[i] = sum_j plaintext(i, j) * rot_j(cipher) as pairs
+ * [bs][a | b][Ri_blockNum][t_num]; blocks at and above ceil((K+l+1)/gamma) are untouched.  The reference instantiates
+ * (gs, bs) = (16, 4), (16, 2), (8, 2); here 1 <= gs <= 16, 1 <= bs <= 8.  All four tables are host arrays. */
+int ckks_giant_rotate_mult_plain_t(ckks_ctx* ctx, uint64_t* bs_cipher_T, const uint64_t* PQ_to_T, const uint64_t* modUp_QjtoT,
+                                   const uint64_t* const* rotKeys_host, const int* rotSlots_host, const uint64_t* const* plaintextT_host,
+                                   const int* accNum_host, int bs, int gs, int l);
+/* EncodingMatrix::Baby_Rotate (Bootstrapping_C2S_S2C_impl.cuh:154-228): output (a pair in T, NTT domain) += the pair `input`
+ * rotated with each of the rotNum <= 16 keys given (NULL entries are skipped); modUp_QjtoT holds the digits of input's a part
+ * after its ModDown.  output != input. */
+int ckks_baby_rotate(ckks_ctx* ctx, uint64_t* output, const uint64_t* modUp_QjtoT, const uint64_t* input, int rotNum,
+                     const uint64_t* const* rotKeys_host, const int* rotSlots_host, int l);
+/* One level of EncodingMatrix::EvalCoeffsToSlots / EvalSlotsToCoeffs (Bootstrapping_C2S_S2C_impl.cuh:254-382, 531-625) up to, not
+ * including, its rescale: cipher (pair of L+1 limbs, COEFFICIENT domain, level l) becomes, in place,
+ * sum_{i<bs} rot_out[i]( sum_{j<accNum[i]} plaintext(i, j) * rot_in[j](cipher) ); a rotation by 0 slots needs no key, rot_out[0] is
+ * not applied (as in the reference).  A missing key for a non-zero rotation returns CKKS_E_STATE.
+ * scratch: ckks_bsgs_scratch_words(ctx, bs) words. */
+int ckks_bsgs_scratch_words(const ckks_ctx* ctx, int bs, size_t* words);
+int ckks_bsgs_level_23(ckks_ctx* ctx, uint64_t* cipher, int l, const uint64_t* const* plaintextT_host, const int* accNum_host,
+                       const int* rot_in_host, const uint64_t* const* rot_in_keys_host, const int* rot_out_host,
+                       const uint64_t* const* rot_out_keys_host, int bs, int gs, uint64_t* scratch);
+
 /* ---- ring-packed PCMM ---- */
 /* PCMM_Context::PCMM_Context (PCMM_Context.cuh:7-57) */
 int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int mlwe_rank, const uint64_t* p_ringpack, int p_count,

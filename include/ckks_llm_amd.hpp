@@ -374,6 +374,12 @@ public:
         cipher_res.scale = cipher.scale;
         cipher_res.slots = cipher.slots;
     }
+    // Scheme_23::rescaleAndEqual_noNTT (Scheme_23.cuh:427-440): rescale of a coefficient-domain ciphertext
+    void rescaleAndEqual_noNTT(Ciphertext& cipher) {
+        check(ckks_rescale_coeff(context.handle, cipher.cipher_device, cipher.l), "rescaleAndEqual_noNTT");
+        cipher.scale = cipher.scale / (long double)context.qVec[(size_t)cipher.l];
+        cipher.l -= 1;
+    }
     // Scheme_23::conjugate_23 (KeySwitch_23.cuh:433-468)
     void conjugate_23(Ciphertext& cipher_res, Ciphertext& cipher) {
         check(ckks_conjugate_23(context.handle, cipher_res.cipher_device, cipher.cipher_device, ConjKey_23 ? ConjKey_23->cipher_device : nullptr,
@@ -413,6 +419,83 @@ private:
         if (!publicKey) throw std::invalid_argument("encryptMsg: no encryption key (addEncKey)");
         context.generateRandom_device(in_enc, (uint64_tt)random_len_for_enc);
         check(ckks_encrypt(context.handle, cipher.cipher_device, mx, publicKey->cipher_device, in_enc, vx_enc, l), "encryptMsg");
+    }
+};
+
+
+// PlaintextT (bootstrapping/Bootstrapping_encoding.h): a plaintext over the T primes, NTT domain, t_num limbs.
+class PlaintextT {
+public:
+    uint64_tt* mx_device = nullptr;
+    int N = 0, t_num = 0;
+    long double scale = 1;
+
+    PlaintextT(int N, int t_num, long double scale) : N(N), t_num(t_num), scale(scale) { mx_device = device_alloc_words((size_t)N * t_num); }
+    PlaintextT(const PlaintextT&) = delete;
+    PlaintextT& operator=(const PlaintextT&) = delete;
+    virtual ~PlaintextT() { device_release(mx_device); }
+};
+
+// The hoisted baby-step / giant-step part of EncodingMatrix (Bootstrapping_C2S_S2C_impl.cuh): Giant_Rotate_And_Mult_PlaintT,
+// Baby_Rotate, and one level of EvalCoeffsToSlots / EvalSlotsToCoeffs around them.  The plaintext diagonals and rotation tables
+// of a level come from the caller: generating them is the bootstrapping's set-up, which is not part of this library.
+class EncodingMatrix {
+public:
+    Scheme_23& scheme;
+    uint64_tt* scratch = nullptr;
+    size_t scratch_words = 0;
+
+    explicit EncodingMatrix(Scheme_23& scheme) : scheme(scheme) {}
+    EncodingMatrix(const EncodingMatrix&) = delete;
+    ~EncodingMatrix() { device_release(scratch); }
+
+    // Bootstrapping_C2S_S2C_impl.cuh:93-152
+    void Giant_Rotate_And_Mult_PlaintT(uint64_tt* bs_cipher_T, uint64_tt* PQ_to_T_temp, int rotNum_here, uint64_tt* modUp_QjtoT_temp,
+                                       std::vector<uint64_tt*> rotKey_pointer, std::vector<int> rotSlots_vec, std::vector<uint64_tt*> plaintextT_pointer,
+                                       std::vector<int> accNum_vec, int bs, int gs, int l) {
+        (void)rotNum_here;                       // carried for the reference's signature; its kernel runs over gs
+        if ((int)rotKey_pointer.size() < gs || (int)rotSlots_vec.size() < gs || (int)plaintextT_pointer.size() < bs * gs || (int)accNum_vec.size() < bs)
+            throw std::invalid_argument("Giant_Rotate_And_Mult_PlaintT: a table is shorter than gs / bs * gs / bs");
+        check(ckks_giant_rotate_mult_plain_t(scheme.context.handle, bs_cipher_T, PQ_to_T_temp, modUp_QjtoT_temp, rotKey_pointer.data(), rotSlots_vec.data(),
+                                             plaintextT_pointer.data(), accNum_vec.data(), bs, gs, l), "Giant_Rotate_And_Mult_PlaintT");
+    }
+    // Bootstrapping_C2S_S2C_impl.cuh:203-228
+    void Baby_Rotate(uint64_tt* output, uint64_tt* modUp_QjtoT_temp, uint64_tt* input, int rotNum_here, std::vector<uint64_tt*> rotKey_pointer,
+                     std::vector<int> rotSlots_vec, int l) {
+        if ((int)rotKey_pointer.size() < rotNum_here || (int)rotSlots_vec.size() < rotNum_here) throw std::invalid_argument("Baby_Rotate: a table is shorter than rotNum_here");
+        check(ckks_baby_rotate(scheme.context.handle, output, modUp_QjtoT_temp, input, rotNum_here, rotKey_pointer.data(), rotSlots_vec.data(), l), "Baby_Rotate");
+    }
+    // One pass of the level loop (Bootstrapping_C2S_S2C_impl.cuh:254-382): cipher is in the COEFFICIENT domain and stays there.
+    // A_s[G + j] is the plaintext of baby step G / g and rotation j, index numRotations has none (:290-300); keys come from
+    // scheme.rotKey_vec_23, a missing one throws std::invalid_argument.
+    void EvalLevel(std::vector<PlaintextT*>& A_s, Ciphertext& cipher, const std::vector<int>& rot_in, const std::vector<int>& rot_out, int b, int g,
+                   int numRotations, bool rescale = true) {
+        if ((int)rot_in.size() < g || (int)rot_out.size() < b) throw std::invalid_argument("EvalLevel: a rotation table is shorter than g / b");
+        std::vector<const uint64_tt*> plain((size_t)b * g, nullptr), in_keys((size_t)g, nullptr), out_keys((size_t)b, nullptr);
+        std::vector<int> acc((size_t)b, 0);
+        for (int i = 0; i < b; i++)
+            for (int j = 0; j < g; j++)
+                if (i * g + j != numRotations && (size_t)(i * g + j) < A_s.size()) {
+                    plain[(size_t)i * g + j] = A_s[(size_t)i * g + j]->mx_device;
+                    acc[(size_t)i]++;
+                }
+        auto key = [&](int r) -> const uint64_tt* {
+            if (r <= 0 || (size_t)r >= scheme.rotKey_vec_23.size() || !scheme.rotKey_vec_23[(size_t)r]) return nullptr;
+            return scheme.rotKey_vec_23[(size_t)r]->cipher_device;
+        };
+        for (int j = 0; j < g; j++) in_keys[(size_t)j] = key(rot_in[(size_t)j]);
+        for (int i = 0; i < b; i++) out_keys[(size_t)i] = key(rot_out[(size_t)i]);
+        size_t words = 0;
+        check(ckks_bsgs_scratch_words(scheme.context.handle, b, &words), "ckks_bsgs_scratch_words");
+        if (words > scratch_words) {
+            device_release(scratch);
+            scratch = device_alloc_words(words);
+            scratch_words = words;
+        }
+        check(ckks_bsgs_level_23(scheme.context.handle, cipher.cipher_device, cipher.l, plain.data(), acc.data(), rot_in.data(), in_keys.data(),
+                                 rot_out.data(), out_keys.data(), b, g, scratch), "EvalLevel");
+        cipher.scale *= A_s.at(0)->scale;
+        if (rescale) scheme.rescaleAndEqual_noNTT(cipher);
     }
 };
 

@@ -1237,6 +1237,192 @@ int orc_conjugate_23(const orc_ctx* c, u64* out, const u64* cipher, const u64* c
 }
 
 // ------------------------------------------------------------------------------------------------
+// hoisted rotations of the slot <-> coefficient transforms (baby-step / giant-step over the T basis)
+// ------------------------------------------------------------------------------------------------
+// index the kernels read for output slot x under the rotation by `slots` (Bootstrapping_C2S_S2C_impl.cuh:37-41, 175-179):
+// with e = 2 * bitrev(x) + 1, bitrev(((5^slots * e mod 2N) - 1) / 2)
+static inline long hoist_perm(const orc_ctx* c, u64 pow, long x) {
+    const u64 mask = 2 * (u64)c->N - 1;
+    u64 e = 2 * (u64)orc_bitrev((uint32_t)x, c->logN) + 1;
+    e = (((pow * e) & mask) - 1) >> 1;
+    return (long)orc_bitrev((uint32_t)e, c->logN);
+}
+// cipher_mul_P_batch as the transforms call it (poly_arithmetic.cuh:863-887, Bootstrapping_C2S_S2C_impl.cuh:270): out is a pair over
+// [P | Q] (K+L+1 limbs each); the special limbs are zero, limb K+i = cipher limb i times (P mod q_i), i <= l; the rest is untouched
+int orc_cipher_mul_p(const orc_ctx* c, u64* out, const u64* cipher, int l) {
+    const long N = c->N; const int K = c->K, L = c->L;
+    if (l < 0 || l > L || K <= 0) return -1;
+    for (int z = 0; z < 2; z++) {
+        std::fill(out + (size_t)z * (K + L + 1) * N, out + ((size_t)z * (K + L + 1) + K) * N, 0);
+        for (int i = 0; i <= l; i++) {
+            const u64 q = c->pqt[K + i];
+            for (long x = 0; x < N; x++)
+                out[((size_t)z * (K + L + 1) + K + i) * N + x] = orc_mulmod(cipher[((size_t)z * (L + 1) + i) * N + x], c->PModqt[i], q);
+        }
+    }
+    return 0;
+}
+// cipher_add_T_batch_device (poly_arithmetic.cuh:143-153, 409-413): a += b on `blocks` groups of t_num limbs modulo the T primes
+int orc_cipher_add_t(const orc_ctx* c, u64* a, const u64* b, int blocks) {
+    const long N = c->N; const int T = c->t_num, base = c->p_num + c->q_num;
+    if (T <= 0 || blocks < 0) return -1;
+    for (int z = 0; z < blocks; z++)
+        for (int k = 0; k < T; k++) {
+            const u64 t = c->pqt[base + k];
+            for (long x = 0; x < N; x++) {
+                const size_t i = ((size_t)z * T + k) * N + x;
+                a[i] = csub_q(a[i] + b[i], t);
+            }
+        }
+    return 0;
+}
+// Scheme_23::rescaleAndEqual_noNTT (Scheme_23.cuh:321-337, 427-440): coefficient-domain pair, limb i < l becomes
+// (c_i + 2 q_i - c_l) * q_l^-1 mod q_i with the last limb used as an integer, not reduced modulo q_i first
+int orc_rescale_coeff(const orc_ctx* c, u64* cipher, int l) {
+    const long N = c->N; const int K = c->K, L = c->L;
+    if (l < 1 || l > L) return -1;
+    const u64* inv = &c->qiInvModql[(size_t)l * (l - 1) / 2]; const u64* inv_s = &c->qiInvModql_shoup[(size_t)l * (l - 1) / 2];
+    for (int z = 0; z < 2; z++)
+        for (int i = 0; i < l; i++) {
+            const u64 q = c->pqt[K + i];
+            for (long x = 0; x < N; x++) {
+                const size_t idx = ((size_t)z * (L + 1) + i) * N + x;
+                u64 ra = cipher[idx] + 2 * q - cipher[((size_t)z * (L + 1) + l) * N + x];
+                ra = csub_q(ra, q);
+                cipher[idx] = orc_mulmod_shoup(ra, inv[i], inv_s[i], q);
+            }
+        }
+    return 0;
+}
+// EncodingMatrix::Giant_Rotate_And_Mult_PlaintT (Bootstrapping_C2S_S2C_impl.cuh:7-152).  For every rotation j < gs of the giant step
+// the rotated pair in the T basis is formed on the fly - without a key (null pointer) the pair P*(a, b) itself, with a key the
+// inner product of the digits of a with the key's two halves, plus P*b, all read at the rotation's index - and multiplied into the
+// accumulators of the baby steps i < bs whose plaintext j exists (j < accNum[i]): 128-bit sums, one reduction at the end.
+// PQ_to_T: [a | b][Ri_blockNum][t_num]; modUp_QjtoT: [digit][t_num]; key: [a | b][dnum][Ri_blockNum][t_num];
+// plaintext (i, j): t_num limbs; bs_cipher_T: [bs][a | b][Ri_blockNum][t_num].  Blocks at and beyond ceil((K+l+1)/gamma) are untouched.
+int orc_giant_rotate_mult_plain_t(const orc_ctx* c, u64* bs_cipher_T, const u64* PQ_to_T, const u64* modUp_QjtoT, const u64* const* rotKeys,
+                                  const int* rotSlots, const u64* const* plaintextT, const int* accNum, int bs, int gs, int l) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum;
+    if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L || bs < 1 || gs < 1 || bs > 16) return -1;
+    const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+    const size_t half = (size_t)RB * T * N;
+    std::vector<u64> pows(gs, 1);
+    for (int j = 0; j < gs; j++) if (rotKeys[j]) pows[j] = orc_rot_group(c, rotSlots[j]);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int blk = 0; blk < blockNum; blk++)
+        for (int k = 0; k < T; k++)
+            for (long x = 0; x < N; x++) {
+                const size_t idx = (size_t)x + ((size_t)blk * T + k) * N;
+                u128 acc_a[16], acc_b[16];
+                for (int i = 0; i < bs; i++) acc_a[i] = acc_b[i] = 0;
+                for (int j = 0; j < gs; j++) {
+                    u64 ea, eb;
+                    if (!rotKeys[j]) {
+                        ea = PQ_to_T[idx]; eb = PQ_to_T[idx + half];
+                    } else {
+                        const long px = hoist_perm(c, pows[j], x);
+                        u128 a1 = 0, a2 = 0;
+                        for (int i = 0; i < cipher_blockNum; i++) {
+                            const u64 d = modUp_QjtoT[((size_t)i * T + k) * N + px];
+                            const size_t kidx = ((size_t)i * T * RB + (size_t)blk * T + k) * N + px;
+                            a1 += (u128)d * rotKeys[j][kidx];
+                            a2 += (u128)d * rotKeys[j][half * dnum + kidx];
+                        }
+                        a2 += PQ_to_T[(size_t)px + ((size_t)blk * T + k) * N + half];
+                        ea = barrett_idx(c, a1, P + Q + k); eb = barrett_idx(c, a2, P + Q + k);
+                    }
+                    for (int i = 0; i < bs; i++)
+                        if (j < accNum[i]) {
+                            const u64 mx = plaintextT[(size_t)i * gs + j][(size_t)k * N + x];
+                            acc_a[i] += (u128)ea * mx; acc_b[i] += (u128)eb * mx;
+                        }
+                }
+                for (int i = 0; i < bs; i++) {
+                    bs_cipher_T[idx + (size_t)(2 * i) * half] = barrett_idx(c, acc_a[i], P + Q + k);
+                    bs_cipher_T[idx + (size_t)(2 * i + 1) * half] = barrett_idx(c, acc_b[i], P + Q + k);
+                }
+            }
+    return 0;
+}
+// EncodingMatrix::Baby_Rotate (Bootstrapping_C2S_S2C_impl.cuh:154-228): output (a pair in the T basis) += the pair `input` rotated
+// with each key given: a += <digits, key_a>, b += <digits, key_b> + input_b, digits / keys / input_b read at the rotation's index
+int orc_baby_rotate(const orc_ctx* c, u64* output, const u64* modUp_QjtoT, const u64* input, int rotNum, const u64* const* rotKeys,
+                    const int* rotSlots, int l) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum;
+    if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L || rotNum < 0) return -1;
+    const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+    const size_t half = (size_t)RB * T * N;
+    for (int r = 0; r < rotNum; r++) {
+        if (!rotKeys[r]) continue;
+        const u64 pow = orc_rot_group(c, rotSlots[r]);
+        std::vector<u64> next_a(half), next_b(half);
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int blk = 0; blk < blockNum; blk++)
+            for (int k = 0; k < T; k++)
+                for (long x = 0; x < N; x++) {
+                    const size_t idx = (size_t)x + ((size_t)blk * T + k) * N;
+                    const long px = hoist_perm(c, pow, x);
+                    u128 a1 = 0, a2 = 0;
+                    for (int i = 0; i < cipher_blockNum; i++) {
+                        const u64 d = modUp_QjtoT[((size_t)i * T + k) * N + px];
+                        const size_t kidx = ((size_t)i * T * RB + (size_t)blk * T + k) * N + px;
+                        a1 += (u128)d * rotKeys[r][kidx];
+                        a2 += (u128)d * rotKeys[r][half * dnum + kidx];
+                    }
+                    a1 += output[idx];
+                    a2 += input[(size_t)px + ((size_t)blk * T + k) * N + half];
+                    a2 += output[idx + half];
+                    next_a[idx] = barrett_idx(c, a1, P + Q + k); next_b[idx] = barrett_idx(c, a2, P + Q + k);
+                }
+        for (int blk = 0; blk < blockNum; blk++)
+            for (int k = 0; k < T; k++) {
+                const size_t o = ((size_t)blk * T + k) * N;
+                std::copy(next_a.begin() + o, next_a.begin() + o + N, output + o);
+                std::copy(next_b.begin() + o, next_b.begin() + o + N, output + half + o);
+            }
+    }
+    return 0;
+}
+// One level of EncodingMatrix::EvalCoeffsToSlots / EvalSlotsToCoeffs (Bootstrapping_C2S_S2C_impl.cuh:254-382, 531-625) without
+// its final rescale: cipher (coefficient domain, level l, in place) becomes sum_i rot_out[i]( sum_{j < accNum[i]} plain[i][j] *
+// rot_in[j](cipher) ).  A rotation by 0 slots takes no key (null).
+int orc_bsgs_level_23(const orc_ctx* c, u64* cipher, int l, const u64* const* plaintextT, const int* accNum, const int* rot_in,
+                      const u64* const* rot_in_keys, const int* rot_out, const u64* const* rot_out_keys, int bs, int gs) {
+    const long N = c->N; const int K = c->K, L = c->L, T = c->t_num, RB = c->Ri_blockNum, g = c->gamma;
+    if (g <= 0 || T <= 0 || K <= 0 || l < 0 || l > L || bs < 1 || gs < 1) return -1;
+    const int cipher_blockNum = ceil_div(l + 1, K), blockNum = ceil_div(K + l + 1, g);
+    const size_t half = (size_t)RB * T * N;
+    std::vector<u64> up((size_t)N * T * c->Qj_blockNum, 0), pq((size_t)2 * (K + L + 1) * N, 0), pqT(2 * half, 0), bsT((size_t)bs * 2 * half, 0),
+        gsT(2 * half, 0), back(2 * half, 0);          // the T -> PQ buffer keeps the T-basis stride between a and b
+    orc_modup_qj_to_t(c, up.data(), cipher, l, 1);                                                   // :262
+    orc_ntt_fwd(c, up.data(), 0, K + L + 1, cipher_blockNum, T, T);                                  // :263
+    orc_cipher_mul_p(c, pq.data(), cipher, l);                                                       // :267
+    orc_modup_pq_to_t(c, pqT.data(), pq.data(), l, 2);                                               // :270
+    orc_ntt_fwd_ext(c, pqT.data(), 0, K + L + 1, blockNum, T, T, RB * T, 2);                         // :272
+    std::vector<const u64*> keys(gs);
+    std::vector<int> slots(gs);
+    for (int j = 0; j < gs; j++) { keys[j] = rot_in[j] != 0 ? rot_in_keys[j] : nullptr; slots[j] = rot_in[j] != 0 ? rot_in[j] : -1; }   // :275-288
+    if (orc_giant_rotate_mult_plain_t(c, bsT.data(), pqT.data(), up.data(), keys.data(), slots.data(), plaintextT, accNum, bs, gs, l)) return -1;
+    for (int i = 1; i < bs; i++) {                                                                   // :326-356
+        u64* part = bsT.data() + (size_t)i * 2 * half;
+        if (rot_out[i] == 0) { orc_cipher_add_t(c, bsT.data(), part, RB * 2); continue; }
+        std::copy(part, part + 2 * half, gsT.begin());
+        orc_ntt_inv_ext(c, part, 0, K + L + 1, blockNum, T, T, RB * T, 2);
+        orc_modup_t_to_pql(c, back.data(), part, l, 1);
+        orc_moddown_pql_to_ql(c, cipher, back.data(), l, 1);
+        orc_modup_qj_to_t(c, up.data(), cipher, l, 1);
+        orc_ntt_fwd(c, up.data(), 0, K + L + 1, cipher_blockNum, T, T);
+        const u64* key1[1] = {rot_out_keys[i]};
+        const int slot1[1] = {rot_out[i]};
+        if (orc_baby_rotate(c, bsT.data(), up.data(), gsT.data(), 1, key1, slot1, l)) return -1;
+    }
+    orc_ntt_inv_ext(c, bsT.data(), 0, K + L + 1, blockNum, T, T, RB * T, 2);                         // :359
+    orc_modup_t_to_pql(c, back.data(), bsT.data(), l, 2);                                            // :361
+    orc_moddown_pql_to_ql(c, cipher, back.data(), l, 2);                                             // :363
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
 // MLWE secret key, repacking keys, MLWE decryption (the key side of the ring-packed PCMM)
 // ------------------------------------------------------------------------------------------------
 // PCMM_Scheme::convertMLWESKfromRLWESK (PCMM_Scheme.cuh:23-48) with ringDown_kernel (ringSwitch.cuh:7-19): the RLWE secret

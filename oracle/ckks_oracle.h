@@ -152,6 +152,17 @@ int orc_keygen_switch_23(const orc_ctx*, uint64_t* swk, const uint64_t* s_to, co
 int orc_mult_23(const orc_ctx*, uint64_t* out, const uint64_t* c1, const uint64_t* c2, const uint64_t* rlk, int l);
 int orc_rotate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* rotkey, long rot, int l);
 int orc_conjugate_23(const orc_ctx*, uint64_t* out, const uint64_t* cipher, const uint64_t* conjkey, int l);
+/* hoisted rotations of the slot <-> coefficient transforms (Bootstrapping_C2S_S2C_impl.cuh) */
+int orc_cipher_mul_p(const orc_ctx*, uint64_t* out, const uint64_t* cipher, int l);
+int orc_cipher_add_t(const orc_ctx*, uint64_t* a, const uint64_t* b, int blocks);
+int orc_rescale_coeff(const orc_ctx*, uint64_t* cipher, int l);
+int orc_giant_rotate_mult_plain_t(const orc_ctx*, uint64_t* bs_cipher_T, const uint64_t* PQ_to_T, const uint64_t* modUp_QjtoT,
+                                  const uint64_t* const* rotKeys, const int* rotSlots, const uint64_t* const* plaintextT, const int* accNum,
+                                  int bs, int gs, int l);
+int orc_baby_rotate(const orc_ctx*, uint64_t* output, const uint64_t* modUp_QjtoT, const uint64_t* input, int rotNum,
+                    const uint64_t* const* rotKeys, const int* rotSlots, int l);
+int orc_bsgs_level_23(const orc_ctx*, uint64_t* cipher, int l, const uint64_t* const* plaintextT, const int* accNum, const int* rot_in,
+                      const uint64_t* const* rot_in_keys, const int* rot_out, const uint64_t* const* rot_out_keys, int bs, int gs);
 
 /* ---- MLWE secret key, repacking keys, MLWE decryption ---- */
 int orc_pcmm_convert_mlwe_sk(const orc_pcmm*, uint64_t* mlwe_sk, const uint64_t* rlwe_sk);

@@ -95,6 +95,10 @@ def lib():
             "orc_keygen_switch_23": (i, [vp, P64, P64, P64, P8, P8]),
             "orc_mult_23": (i, [vp, P64, P64, P64, P64, i]), "orc_rotate_23": (i, [vp, P64, P64, P64, l, i]),
             "orc_conjugate_23": (i, [vp, P64, P64, P64, i]),
+            "orc_cipher_mul_p": (i, [vp, P64, P64, i]), "orc_cipher_add_t": (i, [vp, P64, P64, i]), "orc_rescale_coeff": (i, [vp, P64, i]),
+            "orc_giant_rotate_mult_plain_t": (i, [vp, P64, P64, P64, C.POINTER(P64), C.POINTER(i), C.POINTER(P64), C.POINTER(i), i, i, i]),
+            "orc_baby_rotate": (i, [vp, P64, P64, P64, i, C.POINTER(P64), C.POINTER(i), i]),
+            "orc_bsgs_level_23": (i, [vp, P64, i, C.POINTER(P64), C.POINTER(i), C.POINTER(i), C.POINTER(P64), C.POINTER(i), C.POINTER(P64), i, i]),
             "orc_pcmm_convert_mlwe_sk": (i, [vp, P64, P64]), "orc_pcmm_add_repacking_key": (i, [vp, P64, P64, P64, P8]),
             "orc_pcmm_mlwe_decrypt": (i, [vp, P64, P64, P64, i]),
             "orc_pcmm_decode_coeffs": (i, [vp, C.POINTER(C.c_double), P64, C.c_longlong, i]),
@@ -250,6 +254,38 @@ class OracleContext:
 
     def conjugate_23(self, out, cipher, conjkey, l):
         self._ck(self.L_.orc_conjugate_23(self.h, _ptr(out), _ptr(cipher), _ptr(conjkey), l))
+
+    # hoisted rotations of the slot <-> coefficient transforms (Bootstrapping_C2S_S2C_impl.cuh); a missing key / plaintext is None
+    @staticmethod
+    def _ptr_table(arrs):
+        T = P64 * max(len(arrs), 1)
+        return T(*[(_ptr(a) if a is not None else P64()) for a in arrs])
+
+    @staticmethod
+    def _int_table(vals):
+        T = C.c_int * max(len(vals), 1)
+        return T(*[int(v) for v in vals])
+
+    def cipher_mul_P(self, out, cipher, l):
+        self._ck(self.L_.orc_cipher_mul_p(self.h, _ptr(out), _ptr(cipher), l))
+
+    def cipher_add_T(self, a, b, blocks):
+        self._ck(self.L_.orc_cipher_add_t(self.h, _ptr(a), _ptr(b), blocks))
+
+    def rescaleAndEqual_noNTT(self, cipher, l):
+        self._ck(self.L_.orc_rescale_coeff(self.h, _ptr(cipher), l))
+
+    def Giant_Rotate_And_Mult_PlaintT(self, bs_cipher_T, PQ_to_T, modUp_QjtoT, rotKeys, rotSlots, plaintextT, accNum, bs, gs, l):
+        self._ck(self.L_.orc_giant_rotate_mult_plain_t(self.h, _ptr(bs_cipher_T), _ptr(PQ_to_T), _ptr(modUp_QjtoT), self._ptr_table(rotKeys),
+                                                       self._int_table(rotSlots), self._ptr_table(plaintextT), self._int_table(accNum), bs, gs, l))
+
+    def Baby_Rotate(self, output, modUp_QjtoT, inp, rotKeys, rotSlots, l):
+        self._ck(self.L_.orc_baby_rotate(self.h, _ptr(output), _ptr(modUp_QjtoT), _ptr(inp), len(rotKeys), self._ptr_table(rotKeys),
+                                         self._int_table(rotSlots), l))
+
+    def bsgs_level_23(self, cipher, l, plaintextT, accNum, rot_in, rot_in_keys, rot_out, rot_out_keys, bs, gs):
+        self._ck(self.L_.orc_bsgs_level_23(self.h, _ptr(cipher), l, self._ptr_table(plaintextT), self._int_table(accNum), self._int_table(rot_in),
+                                           self._ptr_table(rot_in_keys), self._int_table(rot_out), self._ptr_table(rot_out_keys), bs, gs))
 
     def decode_coeffs(self, mx, scale, slots, l, is_bitrev=False):
         """Context_23::decode_coeffs (Encoder.cuh:113-186): iNTT of limbs 0..l, CRT to the centred integer modulo q_0..q_l

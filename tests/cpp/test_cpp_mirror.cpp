@@ -247,6 +247,41 @@ static int run() {
         threw = false;
         try { s2.mult_23(res, e1, lvl0); } catch (const std::invalid_argument&) { threw = true; }
         EXPECT(threw, "mult_23 on level 0 throws std::invalid_argument");
+        // one baby-step / giant-step level of the slot <-> coefficient transforms through EncodingMatrix::EvalLevel, with the
+        // rotation key generated above and random plaintexts over T, against the oracle's level on the same words
+        {
+            const int T = c2.t_num, b = 2, g = 2, numRotations = 3;
+            std::vector<PlaintextT*> A;
+            std::vector<std::vector<uint64_tt>> A_host;
+            for (int i = 0; i < b * g; i++) {
+                A.push_back(new PlaintextT((int)n, T, 1.0L));
+                A_host.push_back(uniform_limbs(rng, t13, 1, n));
+                upload(A.back()->mx_device, A_host.back());
+            }
+            const std::vector<int> rot_in = {0, 7}, rot_out = {0, 7};
+            std::vector<const uint64_tt*> o_plain = {A_host[0].data(), A_host[1].data(), A_host[2].data(), nullptr};
+            const int o_acc[2] = {2, 1};
+            const uint64_tt* o_in_keys[2] = {nullptr, o_key.data()};
+            const uint64_tt* o_out_keys[2] = {nullptr, o_key.data()};
+            std::vector<uint64_tt> o_lvl = o_c1;
+            orc_ntt_inv(o2, o_lvl.data(), 0, K, 2, L1, L1);
+            orc_bsgs_level_23(o2, o_lvl.data(), c2.L, o_plain.data(), o_acc, rot_in.data(), o_in_keys, rot_out.data(), o_out_keys, b, g);
+            orc_rescale_coeff(o2, o_lvl.data(), c2.L);
+            Ciphertext lvl(e1);
+            c2.FromNTTInplace(lvl.cipher_device, 0, K, 2, L1, L1);
+            EncodingMatrix em(s2);
+            em.EvalLevel(A, lvl, rot_in, rot_out, b, g, numRotations);
+            std::vector<uint64_tt> got = download(lvl.cipher_device, o_lvl.size());
+            bool same = lvl.l == c2.L - 1;
+            for (int z = 0; z < 2 && same; z++)
+                for (size_t w = 0; w < (size_t)n * (L1 - 1); w++)
+                    if (got[(size_t)z * n * L1 + w] != o_lvl[(size_t)z * n * L1 + w]) { same = false; break; }
+            EXPECT(same, "EncodingMatrix::EvalLevel (hoisted rotations + rescale) == oracle");
+            threw = false;
+            try { em.EvalLevel(A, lvl, {0, 9}, rot_out, b, g, numRotations); } catch (const std::invalid_argument&) { threw = true; }
+            EXPECT(threw, "EvalLevel without a rotation key throws std::invalid_argument");
+            for (PlaintextT* a : A) delete a;
+        }
         orc_ctx_destroy(o2);
     }
 
