@@ -28,6 +28,57 @@ __device__ __forceinline__ long hoist_perm(u64 pow, long x, int logN, u64 mask) 
     return (long)(__brev((unsigned)e) >> (32 - logN));
 }
 
+// Sums of up to 16 products of operands below 2^60 without carries: the operands are split at bit 30 and the four partial
+// products, each below 2^60, are summed in four 64-bit words (16 x (2^30 - 1)^2 < 2^64), one 32 x 32 + 64-bit multiply-add each;
+// the 128-bit value is put together once per sum.  A 64 x 64 -> 128-bit multiply-add in 32-bit pieces with carry chains costs
+// about three times as many instructions, and these kernels are bound by them.
+struct Sum60 {
+    u64 s00, s01, s10, s11;
+};
+__device__ __forceinline__ void mac60(Sum60& s, u64 a, u64 b) {
+    const unsigned a0 = (unsigned)a & 0x3fffffffu, a1 = (unsigned)(a >> 30);
+    const unsigned b0 = (unsigned)b & 0x3fffffffu, b1 = (unsigned)(b >> 30);
+    s.s00 += (u64)a0 * b0;
+    s.s01 += (u64)a0 * b1;
+    s.s10 += (u64)a1 * b0;
+    s.s11 += (u64)a1 * b1;
+}
+__device__ __forceinline__ u128w fold60(const Sum60& s, u64 extra) {       // s00 + (s01 + s10) 2^30 + s11 2^60 + extra
+    u128w r{s.s00, 0};
+    const u64 m = s.s01 + s.s10;
+    const u64 mc = m < s.s01;                              // bit 64 of the middle sum
+    u64 lo = r.lo + (m << 30);
+    r.hi = (m >> 34) + (mc << 30) + (lo < r.lo);
+    r.lo = lo;
+    lo = r.lo + (s.s11 << 60);
+    r.hi += (s.s11 >> 4) + (lo < r.lo);
+    r.lo = lo;
+    lo = r.lo + extra;
+    r.hi += (lo < r.lo);
+    r.lo = lo;
+    return r;
+}
+// FAST: every T prime below 2^60 and at most 16 digits (so at most 16 terms per sum): the carry-free sums above
+template <bool FAST>
+struct Acc;
+template <>
+struct Acc<true> {
+    Sum60 s{0, 0, 0, 0};
+    __device__ __forceinline__ void mac(u64 a, u64 b) { mac60(s, a, b); }
+    __device__ __forceinline__ u128w value(u64 extra) const { return fold60(s, extra); }
+};
+template <>
+struct Acc<false> {
+    u128w s{0, 0};
+    __device__ __forceinline__ void mac(u64 a, u64 b) { mac128(s, a, b); }
+    __device__ __forceinline__ u128w value(u64 extra) const {
+        u128w r = s;
+        r.lo += extra;
+        r.hi += (r.lo < extra);
+        return r;
+    }
+};
+
 struct GiantArgs {
     u64* out;                       // [bs][a | b][Ri_blockNum][t_num] limbs
     const u64* pqT;                 // P * (a, b) in T: [a | b][Ri_blockNum][t_num]
@@ -43,7 +94,7 @@ struct GiantArgs {
 
 // one lane per (block, T prime, slot); per rotation of the giant step the rotated pair is formed once and multiplied into the
 // accumulators of all baby steps
-template <int BS>
+template <int BS, bool FAST>
 __global__ __launch_bounds__(THREADS) void giant_rotate_mult_kernel(GiantArgs a) {
     const long x = (long)blockIdx.x * THREADS + threadIdx.x;
     const int k = blockIdx.y, blk = blockIdx.z;
@@ -52,9 +103,7 @@ __global__ __launch_bounds__(THREADS) void giant_rotate_mult_kernel(GiantArgs a)
     const u64 mask = 2 * (u64)N - 1;
     const size_t half = (size_t)a.RB * a.T * N;
     const size_t limb = ((size_t)blk * a.T + k) * N;
-    u128w acc_a[BS], acc_b[BS];
-#pragma unroll
-    for (int i = 0; i < BS; i++) { acc_a[i] = u128w{0, 0}; acc_b[i] = u128w{0, 0}; }
+    Acc<false> acc_a[BS], acc_b[BS];         // 128-bit sums here: the carry-free form would double their registers
     for (int j = 0; j < a.gs; j++) {
         const u64* key = a.key[j];
         u64 ea, eb;
@@ -63,32 +112,30 @@ __global__ __launch_bounds__(THREADS) void giant_rotate_mult_kernel(GiantArgs a)
             eb = a.pqT[limb + x + half];
         } else {
             const long px = hoist_perm(a.pow[j], x, a.logN, mask);
-            u128w s1{0, 0}, s2{0, 0};
+            Acc<FAST> s1, s2;
             for (int i = 0; i < a.digits; i++) {
                 const u64 d = a.up[((size_t)i * a.T + k) * N + px];
                 const size_t kidx = ((size_t)i * a.T * a.RB + (size_t)blk * a.T + k) * N + px;
-                mac128(s1, d, key[kidx]);
-                mac128(s2, d, key[half * a.dnum + kidx]);
+                s1.mac(d, key[kidx]);
+                s2.mac(d, key[half * a.dnum + kidx]);
             }
             const u64 b0 = a.pqT[limb + px + half];
-            s2.lo += b0;
-            s2.hi += (s2.lo < b0);
-            ea = barrett128(s1, p.q, p.mu_hi, p.mu_lo);
-            eb = barrett128(s2, p.q, p.mu_hi, p.mu_lo);
+            ea = barrett128(s1.value(0), p.q, p.mu_hi, p.mu_lo);
+            eb = barrett128(s2.value(b0), p.q, p.mu_hi, p.mu_lo);
         }
 #pragma unroll
         for (int i = 0; i < BS; i++)
             if (i < a.bs && j < a.acc_num[i]) {
                 const u64 mx = a.plain[i * a.gs + j][(size_t)k * N + x];
-                mac128(acc_a[i], ea, mx);
-                mac128(acc_b[i], eb, mx);
+                acc_a[i].mac(ea, mx);
+                acc_b[i].mac(eb, mx);
             }
     }
 #pragma unroll
     for (int i = 0; i < BS; i++)
         if (i < a.bs) {
-            a.out[limb + x + (size_t)(2 * i) * half] = barrett128(acc_a[i], p.q, p.mu_hi, p.mu_lo);
-            a.out[limb + x + (size_t)(2 * i + 1) * half] = barrett128(acc_b[i], p.q, p.mu_hi, p.mu_lo);
+            a.out[limb + x + (size_t)(2 * i) * half] = barrett128(acc_a[i].value(0), p.q, p.mu_hi, p.mu_lo);
+            a.out[limb + x + (size_t)(2 * i + 1) * half] = barrett128(acc_b[i].value(0), p.q, p.mu_hi, p.mu_lo);
         }
 }
 
@@ -102,6 +149,7 @@ struct BabyArgs {
     long N;
     int logN, T, RB, dnum, digits, prime0, rot_num;
 };
+template <bool FAST>
 __global__ __launch_bounds__(THREADS) void baby_rotate_kernel(BabyArgs a) {
     const long x = (long)blockIdx.x * THREADS + threadIdx.x;
     const int k = blockIdx.y, blk = blockIdx.z;
@@ -117,22 +165,19 @@ __global__ __launch_bounds__(THREADS) void baby_rotate_kernel(BabyArgs a) {
         if (!key) continue;
         any = true;
         const long px = hoist_perm(a.pow[r], x, a.logN, mask);
-        u128w s1{0, 0}, s2{0, 0};
+        Acc<FAST> s1, s2;
         for (int i = 0; i < a.digits; i++) {
             const u64 d = a.up[((size_t)i * a.T + k) * N + px];
             const size_t kidx = ((size_t)i * a.T * a.RB + (size_t)blk * a.T + k) * N + px;
-            mac128(s1, d, key[kidx]);
-            mac128(s2, d, key[half * a.dnum + kidx]);
+            s1.mac(d, key[kidx]);
+            s2.mac(d, key[half * a.dnum + kidx]);
         }
-        s1.lo += oa;
-        s1.hi += (s1.lo < oa);
         const u64 b0 = a.in[limb + px + half];
-        s2.lo += b0;
-        s2.hi += (s2.lo < b0);
-        s2.lo += ob;
-        s2.hi += (s2.lo < ob);
-        oa = barrett128(s1, p.q, p.mu_hi, p.mu_lo);
-        ob = barrett128(s2, p.q, p.mu_hi, p.mu_lo);
+        u128w v1 = s1.value(oa), v2 = s2.value(b0);
+        v2.lo += ob;
+        v2.hi += (v2.lo < ob);
+        oa = barrett128(v1, p.q, p.mu_hi, p.mu_lo);
+        ob = barrett128(v2, p.q, p.mu_hi, p.mu_lo);
     }
     if (any) {
         a.out[limb + x] = oa;
@@ -176,6 +221,14 @@ __global__ __launch_bounds__(THREADS) void rescale_coeff_kernel(u64* a, const Pr
     const size_t idx = ((size_t)z * q_num + i) * N + x;
     const u64 ra = csub(a[idx] + 2 * q - a[((size_t)z * q_num + l) * N + x], q);
     a[idx] = mul_shoup(ra, inv[i], inv_s[i], q);
+}
+
+// the carry-free sums need every operand below 2^60 and at most 16 terms per sum
+bool carry_free_ok(const ckks_ctx* c, int digits) {
+    if (digits > 16 || c->arith_mode == 1) return false;
+    for (int k = 0; k < c->t_num; k++)
+        if (c->pqt[(size_t)c->p_num + c->q_num + k] >= (1ull << 60)) return false;
+    return true;
 }
 
 int need_t_basis(const ckks_ctx* c, int l, const char* who) {
@@ -249,10 +302,17 @@ extern "C" int ckks_giant_rotate_mult_plain_t(ckks_ctx* c, uint64_t* bs_cipher_T
         }
     const int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;
     const dim3 grid((unsigned)(c->N / THREADS), c->t_num, blockNum), block(THREADS);
-    if (bs == 1) hipLaunchKernelGGL(giant_rotate_mult_kernel<1>, grid, block, 0, c->stream, a);
-    else if (bs == 2) hipLaunchKernelGGL(giant_rotate_mult_kernel<2>, grid, block, 0, c->stream, a);
-    else if (bs <= 4) hipLaunchKernelGGL(giant_rotate_mult_kernel<4>, grid, block, 0, c->stream, a);
-    else hipLaunchKernelGGL(giant_rotate_mult_kernel<8>, grid, block, 0, c->stream, a);
+    if (carry_free_ok(c, a.digits)) {
+        if (bs == 1) hipLaunchKernelGGL((giant_rotate_mult_kernel<1, true>), grid, block, 0, c->stream, a);
+        else if (bs == 2) hipLaunchKernelGGL((giant_rotate_mult_kernel<2, true>), grid, block, 0, c->stream, a);
+        else if (bs <= 4) hipLaunchKernelGGL((giant_rotate_mult_kernel<4, true>), grid, block, 0, c->stream, a);
+        else hipLaunchKernelGGL((giant_rotate_mult_kernel<8, true>), grid, block, 0, c->stream, a);
+    } else {
+        if (bs == 1) hipLaunchKernelGGL((giant_rotate_mult_kernel<1, false>), grid, block, 0, c->stream, a);
+        else if (bs == 2) hipLaunchKernelGGL((giant_rotate_mult_kernel<2, false>), grid, block, 0, c->stream, a);
+        else if (bs <= 4) hipLaunchKernelGGL((giant_rotate_mult_kernel<4, false>), grid, block, 0, c->stream, a);
+        else hipLaunchKernelGGL((giant_rotate_mult_kernel<8, false>), grid, block, 0, c->stream, a);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
@@ -280,7 +340,8 @@ extern "C" int ckks_baby_rotate(ckks_ctx* c, uint64_t* output, const uint64_t* m
     }
     if (!any) return CKKS_OK;
     const int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;
-    hipLaunchKernelGGL(baby_rotate_kernel, dim3((unsigned)(c->N / THREADS), c->t_num, blockNum), dim3(THREADS), 0, c->stream, a);
+    if (carry_free_ok(c, a.digits)) hipLaunchKernelGGL(baby_rotate_kernel<true>, dim3((unsigned)(c->N / THREADS), c->t_num, blockNum), dim3(THREADS), 0, c->stream, a);
+    else hipLaunchKernelGGL(baby_rotate_kernel<false>, dim3((unsigned)(c->N / THREADS), c->t_num, blockNum), dim3(THREADS), 0, c->stream, a);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }

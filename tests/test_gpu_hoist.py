@@ -37,11 +37,16 @@ def uniform_T(rng, orc, shape):
     return out
 
 
-@pytest.mark.parametrize("params,logN,l,bs,gs", [(14, 10, None, 2, 8), (15, 9, 2, 4, 16), (13, 11, 3, 3, 5), (14, 8, 0, 1, 1), (15, 10, None, 8, 16),
-                                                 (13, 16, 3, 2, 4)])
-def test_giant_and_baby_rotations_match_oracle(params, logN, l, bs, gs):
+@pytest.mark.parametrize("params,logN,l,bs,gs,generic", [(14, 10, None, 2, 8, False), (15, 9, 2, 4, 16, False), (13, 11, 3, 3, 5, False),
+                                                         (14, 8, 0, 1, 1, False), (15, 10, None, 8, 16, False), (13, 16, 3, 2, 4, False),
+                                                         (15, 9, None, 4, 16, True), (14, 10, 3, 2, 3, True)])
+def test_giant_and_baby_rotations_match_oracle(params, logN, l, bs, gs, generic):
+    """generic: the integer back end is forced, which takes the kernels' 128-bit multiply-add path instead of the carry-free sums
+    that primes below 2^60 allow."""
     pair = ref_pair(params, logN)
     orc, dev = pair.orc, pair.dev
+    if generic:
+        assert dev.L_.ckks_ctx_set_arith_mode(dev.h, 1) == 0
     l = orc.L if l is None else l
     N, K, L, T, RB, dnum = pair.N, orc.K, orc.L, orc.t_num, orc.Ri_blockNum, orc.dnum
     rng = np.random.default_rng(1000 * params + logN)
