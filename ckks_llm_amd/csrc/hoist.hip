@@ -79,6 +79,29 @@ struct Acc<false> {
     }
 };
 
+// Workgroup id -> (256-slot chunk, T prime, block).  The digits of a, P b and the plaintexts of a (chunk, prime) are the same for
+// every block; workgroups whose ids agree modulo 8 share an XCD and its L2 and start in id order, so the blocks of one (chunk,
+// prime) get consecutive places in one XCD's sequence and read those operands from the L2 instead of from memory again (counters:
+// 13.2 GB fetched for 7.4 GB of distinct operands with a plain 3-D grid).
+struct TileIndex {
+    int chunk, k, blk;
+};
+__device__ __forceinline__ TileIndex tile_index(unsigned id, int chunks, int T, int blocks) {
+    TileIndex t;
+    if ((chunks & 7) == 0) {
+        const unsigned xcd = id & 7, j = id >> 3, per = (unsigned)chunks >> 3;
+        t.blk = (int)(j % (unsigned)blocks);
+        const unsigned r = j / (unsigned)blocks;
+        t.chunk = (int)((r % per) * 8 + xcd);
+        t.k = (int)(r / per);
+    } else {
+        t.chunk = (int)(id % (unsigned)chunks);
+        t.k = (int)((id / (unsigned)chunks) % (unsigned)T);
+        t.blk = (int)(id / ((unsigned)chunks * (unsigned)T));
+    }
+    return t;
+}
+
 struct GiantArgs {
     u64* out;                       // [bs][a | b][Ri_blockNum][t_num] limbs
     const u64* pqT;                 // P * (a, b) in T: [a | b][Ri_blockNum][t_num]
@@ -89,15 +112,16 @@ struct GiantArgs {
     const u64* plain[MAX_BS * MAX_GS];
     int acc_num[MAX_BS];
     long N;
-    int logN, T, RB, dnum, digits, prime0, bs, gs;
+    int logN, T, RB, dnum, digits, prime0, bs, gs, blocks;
 };
 
 // one lane per (block, T prime, slot); per rotation of the giant step the rotated pair is formed once and multiplied into the
 // accumulators of all baby steps
 template <int BS, bool FAST>
 __global__ __launch_bounds__(THREADS) void giant_rotate_mult_kernel(GiantArgs a) {
-    const long x = (long)blockIdx.x * THREADS + threadIdx.x;
-    const int k = blockIdx.y, blk = blockIdx.z;
+    const TileIndex ti = tile_index(blockIdx.x, (int)(a.N / THREADS), a.T, a.blocks);
+    const long x = (long)ti.chunk * THREADS + threadIdx.x;
+    const int k = ti.k, blk = ti.blk;
     const PrimeConst p = a.primes[a.prime0 + k];
     const long N = a.N;
     const u64 mask = 2 * (u64)N - 1;
@@ -147,12 +171,13 @@ struct BabyArgs {
     const u64* key[MAX_GS];
     u64 pow[MAX_GS];
     long N;
-    int logN, T, RB, dnum, digits, prime0, rot_num;
+    int logN, T, RB, dnum, digits, prime0, rot_num, blocks;
 };
 template <bool FAST>
 __global__ __launch_bounds__(THREADS) void baby_rotate_kernel(BabyArgs a) {
-    const long x = (long)blockIdx.x * THREADS + threadIdx.x;
-    const int k = blockIdx.y, blk = blockIdx.z;
+    const TileIndex ti = tile_index(blockIdx.x, (int)(a.N / THREADS), a.T, a.blocks);
+    const long x = (long)ti.chunk * THREADS + threadIdx.x;
+    const int k = ti.k, blk = ti.blk;
     const PrimeConst p = a.primes[a.prime0 + k];
     const long N = a.N;
     const u64 mask = 2 * (u64)N - 1;
@@ -301,7 +326,8 @@ extern "C" int ckks_giant_rotate_mult_plain_t(ckks_ctx* c, uint64_t* bs_cipher_T
             if (!a.plain[i * gs + j]) { set_error("Giant_Rotate_And_Mult_PlaintT: a plaintext inside accNum is null"); return CKKS_E_INVALID; }
         }
     const int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;
-    const dim3 grid((unsigned)(c->N / THREADS), c->t_num, blockNum), block(THREADS);
+    a.blocks = blockNum;
+    const dim3 grid((unsigned)(c->N / THREADS) * (unsigned)c->t_num * (unsigned)blockNum), block(THREADS);
     if (carry_free_ok(c, a.digits)) {
         if (bs == 1) hipLaunchKernelGGL((giant_rotate_mult_kernel<1, true>), grid, block, 0, c->stream, a);
         else if (bs == 2) hipLaunchKernelGGL((giant_rotate_mult_kernel<2, true>), grid, block, 0, c->stream, a);
@@ -340,8 +366,10 @@ extern "C" int ckks_baby_rotate(ckks_ctx* c, uint64_t* output, const uint64_t* m
     }
     if (!any) return CKKS_OK;
     const int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;
-    if (carry_free_ok(c, a.digits)) hipLaunchKernelGGL(baby_rotate_kernel<true>, dim3((unsigned)(c->N / THREADS), c->t_num, blockNum), dim3(THREADS), 0, c->stream, a);
-    else hipLaunchKernelGGL(baby_rotate_kernel<false>, dim3((unsigned)(c->N / THREADS), c->t_num, blockNum), dim3(THREADS), 0, c->stream, a);
+    a.blocks = blockNum;
+    const dim3 grid((unsigned)(c->N / THREADS) * (unsigned)c->t_num * (unsigned)blockNum);
+    if (carry_free_ok(c, a.digits)) hipLaunchKernelGGL(baby_rotate_kernel<true>, grid, dim3(THREADS), 0, c->stream, a);
+    else hipLaunchKernelGGL(baby_rotate_kernel<false>, grid, dim3(THREADS), 0, c->stream, a);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
