@@ -422,6 +422,95 @@ class Scheme_23:
                                       cipher.l, *self._ks_buffers()), "ckks_conjugate_23")
         cipher_res.l, cipher_res.scale, cipher_res.slots = cipher.l, cipher.scale, cipher.slots
 
+    # ---- the in-place and derived forms of the members above: host composition over the same entry points, same words ----
+    def _temp(self, like):
+        c = self.context
+        t = getattr(self, "_cipher_temp", None)
+        if t is None:
+            t = self._cipher_temp = Ciphertext(c.N, c.L, like.l, like.slots, like.scale)
+        return t
+
+    def _copy_back(self, dst, src):
+        c = self.context
+        _check(c.L_.ckks_memcpy_d2d(dst.cipher_device.ptr, src.cipher_device.ptr, 8 * c.N * (c.L + 1) * 2), "ckks_memcpy_d2d")
+        dst.l, dst.scale = src.l, src.scale
+
+    def multAndEqual_23(self, cipher1, cipher2):
+        """KeySwitch_23.cuh:238-282."""
+        t = self._temp(cipher1)
+        self.mult_23(t, cipher1, cipher2)
+        self._copy_back(cipher1, t)
+
+    def square(self, cipher1, cipher2):
+        """KeySwitch_23.cuh:346-388: cipher1 = cipher2^2 (2ab, a^2, b^2 are the tensor of cipher2 with itself)."""
+        self.mult_23(cipher1, cipher2, cipher2)
+
+    def squareAndEqual(self, cipher):
+        """KeySwitch_23.cuh:390-430."""
+        t = self._temp(cipher)
+        self.mult_23(t, cipher, cipher)
+        self._copy_back(cipher, t)
+
+    def conjugateAndEqual_23(self, cipher):
+        """KeySwitch_23.cuh:473-506."""
+        t = self._temp(cipher)
+        self.conjugate_23(t, cipher)
+        self._copy_back(cipher, t)
+
+    def leftRotateAndEqual_23(self, cipher, rotSlots):
+        """KeySwitch_23.cuh:509-553."""
+        t = self._temp(cipher)
+        self.leftRotate_23(t, cipher, rotSlots)
+        self._copy_back(cipher, t)
+
+    def rightRotateAndEqual_23(self, cipher, rotSlots):
+        """KeySwitch_23.cuh:618-622: a right rotation by 2^rotSlots slots as the left rotation by N/2 - 2^rotSlots."""
+        self.leftRotateAndEqual_23(cipher, self.context.N // 2 - (1 << rotSlots))
+
+    def leftRotateAddSelf_23(self, cipher, rotSlots):
+        """KeySwitch_23.cuh:583-616: cipher += cipher rotated left by rotSlots."""
+        t = self._temp(cipher)
+        self.leftRotate_23(t, cipher, rotSlots)
+        self.addAndEqual(cipher, t)
+
+    def add(self, cipher_res, cipher1, cipher2):
+        """Scheme_23.cuh:130-141."""
+        c = self.context
+        l = min(cipher1.l, cipher2.l)
+        for z in range(2):
+            o = z * (c.L + 1)
+            c.poly_add_3param_batch_device(cipher_res.cipher_device, cipher1.cipher_device, cipher2.cipher_device, o, o, o, c.K, l + 1)
+        cipher_res.l, cipher_res.scale = l, cipher1.scale
+
+    def addAndEqual(self, cipher1, cipher2):
+        """Scheme_23.cuh:143-152."""
+        scale = cipher1.scale
+        self.add(cipher1, cipher1, cipher2)
+        cipher1.scale = scale
+
+    def sub(self, cipher_res, cipher1, cipher2):
+        """Scheme_23.cuh:268-280 (the result keeps cipher1's level, as there)."""
+        c = self.context
+        l = min(cipher1.l, cipher2.l)
+        for z in range(2):
+            o = z * (c.L + 1)
+            c.poly_sub_3param_batch_device(cipher_res.cipher_device, cipher1.cipher_device, cipher2.cipher_device, o, o, o, c.K, l + 1)
+        cipher_res.l, cipher_res.scale = cipher1.l, cipher1.scale
+
+    def subAndEqual(self, cipher1, cipher2):
+        """Scheme_23.cuh:282-292."""
+        l = min(cipher1.l, cipher2.l)
+        self.sub(cipher1, cipher1, cipher2)
+        cipher1.l = l
+
+    def rescaleToAndEqual(self, cipher, level):
+        """Scheme_23.cuh:407-425: to the coefficient domain, one coefficient-domain rescale per level, back."""
+        c = self.context
+        c.FromNTTInplace(cipher.cipher_device, 0, c.K, 2, cipher.l + 1, c.L + 1)
+        while cipher.l > level:
+            self.rescaleAndEqual_noNTT(cipher)
+        c.ToNTTInplace(cipher.cipher_device, 0, c.K, 2, cipher.l + 1, c.L + 1)
+
     def _next_nonce(self):
         self.nonce += 1
         return self.nonce

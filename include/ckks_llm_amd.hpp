@@ -294,6 +294,7 @@ public:
         delete rlk_23;
         delete ConjKey_23;
         for (Key_decomp* k : rotKey_vec_23) delete k;
+        delete cipher_temp_pool;
         device_release(sxsx);
         device_release(temp_mul);
         device_release(mul_work);
@@ -394,6 +395,85 @@ public:
         check(ckks_rescale(context.handle, cipher.cipher_device, rescale_buffer, cipher.l), "rescaleAndEqual");
         cipher.scale /= (long double)context.qVec[cipher.l];
         cipher.l -= 1;
+    }
+    // ---- the in-place and derived forms: host composition over the same entry points, same words as the separate-result forms ----
+    Ciphertext* cipher_temp_pool = nullptr;             // Scheme_23.cuh:27
+    Ciphertext& temp_like(const Ciphertext& c) {
+        if (!cipher_temp_pool) cipher_temp_pool = new Ciphertext((int)context.N, context.L, c.l, c.slots, c.scale);
+        return *cipher_temp_pool;
+    }
+    void copy_back(Ciphertext& dst, const Ciphertext& src) {
+        check(ckks_memcpy_d2d(dst.cipher_device, src.cipher_device, sizeof(uint64_tt) * (size_t)context.N * (context.L + 1) * 2), "copy back");
+        dst.l = src.l;
+        dst.scale = src.scale;
+    }
+    // KeySwitch_23.cuh:238-282
+    void multAndEqual_23(Ciphertext& cipher1, Ciphertext& cipher2) {
+        Ciphertext& t = temp_like(cipher1);
+        mult_23(t, cipher1, cipher2);
+        copy_back(cipher1, t);
+    }
+    // KeySwitch_23.cuh:346-388: cipher1 = cipher2^2
+    void square(Ciphertext& cipher1, Ciphertext& cipher2) { mult_23(cipher1, cipher2, cipher2); }
+    // KeySwitch_23.cuh:390-430
+    void squareAndEqual(Ciphertext& cipher) {
+        Ciphertext& t = temp_like(cipher);
+        mult_23(t, cipher, cipher);
+        copy_back(cipher, t);
+    }
+    // KeySwitch_23.cuh:473-506
+    void conjugateAndEqual_23(Ciphertext& cipher) {
+        Ciphertext& t = temp_like(cipher);
+        conjugate_23(t, cipher);
+        copy_back(cipher, t);
+    }
+    // KeySwitch_23.cuh:509-553
+    void leftRotateAndEqual_23(Ciphertext& cipher, long rotSlots) {
+        Ciphertext& t = temp_like(cipher);
+        leftRotate_23(t, cipher, rotSlots);
+        copy_back(cipher, t);
+    }
+    // KeySwitch_23.cuh:618-622: right by 2^rotSlots slots = left by N/2 - 2^rotSlots
+    void rightRotateAndEqual_23(Ciphertext& cipher, long rotSlots) { leftRotateAndEqual_23(cipher, context.N / 2 - (1l << rotSlots)); }
+    // KeySwitch_23.cuh:583-616: cipher += cipher rotated left by rotSlots
+    void leftRotateAddSelf_23(Ciphertext& cipher, long rotSlots) {
+        Ciphertext& t = temp_like(cipher);
+        leftRotate_23(t, cipher, rotSlots);
+        addAndEqual(cipher, t);
+    }
+    // Scheme_23.cuh:130-141
+    void add(Ciphertext& cipher_res, Ciphertext& cipher1, Ciphertext& cipher2) {
+        const int l = cipher1.l < cipher2.l ? cipher1.l : cipher2.l, L1 = context.L + 1;
+        for (int z = 0; z < 2; z++)
+            check(ckks_poly_add(context.handle, cipher_res.cipher_device, cipher1.cipher_device, cipher2.cipher_device, z * L1, z * L1, z * L1, context.K, l + 1), "add");
+        cipher_res.l = l;
+        cipher_res.scale = cipher1.scale;
+    }
+    // Scheme_23.cuh:143-152
+    void addAndEqual(Ciphertext& cipher1, Ciphertext& cipher2) {
+        const long double scale = cipher1.scale;
+        add(cipher1, cipher1, cipher2);
+        cipher1.scale = scale;
+    }
+    // Scheme_23.cuh:268-280 (the result keeps cipher1's level, as there)
+    void sub(Ciphertext& cipher_res, Ciphertext& cipher1, Ciphertext& cipher2) {
+        const int l = cipher1.l < cipher2.l ? cipher1.l : cipher2.l, L1 = context.L + 1;
+        for (int z = 0; z < 2; z++)
+            check(ckks_poly_sub(context.handle, cipher_res.cipher_device, cipher1.cipher_device, cipher2.cipher_device, z * L1, z * L1, z * L1, context.K, l + 1), "sub");
+        cipher_res.l = cipher1.l;
+        cipher_res.scale = cipher1.scale;
+    }
+    // Scheme_23.cuh:282-292
+    void subAndEqual(Ciphertext& cipher1, Ciphertext& cipher2) {
+        const int l = cipher1.l < cipher2.l ? cipher1.l : cipher2.l;
+        sub(cipher1, cipher1, cipher2);
+        cipher1.l = l;
+    }
+    // Scheme_23.cuh:407-425: to the coefficient domain, one coefficient-domain rescale per level, back
+    void rescaleToAndEqual(Ciphertext& cipher, int level) {
+        context.FromNTTInplace(cipher.cipher_device, 0, context.K, 2, cipher.l + 1, context.L + 1);
+        while (cipher.l > level) rescaleAndEqual_noNTT(cipher);
+        context.ToNTTInplace(cipher.cipher_device, 0, context.K, 2, cipher.l + 1, context.L + 1);
     }
     // steps 2..9 of Scheme_23::mult_23 (KeySwitch_23.cuh:219-231): d2 (NTT domain, L+1 limbs) -> out = [a | b].
     // A null key throws std::invalid_argument as the missing rotation / relinearisation key does (:198-201).

@@ -207,3 +207,99 @@ def test_mirror_classes_multiply_rotate_conjugate():
     zero = Ciphertext(N, L, 0, N // 2, 1)
     with pytest.raises(ValueError):
         scheme.mult_23(res, c[0], zero)                                     # level 0 (KeySwitch_23.cuh:194-197)
+
+
+def test_in_place_and_derived_members_leave_the_same_words():
+    """multAndEqual_23, square, squareAndEqual, conjugateAndEqual_23, leftRotateAndEqual_23, rightRotateAndEqual_23,
+    leftRotateAddSelf_23, add / sub and their in-place forms, rescaleToAndEqual: each against the separate-result member (parity-
+    tested against the oracle above) or against the oracle / numpy directly, word for word."""
+    P = REF_PARAMS[14]
+    logN = 10
+    pair = Pair(logN, P["p"], P["q"], P["t"], P["gamma"])
+    ctx, orc = pair.dev, pair.orc
+    N, L, K = ctx.N, ctx.L, ctx.K
+    sk = SecretKey(ctx, h=32, key=KEY, nonce=21)
+    scheme = Scheme_23(ctx, key=KEY)
+    scheme.addEncKey(sk)
+    scheme.addMultKey_23(sk)
+    scheme.addConjKey_23(sk)
+    r_right = N // 2 - (1 << 3)
+    for r in (3, r_right):
+        scheme.addLeftRotKey_23(sk, r)
+    rng = np.random.default_rng(5)
+    scale = float(1 << 30)
+
+    def fresh(l=None):
+        msg = Plaintext(N, L, L, N // 2, int(scale))
+        ctx.encode_coeffs(DeviceBuffer.from_numpy(rng.uniform(-1, 1, N)), msg)
+        ct = Ciphertext(N, L, L, N // 2, int(scale))
+        scheme.encryptMsg(ct, msg)
+        if l is not None:
+            ct.l = l
+        return ct
+
+    def words(ct, l=None):
+        l = ct.l if l is None else l
+        return ct.cipher_device.download(np.uint64).reshape(2, L + 1, N)[:, : l + 1].copy()
+
+    def clone(ct):
+        c2 = Ciphertext(N, L, ct.l, ct.slots, ct.scale)
+        c2.cipher_device.upload(ct.cipher_device.download(np.uint64))
+        return c2
+
+    a, b = fresh(), fresh(L - 2)
+    res = Ciphertext(N, L, L, N // 2, 1)
+    # multAndEqual_23 (levels differ: the lower one wins)
+    scheme.mult_23(res, a, b)
+    a2 = clone(a)
+    scheme.multAndEqual_23(a2, b)
+    assert a2.l == L - 2 and a2.scale == a.scale * b.scale and np.array_equal(words(a2), words(res))
+    # square / squareAndEqual = the product of a ciphertext with itself
+    scheme.mult_23(res, a, a)
+    sq = Ciphertext(N, L, L, N // 2, 1)
+    scheme.square(sq, a)
+    assert sq.l == a.l and np.array_equal(words(sq), words(res))
+    a2 = clone(a)
+    scheme.squareAndEqual(a2)
+    assert a2.scale == a.scale * a.scale and np.array_equal(words(a2), words(res))
+    # conjugate / rotations in place
+    scheme.conjugate_23(res, a)
+    a2 = clone(a)
+    scheme.conjugateAndEqual_23(a2)
+    assert np.array_equal(words(a2), words(res))
+    scheme.leftRotate_23(res, a, 3)
+    a2 = clone(a)
+    scheme.leftRotateAndEqual_23(a2, 3)
+    assert np.array_equal(words(a2), words(res))
+    rot3 = words(res)
+    scheme.leftRotate_23(res, a, r_right)
+    a2 = clone(a)
+    scheme.rightRotateAndEqual_23(a2, 3)                                     # right by 2^3 slots
+    assert np.array_equal(words(a2), words(res))
+    # leftRotateAddSelf_23, add, sub against numpy on the residues
+    q = np.array(ctx.qVec, dtype=object)[None, :, None]
+    a2 = clone(a)
+    scheme.leftRotateAddSelf_23(a2, 3)
+    assert np.array_equal(words(a2).astype(object), (words(a).astype(object) + rot3.astype(object)) % q[:, : L + 1])
+    lo = L - 2
+    scheme.add(res, a, b)
+    assert res.l == lo and np.array_equal(words(res).astype(object), (words(a, lo).astype(object) + words(b).astype(object)) % q[:, : lo + 1])
+    scheme.sub(res, a, b)
+    assert res.l == a.l and np.array_equal(words(res, lo).astype(object), (words(a, lo).astype(object) - words(b).astype(object)) % q[:, : lo + 1])
+    a2 = clone(a)
+    scheme.addAndEqual(a2, b)
+    assert a2.l == lo and a2.scale == a.scale and np.array_equal(words(a2).astype(object), (words(a, lo).astype(object) + words(b).astype(object)) % q[:, : lo + 1])
+    a2 = clone(a)
+    scheme.subAndEqual(a2, b)
+    assert a2.l == lo and np.array_equal(words(a2).astype(object), (words(a, lo).astype(object) - words(b).astype(object)) % q[:, : lo + 1])
+    # rescaleToAndEqual against the oracle's steps
+    a2 = clone(a)
+    want = a.cipher_device.download(np.uint64).copy()
+    orc.FromNTTInplace(want, 0, K, 2, L + 1, L + 1)
+    for l in range(L, L - 3, -1):
+        orc.rescaleAndEqual_noNTT(want, l)
+    orc.ToNTTInplace(want, 0, K, 2, L - 2, L + 1)
+    scheme.rescaleToAndEqual(a2, L - 3)
+    assert a2.l == L - 3 and np.array_equal(words(a2), want.reshape(2, L + 1, N)[:, : L - 2])
+    prod = float(np.prod([float(x) for x in ctx.qVec[L - 2:]]))
+    assert abs(a2.scale * prod / a.scale - 1) < 1e-9
