@@ -58,7 +58,7 @@ u64 orc_barrett128(u64 a_hi, u64 a_lo, u64 q, u64 mu_hi, u64 mu_lo) {
     u128 s = (u128)a_lo * mu_hi + tmp;       // mad.lo.cc / madc.hi
     u64 tmp2 = (u64)s;
     u64 res = (u64)(s >> 64);
-    u128 s2 = (u128)a_hi * mu_lo + tmp2;     // round 2
+    u128 s2 = (u128)a_hi * mu_lo + tmp2;     // second cross product
     res += (u64)(s2 >> 64);                  // madc.hi with carry-in folded in s2
     res += a_hi * mu_hi;                     // mad.lo
     u64 r = a_lo - res * q;
