@@ -105,4 +105,15 @@ size_t ntt_sched_bytes();
 size_t ntt_sched_error_offset();
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
+// Forward transform whose first pass reads its input from MLWE samples (the embedding of the ring packing) instead of dev:
+// coefficient pos of polynomial y = coefficient pos >> logk of row y of sample (pos mod 2^logk) >> loggap, zero where pos mod 2^logk
+// is no multiple of 2^loggap; on the limbs of prime start_mod_idx the value is lifted around zero from q0 to p0.
+// mlwe: DEVICE table of sample pointers, each [(k+1)][n1] words of one modulus.
+struct NttEmbedSource {
+    const uint64_t* const* mlwe;
+    uint64_t p0, q0;
+    int logk, loggap, n1;
+};
+int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
+                        const NttEmbedSource& src);
 }  // namespace ckks

@@ -192,6 +192,13 @@ struct NttArgs {
     long batch_stride_limbs;
     unsigned limb_base, limbs_total;      // this launch covers limbs limb_base .. limb_base + gridDim.y - 1 of limbs_total
     char* mid;                            // compact inter-pass buffer (MID_LIMB_BYTES per limb of the launch) or nullptr
+    // Forward transforms of polynomials that exist only as scattered MLWE samples (the embedding of the ring packing): when
+    // embed_mlwe is set the first pass takes coefficient pos of polynomial y from sample (pos mod k) / gap, coefficient
+    // pos / k (zero where pos mod k is no multiple of gap), lifted around zero from q0 to p0 on the limbs of the first prime.
+    const u64* const* embed_mlwe = nullptr;
+    u64 embed_p0 = 0, embed_q0 = 0;
+    int embed_logk = 0, embed_loggap = 0, embed_n1 = 0;
+    int embed_no_wrap = 0;                // q0 / 2 < p0: the lift p0 - (q0 - x) never wraps, the reference's `% p0` is the identity
 };
 
 // Compact inter-pass form (N = 2^16, FP64 back end, q < 2^39): 5 bytes per value instead of 8, in a separate buffer laid out
@@ -213,6 +220,18 @@ __device__ __forceinline__ u64* limb_ptr(const NttArgs& a, unsigned limb, long N
     unsigned y = r % a.poly_num, z = r / a.poly_num;
     prime = a.start_mod_idx + (int)j;
     return a.data + ((long)z * a.batch_stride_limbs + (long)y * a.poly_mod_len + a.start_poly_idx + j) * N;
+}
+
+// residue modulo q0 -> residue modulo p0 of the same centred value (mlweCipherEmbedding_new_kernel, PCMM_Scheme.cuh:335-339:
+// x > q0/2 ? (p0 - (q0 - x)) % p0 : x).  The 64-bit remainder is a long instruction sequence; with q0 / 2 < p0 it is the identity.
+__device__ __forceinline__ u64 embed_lift(u64 x, const NttArgs& a) {
+    if (x <= a.embed_q0 / 2) return x;
+    const u64 t = a.embed_p0 - (a.embed_q0 - x);
+    return a.embed_no_wrap ? t : t % a.embed_p0;
+}
+__device__ __forceinline__ unsigned limb_poly(const NttArgs& a, unsigned limb) {
+    limb += a.limb_base;
+    return (limb % (a.limbs_total / a.mod_num)) % a.poly_num;
 }
 
 constexpr int s1_of(int S) { return (S + 1) / 2; }
@@ -237,9 +256,10 @@ struct StridedCfg {
     static constexpr int THREADS = G * CW, TILES = N2 / CW, LDS_WORDS = N1 * CW;
 };
 
-template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false>
+template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool EMBED = false>
 __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                             typename AR::V* lds, unsigned tid, char* mid_limb = nullptr) {
+                                             typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const NttArgs* ea = nullptr,
+                                             unsigned poly = 0, bool lift = false) {
     typedef StridedCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     typedef typename AR::V V;
@@ -247,8 +267,50 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
     u64* col = limb + tile * CW + cl;
     V v[R];
     if (!INVERSE) {
+        if constexpr (EMBED) {
+            const unsigned kmask = (1u << ea->embed_logk) - 1, gmask = (1u << ea->embed_loggap) - 1;
+            if (SA == 8 && SB == 8 && ea->embed_logk == 9) {
+                // N = 2^16, rank 512 (the BERT layer's ring): the tile's 16 columns x 256 rows are 128 coefficients of each of 32 sample
+                // rows.  Staged through LDS so that a wave reads 512 contiguous bytes of one sample row; the 16-byte k index is
+                // xor-swizzled with the column so that neither the staging writes nor the register reads conflict on the banks.
+                // all sample pointers first, then all coefficients, unconditionally (a coefficient that the embedding leaves zero is
+                // read and dropped): sixteen independent loads in flight per lane instead of sixteen pointer-then-data round trips
+                const u64* row[16];
+                u64 x[16];
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ar.from_canonical(load_word<COHERENT>(col + (long)(g + j * G) * N2));
+                for (int it = 0; it < 16; it++) {
+                    const unsigned sidx = (it * 256 + tid) >> 7;
+                    const unsigned off = (sidx >> 4) * 256 + tile * CW + (sidx & 15);
+                    row[it] = ea->embed_mlwe[off >> ea->embed_loggap] + (long)poly * ea->embed_n1 + (tid & 127);
+                }
+#pragma unroll
+                for (int it = 0; it < 16; it++) x[it] = *row[it];
+#pragma unroll
+                for (int it = 0; it < 16; it++) {
+                    const unsigned sidx = (it * 256 + tid) >> 7, n = tid & 127, clx = sidx & 15;
+                    const unsigned off = (sidx >> 4) * 256 + tile * CW + clx;
+                    u64 y = (off & gmask) == 0 ? x[it] : 0;
+                    if (lift) y = embed_lift(y, *ea);
+                    lds[sidx * 128 + (n ^ (clx << 1))] = ar.from_canonical(y);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < R; j++) v[j] = lds[((g & 1) * 16 + cl) * 128 + (((g >> 1) + 8 * j) ^ (cl << 1))];
+                __syncthreads();
+            } else
+#pragma unroll
+            for (int j = 0; j < R; j++) {
+                const unsigned pos = (g + j * G) * N2 + tile * CW + cl;
+                const unsigned n = pos >> ea->embed_logk, off = pos & kmask;
+                const u64 raw = ea->embed_mlwe[off >> ea->embed_loggap][(long)poly * ea->embed_n1 + n];     // unconditional: loads overlap
+                u64 x = (off & gmask) == 0 ? raw : 0;
+                if (lift) x = embed_lift(x, *ea);
+                v[j] = ar.from_canonical(x);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < R; j++) v[j] = ar.from_canonical(load_word<COHERENT>(col + (long)(g + j * G) * N2));
+        }
         fwd_spread<AR, SA, S1>(v, tw, 1u, ar);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
@@ -301,15 +363,16 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
     }
 }
 
-template <class AR, int SA, int SB, bool INVERSE, bool COMPACT = false>
+template <class AR, int SA, int SB, bool INVERSE, bool COMPACT = false, bool EMBED = false>
 __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pass(NttArgs a) {
     constexpr long N = 1l << (SA + SB);
     __shared__ typename AR::V lds[StridedCfg<SA, SB>::LDS_WORDS];
     int prime;
     u64* limb = limb_ptr(a, blockIdx.y, N, prime);
     const AR ar(a.primes[prime]);
-    strided_tile<AR, SA, SB, INVERSE, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
-                                                      COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr);
+    strided_tile<AR, SA, SB, INVERSE, false, COMPACT, EMBED>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
+                                                             COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr, &a,
+                                                             EMBED ? limb_poly(a, blockIdx.y) : 0u, EMBED && prime == a.start_mod_idx);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -586,7 +649,8 @@ static void launch_passes(ckks_ctx* c, const NttArgs& args, int n, bool inverse)
     dim3 gs(CS::TILES, n), bs(CS::THREADS);
     dim3 gr(CR::TILES, n), br(CR::THREADS);
     if (!inverse) {
-        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT>), gs, bs, 0, c->stream, args);
+        if (args.embed_mlwe) hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT, true>), gs, bs, 0, c->stream, args);
+        else hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT>), gs, bs, 0, c->stream, args);
         if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
         hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false, COMPACT>), gr, br, 0, c->stream, args);
     } else {
@@ -700,8 +764,26 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
     }
 }
 
+static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src);
+
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse) {
+    return launch_ntt_from(c, dev, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, batch_stride_limbs, batch, inverse, nullptr);
+}
+// forward transform of poly_num polynomials that the first pass gathers from MLWE samples instead of reading them from dev
+int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
+                        const NttEmbedSource& src) {
+    if (!src.mlwe || src.logk < 0 || src.loggap < 0 || src.loggap > src.logk || src.n1 <= 0 || ((long)src.n1 << src.logk) != c->N) {
+        set_error("NTT: bad embedding source");
+        return CKKS_E_INVALID;
+    }
+    if (c->ntt_mode == 3) { set_error("NTT: the embedding source needs the two-launch transform"); return CKKS_E_INVALID; }
+    return launch_ntt_from(c, dev, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, 0, 1, false, &src);
+}
+
+static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src) {
     if (!c || !dev) { set_error("NTT: null argument"); return CKKS_E_INVALID; }
     if (poly_num <= 0 || mod_num <= 0 || batch <= 0) return CKKS_OK;      // empty batch: nothing to do
     if (start_mod_idx < 0 || start_mod_idx + mod_num > c->nprimes || start_poly_idx < 0 || poly_mod_len < 0) {
@@ -724,6 +806,12 @@ int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx
     args.mod_num = mod_num;
     args.poly_mod_len = poly_mod_len;
     args.batch_stride_limbs = batch_stride_limbs;
+    if (src) {
+        args.embed_mlwe = (const u64* const*)src->mlwe;
+        args.embed_p0 = src->p0; args.embed_q0 = src->q0;
+        args.embed_logk = src->logk; args.embed_loggap = src->loggap; args.embed_n1 = src->n1;
+        args.embed_no_wrap = src->q0 / 2 < src->p0 ? 1 : 0;
+    }
     if (f64) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
         return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok);

@@ -342,13 +342,13 @@ struct EmbedArgs {
     const u64* const* mlwe;       // mlwe_num pointers, each [(k+1)][N1] (one modulus)
     u64* embed;                   // [(k+1)][2][N]
     long N;
-    int N1, rank, mlwe_num;
+    int N1, rank, mlwe_num, first_poly;
     u64 p0, q0;
 };
 constexpr int EMBED_ROWS = 8;     // coefficients n of the small ring per workgroup
 __global__ __launch_bounds__(256) void mlwe_embed_kernel(EmbedArgs a) {
     extern __shared__ u64 tile[];                       // [EMBED_ROWS][rank]
-    const int k = a.rank, i = blockIdx.y, n0 = blockIdx.x * EMBED_ROWS, gap = k / a.mlwe_num;
+    const int k = a.rank, i = blockIdx.y + a.first_poly, n0 = blockIdx.x * EMBED_ROWS, gap = k / a.mlwe_num;
     for (int t = threadIdx.x; t < EMBED_ROWS * k; t += 256) tile[t] = 0;
     __syncthreads();
     // 8 lanes read 64 contiguous bytes of one sample; the tile turns (sample, n) into (n, position inside the big coefficient group)
@@ -362,7 +362,12 @@ __global__ __launch_bounds__(256) void mlwe_embed_kernel(EmbedArgs a) {
         const u64 v = tile[t];
         const long pos = (long)n0 * k + t;              // (n0 + t / k) * k + t % k
         big[a.N + pos] = v;                                                         // mod q0
-        big[pos] = v > a.q0 / 2 ? (a.p0 - (a.q0 - v)) % a.p0 : v;                   // mod p0, lifted around zero (:335-339)
+        u64 lifted = v;                                                             // mod p0, lifted around zero (:335-339)
+        if (v > a.q0 / 2) {
+            lifted = a.p0 - (a.q0 - v);
+            if (a.q0 / 2 >= a.p0) lifted %= a.p0;                                   // the reference's `% p0`; the identity when q0 / 2 < p0
+        }
+        big[pos] = lifted;
     }
 }
 
@@ -428,8 +433,16 @@ extern "C" int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* c
     EmbedArgs ea;
     ea.mlwe = (const u64* const*)h->d_ptrs; ea.embed = embed_scratch; ea.N = c->N; ea.N1 = N1; ea.rank = k; ea.mlwe_num = mlwe_num;
     ea.p0 = h->pq[0]; ea.q0 = h->pq[1];
-    hipLaunchKernelGGL(mlwe_embed_kernel, dim3(N1 / EMBED_ROWS, k + 1), dim3(256), (size_t)EMBED_ROWS * k * sizeof(u64), c->stream, ea);
-    if ((rc = launch_ntt(c, embed_scratch, 0, K - 1, k, 2, 2, 0, 1, false))) return rc;            // :389
+    // Only the b polynomial is written out in coefficient form (the ModDown adds it at the end).  The k "a" polynomials are
+    // needed in NTT form only: the first pass of their transform gathers them from the samples, which saves writing and
+    // re-reading 2 k limbs (a quarter of this entry point's memory traffic).
+    ea.first_poly = k;
+    hipLaunchKernelGGL(mlwe_embed_kernel, dim3(N1 / EMBED_ROWS, 1), dim3(256), (size_t)EMBED_ROWS * k * sizeof(u64), c->stream, ea);
+    NttEmbedSource src;
+    src.mlwe = (const uint64_t* const*)h->d_ptrs; src.p0 = h->pq[0]; src.q0 = h->pq[1]; src.n1 = N1;
+    src.logk = 0; while ((1 << src.logk) < k) src.logk++;
+    src.loggap = 0; while ((mlwe_num << src.loggap) < k) src.loggap++;
+    if ((rc = launch_ntt_embedded(c, embed_scratch, 0, K - 1, k, 2, 2, src))) return rc;           // :389
     RepackArgs ra;
     ra.embed = embed_scratch; ra.keys = repacking_keys; ra.acc = mult_scratch; ra.rlwe = rlwe_out; ra.pq = h->d_pq; ra.N = c->N;
     ra.rank = k; ra.L = c->L;
