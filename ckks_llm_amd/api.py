@@ -766,3 +766,137 @@ class PCMM_Scheme:
     def PPMM_strided(self, plain_mat, mlwe_all, out, mat_M, mat_N, mod_num, scaler):
         _check(self.L_.pcmm_ppmm_strided(self.pcmm_context.h, _addr(plain_mat), _addr(mlwe_all), _addr(out), mat_M, mat_N,
                                          mod_num, float(scaler)), "pcmm_ppmm_strided")
+
+
+class Bert_model_weights:
+    """Bert_model_weights (src/bert/Load_bert.cuh:11-348): the fp32 tensors of a BERT-base `model.safetensors` as device buffers
+    under the reference's member names (per-layer members are lists of 12).  File format: 8 bytes little-endian header length, a
+    JSON header {name: {"dtype", "shape", "data_offsets": [begin, end]}}, then the tensor bytes.  A tensor that is absent, not
+    F32 or out of the file's range stays None and is listed in `missing`."""
+
+    GLOBAL = {
+        "embeddings_LayerNorm_beta": "bert.embeddings.LayerNorm.beta", "embeddings_LayerNorm_gamma": "bert.embeddings.LayerNorm.gamma",
+        "embeddings_position_embeddings_weight": "bert.embeddings.position_embeddings.weight",
+        "embeddings_token_type_embeddings_weight": "bert.embeddings.token_type_embeddings.weight",
+        "embeddings_word_embeddings_weight": "bert.embeddings.word_embeddings.weight",
+        "pooler_dense_bias": "bert.pooler.dense.bias", "pooler_dense_weight": "bert.pooler.dense.weight",
+        "cls_predictions_bias": "cls.predictions.bias",
+        "cls_predictions_transform_LayerNorm_beta": "cls.predictions.transform.LayerNorm.beta",
+        "cls_predictions_transform_LayerNorm_gamma": "cls.predictions.transform.LayerNorm.gamma",
+        "cls_predictions_transform_dense_bias": "cls.predictions.transform.dense.bias",
+        "cls_predictions_transform_dense_weight": "cls.predictions.transform.dense.weight",
+        "cls_seq_relationship_bias": "cls.seq_relationship.bias", "cls_seq_relationship_weight": "cls.seq_relationship.weight",
+    }
+    LAYER = ["attention.output.LayerNorm.beta", "attention.output.LayerNorm.gamma", "attention.output.dense.bias",
+             "attention.output.dense.weight", "attention.self.key.bias", "attention.self.key.weight", "attention.self.query.bias",
+             "attention.self.query.weight", "attention.self.value.bias", "attention.self.value.weight", "intermediate.dense.bias",
+             "intermediate.dense.weight", "output.LayerNorm.beta", "output.LayerNorm.gamma", "output.dense.bias", "output.dense.weight"]
+
+    def __init__(self, model_catalog):
+        import json
+        import os
+        self.num_layers = 12
+        self.opened, self.missing, self.loaded = False, [], []
+        for member in self.GLOBAL:
+            setattr(self, member, None)
+        for leaf in self.LAYER:
+            setattr(self, leaf.replace(".", "_"), [None] * self.num_layers)
+        fname = model_catalog + "model.safetensors"                       # Load_bert.cuh:50
+        if not os.path.exists(fname):
+            print("Failed to open model file: " + fname)
+            return
+        with open(fname, "rb") as f:
+            head = f.read(8)
+            size = os.path.getsize(fname)
+            n = int.from_bytes(head, "little") if len(head) == 8 else -1
+            if n < 0 or 8 + n > size:
+                print("Failed to read header size from: " + fname)
+                return
+            header = json.loads(f.read(n))
+            self.opened = True
+            data_bytes = size - 8 - n
+
+            def load(name):
+                e = header.get(name)
+                if not isinstance(e, dict) or e.get("dtype") != "F32":
+                    self.missing.append(name)
+                    return None
+                begin, end = e["data_offsets"]
+                if begin < 0 or end < begin or end > data_bytes or (end - begin) % 4:
+                    self.missing.append(name)
+                    return None
+                f.seek(8 + n + begin)
+                buf = DeviceBuffer.from_numpy(np.frombuffer(f.read(end - begin), dtype=np.float32))
+                self.loaded.append((name, end - begin))
+                return buf
+
+            for member, name in self.GLOBAL.items():
+                setattr(self, member, load(name))
+            for i in range(self.num_layers):
+                for leaf in self.LAYER:
+                    getattr(self, leaf.replace(".", "_"))[i] = load("bert.encoder.layer.%d.%s" % (i, leaf))
+
+
+class Bert:
+    """The PCMM calls of the linear layers of Bert (src/bert/Bert.h:15-66; Bert.cuh:155-169, 204-211, 249-257, 296-302, 404-489):
+    gather of the input ciphertexts into MLWE samples, PPMM with the layer's weight, ring packing of the product rows, with the
+    reference's sample counts and offsets.  Ciphertexts enter and leave in coefficient packing; the slot <-> coefficient
+    conversions, EvalMod and the non-linear layers that the reference runs in between are not part of this library.
+    The gather writes PPMM's operand planes directly, which needs ring-pack primes below 2^39."""
+
+    def __init__(self, model_catalog, context, scheme, pcmm_scheme, sk, target_scale=float(1 << 49)):
+        self.context, self.scheme, self.pcmm_scheme, self.sk = context, scheme, pcmm_scheme, sk
+        self.model_weights = Bert_model_weights(model_catalog)
+        pc = pcmm_scheme.pcmm_context
+        self.PCMM_N1, self.mlwe_rank, self.q_ringpack_count = pc.N1, pc.mlwe_rank, pc.ringpack_q_count
+        self.N, self.L = context.N, context.L
+        if self.mlwe_rank * self.PCMM_N1 != self.N:
+            raise ValueError("Bert: the PCMM context's rank is not N / N1")
+        self.target_scale = target_scale                                  # the reference fixes 2^49 (PPMM_kernel.cuh:283)
+        self.ppmm_output = None
+        self.embeded_mlwe_buffer = DeviceBuffer(8 * (self.mlwe_rank + 1) * 2 * self.N)
+        self.mult_key_output = DeviceBuffer(8 * 4 * self.N)
+
+    def linear(self, plain_mat, M, Nin, parts_in, parts_out):
+        """parts_in: (ciphertext, count, offset, extract); parts_out: (ciphertext, count, offset)."""
+        ps, pc = self.pcmm_scheme, self.pcmm_scheme.pcmm_context
+        mods, C = self.q_ringpack_count, (self.mlwe_rank + 1) * self.PCMM_N1
+        if self.ppmm_output is None or self.ppmm_output.nbytes < 8 * M * mods * C:
+            self.ppmm_output = DeviceBuffer(8 * M * mods * C)
+        in_scale = parts_in[0][0].scale
+        scaler = float(int(pc.q_ringpack[1] * self.target_scale / in_scale))        # PPMM_kernel.cuh:283-284
+        ps.packed_begin(Nin, mods)
+        for ct, count, offset, extract in parts_in:
+            ps.rlweCipherDecompose_packed(ct.cipher_device, extract, offset, ct.l, take=count)
+        ps.PPMM_packed(plain_mat, self.ppmm_output, M, scaler)
+        rows = [self.ppmm_output.ptr + 8 * m * mods * C for m in range(M)]          # row m, first modulus
+        for ct, count, offset in parts_out:
+            ps.mlweCipherPacking(ct.cipher_device, rows, count, offset, ps.repackingKeys, self.embeded_mlwe_buffer, self.mult_key_output)
+            ct.l, ct.scale = 0, in_scale * scaler / pc.q_ringpack[1]
+
+    def PCMM_768_768(self, plain_mat, rlwe_cipher, res_cipher, do_s2c):
+        """do_s2c = 0: two inputs of 512 samples, the first 768 multiplied (Bert.cuh:416-417, 425); 1: three of 256 (:404-412)."""
+        if do_s2c == 1:
+            parts = [(rlwe_cipher[0], 256, 0, 256), (rlwe_cipher[1], 256, 256, 256), (rlwe_cipher[2], 256, 512, 256)]
+        else:
+            parts = [(rlwe_cipher[0], 512, 0, 512), (rlwe_cipher[1], 256, 512, 512)]
+        self.linear(plain_mat, 768, 768, parts, [(res_cipher[0], 256, 0), (res_cipher[1], 256, 256), (res_cipher[2], 256, 512)])
+
+    def mul_W_QKV(self, X, resQ, resK, resV, layer, do_s2c=1):
+        w = self.model_weights
+        self.PCMM_768_768(w.attention_self_query_weight[layer], X, resQ, do_s2c)
+        self.PCMM_768_768(w.attention_self_key_weight[layer], X, resK, do_s2c)
+        self.PCMM_768_768(w.attention_self_value_weight[layer], X, resV, do_s2c)
+
+    def attn_output(self, O, res, layer, do_s2c=1):
+        self.PCMM_768_768(self.model_weights.attention_output_dense_weight[layer], O, res, do_s2c)
+
+    def intermediate(self, O, layer, res):
+        """Bert.cuh:249-257: 512 samples of O[0] and 256 of O[2]; 3072 x 768; rows 512 i .. into res[2 i]."""
+        self.linear(self.model_weights.intermediate_dense_weight[layer], 3072, 768, [(O[0], 512, 0, 512), (O[2], 256, 512, 256)],
+                    [(res[2 * i], 512, 512 * i) for i in range(6)])
+
+    def layer_output(self, O, layer):
+        """Bert.cuh:290-302: 512 samples of each O[2 i]; 768 x 3072; rows 0..511 into O[0], 512..767 into O[2]."""
+        self.linear(self.model_weights.output_dense_weight[layer], 768, 3072, [(O[2 * i], 512, 512 * i, 512) for i in range(6)],
+                    [(O[0], 512, 0), (O[2], 256, 512)])

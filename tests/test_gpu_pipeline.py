@@ -154,3 +154,68 @@ def test_bert_base_layer_on_encrypted_activations():
         assert np.abs(got[:, 1:512:2]).max() < 2.0 ** -9                    # the positions between the packed samples hold noise only
         assert np.median(err) < 2.0 ** -13
     assert np.abs(want).max() > 2.0 and max(worst) < 2.0 ** -10, worst
+
+
+def test_bert_mirror_layers_with_loaded_weights(tmp_path):
+    """The Python mirrors of Bert_model_weights and Bert: weights from a `model.safetensors` written with the safetensors package,
+    PCMM_768_768 (two inputs of 512 samples) and layer_output (768 x 3072, six inputs) on encrypted activations at N = 2^16,
+    decrypted and compared with the plain products."""
+    from safetensors.numpy import save_file
+    from ckks_llm_amd import Bert, Ciphertext, MLWESecretKey, Plaintext, Scheme_23, SecretKey
+    rng = np.random.default_rng(9)
+    pre = "bert.encoder.layer.0."
+    tensors = {pre + "attention.self.query.weight": rng.normal(0, 0.02, (768, 768)).astype(np.float32),
+               pre + "output.dense.weight": rng.normal(0, 0.02, (768, 3072)).astype(np.float32),
+               pre + "output.dense.bias": rng.normal(0, 0.02, 768).astype(np.float32),
+               "cls.seq_relationship.bias": np.zeros(2, np.float16)}
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    logN, N1 = 16, 128
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    ctx = Context_23(logN, [P0], [Q0, Q1])
+    N, L, k = ctx.N, ctx.L, ctx.N // N1
+    key = bytes(range(1, 33))
+    scheme = Scheme_23(ctx, key=key)
+    sk = SecretKey(ctx, h=192, key=key, nonce=1)
+    pc = PCMM_Context(N1, k, [P0], [Q0, Q1], ctx)
+    ps = PCMM_Scheme(pc, key=key)
+    mlwe_sk = MLWESecretKey(N1, pc.ringpack_pq_count - 1, k)
+    ps.convertMLWESKfromRLWESK(mlwe_sk, sk)
+    scheme.addEncKey(sk)
+    ps.addRepakcingKey(mlwe_sk, sk)
+    bert = Bert(str(tmp_path) + "/", ctx, scheme, ps, sk, target_scale=float(1 << 26))
+    w = bert.model_weights
+    assert w.opened and len(w.loaded) == 3 and len(w.missing) == 14 + 16 * 12 - 3 and "cls.seq_relationship.bias" in w.missing
+    assert np.array_equal(w.output_dense_bias[0].download(np.float32), tensors[pre + "output.dense.bias"])
+    assert w.output_dense_bias[1] is None and w.pooler_dense_weight is None
+    x_scale = 1 << 33
+    d_vals = DeviceBuffer(8 * N)
+
+    def encrypt_part(X, first, count, extract):
+        coeffs = np.zeros((N1, k))
+        coeffs[:, 0:count * (k // extract):k // extract] = X[:, first:first + count]
+        msg = Plaintext(N, L, L, N // 2, x_scale)
+        ctx.encode_coeffs(DeviceBuffer.from_numpy(coeffs.reshape(-1)), msg)
+        ct = Ciphertext(N, L, L, N // 2, x_scale)
+        scheme.encryptMsg(ct, msg)
+        return ct
+
+    def worst_error(ct, Y, first, count):
+        dec = Plaintext(N, L, 0, N // 2, 1)
+        scheme.decryptMsg(dec, sk, ct)
+        ctx.decode_coeffs(dec, d_vals)
+        got = d_vals.download(np.float64).reshape(N1, k)
+        return np.abs(got[:, 0:count * (k // count):k // count] - Y[:, first:first + count]).max()
+
+    X = rng.normal(0, 1, (N1, 768))
+    Y = X @ tensors[pre + "attention.self.query.weight"].astype(np.float64).T
+    ins = [encrypt_part(X, 0, 512, 512), encrypt_part(X, 512, 256, 512)]
+    outs = [Ciphertext(N, L, 0, N // 2, 1) for _ in range(3)]
+    bert.PCMM_768_768(w.attention_self_query_weight[0], ins, outs, 0)
+    assert max(worst_error(outs[j], Y, 256 * j, 256) for j in range(3)) < 2.0 ** -10
+    X = rng.normal(0, 0.6, (N1, 3072))
+    Y = X @ tensors[pre + "output.dense.weight"].astype(np.float64).T
+    O = [None] * 12
+    for i in range(6):
+        O[2 * i] = encrypt_part(X, 512 * i, 512, 512)
+    bert.layer_output(O, 0)
+    assert O[0].l == 0 and max(worst_error(O[0], Y, 0, 512), worst_error(O[2], Y, 512, 256)) < 2.0 ** -10
