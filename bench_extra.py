@@ -6,9 +6,9 @@ MFMA_I8_PEAK_MACS = 2.5166e15      # 5.033 POP/s dense int8
 HBM_PEAK = 8.0e12
 
 
-def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3):
+def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None):
     from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
-    primes = P.CFG2_Q[:L]
+    primes = list(primes[:L]) if primes is not None else P.CFG2_Q[:L]
     ctx = Context_23(16, [], primes)
     rank = (1 << 16) // N1
     C = (rank + 1) * N1
@@ -42,7 +42,7 @@ def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3):
     DW, DC, path = sch.pcmm_context.info("last_DW"), sch.pcmm_context.info("last_DC"), sch.pcmm_context.info("last_path")
     word_macs = float(M) * Kin * C * L
     macs = word_macs * DW * DC
-    res = {"workload": "configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (3 if M == 768 else 4, M, Kin, N1, L, C),
+    res = {"workload": label or "configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (3 if M == 768 else 4, M, Kin, N1, L, C),
            "ms": round(best, 3), "word_MAC_per_s": round(word_macs / (best * 1e-3), 1), "int8_MAC_per_s": round(macs / (best * 1e-3), 1),
            "D_w": DW, "D_c": DC, "kernel": "int8 MFMA" if path == 1 else "generic u128",
            "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
@@ -251,5 +251,6 @@ def bench_hoisted_level(P, gs=16, bs=4, reps=3):
 
 
 def run(P):
-    return {"ppmm": bench_ppmm(P), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P),
+    ref_label = "PPMM 768x768 as the reference's BERT layer calls it: its own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens"
+    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}

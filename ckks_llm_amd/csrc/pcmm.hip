@@ -634,6 +634,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             cst[4 * PPMM_MAX_MODS + i] = dbits(cst[i], qi);
         }
         cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 32, qi), qi);
+        cst[3 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 64, qi), qi);
     }
     uint64_t* d_cst = (uint64_t*)(h->d_absmax + 1);
     CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
@@ -649,18 +650,22 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
     a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
     a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np;
-    // digit counts: DW digits cover |A| < 2^(8*DW-1); DC digits cover residues < 2^(8*DC-1)
-    int DW = 1; while (DW < 8 && absmax >= (1ull << (8 * DW - 1))) DW++;
-    int DC = 1; while (DC < 8 && qmax >= (1ull << (8 * DC - 1))) DC++;
+    // digit counts.  d balanced digits in [-128, 127] reach from -0x80..80 up to +0x7f..7f (d bytes each), NOT up to 2^(8d-1) - 1:
+    // the bytes of x + 0x80..80 must not carry into byte d.  DW digits must hold +-|A|max, DC digits every residue 0 .. qmax - 1.
+    auto top = [](int d) { unsigned long long v = 0; for (int i = 0; i < d; i++) v = (v << 8) | 0x7f; return v; };
+    int DW = 1; while (DW < 8 && absmax > top(DW)) DW++;
+    int DC = 1; while (DC < 8 && qmax - 1 > top(DC)) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
-    const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && qmax < (1ull << 39) && DW <= 4 && DC <= 5 &&
+    // residues in 5 digits (q < 2^39) with up to 4 plaintext digits, or in 7 digits (q < 2^50) with up to 3
+    const bool width_ok = (DC <= 5 && DW <= 4) || (DC <= 7 && qmax < (1ull << 50) && DW <= 3 && !packed);
+    const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && width_ok &&
                          (long)Kpad * (DW <= 3 ? 3 : 4) <= 16384 && absmax < qmin && qmin > (1ull << 25);
     if (packed && !mfma_ok) { set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
         hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
-        size_t need = ppmm_bdig_bytes(a);
+        size_t need = ppmm_bdig_bytes(a, DC);
         if (packed && need > h->Bdig_cap) { set_error("PPMM on digit planes: planes not opened for this shape"); return CKKS_E_STATE; }
         if (need > h->Bdig_cap) {
             if (h->d_Bdig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Bdig); h->d_Bdig = nullptr; h->Bdig_cap = 0; }
@@ -669,7 +674,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             h->Bdig_cap = need;
         }
         if (!packed) h->packed_K = h->packed_mods = 0;     // the planes now hold this call's operands
-        rc = launch_ppmm_mfma_impl(c->stream, a, DW, h->d_Bdig, !packed);
+        rc = launch_ppmm_mfma_impl(c->stream, a, DW, DC, h->d_Bdig, !packed);
         if (rc) return rc;
     } else {
         dim3 grid((unsigned)((C + 255) / 256), M), block(256);
@@ -704,7 +709,7 @@ extern "C" int pcmm_packed_begin(pcmm_ctx* h, int Kin, int mod_num) {
         return CKKS_E_INVALID;
     }
     for (int i = 0; i < mod_num; i++)
-        if (h->pq[h->np + i] >= (1ull << 39)) { set_error("pcmm_packed_begin: the digit planes hold primes below 2^39"); return CKKS_E_INVALID; }
+        if (h->pq[h->np + i] - 1 > 0x7f7f7f7f7full) { set_error("pcmm_packed_begin: the digit planes hold residues up to 0x7f7f7f7f7f (primes just below 2^39)"); return CKKS_E_INVALID; }
     const int Kpad = (Kin + 191) / 192 * 192;
     const size_t need = (size_t)mod_num * Kpad * C * 5;
     if (need > h->Bdig_cap) {

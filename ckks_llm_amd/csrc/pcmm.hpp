@@ -31,7 +31,7 @@ struct pcmm_ctx {
 namespace ckks {
 
 // per-call constants of the PPMM epilogue, one row of PPMM_MAX_MODS words each:
-//   [0] q_last^-1 mod q_i   [1] its Shoup word   [2] 2^32 mod q_i   [3] unused   [4] q_last^-1 mod q_i
+//   [0] q_last^-1 mod q_i   [1] its Shoup word   [2] 2^32 mod q_i   [3] 2^64 mod q_i   [4] q_last^-1 mod q_i
 //   rows 2..4 are balanced representatives stored as IEEE double bit patterns (FP64 epilogue)
 constexpr int PPMM_MAX_MODS = 64;
 constexpr int PPMM_CONST_ROWS = 5;
@@ -50,7 +50,7 @@ struct PpmmArgs {
     int M, Kin, Mpad, Kpad, mod_num, np;
 };
 
-size_t ppmm_bdig_bytes(const PpmmArgs& a);
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig, bool pack);
+size_t ppmm_bdig_bytes(const PpmmArgs& a, int DC);
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC, int8_t* bdig, bool pack);
 
 }  // namespace ckks

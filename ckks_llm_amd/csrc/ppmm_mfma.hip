@@ -8,7 +8,9 @@
 //     sum_n A*Ct = sum_{e<DW+DC-1} 256^e * S_e ,   S_e = sum_{d+j=e} sum_n a_d*b_j    (int32, |S_e| <= min(DW,DC)*Kin*2^14)
 // One v_mfma_i32_16x16x64_i8 per (d, j, 16x16 tile, 64 k) accumulates into the anti-diagonal accumulator S_{d+j}.
 // The epilogue recombines the S_e without rounding in FP64 (four diagonals at a time stay below 2^53), reduces modulo q_i
-// (q_i < 2^39) and applies the fused rescale (PPMM_kernel.cuh:213-249).
+// and applies the fused rescale (PPMM_kernel.cuh:213-249).
+// Two residue widths are built: DC = 5 digits for q_i < 2^39 (the 36-bit sets of the benchmarks) and DC = 7 digits for
+// q_i < 2^50 (the reference's own 49-bit ring-pack primes), the latter with DW <= 3.
 //
 #include <type_traits>
 
@@ -19,7 +21,6 @@ namespace ckks {
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int CT = 64, KS = 64;                  // column tile and K step; the row tile is 16 rows per wave of the workgroup
-constexpr int DCMAX = 5;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
 // 16 bytes per lane from global memory straight into LDS (no registers held while the load is in flight):
@@ -50,8 +51,10 @@ __device__ __forceinline__ double balance_f64(double x, double q, double qinv) {
 // One workgroup (256 lanes) handles 64 k x 64 columns: coalesced 512 B row reads, a byte transpose in registers,
 // LDS to gather the 4 waves' quarter rows, then 16 B per lane coalesced writes.
 // ------------------------------------------------------------------------------------------------------------
+template <int DC>
 __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __restrict__ bdig) {
-    constexpr int DC = DCMAX;
+    static_assert(DC == 5 || DC == 7, "residue digits");
+    constexpr u64 BIAS = DC == 5 ? 0x8080808080ull : 0x80808080808080ull;         // bytes of x + BIAS = balanced digit + 128
     __shared__ __align__(16) int8_t tile[DC][CT][KS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const unsigned c0 = blockIdx.x * CT;
@@ -63,7 +66,7 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
     for (int g = 0; g < 4; g++) {
         u64 y[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) y[i] = a.mlwe[ks * KS + 16 * wave + 4 * g + i][col_word] + 0x8080808080ull;   // bytes = digit + 128
+        for (int i = 0; i < 4; i++) y[i] = a.mlwe[ks * KS + 16 * wave + 4 * g + i][col_word] + BIAS;
         const unsigned x0 = (unsigned)y[0], x1 = (unsigned)y[1], x2 = (unsigned)y[2], x3 = (unsigned)y[3];
         const unsigned t0 = __byte_perm(x0, x1, 0x5140), t1 = __byte_perm(x0, x1, 0x7362);
         const unsigned t2 = __byte_perm(x2, x3, 0x5140), t3 = __byte_perm(x2, x3, 0x7362);
@@ -71,9 +74,18 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
         dw[1 * 4 + g] = __byte_perm(t0, t2, 0x7632) ^ 0x80808080u;
         dw[2 * 4 + g] = __byte_perm(t1, t3, 0x5410) ^ 0x80808080u;
         dw[3 * 4 + g] = __byte_perm(t1, t3, 0x7632) ^ 0x80808080u;
-        const unsigned h01 = __byte_perm((unsigned)(y[0] >> 32), (unsigned)(y[1] >> 32), 0x0040);
-        const unsigned h23 = __byte_perm((unsigned)(y[2] >> 32), (unsigned)(y[3] >> 32), 0x0040);
-        dw[4 * 4 + g] = __byte_perm(h01, h23, 0x5410) ^ 0x80808080u;
+        if constexpr (DC == 5) {
+            const unsigned h01 = __byte_perm((unsigned)(y[0] >> 32), (unsigned)(y[1] >> 32), 0x0040);
+            const unsigned h23 = __byte_perm((unsigned)(y[2] >> 32), (unsigned)(y[3] >> 32), 0x0040);
+            dw[4 * 4 + g] = __byte_perm(h01, h23, 0x5410) ^ 0x80808080u;
+        } else {
+            const unsigned h0 = (unsigned)(y[0] >> 32), h1 = (unsigned)(y[1] >> 32), h2 = (unsigned)(y[2] >> 32), h3 = (unsigned)(y[3] >> 32);
+            const unsigned u0 = __byte_perm(h0, h1, 0x5140), u1 = __byte_perm(h0, h1, 0x7362);
+            const unsigned u2 = __byte_perm(h2, h3, 0x5140), u3 = __byte_perm(h2, h3, 0x7362);
+            dw[4 * 4 + g] = __byte_perm(u0, u2, 0x5410) ^ 0x80808080u;
+            dw[5 * 4 + g] = __byte_perm(u0, u2, 0x7632) ^ 0x80808080u;
+            dw[6 * 4 + g] = __byte_perm(u1, u3, 0x5410) ^ 0x80808080u;
+        }
     }
     // LDS chunk index xor-swizzled with the column so that the 64-byte-strided 16-byte stores spread over the banks
 #pragma unroll
@@ -103,9 +115,10 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
 //   NWAVES = 8, RING = 3: 128 x 64 tile, one workgroup per CU (135 KiB of LDS), loads issued two steps ahead.
 // The other shape that fits the LDS (NWAVES = 4, RING = 2: 64 x 64 tile, 64 KiB, two workgroups per CU that drift out of phase)
 // was measured and is no faster (its single step of load lead time costs what the overlap of the two workgroups gains).
-template <int DW, int NWAVES, int RING>
+template <int DW, int NWAVES, int RING, int DC>
 __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_block) {
-    constexpr int DC = DCMAX, ND = DW + DC - 1, MT = 16 * NWAVES;
+    constexpr int ND = DW + DC - 1, MT = 16 * NWAVES;
+    constexpr bool WIDE = DC > 5;                                // residues of up to 50 bits: three groups of diagonals, wider r_last
     constexpr int A_SLABS = DW * (MT / 16), B_SLABS = DC * 4;    // 1 KiB slabs per step
     constexpr int A_PER_WAVE = (A_SLABS + NWAVES - 1) / NWAVES, B_PER_WAVE = (B_SLABS + NWAVES - 1) / NWAVES;
     constexpr int AHEAD = RING - 1;                              // how many steps ahead of its use a slot is refilled
@@ -228,8 +241,9 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
     // r_last (residues modulo the last prime, < 2^39) of this lane's 16 outputs, kept in registers for the fused rescale
     // of the other primes: low words, and the 7 high bits packed four to a word.
     unsigned rl_lo[2][4][2], rl_hi[2][2];
+    double rl_wide[WIDE ? 2 : 1][WIDE ? 2 : 1][WIDE ? 4 : 1];           // the wide form keeps r_last as doubles
     // constants of the prime in work, requested before its K loop so that the epilogue does not start with a round trip to memory
-    double q = 0, qinv = 0, c32 = 0, qli = 0;
+    double q = 0, qinv = 0, c32 = 0, c64 = 0, qli = 0;
     auto epilogue = [&](int im, auto last_c, auto full_c) {
         constexpr bool LAST = decltype(last_c)::value, FULL = decltype(full_c)::value;
         // The output addressing starts from a value the optimiser cannot hoist above the K loop (it would otherwise keep
@@ -249,6 +263,50 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
             }
 #pragma unroll
             for (int nt = 0; nt < 2; nt++) {
+                if constexpr (WIDE) {
+                    // q < 2^50.  Groups of four diagonals y0 (e < 4), y1 (4 <= e < 8), y2 (e >= 8), each exact below 2^53; y0 and y1
+                    // are first brought to (-q/2, q/2] so that the products with 2^32 and 2^64 mod q stay below 2^99 (quotients below
+                    // 2^49: the estimate rint(h / q) is off by less than one) and every sum below stays an integer under 2^53.
+                    double y0[4], y1[4], y2[4], t[4];
+                    constexpr int E1 = ND - 1 < 7 ? ND - 1 : 7;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) { y0[r] = (double)acc[3][mt][nt][r]; y1[r] = (double)acc[E1][mt][nt][r]; y2[r] = ND > 8 ? (double)acc[ND - 1][mt][nt][r] : 0.0; }
+#pragma unroll
+                    for (int e = 2; e >= 0; e--)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) y0[r] = __builtin_fma(y0[r], 256.0, (double)acc[e][mt][nt][r]);
+#pragma unroll
+                    for (int e = E1 - 1; e >= 4; e--)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) y1[r] = __builtin_fma(y1[r], 256.0, (double)acc[e][mt][nt][r]);
+#pragma unroll
+                    for (int e = ND - 2; e >= 8; e--)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) y2[r] = __builtin_fma(y2[r], 256.0, (double)acc[e][mt][nt][r]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y0[r] = balance_f64(y0[r], q, qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y1[r] = balance_f64(y1[r], q, qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y1[r] = mulmod_f64(y1[r], c32, q, qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) y2[r] = mulmod_f64(y2[r], c64, q, qinv);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) t[r] = balance_f64(y0[r] + y1[r] + y2[r], q, qinv);
+                    if (!LAST) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) t[r] = balance_f64(mulmod_f64(t[r] - rl_wide[WIDE ? mt : 0][WIDE ? nt : 0][WIDE ? r : 0], qli, q, qinv), q, qinv);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const double res = t[r] < 0.0 ? t[r] + q : t[r];
+                        if (LAST) rl_wide[WIDE ? mt : 0][WIDE ? nt : 0][WIDE ? r : 0] = res;
+                        const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
+                        if (FULL) orow[r][nt * 16] = ures;
+                        else if (mrow + mt * 16 + r < a.M) orow[r][nt * 16] = ures;
+                    }
+                    continue;
+                }
                 // The four outputs of a lane in one MFMA tile advance together, one operation at a time: every operation below is
                 // a chain link of one output, and four independent links in flight hide the FP64 pipeline latency.
                 // Horner inside each group of four diagonals: y_g = sum_{i<4} 256^i S_{4g+i}; |S_e| <= DW * Kpad * 2^14 and the
@@ -318,6 +376,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
         q = a.pq[a.np + im].qd;
         qinv = a.pq[a.np + im].qinv_d;
         c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
+        if (WIDE) c64 = __longlong_as_double((long long)a.consts[3 * PPMM_MAX_MODS + im]);   // 2^64 mod q (balanced)
         qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
 #pragma unroll
         for (int e = 0; e < ND; e++)
@@ -341,25 +400,29 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
     }
 }
 
-size_t ppmm_bdig_bytes(const PpmmArgs& a) { return (size_t)a.mod_num * a.Kpad * a.C * DCMAX; }
+size_t ppmm_bdig_bytes(const PpmmArgs& a, int DC) { return (size_t)a.mod_num * a.Kpad * a.C * (DC <= 5 ? 5 : 7); }
 
-template <int DW>
+template <int DW, int DC>
 static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool pack) {
     const int c_tiles = (int)(a.C / CT);
-    if (pack) hipLaunchKernelGGL(ppmm_pack_kernel, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
+    if (pack) hipLaunchKernelGGL(ppmm_pack_kernel<DC>, dim3(c_tiles, a.Kpad / KS, a.mod_num), dim3(256), 0, stream, a, bdig);
     const int m_tiles = a.Mpad / 128;
     int m_block = 1;                                   // row tiles per patch: the largest divisor of m_tiles up to 6
     for (int d = 2; d <= 6; d++) if (m_tiles % d == 0) m_block = d;
     const unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
-    hipLaunchKernelGGL((ppmm_mfma_kernel<DW, 8, 3>), dim3(blocks), dim3(512), 0, stream, a, (const int8_t*)bdig, c_tiles, m_block);
+    hipLaunchKernelGGL((ppmm_mfma_kernel<DW, 8, 3, DC>), dim3(blocks), dim3(512), 0, stream, a, (const int8_t*)bdig, c_tiles, m_block);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
 
-// pack = false: the digit planes were written by the caller (the gather that emits them directly)
-int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int8_t* bdig, bool pack) {
-    if (DW <= 3) return launch_dw<3>(stream, a, bdig, pack);
-    return launch_dw<4>(stream, a, bdig, pack);
+// pack = false: the digit planes were written by the caller (the gather that emits them directly; 5 residue digits only)
+int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC, int8_t* bdig, bool pack) {
+    if (DC > 5) {
+        if (DW > 3 || !pack) { set_error("PPMM: 7 residue digits go with at most 3 plaintext digits and the pack pass"); return CKKS_E_INVALID; }
+        return launch_dw<3, 7>(stream, a, bdig, pack);
+    }
+    if (DW <= 3) return launch_dw<3, 5>(stream, a, bdig, pack);
+    return launch_dw<4, 5>(stream, a, bdig, pack);
 }
 
 }  // namespace ckks

@@ -286,7 +286,11 @@ int pcmm_decode_coeffs(pcmm_ctx* h, double* vals, const uint64_t* plain, uint64_
 /* PCMM_Scheme::PPMM device part (PPMM_kernel.cuh:93-252, launch :294-340):
  * out[m][mod][c] = fused-rescaled sum_n trunc(W[m][n]*scaler) * mlwe[n][mod][c] mod q_mod, for mod_num ring-pack
  * primes (the reference fixes mod_num = 2), c < (rank+1)*N1.  W: device fp32 row-major [M][Kin];
- * mlwe_ptrs_host: Kin device pointers; out: device [M][mod_num][(rank+1)*N1]. */
+ * mlwe_ptrs_host: Kin device pointers; out: device [M][mod_num][(rank+1)*N1].
+ * Runs on the int8 matrix cores when (rank+1)*N1 is a multiple of 64, the rows are 16-byte aligned and the operands fit balanced
+ * base-256 digits: residues in 5 digits (primes up to 0x7f7f7f7f80, i.e. the 36-bit sets) with |trunc(W*scaler)| <= 0x7f7f7f7f, or
+ * residues in 7 digits (primes below 2^50, i.e. the reference's own 49-bit ring-pack primes) with |trunc(W*scaler)| <= 0x7f7f7f;
+ * anything else takes a one-output-per-lane kernel with 128-bit accumulation (pcmm_info "last_path" tells which ran). */
 int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_host, uint64_t* out_dev, int M,
               int Kin, int mod_num, double scaler);
 /* same contraction with the MLWE operands in one contiguous device array [Kin][mod_num][(rank+1)*N1] */

@@ -209,7 +209,7 @@ public:
     int mat_M = 768, mat_N = 768;
     int N;
     int L;
-    // true: the gather writes PPMM's operand planes directly (ring-pack primes below 2^39); false: rlweCipherDecompose into
+    // true: the gather writes PPMM's operand planes directly (ring-pack primes that fit five balanced digits, i.e. just below 2^39); false: rlweCipherDecompose into
     // mlwe_cipher_buffer and PPMM, call for call as the reference
     bool packed_gather;
 
@@ -223,7 +223,7 @@ public:
         mlwe_rank = N / PCMM_N1;                                                                       // Bert.cuh:24
         if (mlwe_rank != pcmm_scheme.pcmm_context.mlwe_rank) throw std::invalid_argument("Bert: the PCMM context's rank is not N / N1");
         packed_gather = true;
-        for (uint64_tt q : pcmm_scheme.pcmm_context.q_ringpack) packed_gather = packed_gather && q < (1ull << 39);
+        for (uint64_tt q : pcmm_scheme.pcmm_context.q_ringpack) packed_gather = packed_gather && q - 1 <= 0x7f7f7f7f7full;      // five balanced residue digits
         for (int i = 0; i < decomp_num; i++)
             mlwe_cipher_buffer.push_back(new MLWECiphertext(PCMM_N1, q_ringpack_count - 1, q_ringpack_count - 1, mlwe_rank, 0));
     }

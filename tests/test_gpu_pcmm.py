@@ -92,15 +92,73 @@ def test_ppmm_small_36bit(mod_num):
     assert dev.pcmm_context.info("last_DW") == 4
 
 
+@pytest.mark.parametrize("wide", [False, True])
+def test_ppmm_plaintext_digit_edge(wide):
+    """d balanced base-256 digits reach +-0x7f..7f, not 2^(8d-1) - 1: a plaintext entry of 0x7f7f7f stays on three digits, 0x7f7f80
+    needs four (with 7-digit residues that means the generic kernel); both must come out right, on whole rows of such entries."""
+    q = REF_PARAMS[16]["q"][:2] if wide else CFG2_Q[:2]
+    pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
+    C = (rank + 1) * 128
+    M, Kin, scaler = 16, 64, float(2 ** 20)
+    mlwe = [limbs_uniform(700 + n, q, 1, C)[0] for n in range(Kin)]
+    for edge, want_dw in ((0x7F7F7F, 3), (0x7F7F80, 4)):
+        W = np.zeros((M, Kin), dtype=np.float32)
+        W[0, :] = edge / 2.0 ** 20
+        W[1, :] = -edge / 2.0 ** 20
+        W[2, ::2] = edge / 2.0 ** 20
+        want = np.zeros((M, 2, C), dtype=np.uint64)
+        orc.PPMM(W, [m.reshape(-1) for m in mlwe], want.reshape(-1), M, Kin, 2, scaler)
+        dout = DeviceBuffer(want.nbytes)
+        dev.PPMM(DeviceBuffer.from_numpy(W), [to_dev(m) for m in mlwe], dout, M, Kin, 128, Kin, 2, scaler)
+        assert dev.pcmm_context.info("last_absmax") == edge and dev.pcmm_context.info("last_DW") == want_dw
+        assert dev.pcmm_context.info("last_path") == (0 if wide and want_dw == 4 else 1)
+        assert np.array_equal(from_dev(dout, want.shape), want)
+
+
 def test_ppmm_reference_shape_50bit_primes():
     """The reference's own shape: two 50-bit ring-pack primes {q0, q1}, p_ringpack = {p_last}
-    (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284)."""
+    (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284).  Residues of up to 50 bits take the MFMA
+    kernel with 7 digits as long as the plaintext matrix fits 3; beyond that the generic kernel."""
     P = REF_PARAMS[15]
     q = P["q"][:2]
     pair, dev, orc, rank = make(10, 128, q, P["p"][:1], [P["p"][0]], q)
     scaler = float(int(q[1] * float(2 ** 49) / float(2 ** 49)))
-    assert run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1) == 0          # generic kernel
-    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1) == 0
+    assert run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1) == 1          # MFMA kernel, 7 residue digits
+    assert dev.pcmm_context.info("last_DC") == 7 and dev.pcmm_context.info("last_DW") <= 3
+    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1) == 1
+    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, float(2 ** 33), seed=7, w_std=0.1) == 0            # |A| needs 4 digits: generic kernel
+
+
+@pytest.mark.parametrize("mod_num", [1, 2, 3])
+def test_ppmm_wide_primes_with_extreme_operands(mod_num):
+    """49- to 50-bit primes (the reference's logN = 16 set, some just above 2^49) through the 7-digit MFMA kernel: row and K padding,
+    plaintext entries at the edge of 3 digits, residues 0, 1, q - 1, (q - 1) / 2 and (q + 1) / 2 in whole columns and whole samples."""
+    q = REF_PARAMS[16]["q"][:3]
+    assert max(q) > 1 << 49 and max(q) < 1 << 50
+    N1, M, Kin = 128, 130, 200
+    pair, dev, orc, rank = make(10, N1, q + REF_PARAMS[16]["q"][3:4], REF_PARAMS[16]["p"][:1], [REF_PARAMS[16]["p"][0]], q)
+    C = (rank + 1) * N1
+    rng = np.random.default_rng(40 + mod_num)
+    scaler = float(2 ** 20)
+    W = rng.uniform(-7.9, 7.9, (M, Kin)).astype(np.float32)
+    W[3, :] = 0x7F7F7F / 2.0 ** 20                                        # the largest |A| that three balanced digits hold
+    W[4, :] = -0x7F7F7F / 2.0 ** 20
+    W[5, :] = 0.0
+    mlwe = [limbs_uniform(900 + n, q[:mod_num], 1, C)[0] for n in range(Kin)]
+    for j in range(mod_num):
+        edge = [0, 1, q[j] - 1, (q[j] - 1) // 2, (q[j] + 1) // 2]
+        for n in range(Kin):
+            for t, v in enumerate(edge):
+                mlwe[n][j][64 * t + 3] = v                                # whole columns of one edge value
+                mlwe[n][j][C - 1 - t] = edge[(t + n) % 5]                 # mixed along K
+        for t, v in enumerate(edge):
+            mlwe[7 + t][j][:] = v                                         # whole samples
+    want = np.zeros((M, mod_num, C), dtype=np.uint64)
+    orc.PPMM(W, [m.reshape(-1) for m in mlwe], want.reshape(-1), M, Kin, mod_num, scaler)
+    dout = DeviceBuffer(want.nbytes)
+    dev.PPMM(DeviceBuffer.from_numpy(W), [to_dev(m) for m in mlwe], dout, M, Kin, N1, Kin, mod_num, scaler)
+    assert dev.pcmm_context.info("last_path") == 1 and dev.pcmm_context.info("last_DC") == 7 and dev.pcmm_context.info("last_DW") == 3
+    assert np.array_equal(from_dev(dout, want.shape), want)
 
 
 def test_ppmm_shape_errors():
@@ -180,14 +238,14 @@ def test_small_ring_ntt(N1):
         dev.pcmm_context.ToNTTInplace(d, polys, 3, 0, 1, batch)              # moduli 1..3 of three
 
 
-@pytest.mark.parametrize("M,Kin", [(768, 768), (4096, 4096)])
-def test_ppmm_full_size_sampled_against_oracle(M, Kin):
+@pytest.mark.parametrize("M,Kin,wide", [(768, 768, False), (4096, 4096, False), (768, 768, True)])
+def test_ppmm_full_size_sampled_against_oracle(M, Kin, wide):
     """BASELINE configs 4 and 5 at their real shape (N = 2^16, N1 = 128, rank 512, C = 65,664 columns, 12 primes below 2^36, W ~ N(0, 0.02)
     at scale 2^26): the whole product runs on the device; 24 rows of W over three column panels (the first columns, a panel inside the a
     part that straddles a 64-column tile edge, the last columns of the b part) are recomputed by the oracle with the full contraction length
     and compared on every modulus.  Operands: 16 distinct seeded samples, repeated."""
-    L, N1 = 12, 128
-    primes = CFG2_Q[:L]
+    L, N1 = (2, 128) if wide else (12, 128)
+    primes = REF_PARAMS[16]["q"][:2] if wide else CFG2_Q[:L]          # wide: the reference's own two 49-bit ring-pack moduli
     pair = Pair(16, [], primes)
     rank = pair.N // N1
     C = (rank + 1) * N1
@@ -212,6 +270,7 @@ def test_ppmm_full_size_sampled_against_oracle(M, Kin):
     scaler = float(2 ** 26)
     dev.PPMM(DeviceBuffer.from_numpy(W), bufs, dout, M, Kin, N1, Kin, L, scaler)
     assert dev.pcmm_context.info("last_path") == 1 and dev.pcmm_context.info("last_DW") == 3
+    assert dev.pcmm_context.info("last_DC") == (7 if wide else 5)
     rows = sorted(set([0, M - 1, 127, 128] + [int(v) for v in rng.integers(0, M, 20)]))
     Wsub = np.ascontiguousarray(W[rows])
     mlwe = [seeds[n % 16].reshape(-1) for n in range(Kin)]
