@@ -2,6 +2,8 @@
 (encrypt, rlweCipherDecompose, PPMM, mlweCipherPacking, decrypt, compare with the plaintext product, :92-98,195): the decrypted
 coefficients must be the matrix product of W with the coefficient-packed message, up to the scheme's rounding and noise.
 Key generation, encryption and decryption are plain host arithmetic here (they are not on the GPU path)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -90,12 +92,15 @@ def test_encrypt_decompose_ppmm_pack_decrypt(mlwe_num):
     assert worst <= 16 * N, (worst, biggest)
 
 
-def test_bert_base_layer_on_encrypted_activations():
+@pytest.mark.parametrize("activations", ["normal", "reference_file"])
+def test_bert_base_layer_on_encrypted_activations(activations):
     """BASELINE config 4 end to end at its real ring: 128 tokens x 768 activations ~ N(0, 1), coefficient-packed into two RLWE ciphertexts at
     N = 2^16 (ternary secret of weight 192, Gaussian error 3.2, public-key encryption), times W 768 x 768 ~ N(0, 0.02), out as three ring-packed
     ciphertexts of 256 features each - the sequence of Bert::PCMM_Boot_768_768 between its slot/coefficient conversions (Bert.cuh:411-424, 473,
     482, 491) - with every key generated on the device, the gather writing PPMM's operand planes directly, and the decrypted result compared with
-    the plaintext product as the reference's test program does (GetPrecisionStats, precision.cuh:104)."""
+    the plaintext product as the reference's test program does (GetPrecisionStats, precision.cuh:104).  "reference_file" takes the activations
+    from tests/golden/hidden_states.bin, the 128 x 768 fp32 BERT hidden states the reference holds for its own layer test
+    (test_bert_infer.cu:117; values in [-11.1, 4.25], unlike the unit normal ones)."""
     from ckks_llm_amd import Ciphertext, MLWESecretKey, Plaintext, Scheme_23, SecretKey
     logN, N1 = 16, 128
     P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
@@ -113,7 +118,12 @@ def test_bert_base_layer_on_encrypted_activations():
     ps.addRepakcingKey(mlwe_sk, sk)
     rng = np.random.default_rng(4)
     tokens, feat = N1, 768
-    X = rng.normal(0, 1, (tokens, feat))
+    if activations == "reference_file":
+        X = np.fromfile(os.path.join(os.path.dirname(__file__), "golden", "hidden_states.bin"), dtype="<f4").astype(np.float64)
+        assert X.size == tokens * feat and 11.0 < np.abs(X).max() < 11.2
+        X = X.reshape(tokens, feat)
+    else:
+        X = rng.normal(0, 1, (tokens, feat))
     W = rng.normal(0, 0.02, (feat, feat)).astype(np.float32)
     want = X @ W.astype(np.float64).T                                      # [token][output feature]
     x_scale = 1 << 33
@@ -153,7 +163,7 @@ def test_bert_base_layer_on_encrypted_activations():
         worst.append(err.max())
         assert np.abs(got[:, 1:512:2]).max() < 2.0 ** -9                    # the positions between the packed samples hold noise only
         assert np.median(err) < 2.0 ** -13
-    assert np.abs(want).max() > 2.0 and max(worst) < 2.0 ** -10, worst
+    assert np.abs(want).max() > 1.0 and max(worst) < 2.0 ** -10, worst
 
 
 def test_bert_mirror_layers_with_loaded_weights(tmp_path):
