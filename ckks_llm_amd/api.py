@@ -82,9 +82,25 @@ class DeviceBuffer:
 
 
 class Context_23:
-    """Context_23 (Context_23.h:19-279) for the hot path, with explicit prime lists instead of a logN switch."""
+    """Context_23 (Context_23.h:19-279) for the hot path.  `Context_23(logN, p, q, t, gamma)` takes explicit prime lists;
+    `Context_23(logN, logslots, h=64, sigma=3.2)` is the reference's own constructor (Context_23.h:21), which selects the
+    parameter set compiled in for logN = 13..16 (Params.cuh:11-170) and accepts a secret Hamming weight of 64 or 192 only."""
 
-    def __init__(self, logN, p, q, t=(), gamma=0):
+    def __init__(self, logN, p, q=None, t=(), gamma=0):
+        self.logslots, self.h_weight, self.sigma, self.precision = logN - 1, 64, 3.2, 0
+        if isinstance(p, int):                                               # (logN, logslots, h, sigma)
+            from .params import REF_PARAMS
+            self.logslots = p
+            self.h_weight = 64 if q is None else q
+            self.sigma = 3.2 if isinstance(t, tuple) else t
+            if self.h_weight not in (64, 192):
+                raise ValueError("hamming weight error!")                    # Params.cuh:228
+            if logN not in REF_PARAMS:
+                raise ValueError("Context_23: the reference holds parameter sets for logN = 13, 14, 15 and 16 only")
+            r = REF_PARAMS[logN]
+            p, q, t, gamma = r["p"], r["q"], r["t"], r["gamma"]
+            self.precision = 1 << 36 if logN < 15 else 1 << 49               # Params.cuh:15, 36, 58, 85
+        self.slots = 1 << self.logslots
         self.L_ = load_library()
         self.logN, self.N = logN, 1 << logN
         self.pVec, self.qVec, self.tVec = list(p), list(q), list(t)

@@ -3,7 +3,8 @@
 // Same class names, member names, argument order and addressing as the reference's headers, so that code written
 // against Context_23.h / Scheme_23.h / pcmm/PCMM_Scheme.h compiles against this header with
 // `using namespace ckks_llm_amd;`.  Differences, all deliberate:
-//   * primes are passed to the constructor (the reference selects a compiled-in set by logN, Context_23.cuh:12-113);
+//   * Context_23 has a second constructor that takes the primes (the reference only selects a compiled-in set by logN,
+//     Context_23.cuh:12-113; that constructor is here too);
 //   * tables live in the handle, not in process-global __constant__ symbols, so several contexts can coexist;
 //   * scales are long double (the reference uses NTL::RR only for this bookkeeping, Ciphertext.cuh:23);
 //   * C-ABI error codes become exceptions: std::invalid_argument where the reference throws it
@@ -42,22 +43,91 @@ inline void device_release(uint64_tt*& p) {
     p = nullptr;
 }
 
+// The reference's compiled-in parameter sets (Params.cuh:11-170: logN = 13, 14, 15, 16): Q, P and T primes, gamma and the
+// default plaintext precision.  Data only; the bootstrapping polynomials the same function sets are not part of this library.
+struct ReferenceParams {
+    std::vector<uint64_tt> q, p, t;
+    int gamma = 0;
+    long precision = 0;
+};
+inline ReferenceParams reference_params(long logN) {
+    ReferenceParams r;
+    switch (logN) {
+    case 13:
+        r.q = {
+            0x4001b00001, 0xfff9c0001, 0xfff8e0001, 0xfff840001, 0xfff700001,};
+        r.p = {
+            0x10a19000001,};
+        r.t = {
+            0xffffffffffc0001, 0xfffffffff840001, 0xfffffffff6a0001,};
+        r.gamma = 3; r.precision = 1l << 36;
+        break;
+    case 14:
+        r.q = {
+            0x4001b00001, 0xfff9c0001, 0xfff8e0001, 0xfff840001, 0xfff700001, 0xfff640001, 0x1000a20001, 0x1000b40001,
+            0x1000f60001, 0x10011a0001,};
+        r.p = {
+            0x10a19000001, 0x10a3b000001,};
+        r.t = {
+            0xffffffffffc0001, 0xfffffffff840001, 0xfffffffff6a0001, 0xfffffffff5a0001,};
+        r.gamma = 3; r.precision = 1l << 36;
+        break;
+    case 15:
+        r.q = {
+            0x20000018e0001, 0x2000001c00001, 0x2000001ca0001, 0x2000001d20001, 0x1fffffee80001, 0x1fffffede0001,
+            0x1fffffec40001, 0x1fffffe780001, 0x2000000ce0001, 0x20000013a0001, 0x20000013c0001, 0x20000015a0001,};
+        r.p = {
+            0x2000002600001, 0x20000027e0001, 0x2000002800001, 0x20000029e0001,};
+        r.t = {
+            0xffffffffffc0001, 0xfffffffff840001, 0xfffffffff6a0001, 0xfffffffff5a0001, 0xfffffffff2a0001,
+            0xfffffffff240001, 0xffffffffefe0001,};
+        r.gamma = 4; r.precision = 1l << 49;
+        break;
+    case 16:
+        r.q = {
+            0x20000018e0001, 0x2000001c00001, 0x2000001ca0001, 0x2000001d20001, 0x1fffffee80001, 0x1fffffede0001,
+            0x1fffffec40001, 0x1fffffe780001, 0x2000000ce0001, 0x20000013a0001, 0x20000013c0001, 0x20000015a0001,
+            0x1ffffffea0001, 0x1ffffffd40001, 0x1ffffffba0001, 0x1ffffffb40001, 0x20000001a0001, 0x20000005e0001,
+            0x2000000860001, 0x2000000b00001, 0x1ffffffb00001, 0x1ffffffa20001, 0x1ffffff780001, 0x1ffffff5c0001,
+            0x1fffffe5a0001, 0x1fffffe480001, 0x1fffffde80001, 0x1fffffde20001,};
+        r.p = {
+            0x2000002600001, 0x20000027e0001, 0x2000002800001, 0x20000029e0001,};
+        r.t = {
+            0xffffffffffc0001, 0xfffffffff840001, 0xfffffffff6a0001, 0xfffffffff5a0001, 0xfffffffff2a0001,
+            0xfffffffff240001, 0xffffffffefe0001, 0xffffffffeca0001,};
+        r.gamma = 4; r.precision = 1l << 49;
+        break;
+    default:
+        throw std::invalid_argument("Context_23: the reference holds parameter sets for logN = 13, 14, 15 and 16 only");
+    }
+    return r;
+}
+
 // Context_23 (Context_23.h:19-279): prime sets, tables, NTT and basis conversion.
 class Context_23 {
 public:
     long logN, N;
     int p_num, q_num, t_num, gamma, K, L, dnum, Ri_blockNum, Qj_blockNum;
     std::vector<uint64_tt> pVec, qVec, tVec;
+    long logslots = 0, slots = 0, M = 0, Nh = 0, logNh = 0, h = 64, precision = 0;     // Context_23.h:62-89
+    double sigma = 3.2;
     ckks_ctx* handle = nullptr;
 
     Context_23(long logN, const std::vector<uint64_tt>& p, const std::vector<uint64_tt>& q,
                const std::vector<uint64_tt>& t = {}, int gamma = 0)
         : logN(logN), N(1l << logN), p_num((int)p.size()), q_num((int)q.size()), t_num((int)t.size()), gamma(gamma),
           K((int)p.size()), L((int)q.size() - 1), pVec(p), qVec(q), tVec(t) {
-        check(ckks_ctx_create(&handle, (int)logN, p.data(), p_num, q.data(), q_num, t.data(), t_num, gamma), "Context_23");
-        dnum = (int)info("dnum");
-        Ri_blockNum = (int)info("Ri_blockNum");
-        Qj_blockNum = (int)info("Qj_blockNum");
+        create();
+    }
+    // The reference's own constructor (Context_23.h:21, Context_23.cuh:12-52): the parameter set compiled in for logN, the
+    // secret's Hamming weight 64 or 192 ("hamming weight error!" otherwise, Params.cuh:228).
+    Context_23(long logN, long logslots, long h = 64, double sigma = 3.2)
+        : logN(logN), N(1l << logN), logslots(logslots), slots(1l << logslots), h(h), sigma(sigma) {
+        if (h != 64 && h != 192) throw std::invalid_argument("hamming weight error!");
+        ReferenceParams r = reference_params(logN);
+        pVec = r.p; qVec = r.q; tVec = r.t; gamma = r.gamma; precision = r.precision;
+        p_num = K = (int)pVec.size(); q_num = (int)qVec.size(); t_num = (int)tVec.size(); L = q_num - 1;
+        create();
     }
     Context_23(const Context_23&) = delete;
     Context_23& operator=(const Context_23&) = delete;
@@ -68,6 +138,16 @@ public:
         check(ckks_ctx_info(handle, name, &v), "ckks_ctx_info");
         return v;
     }
+private:
+    void create() {
+        M = N << 1; Nh = N >> 1; logNh = logN - 1;
+        if (!slots) { slots = Nh; logslots = logNh; }
+        check(ckks_ctx_create(&handle, (int)logN, pVec.data(), p_num, qVec.data(), q_num, tVec.data(), t_num, gamma), "Context_23");
+        dnum = (int)info("dnum");
+        Ri_blockNum = (int)info("Ri_blockNum");
+        Qj_blockNum = (int)info("Qj_blockNum");
+    }
+public:
 
     // Context_23.h:42-45
     void ToNTTInplace(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len) {

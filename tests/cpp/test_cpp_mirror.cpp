@@ -57,6 +57,32 @@ static int run() {
     context.FromNTTInplace(ct.cipher_device, 0, context.K, 2, context.L + 1, context.L + 1);
     EXPECT(download(ct.cipher_device, h.size()) == h, "FromNTTInplace(ToNTTInplace(x)) == x");
 
+    // ---- the reference's own constructor: Context_23(logN, logslots, h, sigma) picks the compiled-in set (Params.cuh:11-30) ----
+    {
+        Context_23 ref13(13, 12);
+        EXPECT(ref13.q_num == 5 && ref13.p_num == 1 && ref13.t_num == 3 && ref13.gamma == 3 && ref13.slots == 4096 &&
+               ref13.qVec[0] == 0x4001b00001ull && ref13.pVec[0] == 0x10a19000001ull && ref13.tVec[2] == 0xfffffffff6a0001ull &&
+               ref13.precision == (1l << 36) && ref13.h == 64 && ref13.dnum == 5,
+               "Context_23(13, 12) holds the reference's logN = 13 set");
+        const long n13 = ref13.N;
+        orc_ctx* o13 = orc_ctx_create(13, ref13.pVec.data(), 1, ref13.qVec.data(), 5, ref13.tVec.data(), 3, 3);
+        std::vector<uint64_tt> all = ref13.pVec;
+        all.insert(all.end(), ref13.qVec.begin(), ref13.qVec.end());
+        all.insert(all.end(), ref13.tVec.begin(), ref13.tVec.end());
+        std::vector<uint64_tt> x = uniform_limbs(rng, all, 1, n13), w = x;
+        uint64_tt* d = device_alloc_words(x.size());
+        upload(d, x);
+        ref13.ToNTTInplace(d, 0, 0, 1, (int)all.size(), (int)all.size());           // all nine primes in pqt order
+        orc_ntt_fwd(o13, w.data(), 0, 0, 1, (int)all.size(), (int)all.size());
+        EXPECT(download(d, x.size()) == w, "ToNTTInplace over [P | Q | T] of the logN = 13 set == oracle");
+        device_release(d);
+        orc_ctx_destroy(o13);
+        bool bad_h = false, bad_n = false;
+        try { Context_23 c(13, 12, 100); } catch (const std::invalid_argument&) { bad_h = true; }
+        try { Context_23 c(12, 11); } catch (const std::invalid_argument&) { bad_n = true; }
+        EXPECT(bad_h && bad_n, "Hamming weight other than 64 / 192 and an unknown logN throw std::invalid_argument");
+    }
+
     // ---- rescaleAndEqual: level L -> L-1 against the oracle, then std::invalid_argument at level 0 ----
     upload(ct.cipher_device, want);                       // NTT-domain content
     std::vector<uint64_tt> want_rs = want;

@@ -4,7 +4,7 @@ exact for power-of-two scales and within one unit in the last place otherwise.""
 import numpy as np
 import pytest
 
-from ckks_llm_amd import CkksError, Ciphertext, DeviceBuffer, Plaintext, Scheme_23, SecretKey
+from ckks_llm_amd import CkksError, Ciphertext, Context_23, DeviceBuffer, Plaintext, Scheme_23, SecretKey
 from oracle import oracle_py as O
 from tests.gpu_common import Pair, to_dev, from_dev
 from tests.params import CFG2_Q, CFG3_P
@@ -273,3 +273,32 @@ def test_mirror_classes_encrypt_decrypt_decode():
     ctx.decode_coeffs(out, d_vals)
     got = d_vals.download(np.float64)
     assert np.abs(got - vals).max() <= (noise / q[2] + N + 2) / 2.0 ** 20
+
+
+def test_reference_constructor_selects_the_compiled_in_sets():
+    """Context_23(logN, logslots, h, sigma), the reference's own constructor (Context_23.h:21): prime sets, gamma and precision of
+    Params.cuh:11-170, the derived counts of Context_23.cuh:24-35, and one transform over all of [P | Q | T] against the oracle."""
+    from ckks_llm_amd.params import REF_PARAMS
+    for logN, counts in ((13, (1, 5, 3, 3)), (14, (2, 10, 4, 3)), (15, (4, 12, 7, 4)), (16, (4, 28, 8, 4))):
+        ctx = Context_23(logN, logN - 1)
+        assert (ctx.p_num, ctx.q_num, ctx.t_num, ctx.gamma) == counts
+        assert ctx.slots == 1 << (logN - 1) and ctx.precision == (1 << 36 if logN < 15 else 1 << 49)
+        assert ctx.dnum == ctx.q_num // ctx.p_num and ctx.Ri_blockNum == -(-(ctx.p_num + ctx.q_num) // ctx.gamma)
+        assert ctx.Qj_blockNum == -(-ctx.q_num // ctx.p_num)
+        if logN > 14:
+            continue
+        r = REF_PARAMS[logN]
+        primes = r["p"] + r["q"] + r["t"]
+        rng = np.random.default_rng(logN)
+        x = np.stack([rng.integers(0, q, ctx.N, dtype=np.uint64) for q in primes])
+        d = DeviceBuffer.from_numpy(x)
+        ctx.ToNTTInplace(d, 0, 0, 1, len(primes), len(primes))
+        orc = O.OracleContext(logN, r["p"], r["q"], r["t"], r["gamma"])
+        want = x.copy()
+        orc.ToNTTInplace(want, 0, 0, 1, len(primes), len(primes))
+        assert np.array_equal(d.download(np.uint64).reshape(x.shape), want)
+    with pytest.raises(ValueError, match="hamming weight error"):
+        Context_23(13, 12, 100)
+    with pytest.raises(ValueError):
+        Context_23(12, 11)
+    assert Context_23(16, 15, 192).h_weight == 192
