@@ -306,9 +306,12 @@ class Ciphertext:
 
 class SecretKey:
     """SecretKey (SecretKey.cuh:9-31): sparse ternary secret of Hamming weight <= h over [P | Q], NTT domain, sampled from
-    5*h bytes of the context's stream under (key, nonce)."""
+    5*h bytes of the context's stream under (key, nonce).  h = None takes the context's Hamming weight, as the reference's
+    SecretKey(context) does (SecretKey.cuh:20-29)."""
 
-    def __init__(self, context, h=64, key=bytes(32), nonce=0):
+    def __init__(self, context, h=None, key=bytes(32), nonce=0):
+        if h is None:
+            h = context.h_weight
         self.N, self.L, self.K = context.N, context.L, context.K
         self.sx_device = DeviceBuffer(8 * self.N * (self.K + self.L + 1))
         rnd = DeviceBuffer(5 * h + 64)

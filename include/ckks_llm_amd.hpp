@@ -244,7 +244,9 @@ public:
     uint64_tt* sx_device = nullptr;
     int N, L, K;
 
-    explicit SecretKey(Context_23& context, int h = 64) : N((int)context.N), L(context.L), K(context.K) {
+    // h < 0: the context's Hamming weight, as the reference's SecretKey(context) takes it (SecretKey.cuh:20-29)
+    explicit SecretKey(Context_23& context, int h = -1) : N((int)context.N), L(context.L), K(context.K) {
+        if (h < 0) h = (int)context.h;
         sx_device = device_alloc_words((size_t)N * (K + L + 1));
         uint64_tt* rnd = device_alloc_words((size_t)(5 * h + 7) / 8 + 8);
         context.generateRandom_device(reinterpret_cast<uint8_t*>(rnd), (uint64_tt)5 * h);
@@ -742,6 +744,9 @@ public:
         embeded_mlwe_buffer = device_alloc_words((size_t)(pcmm_context.mlwe_rank + 1) * N * (pcmm_context.ringpack_pq_count - 1));
         mult_key_output = device_alloc_words(2 * N * (pcmm_context.ringpack_pq_count - 1));
     }
+    // The reference's signature (PCMM_Scheme.h:19).  It keeps the secret key only for coeffBitRev, a debugging member that
+    // decrypts and encrypts again (PCMM_Scheme.cuh:515-528) and is not part of this library, so the key is not kept here.
+    PCMM_Scheme(PCMM_Context& pcmm_context, Scheme_23& scheme, SecretKey&) : PCMM_Scheme(pcmm_context, scheme) {}
     PCMM_Scheme(const PCMM_Scheme&) = delete;
     ~PCMM_Scheme() {
         device_release(ppmm_output);

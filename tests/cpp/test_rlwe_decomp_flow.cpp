@@ -58,7 +58,7 @@ static int run() {
 
     SecretKey sk(context, 192);
     PCMM_Context pcmm_context(PCMM_N1, mlwe_rank, p_ringpack, q_ringpack, context);
-    PCMM_Scheme pcmm_scheme(pcmm_context, scheme);
+    PCMM_Scheme pcmm_scheme(pcmm_context, scheme, sk);
     const int pq_ringpack_count = pcmm_context.ringpack_pq_count;
     MLWESecretKey mlwe_sk(PCMM_N1, pq_ringpack_count - 1, mlwe_rank);
     pcmm_scheme.convertMLWESKfromRLWESK(mlwe_sk, sk);

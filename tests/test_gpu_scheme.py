@@ -301,4 +301,8 @@ def test_reference_constructor_selects_the_compiled_in_sets():
         Context_23(13, 12, 100)
     with pytest.raises(ValueError):
         Context_23(12, 11)
-    assert Context_23(16, 15, 192).h_weight == 192
+    ctx = Context_23(13, 12, 192)
+    sk = SecretKey(ctx)                                                      # the context's Hamming weight
+    ctx.FromNTTInplace(sk.sx_device, 0, 0, 1, 1, ctx.K + ctx.L + 1)
+    s0 = sk.sx_device.download(np.uint64, ctx.N)
+    assert ctx.h_weight == 192 and 150 < np.count_nonzero(s0) <= 192 and set(np.unique(s0)) <= {0, 1, ctx.pVec[0] - 1}
