@@ -339,6 +339,9 @@ extern "C" int ckks_keyswitch_23(ckks_ctx* c, uint64_t* out, uint64_t* d2, const
     if ((rc = ckks_external_product_t(c, ext, up, swk, l))) return rc;                              // :225
     if ((rc = launch_ntt(c, ext, 0, K + L + 1, swk_blockNum, T, T, (long)RB * T, 2, true))) return rc;   // :226
     if ((rc = ckks_modup_t_to_pql(c, buf, ext, l, 2))) return rc;                                   // :228
+    bool fused = false;
+    if ((rc = launch_ks_moddown_fused(c, out, buf, (long)RB * T * c->N, l, L + 1, false, &fused))) return rc;  // :229 and :231 in two launches
+    if (fused) return CKKS_OK;
     if ((rc = ckks_moddown_pql_to_ql(c, out, buf, l, 2))) return rc;                                // :229
     return launch_ntt(c, out, 0, K, 2, l + 1, L + 1, 0, 1, false);                                  // :231
 }
@@ -372,9 +375,19 @@ extern "C" int ckks_hybrid_keyswitch(ckks_ctx* c, uint64_t* out, uint64_t* in_nt
     int rc;
     if ((rc = launch_ntt(c, in_ntt, 0, P, 1, l + 1, Q, 0, 1, true))) return rc;
     if ((rc = ckks_hybrid_modup(c, dig, in_ntt, l))) return rc;
-    if ((rc = launch_ntt(c, dig, 0, 0, dn, P + l + 1, W, 0, 1, false))) return rc;
-    if ((rc = ckks_hybrid_inner_product(c, ip, dig, evk, l))) return rc;
-    if ((rc = launch_ntt(c, ip, 0, 0, 2, P + l + 1, W, 0, 1, true))) return rc;
+    bool fused = false;
+    const int dnum = (Q + P - 1) / P;
+    // with the one-launch middle the sums' special-prime limbs come out already scaled for the ModDown that follows
+    if ((rc = launch_ks_row_fused(c, dig, ip, evk, dn, P + l + 1, W, W, (long)dnum * W, true, &fused))) return rc;
+    if (!fused) {
+        if ((rc = launch_ntt(c, dig, 0, 0, dn, P + l + 1, W, 0, 1, false))) return rc;
+        if ((rc = ckks_hybrid_inner_product(c, ip, dig, evk, l))) return rc;
+        if ((rc = launch_ntt(c, ip, 0, 0, 2, P + l + 1, W, 0, 1, true))) return rc;
+    }
+    const bool scaled = fused;
+    if ((rc = launch_ks_moddown_fused(c, out, ip, (long)W * c->N, l, Q, scaled, &fused))) return rc;
+    if (fused) return CKKS_OK;
+    if (scaled) { set_error("hybrid_keyswitch: internal: the two one-launch steps apply under the same conditions"); return CKKS_E_UNAVAILABLE; }
     if ((rc = ckks_hybrid_moddown(c, out, ip, l))) return rc;
     return launch_ntt(c, out, 0, P, 2, l + 1, Q, 0, 1, false);
 }

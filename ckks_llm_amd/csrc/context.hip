@@ -307,6 +307,17 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
     int rc = CKKS_OK;
     auto up = [&](int r) { if (rc == CKKS_OK) rc = r; };
     up(upload(&c->d_primes, pc));
+    {
+        // The same constants with N^-1 (and the last inverse twiddle, which carries N^-1) of every special prime p_i multiplied by
+        // (P/p_i)^-1 mod p_i: an inverse transform run with this table leaves, on the special-prime limbs, the scaled residues that
+        // ModDown starts from (BasisConv.cuh:283-289) instead of the plain coefficients.  FP64 back end only.
+        std::vector<ckks::PrimeConst> pm = pc;
+        for (int i = 0; i < K; i++) {
+            pm[i].n_inv_d = balanced_double(H::mulmod(pc[i].n_inv, c->pHatInvVecModp[i], pV[i]), pV[i]);
+            pm[i].w1n_d = balanced_double(H::mulmod(pc[i].w1n, c->pHatInvVecModp[i], pV[i]), pV[i]);
+        }
+        up(upload(&c->d_primes_moddown, pm));
+    }
     up(upload(&c->d_tw_fwd, twf));
     up(upload(&c->d_tw_inv, twi));
     up(upload(&c->d_twd_fwd, twdf));
@@ -338,7 +349,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
 extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     if (!c) return CKKS_OK;
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {c->d_primes, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
+    void* ptrs[] = {c->d_primes, c->d_primes_moddown, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
                     c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_sched, c->d_ntt_mid};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     for (auto& e : c->decode_tabs) (void)hipFree(e.dev);

@@ -68,6 +68,7 @@ struct ckks_ctx {
 
     // device tables
     ckks::PrimeConst* d_primes = nullptr;
+    ckks::PrimeConst* d_primes_moddown = nullptr;   // d_primes with (P/p_i)^-1 folded into the inverse transform's final constants of p_i
     ulonglong2* d_tw_fwd = nullptr;       // [prime][N] (w, shoup(w)), index = reference psi_table index
     ulonglong2* d_tw_inv = nullptr;       // [prime][N] from psiinv_table
     double* d_twd_fwd = nullptr;          // [prime][N] balanced doubles, FP64 back end (0 entries for large primes)
@@ -105,6 +106,16 @@ size_t ntt_sched_bytes();
 size_t ntt_sched_error_offset();
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
+// Middle of the hybrid key switch (forward transform of the digits, inner product with the key, inverse transform of the two sums)
+// with the three row-pass-side steps in one launch; *done = false where it does not apply (the caller then runs the separate steps).
+// scale_special: the sums' special-prime limbs (the first p_num) come out multiplied by (P/p_i)^-1 mod p_i, ready for
+// launch_ks_moddown_fused(..., pre_scaled = true).
+int launch_ks_row_fused(ckks_ctx* c, uint64_t* digits, uint64_t* sums, const uint64_t* key, int ndigits, int mod_num, int poly_mod_len,
+                        long key_digit_stride, long key_z_stride, bool scale_special, bool* done);
+// End of a key switch (ModDown of two extended polynomials, forward transform of the results) with the ModDown inside the first
+// pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).
+int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
+                            bool* done);
 // Forward transform whose first pass reads its input from MLWE samples (the embedding of the ring packing) instead of dev:
 // coefficient pos of polynomial y = coefficient pos >> logk of row y of sample (pos mod 2^logk) >> loggap, zero where pos mod 2^logk
 // is no multiple of 2^loggap; on the limbs of prime start_mod_idx the value is lifted around zero from q0 to p0.

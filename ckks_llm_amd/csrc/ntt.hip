@@ -641,6 +641,8 @@ __global__ __launch_bounds__(256) void ntt_fused_kernel(NttArgs a, NttSched* sch
 
 size_t ntt_sched_bytes() { return sizeof(NttSched); }
 
+static int ensure_mid(ckks_ctx* c, size_t need);
+
 // launches of one chunk of limbs; COMPACT selects the 5-byte inter-pass buffer
 template <class AR, int SA, int SB, bool COMPACT>
 static void launch_passes(ckks_ctx* c, const NttArgs& args, int n, bool inverse) {
@@ -670,12 +672,8 @@ static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, b
         // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
         const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
         if (chunk > max_limbs) chunk = max_limbs;
-        const size_t need = (size_t)chunk * MID_LIMB_BYTES;
-        if (need > c->ntt_mid_cap) {
-            if (c->d_ntt_mid) { (void)hipDeviceSynchronize(); (void)hipFree(c->d_ntt_mid); c->d_ntt_mid = nullptr; c->ntt_mid_cap = 0; }
-            if (hipMalloc(&c->d_ntt_mid, need) != hipSuccess) { set_error("NTT: cannot allocate the inter-pass buffer"); return CKKS_E_NOMEM; }
-            c->ntt_mid_cap = need;
-        }
+        const int rc_mid = ensure_mid(c, (size_t)chunk * MID_LIMB_BYTES);
+        if (rc_mid) return rc_mid;
         args.mid = (char*)c->d_ntt_mid;
     } else {
         args.mid = nullptr;
@@ -762,6 +760,267 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
         case 16: return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
         default: set_error("NTT: logN must be in [8, 16]"); return CKKS_E_INVALID;
     }
+}
+
+
+// ------------------------------------------------------------------------------------------------------------
+// Middle of the hybrid key switch in one launch: the row pass of the forward transform of every digit, the inner product with
+// the key over the digits, and the row pass of the inverse transform of both sums, on one tile of 16 rows of one limb.
+// Between the two row passes the data of a tile never leaves the workgroup: the digits' transforms are multiplied in
+// registers (in the lane layout in which the row pass stores, so the key is read in full lines), the sums go straight into
+// the inverse row pass.  Against the three launches it replaces this saves one write and one read of every digit limb and
+// of both sums.  Same integers as the separate launches: every step is exact modulo the prime.
+// N = 2^16, FP64 back end, 5-byte inter-pass form on both sides.
+// ------------------------------------------------------------------------------------------------------------
+struct KsRowArgs {
+    const char* mid_in;          // inter-pass buffer of the digits' forward transform, limb index o * ndigits + d
+    char* mid_out;               // inter-pass buffer of the sums' inverse transform, limb index o * 2 + z
+    const u64* key;              // limb (z * key_z_stride + d * key_digit_stride + o), canonical residues in the NTT domain
+    const PrimeConst* primes;
+    const double* tw_fwd;
+    const double* tw_inv;
+    int ndigits;
+    long key_digit_stride, key_z_stride;
+};
+__global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
+    typedef RowCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
+    constexpr long N = 1l << 16;
+    static_assert(R == 16 && U == 16 && ROWS == 16, "tile shape");
+    __shared__ double lds[C::LDS_WORDS];
+    const unsigned tile = blockIdx.x, o = blockIdx.y, tid = threadIdx.x;
+    const F64Arith ar(a.primes[o]);
+    const double* twf = a.tw_fwd + (long)o * N;
+    const double* twi = a.tw_inv + (long)o * N;
+    const unsigned u = tid % U, rl = tid / U;
+    const unsigned row = tile * ROWS + rl;
+    double* lrow = lds + rl * C::PITCH;
+    const unsigned tw_off = N1 + row;
+    double acc[2][R];
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[0][j] = acc[1][j] = 0.0;
+    // raw 5-byte values of the digit in work, requested one digit ahead
+    unsigned raw_lo[R], raw_hi[R];
+    auto request = [&](int d) {
+        const char* mid_limb = a.mid_in + ((long)o * a.ndigits + d) * MID_LIMB_BYTES;
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            const char* piece = mid_piece(const_cast<char*>(mid_limb), j, tile);
+            raw_lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
+            raw_hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
+        }
+    };
+    request(0);
+    for (int d = 0; d < a.ndigits; d++) {
+        const u64* ka = a.key + ((long)d * a.key_digit_stride + o) * N + (long)row * N2 + u;
+        const u64* kb = ka + a.key_z_stride * N;
+        double v[R];
+        unsigned two = tw_off;                              // opaque per digit: the twiddle loads stay inside the loop (they hit the
+        asm volatile("" : "+v"(two));                       // cache) instead of occupying registers across it
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = ar.dec40(raw_lo[j], (raw_hi[j] >> (8 * (rl & 3))) & 0xffu);
+        fwd_spread<F64Arith, 8, S1>(v, twf, two, ar);
+        // the first writes of a digit go to the words this lane read last in the digit before: no barrier needed in between
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
+        fwd_packed<F64Arith, 8, S1>(v, twf, two, u, ar);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
+        u64 k0[R], k1[R];                                   // requested once the butterflies' registers are free
+#pragma unroll
+        for (int j = 0; j < R; j++) { k0[j] = ka[j * U]; k1[j] = kb[j * U]; }
+        if (d + 1 < a.ndigits) request(d + 1);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            const double x = ar.balance(lrow[padded(u + j * U)]);                 // column u + 16 j of the row, |x| <= q/2
+            acc[0][j] += ar.mulmod(x, (double)(long long)k0[j]);                  // each term in (-0.51 q, 0.51 q)
+            acc[1][j] += ar.mulmod(x, (double)(long long)k1[j]);
+        }
+    }
+#pragma unroll
+    for (int z = 0; z < 2; z++) {
+        char* mid_limb = a.mid_out + ((long)o * 2 + z) * MID_LIMB_BYTES;
+        double v[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = ar.balance(acc[z][j]);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
+        inv_packed<F64Arith, 8, S1>(v, twi, tw_off, u, ar);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = lrow[padded(u + j * U)];
+        inv_spread<F64Arith, 8, S1, 0>(v, twi, tw_off, ar);
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            char* piece = mid_piece(mid_limb, j, tile);
+            const u64 e = ar.enc40(v[j]);
+            *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
+            *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// End of a key switch: ModDown and the first pass of the forward transform of its result in one launch.  The strided pass
+// of limb q_i of polynomial z takes each of its inputs from the K special-prime limbs and limb q_i of the extended
+// polynomial (BasisConv.cuh:257-326: out = (c_q - sum_i [c_p_i * pHat_i^-1]_p_i * pHat_i) * P^-1 mod q) instead of reading
+// a stored result, so the ModDown output is never written in the coefficient domain.  The special-prime limbs are read once
+// per output prime (from the L2 after the first); the arithmetic is that of the stand-alone FP64 ModDown kernel.
+// ------------------------------------------------------------------------------------------------------------
+struct KsModDownArgs {
+    const u64* in;               // two extended polynomials, coefficient domain: limb i < K modulo p_i, limb K + i modulo q_i
+    long in_z_stride;            // words between the two polynomials
+    char* mid;                   // inter-pass buffer of the forward transform of the results, limb index i * 2 + z
+    const PrimeConst* primes;
+    const double* tw_fwd;
+    const u64* pHatVecModq;      // [q index][K]
+    const u64* pHatInv;          // [K]
+    const u64* PinvModq;         // [q index]
+    int K;
+    int pre_scaled;              // the special-prime limbs already hold [c_p_i * pHat_i^-1]_p_i (canonical)
+};
+__device__ __forceinline__ double exact_u2d(u64 x) {                  // x < 2^52
+    return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0;
+}
+__device__ __forceinline__ double canon_f(const F64Arith& ar, double r) {       // any |r| < 2^52 -> [0, q)
+    r = ar.balance(r);
+    return r < 0.0 ? r + ar.q : r;
+}
+__global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a) {
+    typedef StridedCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    const unsigned tile = blockIdx.x, iq = blockIdx.y >> 1, z = blockIdx.y & 1, tid = threadIdx.x;
+    const unsigned cl = tid % CW, g = tid / CW;
+    const int prime = a.K + (int)iq;
+    const F64Arith ar(a.primes[prime]);
+    const u64* col = a.in + (long)z * a.in_z_stride + tile * CW + cl;
+    double acc[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[j] = 0.0;
+    // the limbs are read one ahead of their use: limb i + 1 (or, after the last special prime, limb q) travels while limb i is worked on
+    u64 x[R], xn[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) x[j] = col[(long)(g + j * G) * N2];
+    for (int i = 0; i < a.K; i++) {
+        const F64Arith ap(a.primes[i]);
+        const double hinv = exact_u2d(a.pHatInv[i]), hat = exact_u2d(a.pHatVecModq[(long)iq * a.K + i]);
+        const u64* nl = col + (long)(i + 1 < a.K ? i + 1 : prime) * N;
+#pragma unroll
+        for (int j = 0; j < R; j++) xn[j] = nl[(long)(g + j * G) * N2];
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            // the canonical representative of each scaled special-prime residue enters the sum, as in the stand-alone kernel
+            if (a.K == 1) acc[j] = exact_u2d(x[j]);                                                  // BasisConv.cuh:274
+            else if (a.pre_scaled) acc[j] += ar.mulmod(exact_u2d(x[j]), hat);
+            else acc[j] += ar.mulmod(canon_f(ap, ap.mulmod(exact_u2d(x[j]), hinv)), hat);
+        }
+#pragma unroll
+        for (int j = 0; j < R; j++) x[j] = xn[j];
+    }
+    const double pinv = exact_u2d(a.PinvModq[iq]);
+    double v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = ar.mulmod(ar.q - canon_f(ar, acc[j]) + exact_u2d(x[j]), pinv);      // in (-0.51 q, 0.51 q)
+    const double* tw = a.tw_fwd + (long)prime * N;
+    fwd_spread<F64Arith, 8, S1>(v, tw, 1u, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
+    fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
+    // lane (cl, g) holds rows 16g .. 16g+15 of column cl: piece (tile, g), the forward layout of the 5-byte form
+    char* piece = mid_piece(a.mid + (long)blockIdx.y * MID_LIMB_BYTES, tile, g);
+    unsigned hi[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const u64 e = ar.enc40(v[j]);
+        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
+        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
+    }
+#pragma unroll
+    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+}
+
+static int ensure_mid(ckks_ctx* c, size_t need) {
+    if (need <= c->ntt_mid_cap) return CKKS_OK;
+    if (c->d_ntt_mid) { (void)hipDeviceSynchronize(); (void)hipFree(c->d_ntt_mid); c->d_ntt_mid = nullptr; c->ntt_mid_cap = 0; }
+    if (hipMalloc(&c->d_ntt_mid, need) != hipSuccess) { set_error("NTT: cannot allocate the inter-pass buffer"); return CKKS_E_NOMEM; }
+    c->ntt_mid_cap = need;
+    return CKKS_OK;
+}
+
+// digits: ndigits polynomials of poly_mod_len limbs, coefficient domain on the limbs of primes 0 .. mod_num-1; sums: two such
+// polynomials, written in the coefficient domain.  *done = false (and nothing launched) where the one-launch middle does not apply.
+int launch_ks_row_fused(ckks_ctx* c, uint64_t* digits, uint64_t* sums, const uint64_t* key, int ndigits, int mod_num, int poly_mod_len,
+                        long key_digit_stride, long key_z_stride, bool scale_special, bool* done) {
+    *done = false;
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the three launches
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || ndigits <= 0 || mod_num <= 0) return CKKS_OK;
+    for (int j = 0; j < mod_num; j++)
+        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    const size_t in_bytes = (size_t)ndigits * mod_num * MID_LIMB_BYTES, out_bytes = (size_t)2 * mod_num * MID_LIMB_BYTES;
+    if (in_bytes + out_bytes > (1ul << 30)) return CKKS_OK;
+    int rc = ensure_mid(c, in_bytes + out_bytes);
+    if (rc) return rc;
+    typedef StridedCfg<8, 8> CS;
+    NttArgs args;
+    args.primes = c->d_primes;
+    args.start_poly_idx = 0; args.start_mod_idx = 0; args.mod_num = mod_num; args.poly_mod_len = poly_mod_len;
+    args.batch_stride_limbs = 0; args.limb_base = 0;
+    // first pass of the digits' forward transform
+    args.data = (u64*)digits; args.poly_num = ndigits; args.limbs_total = (unsigned)(ndigits * mod_num);
+    args.tw = c->d_twd_fwd; args.mid = (char*)c->d_ntt_mid;
+    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, false, true>), dim3(CS::TILES, ndigits * mod_num), dim3(CS::THREADS), 0, c->stream, args);
+    KsRowArgs k;
+    k.mid_in = (const char*)c->d_ntt_mid; k.mid_out = (char*)c->d_ntt_mid + in_bytes; k.key = (const u64*)key; k.primes = c->d_primes;
+    k.tw_fwd = c->d_twd_fwd; k.tw_inv = c->d_twd_inv; k.ndigits = ndigits; k.key_digit_stride = key_digit_stride; k.key_z_stride = key_z_stride;
+    hipLaunchKernelGGL(ks_row_fused_kernel, dim3(RowCfg<8, 8>::TILES, mod_num), dim3(256), 0, c->stream, k);
+    // second pass of the sums' inverse transform
+    args.data = (u64*)sums; args.poly_num = 2; args.limbs_total = (unsigned)(2 * mod_num);
+    args.tw = c->d_twd_inv; args.mid = k.mid_out;
+    if (scale_special) args.primes = c->d_primes_moddown;
+    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, 2 * mod_num), dim3(CS::THREADS), 0, c->stream, args);
+    CKKS_HIP_TRY(hipGetLastError());
+    *done = true;
+    return CKKS_OK;
+}
+
+// in: two extended polynomials [P | Q_l] in the coefficient domain, in_z_stride words apart; out: two polynomials of
+// out_poly_mod_len limbs, written in the NTT domain on limbs 0 .. l.  *done = false (nothing launched) where it does not apply.
+int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
+                            bool* done) {
+    *done = false;
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || c->p_num <= 0 || l < 0) return CKKS_OK;
+    for (int j = 0; j < c->K + l + 1; j++)
+        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    const int limbs = 2 * (l + 1);
+    int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
+    if (rc) return rc;
+    KsModDownArgs m;
+    m.in = (const u64*)in; m.in_z_stride = in_z_stride; m.mid = (char*)c->d_ntt_mid; m.primes = c->d_primes; m.tw_fwd = c->d_twd_fwd;
+    m.pHatVecModq = c->d_pHatVecModq; m.pHatInv = c->d_pHatInvVecModp; m.PinvModq = c->d_PinvModq; m.K = c->K; m.pre_scaled = pre_scaled ? 1 : 0;
+    hipLaunchKernelGGL(ks_moddown_strided_kernel, dim3(StridedCfg<8, 8>::TILES, limbs), dim3(256), 0, c->stream, m);
+    NttArgs args;
+    args.data = (u64*)out; args.primes = c->d_primes; args.tw = c->d_twd_fwd;
+    args.start_poly_idx = 0; args.start_mod_idx = c->K; args.poly_num = 2; args.mod_num = l + 1; args.poly_mod_len = out_poly_mod_len;
+    args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)limbs; args.mid = (char*)c->d_ntt_mid;
+    hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), dim3(RowCfg<8, 8>::TILES, limbs), dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+    CKKS_HIP_TRY(hipGetLastError());
+    *done = true;
+    return CKKS_OK;
 }
 
 static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,

@@ -152,18 +152,26 @@ def test_hybrid_keyswitch_stages(logN, nq, np_, arith_mode):
         assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), ("keyswitch", l)
 
 
-def test_config3_full_size_keyswitch():
+@pytest.mark.parametrize("l", [23, 9])
+def test_config3_full_size_keyswitch(l):
     """BASELINE config 3 at full size: N = 2^16, 24 Q + 6 P primes, dnum = 4, seed 3; parity with the oracle on the
-    whole switch output (every residue)."""
+    whole switch output (every residue), at the top level and at a level whose last digit is partial (10 limbs in digits of 6).
+    At this ring size the middle of the switch (row passes of both transforms around the inner product) is one launch; the
+    same call with the transforms forced to two launches each (ntt mode 1) takes the separate steps and must give the same words."""
     q, p = CFG2_Q, CFG3_P
     pair = Pair(16, p, q)
     o, d, N = pair.orc, pair.dev, pair.N
-    W, nq, np_, l = 30, 24, 6, 23
+    W, nq, np_ = 30, 24, 6
+    dn = -(-(l + 1) // np_)
     evk = limbs_uniform(3, p + q, 2 * 4, N)
-    inp = limbs_uniform(33, q, 1, N)[0]
+    inp = np.zeros((nq, N), dtype=np.uint64)
+    inp[:l + 1] = limbs_uniform(33, q[:l + 1], 1, N)[0]
     wks = np.zeros((2, nq, N), dtype=np.uint64)
     o.hybrid_keyswitch(wks.reshape(-1), inp.copy().reshape(-1), evk.reshape(-1), l)
-    dks = to_dev(np.zeros_like(wks))
-    scratch = DeviceBuffer(8 * (4 + 2) * W * N)
-    d.hybrid_keyswitch(dks, to_dev(inp), to_dev(evk), l, scratch)
-    assert np.array_equal(from_dev(dks, wks.shape), wks)
+    devk = to_dev(evk)
+    for mode in (0, 1):
+        d.set_ntt_mode(mode)
+        dks = to_dev(np.zeros_like(wks))
+        scratch = DeviceBuffer(8 * (dn + 2) * W * N)
+        d.hybrid_keyswitch(dks, to_dev(inp), devk, l, scratch)
+        assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), mode
