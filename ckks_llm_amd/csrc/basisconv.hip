@@ -373,13 +373,13 @@ extern "C" int ckks_hybrid_keyswitch(ckks_ctx* c, uint64_t* out, uint64_t* in_nt
     uint64_t* dig = scratch;
     uint64_t* ip = scratch + (size_t)dn * W * c->N;
     int rc;
-    if ((rc = launch_ntt(c, in_ntt, 0, P, 1, l + 1, Q, 0, 1, true))) return rc;
-    if ((rc = ckks_hybrid_modup(c, dig, in_ntt, l))) return rc;
     bool fused = false;
-    const int dnum = (Q + P - 1) / P;
-    // with the one-launch middle the sums' special-prime limbs come out already scaled for the ModDown that follows
-    if ((rc = launch_ks_row_fused(c, dig, ip, evk, dn, P + l + 1, W, W, (long)dnum * W, true, &fused))) return rc;
+    // Where it applies (N = 2^16, primes below 2^39): five launches up to the sums in the coefficient domain, the digit area of the
+    // scratch serving as work space, the input left as it is; the sums' special-prime limbs come out scaled for the ModDown below.
+    if ((rc = launch_hybrid_front_fused(c, in_ntt, dig, ip, evk, l, &fused))) return rc;
     if (!fused) {
+        if ((rc = launch_ntt(c, in_ntt, 0, P, 1, l + 1, Q, 0, 1, true))) return rc;
+        if ((rc = ckks_hybrid_modup(c, dig, in_ntt, l))) return rc;
         if ((rc = launch_ntt(c, dig, 0, 0, dn, P + l + 1, W, 0, 1, false))) return rc;
         if ((rc = ckks_hybrid_inner_product(c, ip, dig, evk, l))) return rc;
         if ((rc = launch_ntt(c, ip, 0, 0, 2, P + l + 1, W, 0, 1, true))) return rc;

@@ -233,6 +233,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
     std::vector<ckks::ConvBlock> blocks;
     auto iota = [](int lo, int hi) { std::vector<int> v; for (int i = lo; i < hi; i++) v.push_back(i); return v; };
     c->plan_pq_to_t.resize(L + 1); c->plan_qj_to_t.resize(L + 1); c->plan_t_to_pq.resize(L + 1); c->plan_hybrid.resize(L + 1);
+    c->plan_hybrid_all.resize(L + 1);
     for (int l = 0; l <= L; l++) {
         if (gamma > 0 && t_num > 0) {
             // [P|Q] gamma-block -> T (BasisConv.cuh:7-79).  The constants are those of the WHOLE block of [P|Q_L]
@@ -294,10 +295,22 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
                 for (int j = 0; j < hi - lo; j++) { blk.copy_prime[j] = (short)(lo + j); blk.copy_limb[j] = (short)(p_num + lo + j); }
                 blocks.push_back(blk);
             }
+            // the same digits with EVERY prime of [P | Q_l] as a target, target k = prime k (for a prime of the digit itself the
+            // constants reduce to "the residue back": (D/d_j) mod d_j0 = 0 for j != j0, D mod d_j0 = 0), for the key switch whose
+            // ModUp runs inside the first pass of the digits' forward transform
+            if (p_num + l + 1 <= ckks::CONV_MAX_TGT) {
+                c->plan_hybrid_all[l].first = (int)blocks.size(); c->plan_hybrid_all[l].count = nb;
+                for (int b = 0; b < nb; b++) {
+                    int lo = b * p_num, hi = std::min(lo + p_num, l + 1);
+                    ckks::ConvBlock blk;
+                    fill_conv_block(blk, pqt, iota(p_num + lo, p_num + hi), iota(lo, hi), iota(0, p_num + l + 1), iota(0, p_num + l + 1));
+                    blocks.push_back(blk);
+                }
+            }
         }
     }
 
-    for (auto* plans : {&c->plan_pq_to_t, &c->plan_qj_to_t, &c->plan_t_to_pq, &c->plan_hybrid})
+    for (auto* plans : {&c->plan_pq_to_t, &c->plan_qj_to_t, &c->plan_t_to_pq, &c->plan_hybrid, &c->plan_hybrid_all})
         for (ckks::ConvPlan& pl : *plans) {
             pl.f64_ok = pl.count > 0;
             for (int b = 0; b < pl.count; b++) pl.f64_ok = pl.f64_ok && blocks[pl.first + b].f64_ok;
@@ -317,6 +330,25 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
             pm[i].w1n_d = balanced_double(H::mulmod(pc[i].w1n, c->pHatInvVecModp[i], pV[i]), pV[i]);
         }
         up(upload(&c->d_primes_moddown, pm));
+    }
+    if (p_num > 0) {
+        // One table per level l with N^-1 (and the last inverse twiddle) of every prime q_i, i <= l, multiplied by (D/q_i)^-1 mod q_i,
+        // D = the product of the primes of q_i's digit at that level: an inverse transform run with it leaves the scaled residues
+        // y_i that the exact conversion starts from (BasisConv.cuh:18-24).  FP64 back end only.
+        std::vector<ckks::PrimeConst> pu;
+        for (int l = 0; l <= L; l++) {
+            std::vector<ckks::PrimeConst> t = pc;
+            for (int b = 0; b < c->plan_hybrid[l].count; b++) {
+                const ckks::ConvBlock& blk = blocks[c->plan_hybrid[l].first + b];
+                for (int j = 0; j < blk.nsrc; j++) {
+                    const int i = blk.src_prime[j];
+                    t[i].n_inv_d = balanced_double(H::mulmod(pc[i].n_inv, blk.hatinv[j], pqt[i]), pqt[i]);
+                    t[i].w1n_d = balanced_double(H::mulmod(pc[i].w1n, blk.hatinv[j], pqt[i]), pqt[i]);
+                }
+            }
+            pu.insert(pu.end(), t.begin(), t.end());
+        }
+        up(upload(&c->d_primes_modup, pu));
     }
     up(upload(&c->d_tw_fwd, twf));
     up(upload(&c->d_tw_inv, twi));
@@ -349,7 +381,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
 extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     if (!c) return CKKS_OK;
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {c->d_primes, c->d_primes_moddown, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
+    void* ptrs[] = {c->d_primes, c->d_primes_moddown, c->d_primes_modup, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
                     c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_sched, c->d_ntt_mid};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     for (auto& e : c->decode_tabs) (void)hipFree(e.dev);

@@ -68,13 +68,14 @@ struct ckks_ctx {
 
     // device tables
     ckks::PrimeConst* d_primes = nullptr;
+    ckks::PrimeConst* d_primes_modup = nullptr;     // [level][prime]: d_primes with the digit's (D/q_i)^-1 folded in the same way
     ckks::PrimeConst* d_primes_moddown = nullptr;   // d_primes with (P/p_i)^-1 folded into the inverse transform's final constants of p_i
     ulonglong2* d_tw_fwd = nullptr;       // [prime][N] (w, shoup(w)), index = reference psi_table index
     ulonglong2* d_tw_inv = nullptr;       // [prime][N] from psiinv_table
     double* d_twd_fwd = nullptr;          // [prime][N] balanced doubles, FP64 back end (0 entries for large primes)
     double* d_twd_inv = nullptr;
     ckks::ConvBlock* d_conv = nullptr;    // all conversion blocks
-    std::vector<ckks::ConvPlan> plan_pq_to_t, plan_qj_to_t, plan_t_to_pq, plan_hybrid;   // indexed by level l
+    std::vector<ckks::ConvPlan> plan_pq_to_t, plan_qj_to_t, plan_t_to_pq, plan_hybrid, plan_hybrid_all;   // indexed by level l
     // ModDown / rescale constants on device
     uint64_t* d_pHatVecModq = nullptr;    // [L+1][K]
     uint64_t* d_pHatInvVecModp = nullptr; // [K] then [K] Shoup words
@@ -106,12 +107,14 @@ size_t ntt_sched_bytes();
 size_t ntt_sched_error_offset();
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
-// Middle of the hybrid key switch (forward transform of the digits, inner product with the key, inverse transform of the two sums)
-// with the three row-pass-side steps in one launch; *done = false where it does not apply (the caller then runs the separate steps).
-// scale_special: the sums' special-prime limbs (the first p_num) come out multiplied by (P/p_i)^-1 mod p_i, ready for
-// launch_ks_moddown_fused(..., pre_scaled = true).
-int launch_ks_row_fused(ckks_ctx* c, uint64_t* digits, uint64_t* sums, const uint64_t* key, int ndigits, int mod_num, int poly_mod_len,
-                        long key_digit_stride, long key_z_stride, bool scale_special, bool* done);
+// Hybrid key switch up to the inverse transform of the two sums, in five launches where the separate steps take nine:
+//   inverse transform of the input (two passes; the second leaves the residues scaled for the exact conversion, in `work`),
+//   the conversion's quotient estimate per digit and coefficient, the conversion inside the first pass of every digit limb's
+//   forward transform, the row passes of both transforms around the inner product with the key, the last pass of the sums' inverse
+//   transform.  in_ntt: l + 1 limbs of a polynomial of q_num limbs, NTT domain, left untouched; work: at least l + 2 limbs;
+//   sums: two polynomials of poly_mod_len limbs, coefficient domain on return, their first p_num limbs multiplied by (P/p_i)^-1 mod p_i
+//   (ready for launch_ks_moddown_fused(..., pre_scaled = true)).  *done = false where it does not apply (nothing launched).
+int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done);
 // End of a key switch (ModDown of two extended polynomials, forward transform of the results) with the ModDown inside the first
 // pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,

@@ -781,6 +781,11 @@ struct KsRowArgs {
     const double* tw_inv;
     int ndigits;
     long key_digit_stride, key_z_stride;
+    // Limb o >= p_num of digit (o - p_num) / p_num is the input itself: the digit's own residues pass through the conversion and
+    // the forward transform of a coefficient form gives the NTT-domain input back.  With in_ntt set (limb o - p_num of the input,
+    // canonical, NTT domain) that digit's term is taken from there and its transform is never computed.
+    const u64* in_ntt;
+    int p_num;
 };
 __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
     typedef RowCfg<8, 8> C;
@@ -810,10 +815,26 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
             raw_hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
         }
     };
-    request(0);
+    const int own = a.in_ntt && (int)o >= a.p_num ? ((int)o - a.p_num) / a.p_num : -1;
+    if (own != 0) request(0);
+    else if (a.ndigits > 1) request(1);
     for (int d = 0; d < a.ndigits; d++) {
         const u64* ka = a.key + ((long)d * a.key_digit_stride + o) * N + (long)row * N2 + u;
         const u64* kb = ka + a.key_z_stride * N;
+        if (d == own) {
+            const u64* xp = a.in_ntt + (long)((int)o - a.p_num) * N + (long)row * N2 + u;
+            u64 xi[R], k0[R], k1[R];
+#pragma unroll
+            for (int j = 0; j < R; j++) { xi[j] = xp[j * U]; k0[j] = ka[j * U]; k1[j] = kb[j * U]; }
+#pragma unroll
+            for (int j = 0; j < R; j++) {
+                const double x = ar.balance((double)(long long)xi[j]);
+                acc[0][j] += ar.mulmod(x, (double)(long long)k0[j]);
+                acc[1][j] += ar.mulmod(x, (double)(long long)k1[j]);
+            }
+            continue;
+        }
+        const int nxt = d + 1 == own ? d + 2 : d + 1;
         double v[R];
         unsigned two = tw_off;                              // opaque per digit: the twiddle loads stay inside the loop (they hit the
         asm volatile("" : "+v"(two));                       // cache) instead of occupying registers across it
@@ -833,7 +854,7 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
         u64 k0[R], k1[R];                                   // requested once the butterflies' registers are free
 #pragma unroll
         for (int j = 0; j < R; j++) { k0[j] = ka[j * U]; k1[j] = kb[j * U]; }
-        if (d + 1 < a.ndigits) request(d + 1);
+        if (nxt < a.ndigits) request(nxt);
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; j++) {
@@ -900,7 +921,8 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     constexpr long N = 1l << 16;
     __shared__ double lds[C::LDS_WORDS];
-    const unsigned tile = blockIdx.x, iq = blockIdx.y >> 1, z = blockIdx.y & 1, tid = threadIdx.x;
+    // tiles are the slow grid dimension: the workgroups in flight share a few tiles' worth of special-prime columns, which the L2 holds
+    const unsigned tile = blockIdx.y, limb = blockIdx.x, iq = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const unsigned cl = tid % CW, g = tid / CW;
     const int prime = a.K + (int)iq;
     const F64Arith ar(a.primes[prime]);
@@ -941,7 +963,7 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
     // lane (cl, g) holds rows 16g .. 16g+15 of column cl: piece (tile, g), the forward layout of the 5-byte form
-    char* piece = mid_piece(a.mid + (long)blockIdx.y * MID_LIMB_BYTES, tile, g);
+    char* piece = mid_piece(a.mid + (long)limb * MID_LIMB_BYTES, tile, g);
     unsigned hi[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < R; j++) {
@@ -961,13 +983,98 @@ static int ensure_mid(ckks_ctx* c, size_t need) {
     return CKKS_OK;
 }
 
-// digits: ndigits polynomials of poly_mod_len limbs, coefficient domain on the limbs of primes 0 .. mod_num-1; sums: two such
-// polynomials, written in the coefficient domain.  *done = false (and nothing launched) where the one-launch middle does not apply.
-int launch_ks_row_fused(ckks_ctx* c, uint64_t* digits, uint64_t* sums, const uint64_t* key, int ndigits, int mod_num, int poly_mod_len,
-                        long key_digit_stride, long key_z_stride, bool scale_special, bool* done) {
+// ------------------------------------------------------------------------------------------------------------
+// Start of the hybrid key switch: the exact conversion of every digit (BasisConv.cuh:18-58) inside the first pass of the
+// forward transform of the digit's limbs.  y: the digit residues already scaled by (D/d_j)^-1 (left by the inverse transform
+// that ran with the scaled constants), v: the quotient estimates.  Workgroup (tile, o * ndigits + d) produces the 16 columns
+// of limb o of digit d: sum_j y_j * ((D/d_j) mod r_o) - v * (D mod r_o), then the strided pass on them.  For a prime of the
+// digit itself the constants give the residue back.  The extended digits are never written in the coefficient domain.
+// ------------------------------------------------------------------------------------------------------------
+struct KsModUpArgs {
+    const u64* y;                // l + 1 limbs
+    signed char* v;              // [digit][N]
+    char* mid;                   // inter-pass buffer of the digits' forward transform, limb index o * ndigits + d
+    const ConvBlock* blocks;     // one per digit, target k = prime k
+    const PrimeConst* primes;
+    const double* tw_fwd;
+    int ndigits, p_num;
+};
+__global__ __launch_bounds__(256) void ks_modup_quotient_kernel(KsModUpArgs a) {
+    constexpr long N = 1l << 16;
+    const ConvBlock& __restrict__ b = a.blocks[blockIdx.y];
+    const long x = (long)blockIdx.x * 256 + threadIdx.x;
+    double vv = 0.0;
+    for (int j = 0; j < b.nsrc; j++) vv += exact_u2d(a.y[(long)b.src_limb[j] * N + x]) / a.primes[b.src_prime[j]].qd;   // in index order
+    a.v[(long)blockIdx.y * N + x] = (signed char)(int)vv;
+}
+__global__ __launch_bounds__(256) void ks_modup_strided_kernel(KsModUpArgs a) {
+    typedef StridedCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    // tiles are the slow grid dimension: the workgroups in flight share a few tiles' worth of columns of y, which the L2 holds
+    const unsigned tile = blockIdx.y, limb = blockIdx.x, o = limb / a.ndigits, d = limb % a.ndigits, tid = threadIdx.x;
+    const unsigned cl = tid % CW, g = tid / CW;
+    if ((int)o >= a.p_num && ((int)o - a.p_num) / a.p_num == (int)d) return;       // the digit's own limb: taken from the input later
+    const ConvBlock& __restrict__ b = a.blocks[d];
+    const F64Arith ar(a.primes[o]);
+    const unsigned col = tile * CW + cl;
+    const int nsrc = b.nsrc;
+    double acc[R];
+    {
+        const signed char* vp = a.v + (long)d * N + col;
+        const double dm = b.dmod_d[o];
+#pragma unroll
+        for (int j = 0; j < R; j++) acc[j] = -(double)vp[(long)(g + j * G) * N2] * dm;        // |v| <= nsrc, |dmod| <= q/2: exact
+    }
+    // the limbs are read one ahead of their use
+    u64 x[R], xn[R];
+    {
+        const u64* yl = a.y + (long)b.src_limb[0] * N + col;
+#pragma unroll
+        for (int j = 0; j < R; j++) x[j] = yl[(long)(g + j * G) * N2];
+    }
+    for (int s = 0; s < nsrc; s++) {
+        const double hat = b.hat_d[o][s];
+        const u64* yl = a.y + (long)b.src_limb[s + 1 < nsrc ? s + 1 : s] * N + col;
+#pragma unroll
+        for (int j = 0; j < R; j++) xn[j] = yl[(long)(g + j * G) * N2];
+#pragma unroll
+        for (int j = 0; j < R; j++) acc[j] += ar.mulmod(exact_u2d(x[j]), hat);
+#pragma unroll
+        for (int j = 0; j < R; j++) x[j] = xn[j];
+    }
+    double v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = ar.balance(acc[j]);
+    const double* tw = a.tw_fwd + (long)o * N;
+    fwd_spread<F64Arith, 8, S1>(v, tw, 1u, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
+    fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
+    char* piece = mid_piece(a.mid + (long)limb * MID_LIMB_BYTES, tile, g);
+    unsigned hi[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const u64 e = ar.enc40(v[j]);
+        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
+        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
+    }
+#pragma unroll
+    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+}
+
+int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done) {
     *done = false;
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the three launches
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || ndigits <= 0 || mod_num <= 0) return CKKS_OK;
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
+    const int P = c->p_num, Q = c->q_num, W = P + Q;
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || P <= 0 || l < 0 || l > c->L) return CKKS_OK;
+    const int mod_num = P + l + 1, ndigits = (l + 1 + P - 1) / P, dnum = (Q + P - 1) / P;
+    const ConvPlan& plan = c->plan_hybrid_all[l];
+    if (plan.count != ndigits || !plan.f64_ok || !c->d_primes_modup) return CKKS_OK;
     for (int j = 0; j < mod_num; j++)
         if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
     const size_t in_bytes = (size_t)ndigits * mod_num * MID_LIMB_BYTES, out_bytes = (size_t)2 * mod_num * MID_LIMB_BYTES;
@@ -975,22 +1082,33 @@ int launch_ks_row_fused(ckks_ctx* c, uint64_t* digits, uint64_t* sums, const uin
     int rc = ensure_mid(c, in_bytes + out_bytes);
     if (rc) return rc;
     typedef StridedCfg<8, 8> CS;
+    typedef RowCfg<8, 8> CR;
+    const long N = c->N;
+    char* mid = (char*)c->d_ntt_mid;
+    // inverse transform of the input; the second pass writes the scaled residues to `work` and leaves the input alone
     NttArgs args;
-    args.primes = c->d_primes;
-    args.start_poly_idx = 0; args.start_mod_idx = 0; args.mod_num = mod_num; args.poly_mod_len = poly_mod_len;
-    args.batch_stride_limbs = 0; args.limb_base = 0;
-    // first pass of the digits' forward transform
-    args.data = (u64*)digits; args.poly_num = ndigits; args.limbs_total = (unsigned)(ndigits * mod_num);
-    args.tw = c->d_twd_fwd; args.mid = (char*)c->d_ntt_mid;
-    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, false, true>), dim3(CS::TILES, ndigits * mod_num), dim3(CS::THREADS), 0, c->stream, args);
+    args.primes = c->d_primes; args.tw = c->d_twd_inv; args.mid = mid;
+    args.start_poly_idx = 0; args.start_mod_idx = P; args.poly_num = 1; args.mod_num = l + 1; args.poly_mod_len = Q;
+    args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)(l + 1);
+    args.data = (u64*)in_ntt;
+    hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, true, true>), dim3(CR::TILES, l + 1), dim3(CR::THREADS), 0, c->stream, args);
+    args.data = (u64*)work; args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
+    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, l + 1), dim3(CS::THREADS), 0, c->stream, args);
+    // quotient estimates, then the conversion inside the first pass of the digits' forward transform
+    KsModUpArgs u;
+    u.y = (const u64*)work; u.v = (signed char*)(work + (size_t)(l + 1) * N); u.mid = mid; u.blocks = c->d_conv + plan.first;
+    u.primes = c->d_primes; u.tw_fwd = c->d_twd_fwd; u.ndigits = ndigits; u.p_num = P;
+    hipLaunchKernelGGL(ks_modup_quotient_kernel, dim3((unsigned)(N / 256), ndigits), dim3(256), 0, c->stream, u);
+    hipLaunchKernelGGL(ks_modup_strided_kernel, dim3(ndigits * mod_num, CS::TILES), dim3(256), 0, c->stream, u);
+    // row passes of both transforms around the inner product
     KsRowArgs k;
-    k.mid_in = (const char*)c->d_ntt_mid; k.mid_out = (char*)c->d_ntt_mid + in_bytes; k.key = (const u64*)key; k.primes = c->d_primes;
-    k.tw_fwd = c->d_twd_fwd; k.tw_inv = c->d_twd_inv; k.ndigits = ndigits; k.key_digit_stride = key_digit_stride; k.key_z_stride = key_z_stride;
-    hipLaunchKernelGGL(ks_row_fused_kernel, dim3(RowCfg<8, 8>::TILES, mod_num), dim3(256), 0, c->stream, k);
-    // second pass of the sums' inverse transform
-    args.data = (u64*)sums; args.poly_num = 2; args.limbs_total = (unsigned)(2 * mod_num);
-    args.tw = c->d_twd_inv; args.mid = k.mid_out;
-    if (scale_special) args.primes = c->d_primes_moddown;
+    k.mid_in = mid; k.mid_out = mid + in_bytes; k.key = (const u64*)key; k.primes = c->d_primes;
+    k.tw_fwd = c->d_twd_fwd; k.tw_inv = c->d_twd_inv; k.ndigits = ndigits; k.key_digit_stride = W; k.key_z_stride = (long)dnum * W;
+    k.in_ntt = (const u64*)in_ntt; k.p_num = P;
+    hipLaunchKernelGGL(ks_row_fused_kernel, dim3(CR::TILES, mod_num), dim3(256), 0, c->stream, k);
+    // second pass of the sums' inverse transform, special-prime limbs scaled for the ModDown that follows
+    args.data = (u64*)sums; args.primes = c->d_primes_moddown; args.tw = c->d_twd_inv; args.mid = k.mid_out;
+    args.start_mod_idx = 0; args.poly_num = 2; args.mod_num = mod_num; args.poly_mod_len = W; args.limbs_total = (unsigned)(2 * mod_num);
     hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, 2 * mod_num), dim3(CS::THREADS), 0, c->stream, args);
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
@@ -1012,7 +1130,7 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
     KsModDownArgs m;
     m.in = (const u64*)in; m.in_z_stride = in_z_stride; m.mid = (char*)c->d_ntt_mid; m.primes = c->d_primes; m.tw_fwd = c->d_twd_fwd;
     m.pHatVecModq = c->d_pHatVecModq; m.pHatInv = c->d_pHatInvVecModp; m.PinvModq = c->d_PinvModq; m.K = c->K; m.pre_scaled = pre_scaled ? 1 : 0;
-    hipLaunchKernelGGL(ks_moddown_strided_kernel, dim3(StridedCfg<8, 8>::TILES, limbs), dim3(256), 0, c->stream, m);
+    hipLaunchKernelGGL(ks_moddown_strided_kernel, dim3(limbs, StridedCfg<8, 8>::TILES), dim3(256), 0, c->stream, m);
     NttArgs args;
     args.data = (u64*)out; args.primes = c->d_primes; args.tw = c->d_twd_fwd;
     args.start_poly_idx = 0; args.start_mod_idx = c->K; args.poly_num = 2; args.mod_num = l + 1; args.poly_mod_len = out_poly_mod_len;

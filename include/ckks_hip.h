@@ -121,7 +121,8 @@ int ckks_keyswitch_23(ckks_ctx* ctx, uint64_t* out, uint64_t* d2, const uint64_t
 int ckks_hybrid_modup(ckks_ctx* ctx, uint64_t* digits, const uint64_t* in_coeff, int l);
 int ckks_hybrid_inner_product(ckks_ctx* ctx, uint64_t* ip, const uint64_t* digits_ntt, const uint64_t* evk, int l);
 int ckks_hybrid_moddown(ckks_ctx* ctx, uint64_t* out, const uint64_t* in_pq_coeff, int l);
-/* whole switch: in_ntt (q_num limbs, NTT domain; overwritten with its coefficient form) -> out [2][q_num] NTT domain.
+/* whole switch: in_ntt (q_num limbs, NTT domain; on return either overwritten with its coefficient form or left as it was,
+ * depending on the kernels the ring size and primes admit) -> out [2][q_num] NTT domain.
  * scratch: (ceil((l+1)/p_num) + 2) * (p_num+q_num) * N words. */
 int ckks_hybrid_keyswitch(ckks_ctx* ctx, uint64_t* out, uint64_t* in_ntt, const uint64_t* evk, int l, uint64_t* scratch);
 
