@@ -130,4 +130,10 @@ struct NttEmbedSource {
 };
 int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
                         const NttEmbedSource& src);
+// Ring packing up to the inner product with the repacking keys: first pass of the forward transform of the `rank` embedded
+// polynomials (two limbs each, modulo primes prime0 and prime0 + 1, gathered from the samples), then their row pass and the
+// products with the keys in one launch, then the sum over chunks.  work: 2 * rank limbs of scratch; acc: [z][limb][N] sums in
+// the NTT domain.  *done = false where it does not apply (the caller then runs the separate steps).
+int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const uint64_t* keys, int rank, int prime0,
+                              const NttEmbedSource& src, bool* done);
 }  // namespace ckks

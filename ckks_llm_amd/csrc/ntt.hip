@@ -1115,6 +1115,137 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     return CKKS_OK;
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Ring packing: the row pass of the forward transform of the embedded polynomials and their inner product with the repacking
+// keys (mlweCipherPacking, PCMM_Scheme.cuh:389-401) in one launch.  Workgroup (16 rows, limb, chunk) runs the row pass of the
+// polynomials of its chunk one after the other and accumulates their products with both key polynomials in registers; the
+// chunks' partial sums (canonical residues) are added by a second small kernel.  The transformed polynomials, two limbs each,
+// are never written: that is a write and a read of 2 * rank limbs less than the separate launches.
+// ------------------------------------------------------------------------------------------------------------
+struct RepackRowArgs {
+    const char* mid;             // inter-pass buffer of the embedded polynomials' forward transform, limb index im * rank + i
+    const u64* keys;             // key i = [a: 2 limbs | b: 2 limbs], NTT domain
+    u64* partial;                // [chunk][z][im][N]
+    const PrimeConst* primes;
+    const double* tw_fwd;
+    int rank, chunk, prime0;     // limb im is modulo prime prime0 + im of the context
+};
+__global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs a) {
+    typedef RowCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    const unsigned tile = blockIdx.x, im = blockIdx.y, tid = threadIdx.x;
+    const int prime = a.prime0 + (int)im;
+    const F64Arith ar(a.primes[prime]);
+    const double* twf = a.tw_fwd + (long)prime * N;
+    const unsigned u = tid % U, rl = tid / U;
+    const unsigned row = tile * ROWS + rl;
+    double* lrow = lds + rl * C::PITCH;
+    const unsigned tw_off = N1 + row;
+    const int i0 = (int)blockIdx.z * a.chunk, i1 = min(a.rank, i0 + a.chunk);
+    double acc[2][R];
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[0][j] = acc[1][j] = 0.0;
+    unsigned raw_lo[R], raw_hi[R];
+    auto request = [&](int i) {
+        const char* mid_limb = a.mid + ((long)im * a.rank + i) * MID_LIMB_BYTES;
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            const char* piece = mid_piece(const_cast<char*>(mid_limb), j, tile);
+            raw_lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
+            raw_hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
+        }
+    };
+    if (i0 < i1) request(i0);
+    for (int i = i0; i < i1; i++) {
+        const u64* ka = a.keys + ((long)i * 4 + im) * N + (long)row * N2 + u;
+        const u64* kb = ka + 2 * N;
+        double v[R];
+        unsigned two = tw_off;                              // opaque per polynomial: the twiddle loads stay inside the loop
+        asm volatile("" : "+v"(two));
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = ar.dec40(raw_lo[j], (raw_hi[j] >> (8 * (rl & 3))) & 0xffu);
+        fwd_spread<F64Arith, 8, S1>(v, twf, two, ar);
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];           // the words this lane read last: no barrier before
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
+        fwd_packed<F64Arith, 8, S1>(v, twf, two, u, ar);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
+        u64 k0[R], k1[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) { k0[j] = ka[j * U]; k1[j] = kb[j * U]; }
+        if (i + 1 < i1) request(i + 1);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            const double x = ar.balance(lrow[padded(u + j * U)]);
+            acc[0][j] += ar.mulmod(x, (double)(long long)k0[j]);              // each term in (-0.51 q, 0.51 q): exact over any chunk
+            acc[1][j] += ar.mulmod(x, (double)(long long)k1[j]);              // of fewer than 2^13 polynomials
+        }
+    }
+#pragma unroll
+    for (int z = 0; z < 2; z++) {
+        u64* out = a.partial + (((long)blockIdx.z * 2 + z) * 2 + im) * N + (long)row * N2 + u;
+#pragma unroll
+        for (int j = 0; j < R; j++) out[j * U] = ar.canon(ar.balance(acc[z][j]));
+    }
+}
+__global__ __launch_bounds__(256) void repack_reduce_kernel(const u64* partial, u64* acc, const PrimeConst* primes, int prime0, int chunks) {
+    constexpr long N = 1l << 16;
+    const long x = (long)blockIdx.x * 256 + threadIdx.x;
+    const int zi = blockIdx.y;                               // z * 2 + im
+    const F64Arith ar(primes[prime0 + (zi & 1)]);
+    double s = 0.0;
+    for (int ch = 0; ch < chunks; ch++) s += exact_u2d(partial[((long)ch * 4 + zi) * N + x]);      // < chunks * q: exact
+    acc[(long)zi * N + x] = ar.canon(ar.balance(s));
+}
+
+// work: 2 * rank limbs (the area of the embedded polynomials, which this path never writes); acc: [z][im][N] sums, NTT domain.
+// *done = false (nothing launched) where it does not apply.
+int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const uint64_t* keys, int rank, int prime0,
+                              const NttEmbedSource& src, bool* done) {
+    *done = false;
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || rank < 1 || prime0 < 0 || prime0 + 2 > c->nprimes)
+        return CKKS_OK;
+    for (int j = prime0; j < prime0 + 2; j++)
+        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    if (!src.mlwe || src.logk < 0 || src.loggap < 0 || src.loggap > src.logk || src.n1 <= 0 || ((long)src.n1 << src.logk) != c->N ||
+        (1 << src.logk) != rank) return CKKS_OK;
+    int chunks = 16;
+    while (chunks > 1 && (chunks * 4 > 2 * rank || chunks > rank)) chunks >>= 1;
+    const int chunk = (rank + chunks - 1) / chunks;
+    if (chunks * 4 > 2 * rank || chunk >= (1 << 13)) return CKKS_OK;
+    const size_t mid_bytes = (size_t)2 * rank * MID_LIMB_BYTES;
+    if (mid_bytes > (1ul << 30)) return CKKS_OK;
+    int rc = ensure_mid(c, mid_bytes);
+    if (rc) return rc;
+    typedef StridedCfg<8, 8> CS;
+    NttArgs args;
+    args.data = (u64*)work; args.primes = c->d_primes; args.tw = c->d_twd_fwd; args.mid = (char*)c->d_ntt_mid;
+    args.start_poly_idx = 0; args.start_mod_idx = prime0; args.poly_num = rank; args.mod_num = 2; args.poly_mod_len = 2;
+    args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)(2 * rank);
+    args.embed_mlwe = (const u64* const*)src.mlwe;
+    args.embed_p0 = src.p0; args.embed_q0 = src.q0;
+    args.embed_logk = src.logk; args.embed_loggap = src.loggap; args.embed_n1 = src.n1;
+    args.embed_no_wrap = src.q0 / 2 < src.p0 ? 1 : 0;
+    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, false, true, true>), dim3(CS::TILES, 2 * rank), dim3(CS::THREADS), 0, c->stream, args);
+    RepackRowArgs r;
+    r.mid = (const char*)c->d_ntt_mid; r.keys = (const u64*)keys; r.partial = (u64*)work; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd;
+    r.rank = rank; r.chunk = chunk; r.prime0 = prime0;
+    hipLaunchKernelGGL(repack_row_fused_kernel, dim3(RowCfg<8, 8>::TILES, 2, chunks), dim3(256), 0, c->stream, r);
+    hipLaunchKernelGGL(repack_reduce_kernel, dim3((unsigned)(c->N / 256), 4), dim3(256), 0, c->stream, (const u64*)work, (u64*)acc,
+                       (const PrimeConst*)c->d_primes, prime0, chunks);
+    CKKS_HIP_TRY(hipGetLastError());
+    *done = true;
+    return CKKS_OK;
+}
+
 // in: two extended polynomials [P | Q_l] in the coefficient domain, in_z_stride words apart; out: two polynomials of
 // out_poly_mod_len limbs, written in the NTT domain on limbs 0 .. l.  *done = false (nothing launched) where it does not apply.
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,

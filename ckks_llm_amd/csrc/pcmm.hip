@@ -442,12 +442,16 @@ extern "C" int pcmm_mlwe_pack(pcmm_ctx* h, uint64_t* rlwe_out, const uint64_t* c
     src.mlwe = (const uint64_t* const*)h->d_ptrs; src.p0 = h->pq[0]; src.q0 = h->pq[1]; src.n1 = N1;
     src.logk = 0; while ((1 << src.logk) < k) src.logk++;
     src.loggap = 0; while ((mlwe_num << src.loggap) < k) src.loggap++;
-    if ((rc = launch_ntt_embedded(c, embed_scratch, 0, K - 1, k, 2, 2, src))) return rc;           // :389
     RepackArgs ra;
     ra.embed = embed_scratch; ra.keys = repacking_keys; ra.acc = mult_scratch; ra.rlwe = rlwe_out; ra.pq = h->d_pq; ra.N = c->N;
     ra.rank = k; ra.L = c->L;
     ra.pinv = H::invmod(h->pq[0] % h->pq[1], h->pq[1]); ra.pinv_s = H::shoup(ra.pinv, h->pq[1]);
-    hipLaunchKernelGGL(repack_mult_kernel, dim3((unsigned)(c->N / 256), 2), dim3(256), 0, c->stream, ra);
+    bool fused = false;
+    if ((rc = launch_repack_front_fused(c, embed_scratch, mult_scratch, repacking_keys, k, K - 1, src, &fused))) return rc;
+    if (!fused) {
+        if ((rc = launch_ntt_embedded(c, embed_scratch, 0, K - 1, k, 2, 2, src))) return rc;       // :389
+        hipLaunchKernelGGL(repack_mult_kernel, dim3((unsigned)(c->N / 256), 2), dim3(256), 0, c->stream, ra);
+    }
     if ((rc = launch_ntt(c, mult_scratch, 0, K - 1, 2, 2, 2, 0, 1, true))) return rc;              // :405
     hipLaunchKernelGGL(repack_moddown_kernel, dim3((unsigned)(c->N / 256), 2), dim3(256), 0, c->stream, ra);
     CKKS_HIP_TRY(hipGetLastError());
