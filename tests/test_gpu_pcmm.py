@@ -170,7 +170,8 @@ def test_ppmm_shape_errors():
         dev.PPMM(0, [], 0, 4, 4, 128, 5, 2, 1.0)           # mat_N != mlwe_num (:260-263)
 
 
-@pytest.mark.parametrize("logN,N1,mlwe_num", [(12, 128, 32), (12, 128, 8), (10, 64, 16), (16, 128, 512)])
+@pytest.mark.parametrize("logN,N1,mlwe_num", [(12, 128, 32), (12, 128, 8), (10, 64, 16), (16, 128, 512), (16, 128, 64), (16, 256, 256),
+                                              (16, 64, 1024), (16, 4096, 16)])
 def test_mlwe_packing(logN, N1, mlwe_num):
     """mlweCipherPacking through the C ABI against the oracle: embedding, lift to the special prime, NTT, inner product with the
     repacking keys, iNTT, division by the special prime, + (0, b), NTT - bit-exact on random samples and random keys (the
