@@ -302,6 +302,7 @@ extern "C" int ckks_external_product_t(ckks_ctx* c, uint64_t* out, const uint64_
     InnerArgs a;
     a.c = cT; a.key = swk; a.out = out; a.primes = c->d_primes; a.N = c->N;
     a.ndigits = (l + 1 + c->p_num - 1) / c->p_num;                       // cipher_blockNum, ExternalProduct.cuh:87
+    if (a.ndigits > c->dnum) { set_error("external_product_T: the level needs more digits than the key holds (q_num is no multiple of p_num)"); return CKKS_E_INVALID; }
     a.c_mod = c->t_num; a.prime0 = c->p_num + c->q_num;
     a.c_digit_stride = c->t_num; a.key_digit_stride = (long)c->t_num * c->Ri_blockNum;
     a.key_z_stride = (long)c->Ri_blockNum * c->t_num * c->dnum; a.out_z_stride = (long)c->Ri_blockNum * c->t_num;

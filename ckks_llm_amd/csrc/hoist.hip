@@ -307,6 +307,7 @@ extern "C" int ckks_giant_rotate_mult_plain_t(ckks_ctx* c, uint64_t* bs_cipher_T
     a.out = (u64*)bs_cipher_T; a.pqT = (const u64*)PQ_to_T; a.up = (const u64*)modUp_QjtoT; a.primes = c->d_primes;
     a.N = c->N; a.logN = c->logN; a.T = c->t_num; a.RB = c->Ri_blockNum; a.dnum = c->dnum;
     a.digits = (l + 1 + c->p_num - 1) / c->p_num; a.prime0 = c->p_num + c->q_num; a.bs = bs; a.gs = gs;
+    if (a.digits > c->dnum) { set_error("hoisted rotations: the level needs more digits than the keys hold (q_num is no multiple of p_num)"); return CKKS_E_INVALID; }
     for (int j = 0; j < MAX_GS; j++) {
         a.key[j] = j < gs ? (const u64*)rotKeys_host[j] : nullptr;
         a.pow[j] = 1;
@@ -354,6 +355,7 @@ extern "C" int ckks_baby_rotate(ckks_ctx* c, uint64_t* output, const uint64_t* m
     a.out = (u64*)output; a.up = (const u64*)modUp_QjtoT; a.in = (const u64*)input; a.primes = c->d_primes;
     a.N = c->N; a.logN = c->logN; a.T = c->t_num; a.RB = c->Ri_blockNum; a.dnum = c->dnum;
     a.digits = (l + 1 + c->p_num - 1) / c->p_num; a.prime0 = c->p_num + c->q_num; a.rot_num = rotNum;
+    if (a.digits > c->dnum) { set_error("hoisted rotations: the level needs more digits than the keys hold (q_num is no multiple of p_num)"); return CKKS_E_INVALID; }
     bool any = false;
     for (int r = 0; r < MAX_GS; r++) {
         a.key[r] = r < rotNum ? (const u64*)rotKeys_host[r] : nullptr;

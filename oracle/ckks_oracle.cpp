@@ -566,6 +566,7 @@ int orc_external_product_t(const orc_ctx* c, u64* out, const u64* cT, const u64*
     const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum;
     if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L) return -1;
     const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+    if (cipher_blockNum > dnum) return -1;               // q_num is no multiple of p_num: the key holds q_num / p_num digits only
 #pragma omp parallel for collapse(2) schedule(static)
     for (int blk = 0; blk < blockNum; blk++)
         for (int k = 0; k < T; k++)
@@ -1305,6 +1306,7 @@ int orc_giant_rotate_mult_plain_t(const orc_ctx* c, u64* bs_cipher_T, const u64*
     const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, dnum = c->dnum;
     if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L || bs < 1 || gs < 1 || bs > 16) return -1;
     const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+    if (cipher_blockNum > dnum) return -1;
     const size_t half = (size_t)RB * T * N;
     std::vector<u64> pows(gs, 1);
     for (int j = 0; j < gs; j++) if (rotKeys[j]) pows[j] = orc_rot_group(c, rotSlots[j]);

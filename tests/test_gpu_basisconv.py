@@ -92,6 +92,35 @@ def test_external_product_and_keyswitch_23(params):
         assert np.array_equal(from_dev(do, wout.shape)[:, :l + 1], wout[:, :l + 1]), ("keyswitch_23", l)
 
 
+def test_keyswitch_23_full_ring_small_special_primes():
+    """The T-basis switch at N = 2^16 with P and Q primes below 2^39 (36- and 37-bit primes, the reference's 60-bit T primes): at this
+    size its ModDown runs inside the first pass of the final transform; same words as the oracle's separate steps, and as the
+    device's own separate steps (ntt mode 1)."""
+    q, p, t = CFG2_Q[:6], CFG3_P[:2], REF_PARAMS[16]["t"][:3]      # q_num a multiple of p_num, as in every set of the reference
+    pair = Pair(16, p, q, t, 3)
+    o, d, N = pair.orc, pair.dev, pair.N
+    Q, T, RB, QB, dnum, L = o.q_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum, o.dnum, o.L
+    swk = limbs_uniform(7, t, 2 * dnum * RB, N)
+    dswk = to_dev(swk)
+    for l in (L, 2):
+        d2 = np.zeros((Q, N), dtype=np.uint64)
+        d2[:l + 1] = limbs_uniform(20 + l, q[:l + 1], 1, N)[0]
+        wout = np.zeros((2, Q, N), dtype=np.uint64)
+        o.keyswitch_23(wout.reshape(-1), d2.copy().reshape(-1), swk.reshape(-1), l)
+        for mode in (0, 1):
+            d.set_ntt_mode(mode)
+            dd2, do = to_dev(d2), to_dev(np.zeros_like(wout))
+            s1, s2, s3 = DeviceBuffer(8 * N * T * QB), DeviceBuffer(8 * N * T * RB * 2), DeviceBuffer(8 * N * T * RB * 2)
+            s1.zero(); s2.zero(); s3.zero()
+            d.keyswitch_23(do, dd2, dswk, l, s1, s2, s3)
+            assert np.array_equal(from_dev(do, wout.shape)[:, :l + 1], wout[:, :l + 1]), (l, mode)
+    # a context whose q_num is no multiple of p_num has keys of q_num / p_num digits (Context_23.cuh:29): levels that need more are refused
+    odd = Pair(10, p, CFG2_Q[:5], t, 3)
+    with pytest.raises(Exception):
+        odd.dev.external_product_T(to_dev(np.zeros((2, odd.orc.Ri_blockNum * 3, 1024), dtype=np.uint64)),
+                                   to_dev(np.zeros((3, 3, 1024), dtype=np.uint64)), to_dev(np.zeros((2, 2, odd.orc.Ri_blockNum, 3, 1024), dtype=np.uint64)), 4)
+
+
 def test_rescale():
     pair = ref_pair(14, 12)
     o, d, N = pair.orc, pair.dev, pair.N
