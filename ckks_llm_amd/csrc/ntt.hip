@@ -210,6 +210,45 @@ struct NttArgs {
 constexpr int MID_PIECE_BYTES = 1280;
 constexpr long MID_LIMB_BYTES = 256l * MID_PIECE_BYTES;
 __device__ __forceinline__ char* mid_piece(char* mid_limb, unsigned cb, unsigned rb) { return mid_limb + (cb * 16 + rb) * MID_PIECE_BYTES; }
+// Forward first pass, lane (cl, g) holding rows 16g .. 16g+15 of column cl of tile cb: writes its 16 values into piece (cb, g).
+template <class AR>
+__device__ __forceinline__ void mid_store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const typename AR::V (&v)[16], const AR& ar) {
+    char* piece = mid_piece(mid_limb, cb, g);
+    unsigned hi[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const u64 e = ar.enc40(v[j]);
+        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
+        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
+    }
+#pragma unroll
+    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+}
+// Forward second pass, lane (u, rl) of row tile rb taking columns u + 16j of row 16 rb + rl: element (rl, u) of piece (j, rb).
+// The raw words are returned undecoded so that a caller can request them ahead of their use.
+__device__ __forceinline__ void mid_load_row_raw(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, unsigned (&lo)[16], unsigned (&hi)[16]) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const char* piece = mid_piece(const_cast<char*>(mid_limb), j, rb);
+        lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
+        hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
+    }
+}
+template <class AR>
+__device__ __forceinline__ typename AR::V mid_decode_row(const AR& ar, unsigned lo, unsigned hi, unsigned rl) {
+    return ar.dec40(lo, (hi >> (8 * (rl & 3))) & 0xffu);
+}
+// Inverse first pass (row pass) output in the inverse layout of the high bytes: bytes [r_local][c_local].
+template <class AR>
+__device__ __forceinline__ void mid_store_row_inverse(char* mid_limb, unsigned rb, unsigned rl, unsigned u, const typename AR::V (&v)[16], const AR& ar) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        char* piece = mid_piece(mid_limb, j, rb);
+        const u64 e = ar.enc40(v[j]);
+        *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
+        *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
+    }
+}
 
 // limb index of this block -> base pointer and prime.  Limbs are ordered prime-major so that consecutive
 // workgroups reuse one prime's twiddle table while it is hot in L2.
@@ -319,17 +358,7 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
         for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
         fwd_packed<AR, SA, S1>(v, tw, 1u, g, ar);
         if constexpr (COMPACT) {
-            // lane (cl, g) holds rows 16g .. 16g+15 of column cl: piece (tile, g)
-            char* piece = mid_piece(mid_limb, tile, g);
-            unsigned hi[4] = {0, 0, 0, 0};
-#pragma unroll
-            for (int j = 0; j < R; j++) {
-                const u64 e = ar.enc40(v[j]);
-                *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
-                hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
-            }
-#pragma unroll
-            for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+            if constexpr (R == 16) mid_store_columns(mid_limb, tile, g, cl, v, ar);      // the 5-byte form exists for 256 x 256 only
         } else {
 #pragma unroll
             for (int j = 0; j < R; j++) col[(long)(g * R + j) * N2] = ar.to_mid_fwd(v[j]);
@@ -402,13 +431,11 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
     V v[R];
     if (!INVERSE) {
         if constexpr (COMPACT) {
-            // lane (u, rl) takes columns u + 16j of row 16*tile + rl: element (rl, u) of piece (j, tile)
+            if constexpr (R == 16) {
+                unsigned lo[16], hi[16];
+                mid_load_row_raw(mid_limb, tile, rl, u, lo, hi);
 #pragma unroll
-            for (int j = 0; j < R; j++) {
-                const char* piece = mid_piece(mid_limb, j, tile);
-                const unsigned lo = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
-                const unsigned hi = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
-                v[j] = ar.dec40(lo, (hi >> (8 * (rl & 3))) & 0xffu);
+                for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, lo[j], hi[j], rl);
             }
         } else {
 #pragma unroll
@@ -445,13 +472,7 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         if constexpr (COMPACT) {
             // inverse transforms keep the hi bytes as bytes [r_local][c_local]: a wave (16 columns x 4 rows of a piece) stores
             // 64 contiguous bytes per instruction and needs no cross-lane packing
-#pragma unroll
-            for (int j = 0; j < R; j++) {
-                char* piece = mid_piece(mid_limb, j, tile);
-                const u64 e = ar.enc40(v[j]);
-                *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
-                *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
-            }
+            if constexpr (R == 16) mid_store_row_inverse(mid_limb, tile, rl, u, v, ar);
         } else {
 #pragma unroll
             for (int j = 0; j < R; j++) rp[u + j * U] = ar.to_mid_inv(v[j]);
@@ -806,15 +827,7 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
     for (int j = 0; j < R; j++) acc[0][j] = acc[1][j] = 0.0;
     // raw 5-byte values of the digit in work, requested one digit ahead
     unsigned raw_lo[R], raw_hi[R];
-    auto request = [&](int d) {
-        const char* mid_limb = a.mid_in + ((long)o * a.ndigits + d) * MID_LIMB_BYTES;
-#pragma unroll
-        for (int j = 0; j < R; j++) {
-            const char* piece = mid_piece(const_cast<char*>(mid_limb), j, tile);
-            raw_lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
-            raw_hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
-        }
-    };
+    auto request = [&](int d) { mid_load_row_raw(a.mid_in + ((long)o * a.ndigits + d) * MID_LIMB_BYTES, tile, rl, u, raw_lo, raw_hi); };
     const int own = a.in_ntt && (int)o >= a.p_num ? ((int)o - a.p_num) / a.p_num : -1;
     if (own != 0) request(0);
     else if (a.ndigits > 1) request(1);
@@ -839,7 +852,7 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
         unsigned two = tw_off;                              // opaque per digit: the twiddle loads stay inside the loop (they hit the
         asm volatile("" : "+v"(two));                       // cache) instead of occupying registers across it
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ar.dec40(raw_lo[j], (raw_hi[j] >> (8 * (rl & 3))) & 0xffu);
+        for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, raw_lo[j], raw_hi[j], rl);
         fwd_spread<F64Arith, 8, S1>(v, twf, two, ar);
         // the first writes of a digit go to the words this lane read last in the digit before: no barrier needed in between
 #pragma unroll
@@ -880,13 +893,7 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lrow[padded(u + j * U)];
         inv_spread<F64Arith, 8, S1, 0>(v, twi, tw_off, ar);
-#pragma unroll
-        for (int j = 0; j < R; j++) {
-            char* piece = mid_piece(mid_limb, j, tile);
-            const u64 e = ar.enc40(v[j]);
-            *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
-            *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
-        }
+        mid_store_row_inverse(mid_limb, tile, rl, u, v, ar);
     }
 }
 
@@ -962,17 +969,7 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
-    // lane (cl, g) holds rows 16g .. 16g+15 of column cl: piece (tile, g), the forward layout of the 5-byte form
-    char* piece = mid_piece(a.mid + (long)limb * MID_LIMB_BYTES, tile, g);
-    unsigned hi[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int j = 0; j < R; j++) {
-        const u64 e = ar.enc40(v[j]);
-        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
-        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
-    }
-#pragma unroll
-    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+    mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
 }
 
 static int ensure_mid(ckks_ctx* c, size_t need) {
@@ -1055,16 +1052,7 @@ __global__ __launch_bounds__(256) void ks_modup_strided_kernel(KsModUpArgs a) {
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
-    char* piece = mid_piece(a.mid + (long)limb * MID_LIMB_BYTES, tile, g);
-    unsigned hi[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int j = 0; j < R; j++) {
-        const u64 e = ar.enc40(v[j]);
-        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
-        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
-    }
-#pragma unroll
-    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+    mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
 }
 
 int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done) {
@@ -1148,15 +1136,7 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
 #pragma unroll
     for (int j = 0; j < R; j++) acc[0][j] = acc[1][j] = 0.0;
     unsigned raw_lo[R], raw_hi[R];
-    auto request = [&](int i) {
-        const char* mid_limb = a.mid + ((long)im * a.rank + i) * MID_LIMB_BYTES;
-#pragma unroll
-        for (int j = 0; j < R; j++) {
-            const char* piece = mid_piece(const_cast<char*>(mid_limb), j, tile);
-            raw_lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
-            raw_hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
-        }
-    };
+    auto request = [&](int i) { mid_load_row_raw(a.mid + ((long)im * a.rank + i) * MID_LIMB_BYTES, tile, rl, u, raw_lo, raw_hi); };
     if (i0 < i1) request(i0);
     for (int i = i0; i < i1; i++) {
         const u64* ka = a.keys + ((long)i * 4 + im) * N + (long)row * N2 + u;
@@ -1165,7 +1145,7 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
         unsigned two = tw_off;                              // opaque per polynomial: the twiddle loads stay inside the loop
         asm volatile("" : "+v"(two));
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ar.dec40(raw_lo[j], (raw_hi[j] >> (8 * (rl & 3))) & 0xffu);
+        for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, raw_lo[j], raw_hi[j], rl);
         fwd_spread<F64Arith, 8, S1>(v, twf, two, ar);
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];           // the words this lane read last: no barrier before
