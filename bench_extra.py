@@ -79,6 +79,27 @@ def bench_keyswitch(P, reps=10):
                          "frac": round(stage_bytes / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": stage_bytes}}
 
 
+def bench_rescale(P, reps=20):
+    """rescaleAndEqual (Scheme_23.cuh:321-385) of one ciphertext at N = 2^16, 24 primes, from the top level."""
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    q = P.CFG2_Q
+    ctx = Context_23(16, [], q)
+    N, l = 1 << 16, len(q) - 1
+    rng = np.random.default_rng(6)
+    c = np.stack([rng.integers(0, m, (2, N), dtype=np.uint64) for m in q], axis=1)
+    d, scratch = DeviceBuffer.from_numpy(c), DeviceBuffer(8 * 2 * len(q) * N)
+    for _ in range(3):
+        ctx.rescaleAndEqual(d, scratch, l)
+    ctx.timer_start()
+    for _ in range(reps):
+        ctx.rescaleAndEqual(d, scratch, l)
+    ms = ctx.timer_stop() / reps
+    alg = (2 * (l + 1) + 2 * l) * 8 * N        # every limb of the ciphertext read once, every remaining limb written once
+    return {"workload": "rescaleAndEqual: 1 ciphertext, N=2^16, level 23 -> 22 (24 primes <2^36)", "us": round(ms * 1e3, 1),
+            "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
+
+
 def bench_packing(P, N1=128, reps=5):
     """MLWE -> RLWE packing after PPMM (PCMM_Scheme::mlweCipherPacking): rank = 512 samples of N1 = 128 into one ciphertext at
     N = 2^16, one special prime and q0.  Algorithmic bytes: samples in, the embedded polynomials out and through one NTT,
@@ -252,5 +273,5 @@ def bench_hoisted_level(P, gs=16, bs=4, reps=3):
 
 def run(P):
     ref_label = "PPMM 768x768 as the reference's BERT layer calls it: its own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens"
-    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P),
+    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}

@@ -318,6 +318,10 @@ extern "C" int ckks_rescale(ckks_ctx* c, uint64_t* cipher, uint64_t* scratch, in
     const int K = c->K, L = c->L;
     int rc = launch_ntt(c, cipher, l, K + l, 2, 1, L + 1, 0, 1, true);                            // Scheme_23.cuh:372
     if (rc) return rc;
+    const u64* inv_l = (const u64*)c->d_qiInvModql + (size_t)l * (l - 1) / 2;
+    bool fused = false;
+    if ((rc = launch_rescale_fused(c, cipher, l, inv_l, &fused))) return rc;
+    if (fused) return CKKS_OK;
     dim3 grid((unsigned)(c->N / CONV_THREADS), l, 2), block(CONV_THREADS);
     hipLaunchKernelGGL(mod_to_qi_kernel, grid, block, 0, c->stream, (u64*)scratch, (const u64*)cipher, c->d_primes, c->N, K, L + 1, l);
     rc = launch_ntt(c, scratch, 0, K, 2, l, L + 1, 0, 1, false);                                   // :376

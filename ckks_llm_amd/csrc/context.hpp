@@ -115,6 +115,10 @@ int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx
 //   sums: two polynomials of poly_mod_len limbs, coefficient domain on return, their first p_num limbs multiplied by (P/p_i)^-1 mod p_i
 //   (ready for launch_ks_moddown_fused(..., pre_scaled = true)).  *done = false where it does not apply (nothing launched).
 int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done);
+// Rescale after the inverse transform of limb l (cipher: [2][L+1] limbs, inv: q_l^-1 mod q_i for i < l): the reduction of limb l
+// modulo each remaining prime, its forward transform and the final subtraction and scaling in two launches; *done = false where
+// it does not apply.
+int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done);
 // End of a key switch (ModDown of two extended polynomials, forward transform of the results) with the ModDown inside the first
 // pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,

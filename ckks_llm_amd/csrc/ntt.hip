@@ -1226,6 +1226,103 @@ int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const 
     return CKKS_OK;
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Rescale (Scheme_23.cuh:321-385) after the inverse transform of the last limb: the reduction of that limb modulo every
+// remaining prime happens while the first pass of its forward transform loads it, and the final (c_i - x) * q_l^-1 in the
+// second pass, on the values it has just computed, before it stores.  Two launches where the separate steps take four.
+// ------------------------------------------------------------------------------------------------------------
+struct RescaleArgs {
+    u64* cipher;                 // [2][poly_mod_len] limbs; limb l in the coefficient domain, limbs < l in the NTT domain
+    char* mid;                   // limb index i * 2 + z
+    const PrimeConst* primes;
+    const double* tw_fwd;
+    const u64* inv;              // q_l^-1 mod q_i, i < l
+    int l, poly_mod_len, prime0; // limb i is modulo prime prime0 + i
+};
+__global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
+    typedef StridedCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    const unsigned tile = blockIdx.y, limb = blockIdx.x, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
+    const unsigned cl = tid % CW, g = tid / CW;
+    const int prime = a.prime0 + (int)i;
+    const F64Arith ar(a.primes[prime]);
+    const u64* col = a.cipher + ((long)z * a.poly_mod_len + a.l) * N + tile * CW + cl;
+    double v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = ar.balance(exact_u2d(col[(long)(g + j * G) * N2]));      // x mod q_i, |.| <= q_i / 2
+    const double* tw = a.tw_fwd + (long)prime * N;
+    fwd_spread<F64Arith, 8, S1>(v, tw, 1u, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
+    fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
+    mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
+}
+__global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
+    typedef RowCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    const unsigned tile = blockIdx.x, limb = blockIdx.y, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
+    const int prime = a.prime0 + (int)i;
+    const F64Arith ar(a.primes[prime]);
+    const double* tw = a.tw_fwd + (long)prime * N;
+    const unsigned u = tid % U, rl = tid / U;
+    const unsigned row = tile * ROWS + rl;
+    double* lrow = lds + rl * C::PITCH;
+    const unsigned tw_off = N1 + row;
+    u64* rp = a.cipher + ((long)z * a.poly_mod_len + i) * N + (long)row * N2 + u;
+    unsigned lo[R], hi[R];
+    mid_load_row_raw(a.mid + (long)limb * MID_LIMB_BYTES, tile, rl, u, lo, hi);
+    u64 c[R];                                            // the limb's own words, needed after the butterflies
+#pragma unroll
+    for (int j = 0; j < R; j++) c[j] = rp[j * U];
+    double v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, lo[j], hi[j], rl);
+    fwd_spread<F64Arith, 8, S1>(v, tw, tw_off, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
+    fwd_packed<F64Arith, 8, S1>(v, tw, tw_off, u, ar);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
+    __syncthreads();
+    const double inv = exact_u2d(a.inv[i]);
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const double x = ar.balance(lrow[padded(u + j * U)]);
+        rp[j * U] = ar.canon(ar.mulmod(exact_u2d(c[j]) - x, inv));          // |c - x| < 1.5 q
+    }
+}
+// cipher: [2][poly_mod_len] limbs over q_0 .. (prime indices K + i); limb l already in the coefficient domain.
+// *done = false (nothing launched) where it does not apply.
+int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done) {
+    *done = false;
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || l < 1 || l > c->L) return CKKS_OK;
+    for (int j = c->K; j <= c->K + l; j++)
+        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    const int limbs = 2 * l;
+    int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
+    if (rc) return rc;
+    RescaleArgs r;
+    r.cipher = (u64*)cipher; r.mid = (char*)c->d_ntt_mid; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd; r.inv = (const u64*)inv;
+    r.l = l; r.poly_mod_len = c->L + 1; r.prime0 = c->K;
+    hipLaunchKernelGGL(rescale_strided_kernel, dim3(limbs, StridedCfg<8, 8>::TILES), dim3(256), 0, c->stream, r);
+    hipLaunchKernelGGL(rescale_row_kernel, dim3(RowCfg<8, 8>::TILES, limbs), dim3(256), 0, c->stream, r);
+    CKKS_HIP_TRY(hipGetLastError());
+    *done = true;
+    return CKKS_OK;
+}
+
 // in: two extended polynomials [P | Q_l] in the coefficient domain, in_z_stride words apart; out: two polynomials of
 // out_poly_mod_len limbs, written in the NTT domain on limbs 0 .. l.  *done = false (nothing launched) where it does not apply.
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,

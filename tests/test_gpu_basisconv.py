@@ -139,6 +139,30 @@ def test_rescale():
         d.rescaleAndEqual(dc, scratch, 0)                   # level-0 operand (Scheme_23.cuh:192-194 behaviour)
 
 
+def test_rescale_full_ring():
+    """rescaleAndEqual at N = 2^16 on 36-bit primes with a special prime in front (limb i is modulo prime K + i): there the
+    reduction of the last limb and the final subtraction run inside the two passes of the forward transform; same words as the
+    oracle and as the device's separate steps (ntt mode 1), the last limb left in coefficient form, higher limbs untouched."""
+    q, p = CFG2_Q[:7], CFG3_P[:1]
+    pair = Pair(16, p, q)
+    o, d, N = pair.orc, pair.dev, pair.N
+    for l in (6, 3, 1):
+        c = limbs_uniform(60 + l, q, 2, N)
+        c[:, :, :4] = 0
+        for j, qq in enumerate(q):
+            c[:, j, 4] = qq - 1
+        want = c.copy()
+        o.rescaleAndEqual(want.reshape(-1), l)
+        for mode in (0, 1):
+            d.set_ntt_mode(mode)
+            dc = to_dev(c)
+            scratch = DeviceBuffer(8 * 2 * len(q) * N)
+            d.rescaleAndEqual(dc, scratch, l)
+            got = from_dev(dc, c.shape)
+            assert np.array_equal(got[:, :l + 1], want[:, :l + 1]), (l, mode)
+            assert np.array_equal(got[:, l + 1:], c[:, l + 1:]), (l, mode)
+
+
 @pytest.mark.parametrize("arith_mode", [0, 1])
 @pytest.mark.parametrize("logN,nq,np_", [(12, 6, 2), (10, 7, 3), (12, 24, 6), (10, 3, 1)])
 def test_hybrid_keyswitch_stages(logN, nq, np_, arith_mode):
