@@ -972,6 +972,17 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
     mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
 }
 
+// The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
+// transform modes, every prime involved below 2^39.  CKKS_KS_SPLIT (any value) in the environment switches them off, for tuning.
+static bool stage_fusion_applies(const ckks_ctx* c, int first_prime, int prime_count) {
+    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed) return false;
+    if (first_prime < 0 || prime_count < 1 || first_prime + prime_count > c->nprimes) return false;
+    for (int j = first_prime; j < first_prime + prime_count; j++)
+        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return false;
+    return true;
+}
+
 static int ensure_mid(ckks_ctx* c, size_t need) {
     if (need <= c->ntt_mid_cap) return CKKS_OK;
     if (c->d_ntt_mid) { (void)hipDeviceSynchronize(); (void)hipFree(c->d_ntt_mid); c->d_ntt_mid = nullptr; c->ntt_mid_cap = 0; }
@@ -1057,14 +1068,11 @@ __global__ __launch_bounds__(256) void ks_modup_strided_kernel(KsModUpArgs a) {
 
 int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done) {
     *done = false;
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
     const int P = c->p_num, Q = c->q_num, W = P + Q;
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || P <= 0 || l < 0 || l > c->L) return CKKS_OK;
+    if (P <= 0 || l < 0 || l > c->L || !stage_fusion_applies(c, 0, P + l + 1)) return CKKS_OK;
     const int mod_num = P + l + 1, ndigits = (l + 1 + P - 1) / P, dnum = (Q + P - 1) / P;
     const ConvPlan& plan = c->plan_hybrid_all[l];
     if (plan.count != ndigits || !plan.f64_ok || !c->d_primes_modup) return CKKS_OK;
-    for (int j = 0; j < mod_num; j++)
-        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
     const size_t in_bytes = (size_t)ndigits * mod_num * MID_LIMB_BYTES, out_bytes = (size_t)2 * mod_num * MID_LIMB_BYTES;
     if (in_bytes + out_bytes > (1ul << 30)) return CKKS_OK;
     int rc = ensure_mid(c, in_bytes + out_bytes);
@@ -1190,11 +1198,7 @@ __global__ __launch_bounds__(256) void repack_reduce_kernel(const u64* partial, 
 int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const uint64_t* keys, int rank, int prime0,
                               const NttEmbedSource& src, bool* done) {
     *done = false;
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || rank < 1 || prime0 < 0 || prime0 + 2 > c->nprimes)
-        return CKKS_OK;
-    for (int j = prime0; j < prime0 + 2; j++)
-        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    if (rank < 1 || !stage_fusion_applies(c, prime0, 2)) return CKKS_OK;
     if (!src.mlwe || src.logk < 0 || src.loggap < 0 || src.loggap > src.logk || src.n1 <= 0 || ((long)src.n1 << src.logk) != c->N ||
         (1 << src.logk) != rank) return CKKS_OK;
     int chunks = 16;
@@ -1306,10 +1310,7 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
 // *done = false (nothing launched) where it does not apply.
 int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done) {
     *done = false;
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || l < 1 || l > c->L) return CKKS_OK;
-    for (int j = c->K; j <= c->K + l; j++)
-        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    if (l < 1 || l > c->L || !stage_fusion_applies(c, c->K, l + 1)) return CKKS_OK;
     const int limbs = 2 * l;
     int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
     if (rc) return rc;
@@ -1328,10 +1329,7 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
                             bool* done) {
     *done = false;
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;          // tuning hook: keep the separate launches
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed || c->p_num <= 0 || l < 0) return CKKS_OK;
-    for (int j = 0; j < c->K + l + 1; j++)
-        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return CKKS_OK;
+    if (c->p_num <= 0 || l < 0 || l > c->L || !stage_fusion_applies(c, 0, c->K + l + 1)) return CKKS_OK;
     const int limbs = 2 * (l + 1);
     int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
     if (rc) return rc;
