@@ -205,18 +205,20 @@ def test_hybrid_keyswitch_stages(logN, nq, np_, arith_mode):
         assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), ("keyswitch", l)
 
 
-@pytest.mark.parametrize("l", [23, 9])
-def test_config3_full_size_keyswitch(l):
+@pytest.mark.parametrize("nq,np_,l", [(24, 6, 23), (24, 6, 9), (5, 2, 4), (3, 1, 2), (3, 1, 0), (7, 3, 3)])
+def test_config3_full_size_keyswitch(nq, np_, l):
     """BASELINE config 3 at full size: N = 2^16, 24 Q + 6 P primes, dnum = 4, seed 3; parity with the oracle on the
-    whole switch output (every residue), at the top level and at a level whose last digit is partial (10 limbs in digits of 6).
+    whole switch output (every residue), at the top level and at a level whose last digit is partial (10 limbs in digits of 6);
+    then smaller prime sets at the same ring size: a partial last digit at the top level, one special prime (digits of one prime, the
+    ModDown's single-prime branch), level 0, and a level that leaves whole digits unused.
     At this ring size the middle of the switch (row passes of both transforms around the inner product) is one launch; the
     same call with the transforms forced to two launches each (ntt mode 1) takes the separate steps and must give the same words."""
-    q, p = CFG2_Q, CFG3_P
+    q, p = CFG2_Q[:nq], CFG3_P[:np_]
     pair = Pair(16, p, q)
     o, d, N = pair.orc, pair.dev, pair.N
-    W, nq, np_ = 30, 24, 6
+    W = nq + np_
     dn = -(-(l + 1) // np_)
-    evk = limbs_uniform(3, p + q, 2 * 4, N)
+    evk = limbs_uniform(3, p + q, 2 * -(-nq // np_), N)
     inp = np.zeros((nq, N), dtype=np.uint64)
     inp[:l + 1] = limbs_uniform(33, q[:l + 1], 1, N)[0]
     wks = np.zeros((2, nq, N), dtype=np.uint64)
