@@ -100,6 +100,42 @@ def bench_rescale(P, reps=20):
                          "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
 
 
+def bench_mult_23(P, reps=10):
+    """Scheme_23::mult_23 (KeySwitch_23.cuh:192-236) on the reference's own logN = 16 parameter set at the top level: tensor product,
+    key switch through the T basis with a relinearisation key generated on the device, the two additions."""
+    from ckks_llm_amd import Ciphertext, Context_23, DeviceBuffer, Plaintext, Scheme_23, SecretKey
+    ctx = Context_23(16, 15, 192)
+    N, L, K, T, RB = ctx.N, ctx.L, ctx.K, ctx.t_num, ctx.Ri_blockNum
+    key = bytes(range(32))
+    scheme = Scheme_23(ctx, key=key)
+    sk = SecretKey(ctx, key=key, nonce=1)
+    scheme.addEncKey(sk)
+    scheme.addMultKey_23(sk)
+    msg = Plaintext(N, L, L, N // 2, 1 << 40)
+    ctx.encode_coeffs(DeviceBuffer.from_numpy(np.random.default_rng(0).uniform(-1, 1, N)), msg)
+    a, b = Ciphertext(N, L, L, N // 2, 1 << 40), Ciphertext(N, L, L, N // 2, 1 << 40)
+    scheme.encryptMsg(a, msg)
+    scheme.encryptMsg(b, msg)
+    res = Ciphertext(N, L, L, N // 2, 1)
+    for _ in range(3):
+        scheme.mult_23(res, a, b)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(reps):
+        scheme.mult_23(res, a, b)
+    ms = ctx.timer_stop() / reps
+    Q, digits, blocks = L + 1, -(-(L + 1) // K), -(-(K + L + 1) // ctx.gamma)
+    # stage sum of minimal limb moves: tensor product r4Q w3Q, iNTT 2Q, Qj -> T rQ w(digits T), NTT 2 digits T, inner product
+    # r(digits T + 2 digits blocks T) w(2 blocks T), iNTT 4 blocks T, T -> PQ r(2 blocks T) w2(K+Q), ModDown r2(K+Q) w2Q, NTT 4Q, additions r4Q w2Q
+    limbs = 7 * Q + 2 * Q + Q + digits * T + 2 * digits * T + digits * T + 2 * digits * blocks * T + 2 * blocks * T + 4 * blocks * T \
+        + 2 * blocks * T + 2 * (K + Q) + 2 * (K + Q) + 2 * Q + 4 * Q + 6 * Q
+    alg = limbs * 8 * N
+    return {"workload": "mult_23 on the reference's logN=16 parameter set (28 Q + 4 P primes of 49-50 bits, 8 T primes of 60 bits), level 27",
+            "ms": round(ms, 4), "mult_per_s": round(1e3 / ms, 1),
+            "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
+
+
 def bench_packing(P, N1=128, reps=5):
     """MLWE -> RLWE packing after PPMM (PCMM_Scheme::mlweCipherPacking): rank = 512 samples of N1 = 128 into one ciphertext at
     N = 2^16, one special prime and q0.  Algorithmic bytes: samples in, the embedded polynomials out and through one NTT,
@@ -273,5 +309,5 @@ def bench_hoisted_level(P, gs=16, bs=4, reps=3):
 
 def run(P):
     ref_label = "PPMM 768x768 as the reference's BERT layer calls it: its own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens"
-    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P),
+    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "mult_23_ref_params": bench_mult_23(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}
