@@ -668,7 +668,10 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
-        hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad, DW);
+        // every plane the kernel instance reads is written (3 or 4: the instances are built for these widths), also those above the
+        // measured digit count, which are zero for this matrix but may hold an earlier call's digits
+        hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad,
+                           DW <= 3 ? 3 : 4);
         size_t need = ppmm_bdig_bytes(a, DC);
         if (packed && need > h->Bdig_cap) { set_error("PPMM on digit planes: planes not opened for this shape"); return CKKS_E_STATE; }
         if (need > h->Bdig_cap) {

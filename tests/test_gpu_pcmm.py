@@ -115,6 +115,18 @@ def test_ppmm_plaintext_digit_edge(wide):
         assert np.array_equal(from_dev(dout, want.shape), want)
 
 
+@pytest.mark.parametrize("wide", [False, True])
+def test_ppmm_narrower_matrix_after_a_wider_one(wide):
+    """The same context and shape called with plaintext matrices of 3, then 2, then 1, then 2 balanced digits: the kernel instance
+    reads three digit planes whatever the matrix needs, so the planes above the measured width must be rewritten (to zero) on
+    every call and not keep the digits of the call before."""
+    q = REF_PARAMS[16]["q"][:2] if wide else CFG2_Q[:2]
+    pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
+    for step, (scaler, want_dw) in enumerate(((float(2 ** 26), 3), (float(2 ** 17), 2), (float(2 ** 9), 1), (float(2 ** 18), 2))):
+        assert run_ppmm(dev, orc, rank, 128, 40, 70, 2, q, scaler, seed=300 + step) == 1
+        assert dev.pcmm_context.info("last_DW") == want_dw, (step, dev.pcmm_context.info("last_absmax"))
+
+
 def test_ppmm_reference_shape_50bit_primes():
     """The reference's own shape: two 50-bit ring-pack primes {q0, q1}, p_ringpack = {p_last}
     (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284).  Residues of up to 50 bits take the MFMA
