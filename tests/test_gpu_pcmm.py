@@ -127,6 +127,42 @@ def test_ppmm_narrower_matrix_after_a_wider_one(wide):
         assert dev.pcmm_context.info("last_DW") == want_dw, (step, dev.pcmm_context.info("last_absmax"))
 
 
+@pytest.mark.parametrize("wide", [False, True])
+def test_ppmm_random_shapes_on_one_context(wide):
+    """One context, a sequence of calls with random row counts, depths, modulus counts and plaintext magnitudes (1 to 4 digits),
+    extreme plaintext rows and residues in every call: whatever the work space holds from the call before must not reach the next."""
+    qs = REF_PARAMS[16]["q"][:3] if wide else CFG2_Q[:3]
+    p_sp = REF_PARAMS[16]["p"][0] if wide else CFG3_P[0]
+    pair, dev, orc, rank = make(10, 64, list(qs) + [REF_PARAMS[16]["q"][3] if wide else CFG2_Q[3]], [p_sp], [p_sp], list(qs))
+    N1, scaler = 64, float(2 ** 20)
+    C = (rank + 1) * N1
+    rng = np.random.default_rng(777 + wide)
+    widths = set()
+    for it, bits in enumerate((22, 12, 7, 15, 29 if not wide else 23, 9, 18, 13)):
+        mod_num, M, Kin = int(rng.integers(1, 4)), int(rng.integers(4, 200)), int(rng.integers(1, 260))
+        amax = (1 << bits) - 1
+        W = (rng.integers(-amax, amax + 1, (M, Kin)) / scaler).astype(np.float32)
+        W[0, :], W[1, :], W[2, :] = np.float32(amax / scaler), np.float32(-amax / scaler), 0
+        q = qs[:mod_num]
+        mlwe = [limbs_uniform(5000 + 300 * it + n, q, 1, C)[0] for n in range(Kin)]
+        for j in range(mod_num):
+            edge = [0, 1, q[j] - 1, (q[j] - 1) // 2, (q[j] + 1) // 2]
+            for n in range(Kin):
+                for t, v in enumerate(edge):
+                    mlwe[n][j][(7 * t + 3) % C] = v
+                    mlwe[n][j][C - 1 - t] = edge[(t + n) % 5]
+        want = np.zeros((M, mod_num, C), dtype=np.uint64)
+        orc.PPMM(W, [m.reshape(-1) for m in mlwe], want.reshape(-1), M, Kin, mod_num, scaler)
+        dout = DeviceBuffer(want.nbytes)
+        bufs = [to_dev(m) for m in mlwe]
+        dev.PPMM(DeviceBuffer.from_numpy(W), bufs, dout, M, Kin, N1, Kin, mod_num, scaler)
+        widths.add(dev.pcmm_context.info("last_DW"))
+        assert np.array_equal(from_dev(dout, want.shape), want), (it, bits, M, Kin, mod_num, dev.pcmm_context.info("last_path"))
+        for b in bufs + [dout]:
+            b.free()
+    assert widths >= {1, 2, 3}
+
+
 def test_ppmm_reference_shape_50bit_primes():
     """The reference's own shape: two 50-bit ring-pack primes {q0, q1}, p_ringpack = {p_last}
     (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284).  Residues of up to 50 bits take the MFMA
