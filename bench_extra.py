@@ -6,7 +6,7 @@ MFMA_I8_PEAK_MACS = 2.5166e15      # 5.033 POP/s dense int8
 HBM_PEAK = 8.0e12
 
 
-def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None):
+def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None, scaler=None):
     from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
     primes = list(primes[:L]) if primes is not None else P.CFG2_Q[:L]
     ctx = Context_23(16, [], primes)
@@ -31,7 +31,7 @@ def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None)
         b.L_.ckks_memcpy_d2d(b.ptr, seeds[n % 16].ptr, per)
         bufs.append(b)
     out = DeviceBuffer(8 * M * L * C)
-    scaler = float(2 ** 26)
+    scaler = float(2 ** 26) if scaler is None else float(scaler)
     sch.PPMM(dW, bufs, out, M, Kin, N1, Kin, L, scaler)      # warm-up (also allocates the workspace)
     ctx.sync()
     best = 1e30
@@ -44,7 +44,7 @@ def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None)
     macs = word_macs * DW * DC
     res = {"workload": label or "configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (3 if M == 768 else 4, M, Kin, N1, L, C),
            "ms": round(best, 3), "word_MAC_per_s": round(word_macs / (best * 1e-3), 1), "int8_MAC_per_s": round(macs / (best * 1e-3), 1),
-           "D_w": DW, "D_c": DC, "kernel": "int8 MFMA" if path == 1 else "generic u128",
+           "D_w": DW, "D_c": DC, "plaintext_slices": sch.pcmm_context.info("last_slices"), "kernel": "int8 MFMA" if path == 1 else "generic u128",
            "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
                         "unit": "TMAC/s (int8)", "frac": round(macs / (best * 1e-3) / MFMA_I8_PEAK_MACS, 4)}}
     for b in bufs + seeds + [out, dW]:
@@ -308,6 +308,9 @@ def bench_hoisted_level(P, gs=16, bs=4, reps=3):
 
 
 def run(P):
-    ref_label = "PPMM 768x768 as the reference's BERT layer calls it: its own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens"
-    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "mult_23_ref_params": bench_mult_23(P),
+    ref_label = "PPMM 768x768 on the reference's own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens, plaintext scaled by 2^26"
+    ref_scale_label = ("PPMM 768x768 as the reference's BERT layer calls it: its two 49-bit ring-pack moduli and its scaler q1 * 2^49 / scale "
+                       "with scale = 2^49 (PPMM_kernel.cuh:283-284), i.e. 46-bit plaintext entries, N=2^16, 128 tokens")
+    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label),
+            "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "mult_23_ref_params": bench_mult_23(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}

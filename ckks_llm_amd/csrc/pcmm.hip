@@ -205,7 +205,8 @@ __global__ __launch_bounds__(256) void digits_kernel(const long long* A, int8_t*
     unsigned long long biased = 0x8080808080808080ull;
     if (m < M && n < Kin) biased += (unsigned long long)A[(long)m * Kin + n];
     const long pos = ((long)(m >> 4) * (Kpad >> 6) + (n >> 6)) * 1024 + ((n & 63) >> 4) * 256 + (m & 15) * 16 + (n & 15);
-    for (int d = 0; d < DW; d++) dig[(long)d * Mpad * Kpad + pos] = (int8_t)(((biased >> (8 * d)) & 0xff) ^ 0x80);
+    // digits above the eighth are zero: the MFMA path takes |A| below the smallest prime, far below 2^63
+    for (int d = 0; d < DW; d++) dig[(long)d * Mpad * Kpad + pos] = d < 8 ? (int8_t)(((biased >> (8 * d)) & 0xff) ^ 0x80) : (int8_t)0;
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -233,6 +234,44 @@ __global__ __launch_bounds__(256) void ppmm_generic_kernel(PpmmArgs a) {
         } else {
             u64 temp = r + pr.q - r_last;                                   // :244
             o[(long)im * a.C + c] = mul_shoup(temp, a.consts[im], a.consts[PPMM_MAX_MODS + im], pr.q);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Plaintext matrices wider than one MFMA launch takes (more than 4 balanced digits, 3 with the 7-digit residues) are cut into
+// slices of three digits, A = sum_s A_s 2^(24 s): one launch per slice writes the residues of A_s x Ct as they are, and this
+// kernel forms sum_s (2^(24 s) mod q) * slice_s mod q and then the fused rescale of PPMM_kernel.cuh:213-249 - the same
+// integers as one pass over the whole of A, since every step is exact modulo the prime.
+// ------------------------------------------------------------------------------------------------------------
+struct PpmmCombineArgs {
+    u64* out;                     // slice 0 on entry, the result on return; [M][mod_num][C]
+    const u64* more;              // slices 1 .. slices-1, each [M][mod_num][C]
+    const PrimeConst* pq;
+    const u64* consts;            // row 0: q_last^-1 mod q_i, row 1: its Shoup word
+    long C, per_slice;            // per_slice = M * mod_num * C
+    int M, mod_num, np, slices;
+    u64 w[2][PPMM_MAX_MODS];      // 2^24 mod q_i, 2^48 mod q_i
+};
+__global__ __launch_bounds__(256) void ppmm_combine_kernel(PpmmCombineArgs a) {
+    const long c = (long)blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (c >= a.C) return;
+    u64* o = a.out + (long)m * a.C * a.mod_num;
+    const u64* t = a.more + (long)m * a.C * a.mod_num;
+    u64 r_last = 0;
+    for (int im = a.mod_num - 1; im >= 0; im--) {
+        const PrimeConst& pr = a.pq[a.np + im];
+        const long idx = (long)im * a.C + c;
+        u128w acc = {o[idx], 0};
+        for (int s = 1; s < a.slices; s++) mac128(acc, t[(long)(s - 1) * a.per_slice + idx], a.w[s - 1][im]);
+        const u64 r = barrett128(acc, pr.q, pr.mu_hi, pr.mu_lo);
+        if (im == a.mod_num - 1) {
+            r_last = r;
+            o[idx] = r;
+        } else {
+            const u64 temp = r + pr.q - r_last;                             // PPMM_kernel.cuh:244
+            o[idx] = mul_shoup(temp, a.consts[im], a.consts[PPMM_MAX_MODS + im], pr.q);
         }
     }
 }
@@ -269,7 +308,7 @@ extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, 
 extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     if (!h) return CKKS_OK;
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw};
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw, h->d_slices};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     if (h->small) ckks_ctx_destroy(h->small);
     delete h;
@@ -613,7 +652,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     }
     // workspace
     const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 191) / 192 * 192;   // K padded to a multiple of three 64-deep MFMA steps (LDS ring of three slots)
-    size_t needA = (size_t)M * Kin, needD = (size_t)8 * Mpad * Kpad;
+    size_t needA = (size_t)M * Kin, needD = (size_t)9 * Mpad * Kpad;     // up to three slices of three digit planes
     if (needA > h->A_cap) {
         if (h->d_A) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_A); h->d_A = nullptr; }
         CKKS_HIP_TRY(hipMalloc((void**)&h->d_A, needA * sizeof(long long)));
@@ -653,7 +692,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     PpmmArgs a;
     a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
     a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
-    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np;
+    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np; a.raw_all = 0;
     // digit counts.  d balanced digits in [-128, 127] reach from -0x80..80 up to +0x7f..7f (d bytes each), NOT up to 2^(8d-1) - 1:
     // the bytes of x + 0x80..80 must not carry into byte d.  DW digits must hold +-|A|max, DC digits every residue 0 .. qmax - 1.
     auto top = [](int d) { unsigned long long v = 0; for (int i = 0; i < d; i++) v = (v << 8) | 0x7f; return v; };
@@ -661,17 +700,20 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     int DC = 1; while (DC < 8 && qmax - 1 > top(DC)) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
     // residues in 5 digits (q < 2^39) with up to 4 plaintext digits, or in 7 digits (q < 2^50) with up to 3
-    const bool width_ok = (DC <= 5 && DW <= 4) || (DC <= 7 && qmax < (1ull << 50) && DW <= 3 && !packed);
+    // wider plaintext matrices (any int64) go through the same kernels in slices of three digits
+    const bool one_launch = (DC <= 5 && DW <= 4) || (DC <= 7 && qmax < (1ull << 50) && DW <= 3);
+    const int slices = one_launch ? 1 : (DW + 2) / 3;
+    const bool width_ok = (DC <= 5 || (DC <= 7 && qmax < (1ull << 50))) && slices <= 3;
     const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && width_ok &&
-                         (long)Kpad * (DW <= 3 ? 3 : 4) <= 16384 && absmax < qmin && qmin > (1ull << 25);
+                         (long)Kpad * (slices == 1 && DW == 4 ? 4 : 3) <= 16384 && absmax < qmin && qmin > (1ull << 25);
     if (packed && !mfma_ok) { set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
-    h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax;
+    h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax; h->last_slices = mfma_ok ? slices : 0;
     if (mfma_ok) {
         long total = (long)Mpad * Kpad;
         // every plane the kernel instance reads is written (3 or 4: the instances are built for these widths), also those above the
         // measured digit count, which are zero for this matrix but may hold an earlier call's digits
         hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad,
-                           DW <= 3 ? 3 : 4);
+                           slices > 1 ? 3 * slices : DW <= 3 ? 3 : 4);
         size_t need = ppmm_bdig_bytes(a, DC);
         if (packed && need > h->Bdig_cap) { set_error("PPMM on digit planes: planes not opened for this shape"); return CKKS_E_STATE; }
         if (need > h->Bdig_cap) {
@@ -681,8 +723,35 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             h->Bdig_cap = need;
         }
         if (!packed) h->packed_K = h->packed_mods = 0;     // the planes now hold this call's operands
-        rc = launch_ppmm_mfma_impl(c->stream, a, DW, DC, h->d_Bdig, !packed);
-        if (rc) return rc;
+        if (slices == 1) {
+            rc = launch_ppmm_mfma_impl(c->stream, a, DW, DC, h->d_Bdig, !packed);
+            if (rc) return rc;
+        } else {
+            const size_t per_slice = (size_t)M * mod_num * C;
+            if ((slices - 1) * per_slice > h->slices_cap) {
+                if (h->d_slices) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_slices); h->d_slices = nullptr; h->slices_cap = 0; }
+                hipError_t e = hipMalloc((void**)&h->d_slices, (slices - 1) * per_slice * sizeof(uint64_t));
+                if (e != hipSuccess) { set_error("PPMM: cannot allocate the buffers of the plaintext slices"); return CKKS_E_NOMEM; }
+                h->slices_cap = (slices - 1) * per_slice;
+            }
+            PpmmArgs sa = a;
+            sa.raw_all = 1;
+            for (int sl = 0; sl < slices; sl++) {
+                sa.Adig = h->d_Adig + (size_t)3 * sl * Mpad * Kpad;
+                sa.out = sl == 0 ? out : h->d_slices + (size_t)(sl - 1) * per_slice;
+                rc = launch_ppmm_mfma_impl(c->stream, sa, 3, DC, h->d_Bdig, !packed && sl == 0);      // the residue planes are packed once
+                if (rc) return rc;
+            }
+            PpmmCombineArgs ca;
+            ca.out = out; ca.more = h->d_slices; ca.pq = h->d_pq; ca.consts = d_cst; ca.C = C; ca.per_slice = (long)per_slice;
+            ca.M = M; ca.mod_num = mod_num; ca.np = h->np; ca.slices = slices;
+            for (int i = 0; i < mod_num; i++) {
+                const uint64_t qi = h->pq[h->np + i];
+                ca.w[0][i] = H::powmod(2, 24, qi);
+                ca.w[1][i] = H::powmod(2, 48, qi);
+            }
+            hipLaunchKernelGGL(ppmm_combine_kernel, dim3((unsigned)((C + 255) / 256), M), dim3(256), 0, c->stream, ca);
+        }
     } else {
         dim3 grid((unsigned)((C + 255) / 256), M), block(256);
         hipLaunchKernelGGL(ppmm_generic_kernel, grid, block, 0, c->stream, a);
@@ -695,6 +764,7 @@ extern "C" int pcmm_info(const pcmm_ctx* h, const char* name, long* value) {
     if (!h || !name || !value) return CKKS_E_INVALID;
     std::string n(name);
     if (n == "last_path") *value = h->last_path; else if (n == "last_DW") *value = h->last_DW; else if (n == "last_DC") *value = h->last_DC;
+    else if (n == "last_slices") *value = h->last_slices;
     else if (n == "last_absmax") *value = (long)h->last_absmax; else if (n == "N1") *value = h->N1; else if (n == "mlwe_rank") *value = h->rank;
     else { set_error("pcmm_info: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;

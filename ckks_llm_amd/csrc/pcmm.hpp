@@ -21,6 +21,9 @@ struct pcmm_ctx {
     size_t zero_cap = 0;
     int packed_K = 0, packed_mods = 0;       // shape the residue digit planes were opened for by pcmm_packed_begin (0: not open)
     int last_path = -1, last_DW = 0, last_DC = 0;   // what the last PPMM call ran: 1 = MFMA kernel, 0 = generic kernel
+    int last_slices = 0;                     // plaintext digit slices of the last MFMA call (1: one launch with the fused rescale)
+    uint64_t* d_slices = nullptr;            // outputs of the plaintext slices above the first, [slice - 1][M][mod_num][C]
+    size_t slices_cap = 0;
     unsigned long long last_absmax = 0;
     ckks_ctx* small = nullptr;               // tables of the size-N1 transform over the ring-pack primes, built on first use
     uint64_t* d_small_tw = nullptr;          // tables of the size-N1 transform when N1 < 256: [prime][forward | inverse][N1]
@@ -48,6 +51,7 @@ struct PpmmArgs {
     const u64* consts;            // PPMM_CONST_WORDS words, see above
     long C;
     int M, Kin, Mpad, Kpad, mod_num, np;
+    int raw_all;                  // MFMA kernel: store every modulus' residue as it is (no fused rescale); the caller combines slices
 };
 
 size_t ppmm_bdig_bytes(const PpmmArgs& a, int DC);

@@ -394,7 +394,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
         // ---- end of a prime: exact recombination, reduction mod q, fused rescale ----
         // Straight-line code (the prime-position and M-padding cases are resolved once, outside the unrolled loops) so that
         // the independent output chains of a lane can be interleaved.
-        const bool last = im == a.mod_num - 1, full = m0 + MT <= a.M;
+        const bool last = a.raw_all || im == a.mod_num - 1, full = m0 + MT <= a.M;
         if (last) { if (full) epilogue(im, std::true_type{}, std::true_type{}); else epilogue(im, std::true_type{}, std::false_type{}); }
         else      { if (full) epilogue(im, std::false_type{}, std::true_type{}); else epilogue(im, std::false_type{}, std::false_type{}); }
     }
@@ -418,7 +418,7 @@ static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool p
 // pack = false: the digit planes were written by the caller (the gather that emits them directly; 5 residue digits only)
 int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC, int8_t* bdig, bool pack) {
     if (DC > 5) {
-        if (DW > 3 || !pack) { set_error("PPMM: 7 residue digits go with at most 3 plaintext digits and the pack pass"); return CKKS_E_INVALID; }
+        if (DW > 3) { set_error("PPMM: 7 residue digits go with at most 3 plaintext digits per launch"); return CKKS_E_INVALID; }
         return launch_dw<3, 7>(stream, a, bdig, pack);
     }
     if (DW <= 3) return launch_dw<3, 5>(stream, a, bdig, pack);

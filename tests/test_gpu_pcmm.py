@@ -95,7 +95,7 @@ def test_ppmm_small_36bit(mod_num):
 @pytest.mark.parametrize("wide", [False, True])
 def test_ppmm_plaintext_digit_edge(wide):
     """d balanced base-256 digits reach +-0x7f..7f, not 2^(8d-1) - 1: a plaintext entry of 0x7f7f7f stays on three digits, 0x7f7f80
-    needs four (with 7-digit residues that means the generic kernel); both must come out right, on whole rows of such entries."""
+    needs four (with 7-digit residues that means two slices of three digits); both must come out right, on whole rows of such entries."""
     q = REF_PARAMS[16]["q"][:2] if wide else CFG2_Q[:2]
     pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
     C = (rank + 1) * 128
@@ -111,7 +111,8 @@ def test_ppmm_plaintext_digit_edge(wide):
         dout = DeviceBuffer(want.nbytes)
         dev.PPMM(DeviceBuffer.from_numpy(W), [to_dev(m) for m in mlwe], dout, M, Kin, 128, Kin, 2, scaler)
         assert dev.pcmm_context.info("last_absmax") == edge and dev.pcmm_context.info("last_DW") == want_dw
-        assert dev.pcmm_context.info("last_path") == (0 if wide and want_dw == 4 else 1)
+        assert dev.pcmm_context.info("last_path") == 1
+        assert dev.pcmm_context.info("last_slices") == (2 if wide and want_dw == 4 else 1)     # 7-digit residues: two slices of three digits
         assert np.array_equal(from_dev(dout, want.shape), want)
 
 
@@ -138,7 +139,8 @@ def test_ppmm_random_shapes_on_one_context(wide):
     C = (rank + 1) * N1
     rng = np.random.default_rng(777 + wide)
     widths = set()
-    for it, bits in enumerate((22, 12, 7, 15, 29 if not wide else 23, 9, 18, 13)):
+    # up to 34 bits against the 36-bit primes (two slices of three digits), up to 48 against the 49-bit ones (three slices)
+    for it, bits in enumerate((22, 12, 47, 7, 30, 15, 23, 9, 40, 13) if wide else (22, 12, 34, 7, 15, 29, 9, 33, 18, 13)):
         mod_num, M, Kin = int(rng.integers(1, 4)), int(rng.integers(4, 200)), int(rng.integers(1, 260))
         amax = (1 << bits) - 1
         W = (rng.integers(-amax, amax + 1, (M, Kin)) / scaler).astype(np.float32)
@@ -160,13 +162,13 @@ def test_ppmm_random_shapes_on_one_context(wide):
         assert np.array_equal(from_dev(dout, want.shape), want), (it, bits, M, Kin, mod_num, dev.pcmm_context.info("last_path"))
         for b in bufs + [dout]:
             b.free()
-    assert widths >= {1, 2, 3}
+    assert widths >= ({1, 2, 3, 4, 6, 7} if wide else {1, 2, 3, 4, 5})
 
 
 def test_ppmm_reference_shape_50bit_primes():
     """The reference's own shape: two 50-bit ring-pack primes {q0, q1}, p_ringpack = {p_last}
     (test_rlwe_decomp.cu:36-49), scaler = q1 * 2^49 / scale (PPMM_kernel.cuh:283-284).  Residues of up to 50 bits take the MFMA
-    kernel with 7 digits as long as the plaintext matrix fits 3; beyond that the generic kernel."""
+    kernel with 7 digits, in one launch as long as the plaintext matrix fits 3 digits and in slices of three digits beyond."""
     P = REF_PARAMS[15]
     q = P["q"][:2]
     pair, dev, orc, rank = make(10, 128, q, P["p"][:1], [P["p"][0]], q)
@@ -174,7 +176,13 @@ def test_ppmm_reference_shape_50bit_primes():
     assert run_ppmm(dev, orc, rank, 128, 16, 24, 2, q, float(2 ** 20), seed=5, w_std=0.1) == 1          # MFMA kernel, 7 residue digits
     assert dev.pcmm_context.info("last_DC") == 7 and dev.pcmm_context.info("last_DW") <= 3
     assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, scaler / 2 ** 30, seed=6, w_std=0.1) == 1
-    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, float(2 ** 33), seed=7, w_std=0.1) == 0            # |A| needs 4 digits: generic kernel
+    assert run_ppmm(dev, orc, rank, 128, 8, 8, 2, q, float(2 ** 33), seed=7, w_std=0.1) == 1            # |A| needs 4 digits: two slices
+    assert dev.pcmm_context.info("last_slices") == 2
+    # the reference's own scale: scaler = q1 * 2^49 / 2^49 (PPMM_kernel.cuh:283-284), plaintext entries of 46 bits, two slices
+    assert run_ppmm(dev, orc, rank, 128, 40, 70, 2, q, scaler, seed=8, w_std=0.05) == 1
+    assert dev.pcmm_context.info("last_slices") == 2 and dev.pcmm_context.info("last_DW") == 6
+    assert run_ppmm(dev, orc, rank, 128, 40, 70, 2, q, scaler, seed=9, w_std=0.12) == 1                 # 48-bit entries: seven digits
+    assert dev.pcmm_context.info("last_slices") == 3 and dev.pcmm_context.info("last_DW") == 7
 
 
 @pytest.mark.parametrize("mod_num", [1, 2, 3])
