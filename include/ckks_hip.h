@@ -246,7 +246,8 @@ int pcmm_ctx_destroy(pcmm_ctx* h);
 int pcmm_ntt_fwd(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
 int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size);
 /* "N1", "mlwe_rank", and facts about the last PPMM call: "last_path" (1 = int8 MFMA kernel, 0 = generic 128-bit kernel),
- * "last_DW" / "last_DC" (base-256 digits of the plaintext matrix / of the residues), "last_absmax" (max |A|). */
+ * "last_DW" / "last_DC" (base-256 digits of the plaintext matrix / of the residues), "last_slices" (three-digit slices the
+ * plaintext matrix was cut into on the matrix cores, 1 = one launch), "last_absmax" (max |A|). */
 int pcmm_info(const pcmm_ctx* h, const char* name, long* value);
 /* the gather kernel of PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:50-88,115-119): rlwe = [a | b] with
  * L+1 limbs each, COEFFICIENT domain; mlwe_ptrs_host: mlwe_num device pointers, each [(l+1)][(rank+1)][N1]. */
@@ -289,9 +290,11 @@ int pcmm_decode_coeffs(pcmm_ctx* h, double* vals, const uint64_t* plain, uint64_
  * primes (the reference fixes mod_num = 2), c < (rank+1)*N1.  W: device fp32 row-major [M][Kin];
  * mlwe_ptrs_host: Kin device pointers; out: device [M][mod_num][(rank+1)*N1].
  * Runs on the int8 matrix cores when (rank+1)*N1 is a multiple of 64, the rows are 16-byte aligned and the operands fit balanced
- * base-256 digits: residues in 5 digits (primes up to 0x7f7f7f7f80, i.e. the 36-bit sets) with |trunc(W*scaler)| <= 0x7f7f7f7f, or
- * residues in 7 digits (primes below 2^50, i.e. the reference's own 49-bit ring-pack primes) with |trunc(W*scaler)| <= 0x7f7f7f;
- * anything else takes a one-output-per-lane kernel with 128-bit accumulation (pcmm_info "last_path" tells which ran). */
+ * base-256 digits: residues in 5 digits (primes up to 0x7f7f7f7f80, i.e. the 36-bit sets) or in 7 digits (primes below 2^50, i.e.
+ * the reference's own 49-bit ring-pack primes), and |trunc(W*scaler)| below the smallest prime.  One launch takes a plaintext
+ * matrix of up to 4 digits (3 with the 7-digit residues); wider ones, such as the 46-bit entries that the reference's scaler
+ * q1 * 2^49 / scale gives, run as two or three launches over slices of three digits and a combining pass, with the same result.
+ * Anything else takes a one-output-per-lane kernel with 128-bit accumulation (pcmm_info "last_path" tells which ran). */
 int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_host, uint64_t* out_dev, int M,
               int Kin, int mod_num, double scaler);
 /* same contraction with the MLWE operands in one contiguous device array [Kin][mod_num][(rank+1)*N1] */
