@@ -166,6 +166,68 @@ def test_bert_base_layer_on_encrypted_activations(activations):
     assert np.abs(want).max() > 1.0 and max(worst) < 2.0 ** -10, worst
 
 
+def test_layer_on_the_references_own_parameter_set():
+    """The same layer on the reference's own configuration: Context_23(16, 15, 192) (its compiled-in logN = 16 set: 28 Q and 4 P primes
+    of 49 - 50 bits, 8 T primes), ring-pack primes {p_last} and {q0, q1} as its test program picks them (test_rlwe_decomp.cu:36-49),
+    messages at its precision 2^49 and its scaler q1 * 2^49 / scale (PPMM_kernel.cuh:283-284), which makes the plaintext entries 45
+    bits wide.  768 activations x 768 outputs, decrypted and compared with the plain product."""
+    from ckks_llm_amd import Ciphertext, MLWESecretKey, Plaintext, Scheme_23, SecretKey
+    ctx = Context_23(16, 15, 192)
+    N, L, N1 = ctx.N, ctx.L, 128
+    k = N // N1
+    key = bytes(range(32))
+    scheme = Scheme_23(ctx, key=key)
+    sk = SecretKey(ctx, key=key, nonce=1)
+    p_rp, q_rp = [ctx.pVec[-1]], [ctx.qVec[0], ctx.qVec[1]]
+    pc = PCMM_Context(N1, k, p_rp, q_rp, ctx)
+    ps = PCMM_Scheme(pc, key=key)
+    mlwe_sk = MLWESecretKey(N1, pc.ringpack_pq_count - 1, k)
+    ps.convertMLWESKfromRLWESK(mlwe_sk, sk)
+    scheme.addEncKey(sk)
+    ps.addRepakcingKey(mlwe_sk, sk)
+    rng = np.random.default_rng(16)
+    tokens, feat = N1, 768
+    X = rng.normal(0, 0.05, (tokens, feat))
+    W = rng.normal(0, 0.02, (feat, feat)).astype(np.float32)
+    want = X @ W.astype(np.float64).T
+    x_scale = ctx.precision                                                  # 2^49
+    C = (k + 1) * N1
+    samples = []
+    for lo, hi in ((0, 512), (512, 768)):
+        coeffs = np.zeros((tokens, k))
+        coeffs[:, : hi - lo] = X[:, lo:hi]
+        msg = Plaintext(N, L, 1, N // 2, x_scale)
+        ctx.encode_coeffs(DeviceBuffer.from_numpy(coeffs.reshape(-1)), msg)
+        ct = Ciphertext(N, L, 1, N // 2, x_scale)
+        scheme.encryptMsg(ct, msg)
+        part = [DeviceBuffer(8 * 2 * C) for _ in range(512)]
+        ps.rlweCipherDecompose(ct.cipher_device, part, 512, 0, 1)
+        samples += part[: hi - lo]
+    scaler = float(int(q_rp[1] * float(1 << 49) / float(x_scale)))
+    out = DeviceBuffer(8 * feat * 2 * C)
+    ps.PPMM(DeviceBuffer.from_numpy(W), samples, out, feat, feat, N1, feat, 2, scaler)
+    assert pc.info("last_path") == 1 and pc.info("last_DC") == 7 and pc.info("last_DW") == 6 and pc.info("last_slices") == 2
+    rows = [DeviceBuffer(8 * C) for _ in range(feat)]
+    for m in range(feat):
+        rows[m].L_.ckks_memcpy_d2d(rows[m].ptr, out.ptr + 8 * m * 2 * C, 8 * C)
+    out_scale = x_scale * scaler / q_rp[1]
+    embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    dec, d_vals = Plaintext(N, L, 0, N // 2, 1), DeviceBuffer(8 * N)
+    worst = []
+    for j in range(3):
+        res = Ciphertext(N, L, 0, N // 2, out_scale)
+        res.cipher_device.zero()
+        ps.mlweCipherPacking(res.cipher_device, rows[256 * j: 256 * (j + 1)], 256, 0, ps.repackingKeys, embed, mult)
+        res.l, res.scale = 0, out_scale
+        scheme.decryptMsg(dec, sk, res)
+        ctx.decode_coeffs(dec, d_vals)
+        got = d_vals.download(np.float64).reshape(tokens, k)
+        err = np.abs(got[:, 0:512:2] - want[:, 256 * j: 256 * (j + 1)])
+        worst.append(err.max())
+        assert np.median(err) < 2.0 ** -20
+    assert np.abs(want).max() > 0.05 and np.abs(want).max() < 0.4 and max(worst) < 2.0 ** -16, worst
+
+
 def test_bert_mirror_layers_with_loaded_weights(tmp_path):
     """The Python mirrors of Bert_model_weights and Bert: weights from a `model.safetensors` written with the safetensors package,
     PCMM_768_768 (two inputs of 512 samples) and layer_output (768 x 3072, six inputs) on encrypted activations at N = 2^16,
