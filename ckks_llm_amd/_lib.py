@@ -40,6 +40,7 @@ def _declare(L):
         "ckks_ctx_table": (i, [vp, C.c_char_p, u64p, sz, C.POINTER(sz)]),
         "ckks_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "ckks_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
         "ckks_ntt_timed": (i, [vp, vp, i, i, i, i, i, i, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+        "ckks_ntt_noalloc": (i, [vp, vp, i, i, i, i, i, i]), "ckks_ntt_noalloc_max_limbs": (i, []),
         "ckks_ntt_fwd_ext": (i, [vp, vp, i, i, i, i, i, i, i]), "ckks_ntt_inv_ext": (i, [vp, vp, i, i, i, i, i, i, i]),
         "ckks_modup_pq_to_t": (i, [vp, vp, vp, i, i]), "ckks_modup_qj_to_t": (i, [vp, vp, vp, i, i]),
         "ckks_modup_t_to_pql": (i, [vp, vp, vp, i, i]), "ckks_moddown_pql_to_ql": (i, [vp, vp, vp, i, i]),

@@ -168,6 +168,15 @@ class Context_23:
     def FromNTTInplace(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len):
         _check(self.L_.ckks_ntt_inv(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ckks_ntt_inv")
 
+    def ntt_noalloc(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, inverse):
+        """ToNTTInplace / FromNTTInplace without any device allocation (fixed inter-pass area inside the library;
+        at most ntt_noalloc_max_limbs() limbs per call)."""
+        _check(self.L_.ckks_ntt_noalloc(self.h, _addr(device_a), start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len,
+                                        1 if inverse else 0), "ckks_ntt_noalloc")
+
+    def ntt_noalloc_max_limbs(self):
+        return int(self.L_.ckks_ntt_noalloc_max_limbs())
+
     def ntt_timed(self, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, inverse):
         """One transform; returns the HIP-event durations (ms) of its two kernel launches."""
         a, b = C.c_float(), C.c_float()

@@ -369,6 +369,8 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         if (hipMalloc(&c->d_ntt_sched, ckks::ntt_sched_bytes()) != hipSuccess || hipMemset(c->d_ntt_sched, 0, ckks::ntt_sched_bytes()) != hipSuccess) rc = CKKS_E_NOMEM;
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) c->cu_count = cus;
+        c->device = dev;
+        if (rc == CKKS_OK) rc = ckks::ntt_noalloc_init(nullptr);
     }
     if (rc == CKKS_OK && hipEventCreate(&c->ev0) != hipSuccess) rc = CKKS_E_HIP;
     if (rc == CKKS_OK && hipEventCreate(&c->ev1) != hipSuccess) rc = CKKS_E_HIP;
@@ -519,6 +521,10 @@ extern "C" int ckks_ntt_fwd(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, 
 extern "C" int ckks_ntt_inv(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml) {
     return ckks::launch_ntt(c, dev, sp, sm, pn, mn, pml, 0, 1, true);
 }
+extern "C" int ckks_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml, int inverse) {
+    return ckks::launch_ntt_noalloc(c, dev, sp, sm, pn, mn, pml, inverse != 0);
+}
+extern "C" int ckks_ntt_noalloc_max_limbs(void) { return ckks::ntt_noalloc_max_limbs(); }
 extern "C" int ckks_ntt_fwd_ext(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml, int cmn, int bs) {
     return ckks::launch_ntt(c, dev, sp, sm, pn, mn, pml, cmn, bs, false);
 }

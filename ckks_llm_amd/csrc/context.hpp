@@ -88,6 +88,9 @@ struct ckks_ctx {
     int cu_count = 256;
     void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
     size_t ntt_mid_cap = 0;
+    char* mid_fixed = nullptr;            // set for the duration of a call that must not allocate: inter-pass area to use instead
+    size_t mid_fixed_cap = 0;
+    int device = 0;                       // the device that was current when the context was created
     struct DecodeTab { int level, words; void* dev; };
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     void* d_ntt_sched = nullptr;          // scheduler words of the fused NTT kernel (zero between launches)
@@ -105,6 +108,12 @@ int hip_fail(hipError_t e, const char* what);
 // launchers (ntt.hip, basisconv.hip)
 size_t ntt_sched_bytes();
 size_t ntt_sched_error_offset();
+// Address, on the current device, of the file-scope inter-pass area of the transform that allocates nothing (looked up once per
+// device), its capacity in limbs, and that transform (N = 2^16 with the 5-byte inter-pass form, or any ring in place).
+int ntt_noalloc_init(char** ptr_out);
+int ntt_noalloc_max_limbs();
+int launch_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
+                       bool inverse);
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
 // Hybrid key switch up to the inverse transform of the two sums, in five launches where the separate steps take nine:

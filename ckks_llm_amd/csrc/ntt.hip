@@ -25,6 +25,8 @@
 // [0,2q) for IntArith, raw double bit patterns for F64Arith); after the second pass it holds canonical residues.
 #include <cstddef>
 #include <cstdlib>
+#include <mutex>
+#include <string>
 #include <type_traits>
 
 #include "context.hpp"
@@ -691,11 +693,18 @@ static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, b
     const bool compact = CAN_COMPACT && compact_ok && c->ntt_mode != 1;
     if (compact) {
         // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
-        const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
-        if (chunk > max_limbs) chunk = max_limbs;
-        const int rc_mid = ensure_mid(c, (size_t)chunk * MID_LIMB_BYTES);
-        if (rc_mid) return rc_mid;
-        args.mid = (char*)c->d_ntt_mid;
+        if (c->mid_fixed) {
+            // caller-provided inter-pass area (the entry point that allocates nothing): the batch must fit it whole
+            if ((size_t)limbs * MID_LIMB_BYTES > c->mid_fixed_cap) { set_error("NTT: batch larger than the fixed inter-pass area"); return CKKS_E_INVALID; }
+            chunk = limbs;
+            args.mid = c->mid_fixed;
+        } else {
+            const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
+            if (chunk > max_limbs) chunk = max_limbs;
+            const int rc_mid = ensure_mid(c, (size_t)chunk * MID_LIMB_BYTES);
+            if (rc_mid) return rc_mid;
+            args.mid = (char*)c->d_ntt_mid;
+        }
     } else {
         args.mid = nullptr;
     }
@@ -1401,6 +1410,64 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
     }
     args.tw = inverse ? (const void*)c->d_tw_inv : (const void*)c->d_tw_fwd;
     return dispatch_logn<IntArith>(c, args, (int)limbs, inverse, false);
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Transform that allocates nothing.  The two-launch transform at N = 2^16 hands its data from the first pass to the second in
+// the 5-byte inter-pass form, in a buffer that the ordinary entry points allocate and grow on demand.  Callers that cannot
+// allocate (HIP graph capture, serving loops, harnesses that forbid it) get the same transform with that buffer in a
+// file-scope device array instead: NOALLOC_MAX_LIMBS limbs of 320 KiB, held by every GPU the library runs on until the
+// process ends.  All calls on one GPU share the array, so calls that overlap on one GPU (two streams, two host threads)
+// race; the first pass writes every byte the second pass reads, so nothing has to be cleared between calls.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int NOALLOC_MAX_LIMBS = 64;
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)NOALLOC_MAX_LIMBS * MID_LIMB_BYTES];
+static std::mutex g_scratch_mutex;
+static char* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};      // device address of `scratch` on each GPU (each GPU has its own copy)
+
+// address of the array on the current device, looked up once per device (called from ckks_ctx_create, and again by the
+// entry point for a device that no context was created on)
+int ntt_noalloc_init(char** ptr_out) {
+    int dev = -1;
+    CKKS_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { set_error("NTT: device index out of range"); return CKKS_E_INVALID; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        CKKS_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) { set_error("NTT: no device address for the fixed inter-pass area"); return CKKS_E_HIP; }
+        g_scratch_ptr[dev] = (char*)p;
+    }
+    if (ptr_out) *ptr_out = g_scratch_ptr[dev];
+    return CKKS_OK;
+}
+int ntt_noalloc_max_limbs() { return NOALLOC_MAX_LIMBS; }
+
+int launch_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
+                       bool inverse) {
+    if (!c || !dev) { set_error("NTT: null argument"); return CKKS_E_INVALID; }
+    const long limbs = (long)poly_num * mod_num;
+    if (poly_num > 0 && mod_num > 0 && limbs > NOALLOC_MAX_LIMBS) {
+        set_error("ckks_ntt_noalloc: " + std::to_string(limbs) + " limbs in one call, the limit is " + std::to_string(NOALLOC_MAX_LIMBS));
+        return CKKS_E_INVALID;
+    }
+    int cur = -1;
+    CKKS_HIP_TRY(hipGetDevice(&cur));
+    if (cur != c->device) { set_error("ckks_ntt_noalloc: the context was created on another device than the current one"); return CKKS_E_INVALID; }
+    char* ptr = nullptr;
+    int rc = ntt_noalloc_init(&ptr);
+    if (rc) return rc;
+    // two launches, inter-pass data in the fixed area where the 5-byte form applies and in place otherwise
+    const int mode = c->ntt_mode;
+    c->ntt_mode = 0;
+    c->mid_fixed = ptr;
+    c->mid_fixed_cap = (size_t)NOALLOC_MAX_LIMBS * MID_LIMB_BYTES;
+    rc = launch_ntt_from(c, dev, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, 0, 1, inverse, nullptr);
+    c->mid_fixed = nullptr;
+    c->mid_fixed_cap = 0;
+    c->ntt_mode = mode;
+    return rc;
 }
 
 }  // namespace ckks

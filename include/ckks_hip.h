@@ -92,6 +92,17 @@ int ckks_ntt_fwd_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start
 int ckks_ntt_inv_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                      int poly_mod_len, int cipher_mod_num, int batch_size);
 
+/* The same transform as ckks_ntt_fwd (inverse = 0) / ckks_ntt_inv (inverse != 0), for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * The ordinary entry points keep the data between the two launches of a transform at N = 2^16 in a buffer that they allocate
+ * and grow on demand; this one keeps it in a fixed device array inside the library (ckks_ntt_noalloc_max_limbs() limbs of
+ * 320 KiB = 20 MiB per GPU, held until the process ends) and calls no allocating routine.  poly_num * mod_num above that limit
+ * returns CKKS_E_INVALID.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two host threads)
+ * race.  The context must have been created on the current device.  Results are those of ckks_ntt_fwd / ckks_ntt_inv. */
+int ckks_ntt_noalloc(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
+                     int poly_mod_len, int inverse);
+int ckks_ntt_noalloc_max_limbs(void);
+
 /* One transform with HIP-event timing of its two kernel launches (strided pass and row pass; the forward transform
  * runs the strided pass first, the inverse the row pass first).  Replaces the cudaEvent pairs of ntt_throughput.cu:51-60. */
 int ckks_ntt_timed(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
