@@ -36,10 +36,12 @@ def _declare(L):
         "ckks_timer_start": (i, [vp]), "ckks_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
         "ckks_ctx_create": (i, [C.POINTER(vp), i, u64p, i, u64p, i, u64p, i, i]), "ckks_ctx_destroy": (i, [vp]),
         "ckks_set_stream": (i, [vp, vp]), "ckks_ctx_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
-        "ckks_ctx_set_arith_mode": (i, [vp, i]), "ckks_ctx_set_ntt_mode": (i, [vp, i]), "ckks_ctx_check": (i, [vp]),
+        "ckks_ctx_set_arith_mode": (i, [vp, i]), "ckks_ctx_set_ntt_mode": (i, [vp, i]), "ckks_ctx_check": (i, [vp]), "ckks_ctx_set_ntt_chain": (i, [vp, i, i]),
         "ckks_ctx_table": (i, [vp, C.c_char_p, u64p, sz, C.POINTER(sz)]),
         "ckks_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "ckks_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
         "ckks_ntt_timed": (i, [vp, vp, i, i, i, i, i, i, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+        "ckks_ntt_chain_slot": (i, [C.c_uint, C.c_uint, C.c_uint, C.POINTER(C.c_uint), C.POINTER(C.c_uint), C.POINTER(C.c_uint)]),
+        "ckks_ntt_chain_slots": (C.c_uint, [C.c_uint, C.c_uint, C.c_uint]),
         "ckks_ntt_noalloc": (i, [vp, vp, i, i, i, i, i, i]), "ckks_ntt_noalloc_max_limbs": (i, []),
         "ckks_ntt_fwd_ext": (i, [vp, vp, i, i, i, i, i, i, i]), "ckks_ntt_inv_ext": (i, [vp, vp, i, i, i, i, i, i, i]),
         "ckks_modup_pq_to_t": (i, [vp, vp, vp, i, i]), "ckks_modup_qj_to_t": (i, [vp, vp, vp, i, i]),

@@ -139,12 +139,16 @@ class Context_23:
         _check(self.L_.ckks_ctx_set_arith_mode(self.h, mode), "ckks_ctx_set_arith_mode")
 
     def set_ntt_mode(self, mode):
-        """0: automatic, 1: two launches per transform, 2: ticket-scheduled one-launch transform (switched off),
-        3: one workgroup per limb wherever that kernel exists (N >= 2^15)."""
+        """0: automatic, 1: two launches per transform (data in place between them), 2: chained one-launch transform
+        (N >= 2^15), 3: one workgroup per limb (N >= 2^15).  All give the same residues."""
         _check(self.L_.ckks_ctx_set_ntt_mode(self.h, mode), "ckks_ctx_set_ntt_mode")
 
+    def set_ntt_chain(self, skew=0, spin_max=-1):
+        """Tuning / test hook of the chained transform (ntt_mode 2); spin_max = 0 sends every second-pass tile to the finishing launch."""
+        _check(self.L_.ckks_ctx_set_ntt_chain(self.h, skew, spin_max), "ckks_ctx_set_ntt_chain")
+
     def check(self):
-        """Synchronise the context's stream; raises if a bounded wait of the one-launch transform ran out."""
+        """Synchronise the context's stream; raises if HIP reports an error for the launches so far."""
         _check(self.L_.ckks_ctx_check(self.h), "ckks_ctx_check")
 
     def set_stream(self, stream_handle):

@@ -366,7 +366,6 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         up(upload(&c->d_qiInvModql, z));
     }
     if (rc == CKKS_OK) {
-        if (hipMalloc(&c->d_ntt_sched, ckks::ntt_sched_bytes()) != hipSuccess || hipMemset(c->d_ntt_sched, 0, ckks::ntt_sched_bytes()) != hipSuccess) rc = CKKS_E_NOMEM;
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) c->cu_count = cus;
         c->device = dev;
@@ -384,7 +383,7 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     if (!c) return CKKS_OK;
     (void)hipDeviceSynchronize();
     void* ptrs[] = {c->d_primes, c->d_primes_moddown, c->d_primes_modup, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
-                    c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_sched, c->d_ntt_mid};
+                    c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_chain, c->d_ntt_mid};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     for (auto& e : c->decode_tabs) (void)hipFree(e.dev);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
@@ -408,6 +407,7 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
     else if (n == "gamma") *value = c->gamma; else if (n == "dnum") *value = c->dnum;
     else if (n == "Ri_blockNum") *value = c->Ri_blockNum; else if (n == "Qj_blockNum") *value = c->Qj_blockNum;
     else if (n == "arith_mode") *value = c->arith_mode; else if (n == "ntt_mode") *value = c->ntt_mode;
+    else if (n == "ntt_chain_deferred_tiles") return ckks::ntt_chain_deferred(const_cast<ckks_ctx*>(c), value);
     else { ckks::set_error("ckks_ctx_info: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
@@ -419,27 +419,29 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
     return CKKS_OK;
 }
 
-// test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = ticket-scheduled one-launch transform (switched off),
-// 3 = one workgroup per limb wherever that kernel exists (N >= 2^15)
+// test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = chained one-launch transform wherever that kernel exists
+// (N >= 2^15), 3 = one workgroup per limb wherever that kernel exists (N >= 2^15)
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
     if (!c || mode < 0 || mode > 3) return CKKS_E_INVALID;
     c->ntt_mode = mode;
     return CKKS_OK;
 }
 
-// Waits for the context's stream and reports a scheduler wait of the fused NTT kernel that ran out (the transforms of
-// that launch are then incomplete).  The flag is cleared by the call.
+// test / tuning hook of the chained transform: skew = how many limbs a chain's first pass runs ahead of its second pass (0: default),
+// spin_max = polls a second-pass workgroup spends on its limb's completion word before it leaves its tile to the finishing launch
+// (-1: default; 0 sends every tile there, which is how the tests reach that path)
+extern "C" int ckks_ctx_set_ntt_chain(ckks_ctx* c, int skew, int spin_max) {
+    if (!c || skew < 0 || skew > 64 || spin_max < -1) return CKKS_E_INVALID;
+    c->chain_skew = skew;
+    c->chain_spin = spin_max;
+    return CKKS_OK;
+}
+
+// Waits for the context's stream and reports what HIP has to say about the launches so far.
 extern "C" int ckks_ctx_check(ckks_ctx* c) {
     if (!c) return CKKS_E_INVALID;
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
-    unsigned err = 0;
-    char* word = (char*)c->d_ntt_sched + ckks::ntt_sched_error_offset();
-    CKKS_HIP_TRY(hipMemcpy(&err, word, sizeof(err), hipMemcpyDeviceToHost));
-    if (err) {
-        CKKS_HIP_TRY(hipMemset(c->d_ntt_sched, 0, ckks::ntt_sched_bytes()));
-        ckks::set_error("fused NTT: a scheduler wait ran out; the last transforms are incomplete");
-        return CKKS_E_UNAVAILABLE;
-    }
+    CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
 
@@ -524,6 +526,12 @@ extern "C" int ckks_ntt_inv(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, 
 extern "C" int ckks_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml, int inverse) {
     return ckks::launch_ntt_noalloc(c, dev, sp, sm, pn, mn, pml, inverse != 0);
 }
+extern "C" int ckks_ntt_chain_slot(unsigned slot, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile) {
+    if (!second || !k || !tile || !tiles) return CKKS_E_INVALID;
+    ckks::ntt_chain_slot(slot, tiles, skew, second, k, tile);
+    return CKKS_OK;
+}
+extern "C" unsigned ckks_ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return ckks::ntt_chain_slots(kmax, tiles, skew); }
 extern "C" int ckks_ntt_noalloc_max_limbs(void) { return ckks::ntt_noalloc_max_limbs(); }
 extern "C" int ckks_ntt_fwd_ext(ckks_ctx* c, uint64_t* dev, int sp, int sm, int pn, int mn, int pml, int cmn, int bs) {
     return ckks::launch_ntt(c, dev, sp, sm, pn, mn, pml, cmn, bs, false);

@@ -84,7 +84,7 @@ struct ckks_ctx {
     size_t qiInv_count = 0;
 
     int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
-    int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: fused launch wherever it exists
+    int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: chained one-launch transform, 3: one workgroup per limb
     int cu_count = 256;
     void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
     size_t ntt_mid_cap = 0;
@@ -93,7 +93,8 @@ struct ckks_ctx {
     int device = 0;                       // the device that was current when the context was created
     struct DecodeTab { int level, words; void* dev; };
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
-    void* d_ntt_sched = nullptr;          // scheduler words of the fused NTT kernel (zero between launches)
+    int chain_skew = 0, chain_spin = -1;  // chained transform: limbs a chain's first pass runs ahead of its second (0: default), poll limit of a wait (-1: default)
+    void* d_ntt_chain = nullptr;          // completion words of the chained (one-launch) transform, allocated on its first use; zero between transforms
 };
 
 namespace ckks {
@@ -106,8 +107,10 @@ int hip_fail(hipError_t e, const char* what);
     } while (0)
 
 // launchers (ntt.hip, basisconv.hip)
-size_t ntt_sched_bytes();
-size_t ntt_sched_error_offset();
+// chained (one-launch) transform: tiles left to its finishing launch so far, and the host view of its slot order (for tests)
+int ntt_chain_deferred(ckks_ctx* c, long* tiles);
+void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile);
+unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew);
 // Address, on the current device, of the file-scope inter-pass area of the transform that allocates nothing (looked up once per
 // device), its capacity in limbs, and that transform (N = 2^16 with the 5-byte inter-pass form, or any ring in place).
 int ntt_noalloc_init(char** ptr_out);

@@ -47,7 +47,9 @@ struct IntArith {
     __device__ __forceinline__ V from_mid(u64 x) const { return x; }
     __device__ __forceinline__ u64 to_mid_fwd(V x) const { return x; }          // lazy [0,4q)
     __device__ __forceinline__ u64 to_mid_inv(V x) const { return x; }          // lazy [0,2q)
+    static constexpr bool lazy40 = false;
     __device__ __forceinline__ u64 enc40(V x) const { return x; }               // the compact inter-pass form is FP64-only
+    __device__ __forceinline__ u64 enc40_raw(V x) const { return x; }
     __device__ __forceinline__ V dec40(unsigned lo, unsigned) const { return lo; }
     __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return csub(csub(x, q2), q); }
     // Harvey lazy butterflies; ranges as ntt_60bit.cuh:293-318
@@ -73,9 +75,12 @@ struct IntArith {
 struct F64Arith {
     typedef double V;
     typedef double TW;
-    double q, qinv, n_inv, w1n;
-    __device__ __forceinline__ F64Arith(const PrimeConst& pc) : q(pc.qd), qinv(pc.qinv_d), n_inv(pc.n_inv_d), w1n(pc.w1n_d) {}
-    __device__ __forceinline__ V from_canonical(u64 x) const { return (double)(long long)x; }
+    double q, qinv, hqinv, n_inv, w1n;
+    bool lazy40;               // q < 2^36.5: the values between the passes of a forward transform (|x| < 5.1 q) fit 40 bits as they are
+    __device__ __forceinline__ F64Arith(const PrimeConst& pc)
+        : q(pc.qd), qinv(pc.qinv_d), hqinv(0.5 * pc.qinv_d), n_inv(pc.n_inv_d), w1n(pc.w1n_d), lazy40(pc.qd < 97184015999.0) {}
+    // canonical residue (below 2^52) -> double: the word is the mantissa of 2^52 + x
+    __device__ __forceinline__ V from_canonical(u64 x) const { return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0; }
     __device__ __forceinline__ V from_mid(u64 x) const { return __longlong_as_double((long long)x); }
     __device__ __forceinline__ u64 to_mid_fwd(V x) const { return (u64)__double_as_longlong(x); }
     __device__ __forceinline__ V mulmod(V a, TW w) const {          // result in (-0.51 q, 0.51 q)
@@ -85,17 +90,26 @@ struct F64Arith {
         return __builtin_fma(-c, q, h) + l;
     }
     __device__ __forceinline__ V balance(V x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
+    // integer in [0, 2^52) held in a double -> the integer: the mantissa of 2^52 + r
+    __device__ __forceinline__ static u64 bits52(V r) { return (u64)__double_as_longlong(r + 4503599627370496.0) & 0xFFFFFFFFFFFFFull; }
     __device__ __forceinline__ u64 canon(V r) const {               // r in (-q, q) -> [0, q)
         r = r < 0.0 ? r + q : r;
-        return (u64)(long long)r;
+        return bits52(r);
+    }
+    // any integer |x| < 2^10 q -> [0, q) without a sign fix-up: (x + 1/2) / q is at least 1/(2q) > 2^-42 away from every integer
+    // and the product is off by less than 2^-42, so the floor is exactly floor(x / q)
+    __device__ __forceinline__ u64 canon_any(V x) const {
+        const double c = __builtin_floor(__builtin_fma(x, qinv, hqinv));
+        return bits52(__builtin_fma(-c, q, x));
     }
     __device__ __forceinline__ u64 to_mid_inv(V x) const { return (u64)__double_as_longlong(balance(x)); }
     // 40-bit form of a balanced value (q < 2^39, so |r| < 2^38.1): r + 2^39 read from the low mantissa bits of r + 2^52 + 2^39
     __device__ __forceinline__ u64 enc40(V x) const { return (u64)__double_as_longlong(balance(x) + 4504149383184384.0) & 0xFFFFFFFFFFull; }
+    __device__ __forceinline__ u64 enc40_raw(V x) const { return (u64)__double_as_longlong(x + 4504149383184384.0) & 0xFFFFFFFFFFull; }   // |x| < 2^39
     __device__ __forceinline__ V dec40(unsigned lo, unsigned hi8) const {
         return __longlong_as_double((long long)(0x4330000000000000ull | ((u64)hi8 << 32) | lo)) - 4504149383184384.0;
     }
-    __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon(balance(x)); }
+    __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon_any(x); }
     __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
         double t = mulmod(y, w);
         y = x - t;
@@ -108,8 +122,8 @@ struct F64Arith {
     }
     __device__ __forceinline__ void gs_last(V& x, V& y, u64& ox, u64& oy) const {
         double s = x + y, d = x - y;
-        ox = canon(mulmod(s, n_inv));
-        oy = canon(mulmod(d, w1n));
+        ox = canon_any(mulmod(s, n_inv));
+        oy = canon_any(mulmod(d, w1n));
     }
 };
 
@@ -217,11 +231,18 @@ template <class AR>
 __device__ __forceinline__ void mid_store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const typename AR::V (&v)[16], const AR& ar) {
     char* piece = mid_piece(mid_limb, cb, g);
     unsigned hi[4] = {0, 0, 0, 0};
+    u64 e[16];
+    if (ar.lazy40) {                 // uniform over the workgroup: small primes skip the reduction before the 40-bit form
+#pragma unroll
+        for (int j = 0; j < 16; j++) e[j] = ar.enc40_raw(v[j]);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) e[j] = ar.enc40(v[j]);
+    }
 #pragma unroll
     for (int j = 0; j < 16; j++) {
-        const u64 e = ar.enc40(v[j]);
-        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e;
-        hi[j >> 2] |= (unsigned)(e >> 32) << (8 * (j & 3));
+        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e[j];
+        hi[j >> 2] |= (unsigned)(e[j] >> 32) << (8 * (j & 3));
     }
 #pragma unroll
     for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
@@ -539,130 +560,135 @@ __global__ __launch_bounds__(256 * GROUPS) void ntt_limb_kernel(NttArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Fused transform: both passes in ONE launch, the data between them held in the XCD's L2.
+// Chained transform: both passes in ONE launch, the data between them held in the XCD's L2.
 //
-// A two-launch transform moves every limb through HBM twice.  Here the second pass of a limb runs on the same XCD as its
-// first pass, a few microseconds later, while the limb (512 KiB at N = 2^16) is still dirty in that XCD's 4 MiB L2:
-// HBM sees one read and one write per limb.
+// A two-launch transform moves every limb through HBM twice.  Here the second pass of a limb runs on the same XCD as its first
+// pass, a few microseconds later, while the limb's lines (512 KiB at N = 2^16, written in place by the first pass) are still
+// dirty in that XCD's 4 MiB L2: HBM sees one read and one write per limb.
 //
-// Scheduling.  Workgroups are persistent and find out at run time which XCD they sit on (hardware register XCC_ID).  Each
-// XCD has a ticket counter; a ticket is one tile of one pass of one limb, in the order
-//     P1(l0) P1(l1) ... P1(l_SKEW-1) | P1(l_SKEW) P2(l0) | P1(l_SKEW+1) P2(l1) | ...      (TILES tickets per entry)
-// where l_k is the k-th limb this XCD has claimed from a global counter (claimed by whoever draws the first P1 ticket of
-// the entry).  A P2 ticket waits until all first-pass tiles of its limb have signalled completion.  Every wait is for work
-// whose tickets are smaller in the same queue, i.e. held by workgroups that are already running, so the scheme cannot
-// deadlock and does not depend on how many workgroups the hardware puts on which XCD.  Waits are bounded all the same: a
-// wait that runs out raises sched->error and every workgroup leaves.
-// The last workgroup to leave restores the scheduler words to zero for the next launch.
+// Order of work.  The grid is one-dimensional and not persistent.  Workgroup b belongs to chain x = b mod 8 and takes slot
+// s = b / 8 of that chain; the hardware hands consecutive workgroups of a grid to the XCDs in turn, so a chain's workgroups all
+// run on one XCD.  A chain works through the limbs x, x + 8, x + 16, .. in entries of TILES workgroups (one pass of one limb):
+//     P1(k=0) .. P1(k=skew-1) | P1(k=skew) P2(k=0) | P1(k=skew+1) P2(k=1) | ...
+// so that the second pass of a limb is dispatched while later limbs' first passes keep the compute units busy.
+//
+// Synchronisation.  A first-pass workgroup waits for nothing; when its stores have reached the L2 it adds 1 to the limb's
+// completion word.  A second-pass workgroup waits until that word reads TILES.  Workgroups of a grid start in the order of their
+// index, so what it waits for has started before it; the wait is bounded by a poll count all the same.
+// Nothing depends on the placement or on the wait for correctness: every workgroup reads the XCD it really runs on from the
+// hardware register; a first-pass workgroup that finds itself on another XCD than its chain's adds a mark to the completion word
+// instead of the plain 1, and a second-pass workgroup that is on the wrong XCD, sees a mark, or runs out of polls does not touch
+// the data: it records its tile in the limb's `todo` word and leaves.  A second launch (ntt_chain_finish_kernel, one workgroup
+// per limb) runs the recorded tiles - after the kernel boundary every store is visible everywhere - and returns both words to
+// zero for the next transform.  Every workgroup of both launches ends after a bounded number of steps.
 // ------------------------------------------------------------------------------------------------------------
-constexpr unsigned SCHED_CLAIM_PAD = 512;      // entries drawn past the end of the work while the workgroups wind down
-struct NttSched {
-    unsigned next_limb, finished, error, pad;
-    unsigned ticket[8];
-    unsigned done[65536];             // per limb: first-pass tiles completed
-    unsigned claim[8][65536 + SCHED_CLAIM_PAD];     // per XCD, k-th claimed limb + 1 (0 = not yet claimed)
+constexpr unsigned CHAIN_XCDS = 8;
+constexpr unsigned CHAIN_MARK = 0x10000u;          // added by a first-pass workgroup that ran on an unexpected XCD
+struct ChainArgs {
+    unsigned* done;            // [limb] completion word of the first pass
+    unsigned* todo;            // [limb] bit t: second-pass tile t was left to the finishing launch
+    unsigned* stats;           // [0]: tiles left to the finishing launch since the context was created
+    unsigned limbs, kmax, skew, spin_max;
+    unsigned zero;             // 0, but not known to the compiler: "add zero" stays a read-modify-write executed at the L2
+    unsigned long long xcc_of; // nibble x: the XCD that runs chain x
 };
-constexpr unsigned SCHED_END = 0xFFFFFFFFu;
-constexpr unsigned long long SCHED_WAIT_TICKS = 2000000ull;      // bound of one wait: 20 ms of the 100 MHz wall clock
 
-// Every scheduler word is written AND read with read-modify-write atomics (a read is "add 0"): they all execute at the same
-// place in the memory system, so a waiter cannot spin on a stale cached copy.  A wait is bounded in TIME, not in polls (a poll
-// of a word that hundreds of workgroups poll can take tens of microseconds); when it runs out, or when another workgroup's
-// wait has, sched->error is raised and the caller leaves.  Returns the last value read.
-// `zero` is a run-time 0: with a literal the compiler turns the idempotent atomic into a plain cache-level load.
-template <class Pred>
-__device__ __forceinline__ unsigned sched_wait(unsigned* word, Pred satisfied, NttSched* sched, unsigned zero, bool& failed) {
-    const unsigned long long t_end = wall_clock64() + SCHED_WAIT_TICKS;
-    for (unsigned n = 1;; n++) {
-        const unsigned v = atomicAdd(word, zero);
-        if (satisfied(v)) return v;
-        if ((n & 7u) == 0 && (wall_clock64() > t_end || atomicAdd(&sched->error, zero) != 0)) {
-            atomicExch(&sched->error, 1u);
-            failed = true;
-            return v;
-        }
-        __builtin_amdgcn_s_sleep(4);
-    }
+// slot s of a chain -> pass (0 / 1), index k of the limb within the chain, tile.  k >= kmax: an empty slot.
+__host__ __device__ inline void chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned& second, unsigned& k, unsigned& tile) {
+    const unsigned e = s / tiles;
+    tile = s % tiles;
+    if (e < skew) { second = 0; k = e; }
+    else { const unsigned r = e - skew; second = r & 1u; k = second ? r / 2 : skew + r / 2; }
 }
+__host__ __device__ inline unsigned chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return (skew + 2 * kmax) * tiles; }
 
-template <class AR, int SA, int SB, bool INVERSE, int SKEW>
-__global__ __launch_bounds__(256) void ntt_fused_kernel(NttArgs a, NttSched* sched) {
+template <class AR, int SA, int SB, bool INVERSE>
+__global__ __launch_bounds__(256) void ntt_chain_kernel(NttArgs a, ChainArgs ch) {
     typedef StridedCfg<SA, SB> CS;
     typedef RowCfg<SA, SB> CR;
-    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES, "fused kernel: tile shapes must agree");
+    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES && CS::TILES <= 16, "chained kernel: tile shapes");
     constexpr unsigned TILES = CS::TILES;
     constexpr long N = 1l << (SA + SB);
     constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
     typedef typename AR::TW TW;
     __shared__ typename AR::V lds[LDS_WORDS];
-    __shared__ unsigned item[3];                       // limb (or SCHED_END), tile, second pass?
-    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;       // XCC_ID[3:0]
-    const unsigned limbs = a.limbs_total;
-    const unsigned zero = a.limb_base;                 // 0 in every launch of this kernel
-
-    for (;;) {
-        if (threadIdx.x == 0) {
-            const unsigned t = atomicAdd(&sched->ticket[xcc], 1u);
-            const unsigned entry = t / TILES, tile = t % TILES;
-            unsigned k, second;
-            if (entry < SKEW) { k = entry; second = 0; }
-            else { const unsigned r = entry - SKEW; second = r & 1u; k = second ? r / 2 : SKEW + r / 2; }
-            unsigned limb = 0;
-            bool failed = false;
-            if (k >= limbs + SCHED_CLAIM_PAD) {
-                limb = SCHED_END;                                                // far past the end: nothing is recorded any more
-            } else if (!second && tile == 0) {
-                limb = atomicAdd(&sched->next_limb, 1u);
-                if (limb >= limbs) limb = SCHED_END - 1;                         // stored + 1
-                atomicExch(&sched->claim[xcc][k], limb + 1);
-            } else {
-                limb = sched_wait(&sched->claim[xcc][k], [](unsigned v) { return v != 0; }, sched, zero, failed) - 1;
+    __shared__ unsigned go;
+    const unsigned x = blockIdx.x % CHAIN_XCDS;
+    unsigned second, k, tile;
+    chain_slot(blockIdx.x / CHAIN_XCDS, TILES, ch.skew, second, k, tile);
+    const unsigned limb_id = x + CHAIN_XCDS * k;
+    if (k >= ch.kmax || limb_id >= ch.limbs) return;                            // uniform over the workgroup
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;       // XCC_ID[3:0]
+    const bool placed = xcc == (unsigned)((ch.xcc_of >> (4 * x)) & 15u);
+    int prime;
+    u64* limb = limb_ptr(a, limb_id, N, prime);
+    const AR ar(a.primes[prime]);
+    const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
+    if (!second) {
+        if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
+        else row_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
+        // every store of this tile has been acknowledged by the L2 before the completion word moves
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (threadIdx.x == 0) atomicAdd(&ch.done[limb_id], placed ? 1u : CHAIN_MARK + 1u);
+        return;
+    }
+    if (threadIdx.x == 0) {
+        unsigned ok = placed ? 1u : 0u;
+        if (ok) {
+            unsigned v = 0;
+            for (unsigned n = 0; n < ch.spin_max; n++) {
+                v = atomicAdd(&ch.done[limb_id], ch.zero);
+                if (v >= TILES) break;
+                __builtin_amdgcn_s_sleep(8);
             }
-            if (limb >= limbs) limb = SCHED_END;
-            if (second && limb != SCHED_END && !failed)
-                sched_wait(&sched->done[limb], [](unsigned v) { return v >= TILES; }, sched, zero, failed);
-            if (failed) { limb = SCHED_END; second = 1; }                        // leave: the launch is abandoned
-            item[0] = limb; item[1] = tile; item[2] = second;
+            ok = v == TILES ? 1u : 0u;
         }
-        __syncthreads();
-        const unsigned limb_id = item[0], tile = item[1], second = item[2];
-        __syncthreads();
-        if (limb_id == SCHED_END) {
-            if (second) break;              // every later ticket of this queue is past the end as well
-            continue;                       // a first-pass entry past the end: second-pass entries of earlier limbs may follow
-        }
+        if (!ok) atomicOr(&ch.todo[limb_id], 1u << tile);
+        go = ok;
+    }
+    __syncthreads();
+    if (!go) return;
+    // second-pass loads bypass this compute unit's L1 (which may hold pre-transform copies of the same lines) and are served by the L2
+    if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, tile, tw, ar, lds, threadIdx.x);
+    else strided_tile<AR, SA, SB, true, true>(limb, tile, tw, ar, lds, threadIdx.x);
+}
+
+// One workgroup per limb: runs the second-pass tiles that the chained launch left behind, then clears the limb's words.
+template <class AR, int SA, int SB, bool INVERSE>
+__global__ __launch_bounds__(256) void ntt_chain_finish_kernel(NttArgs a, ChainArgs ch) {
+    typedef StridedCfg<SA, SB> CS;
+    typedef RowCfg<SA, SB> CR;
+    constexpr long N = 1l << (SA + SB);
+    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
+    typedef typename AR::TW TW;
+    __shared__ typename AR::V lds[LDS_WORDS];
+    __shared__ unsigned mask_s;
+    const unsigned limb_id = blockIdx.x;
+    if (limb_id >= ch.limbs) return;
+    if (threadIdx.x == 0) mask_s = ch.todo[limb_id];
+    __syncthreads();
+    const unsigned mask = mask_s;
+    if (mask) {
         int prime;
         u64* limb = limb_ptr(a, limb_id, N, prime);
         const AR ar(a.primes[prime]);
         const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
-        if (!second) {
-            if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
-            else row_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
-            // all stores of this tile have reached the L2 before the completion count moves
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
-            if (threadIdx.x == 0) atomicAdd(&sched->done[limb_id], 1u);
-        } else {
-            if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, tile, tw, ar, lds, threadIdx.x);
-            else strided_tile<AR, SA, SB, true, true>(limb, tile, tw, ar, lds, threadIdx.x);
+#pragma unroll 1
+        for (unsigned tile = 0; tile < (unsigned)CS::TILES; tile++) {
+            if (!((mask >> tile) & 1u)) continue;
+            if (!INVERSE) row_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
+            else strided_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
             __syncthreads();
         }
     }
-
-    // the last workgroup out restores the scheduler for the next launch
-    if (threadIdx.x == 0) item[0] = atomicAdd(&sched->finished, 1u);
-    __syncthreads();
-    if (item[0] == gridDim.x - 1) {
-        for (unsigned i = threadIdx.x; i < limbs; i += blockDim.x) sched->done[i] = 0;
-        for (unsigned x = 0; x < 8; x++)
-            for (unsigned i = threadIdx.x; i < limbs + SCHED_CLAIM_PAD; i += blockDim.x) sched->claim[x][i] = 0;
-        if (threadIdx.x < 8) sched->ticket[threadIdx.x] = 0;
-        if (threadIdx.x == 0) { sched->next_limb = 0; sched->finished = 0; }
+    if (threadIdx.x == 0) {
+        ch.done[limb_id] = 0;
+        ch.todo[limb_id] = 0;
+        if (mask) atomicAdd(ch.stats, (unsigned)__builtin_popcount(mask));
     }
 }
-
-size_t ntt_sched_bytes() { return sizeof(NttSched); }
 
 static int ensure_mid(ckks_ctx* c, size_t need);
 
@@ -721,22 +747,62 @@ static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, b
     return CKKS_OK;
 }
 
+constexpr unsigned CHAIN_MAX_LIMBS = 65536;
+static int ensure_chain(ckks_ctx* c) {
+    if (c->d_ntt_chain) return CKKS_OK;
+    const size_t bytes = (2 * (size_t)CHAIN_MAX_LIMBS + 16) * sizeof(unsigned);
+    if (hipMalloc(&c->d_ntt_chain, bytes) != hipSuccess) { set_error("NTT: cannot allocate the completion words of the chained transform"); return CKKS_E_NOMEM; }
+    CKKS_HIP_TRY(hipMemsetAsync(c->d_ntt_chain, 0, bytes, c->stream));
+    return CKKS_OK;
+}
+
 template <class AR, int SA, int SB>
-static int launch_fused(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
-    static const int bpc_env = getenv("CKKS_NTT_BPC") ? atoi(getenv("CKKS_NTT_BPC")) : 0;
-    const int bpc = bpc_env > 0 ? bpc_env : 3;                     // resident workgroups per compute unit
-    long blocks = (long)c->cu_count * bpc;
-    const long tiles = (long)limbs * StridedCfg<SA, SB>::TILES;
-    if (blocks > tiles) blocks = tiles;
+static int launch_chain(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
+    static const int skew_env = getenv("CKKS_NTT_SKEW") ? atoi(getenv("CKKS_NTT_SKEW")) : 0;
+    static const int spin_env = getenv("CKKS_NTT_SPIN") ? atoi(getenv("CKKS_NTT_SPIN")) : 0;
+    static const int lds_env = getenv("CKKS_NTT_CHAIN_LDS") ? atoi(getenv("CKKS_NTT_CHAIN_LDS")) : 0;      // extra LDS per workgroup: fewer resident workgroups
+    int rc = ensure_chain(c);
+    if (rc) return rc;
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
     args.mid = nullptr;
-    NttSched* sched = (NttSched*)c->d_ntt_sched;
-    if (!inverse) hipLaunchKernelGGL((ntt_fused_kernel<AR, SA, SB, false, 1>), dim3((unsigned)blocks), dim3(256), 0, c->stream, args, sched);
-    else hipLaunchKernelGGL((ntt_fused_kernel<AR, SA, SB, true, 1>), dim3((unsigned)blocks), dim3(256), 0, c->stream, args, sched);
+    ChainArgs ch;
+    ch.done = (unsigned*)c->d_ntt_chain;
+    ch.todo = ch.done + CHAIN_MAX_LIMBS;
+    ch.stats = ch.todo + CHAIN_MAX_LIMBS;
+    ch.limbs = (unsigned)limbs;
+    ch.kmax = ((unsigned)limbs + CHAIN_XCDS - 1) / CHAIN_XCDS;
+    ch.skew = c->chain_skew > 0 ? (unsigned)c->chain_skew : skew_env > 0 ? (unsigned)skew_env : 1u;
+    if (ch.skew > ch.kmax) ch.skew = ch.kmax;
+    // about 5 ms of polls by default, far beyond any wait of a healthy launch; 0 polls (a test setting) leaves every second-pass
+    // tile to the finishing launch
+    ch.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : spin_env > 0 ? (unsigned)spin_env : 20000u;
+    ch.zero = 0;
+    ch.xcc_of = 0x76543210ull;
+    const unsigned blocks = chain_slots(ch.kmax, StridedCfg<SA, SB>::TILES, ch.skew) * CHAIN_XCDS;
+    if (!inverse) {
+        hipLaunchKernelGGL((ntt_chain_kernel<AR, SA, SB, false>), dim3(blocks), dim3(256), (size_t)lds_env, c->stream, args, ch);
+        hipLaunchKernelGGL((ntt_chain_finish_kernel<AR, SA, SB, false>), dim3((unsigned)limbs), dim3(256), 0, c->stream, args, ch);
+    } else {
+        hipLaunchKernelGGL((ntt_chain_kernel<AR, SA, SB, true>), dim3(blocks), dim3(256), (size_t)lds_env, c->stream, args, ch);
+        hipLaunchKernelGGL((ntt_chain_finish_kernel<AR, SA, SB, true>), dim3((unsigned)limbs), dim3(256), 0, c->stream, args, ch);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
+// tiles that second-pass workgroups of chained transforms have left to the finishing launch so far (synchronises the stream)
+int ntt_chain_deferred(ckks_ctx* c, long* tiles) {
+    *tiles = 0;
+    if (!c->d_ntt_chain) return CKKS_OK;
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
+    unsigned v = 0;
+    CKKS_HIP_TRY(hipMemcpy(&v, (unsigned*)c->d_ntt_chain + 2 * (size_t)CHAIN_MAX_LIMBS, sizeof(v), hipMemcpyDeviceToHost));
+    *tiles = v;
+    return CKKS_OK;
+}
+// host view of the slot order, for tests
+void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile) { chain_slot(s, tiles, skew, *second, *k, *tile); }
+unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return chain_slots(kmax, tiles, skew); }
 
 template <class AR, int SA, int SB>
 static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
@@ -755,28 +821,18 @@ static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse)
     return CKKS_OK;
 }
 
-// the word of the scheduler block that a bounded wait sets when it runs out
-size_t ntt_sched_error_offset() { return offsetof(NttSched, error); }
-
 template <class AR>
 static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok) {
-    // The one-launch transform (ntt_fused_kernel) is switched off: on MI355X its launches did not complete (the process had to
-    // be ended by a test time-out, twice, the second time with every scheduler wait bounded to 20 ms), and the cause has not
-    // been shown yet.  Mode 2 therefore reports an error instead of launching it; the automatic mode uses two launches.
-    if (c->ntt_mode == 2) {
-        set_error("NTT: the one-launch transform is switched off in this build (its launches did not complete on MI355X)");
-        return CKKS_E_UNAVAILABLE;
+    // mode 2: both passes in one launch, the limb held in the XCD's L2 between them (N >= 2^15)
+    if (!c->ev_mid_armed && c->ntt_mode == 2 && !args.embed_mlwe) {
+        if (c->logN == 16) return launch_chain<AR, 8, 8>(c, args, limbs, inverse);
+        if (c->logN == 15) return launch_chain<AR, 8, 7>(c, args, limbs, inverse);
     }
     // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
     // (the limbs in flight, 0.5 MiB per resident workgroup, exceed the L2 by far), so the automatic mode does not pick it.
     if (!c->ev_mid_armed && c->ntt_mode == 3) {
         if (c->logN == 16) return launch_whole_limb<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_whole_limb<AR, 8, 7>(c, args, limbs, inverse);
-    }
-    constexpr bool fused_enabled = false;
-    if (fused_enabled && c->d_ntt_sched && !c->ev_mid_armed && limbs >= 96) {
-        if (c->logN == 16) return launch_fused<AR, 8, 8>(c, args, limbs, inverse);
-        if (c->logN == 15) return launch_fused<AR, 8, 7>(c, args, limbs, inverse);
     }
     switch (c->logN) {
         case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse, compact_ok);

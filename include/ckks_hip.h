@@ -58,21 +58,29 @@ int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int p_num, cons
                     const uint64_t* t, int t_num, int gamma);
 int ckks_ctx_destroy(ckks_ctx* ctx);
 int ckks_set_stream(ckks_ctx* ctx, void* hip_stream);
-/* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum" */
+/* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum","arith_mode","ntt_mode";
+ * "ntt_chain_deferred_tiles" (synchronises): second-pass tiles that chained transforms have left to their finishing launch */
 int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
 /* 0 (default): FP64 butterflies for primes < 2^41, integer butterflies otherwise; 1: integer butterflies everywhere.
  * Both give the same residues; the switch exists for testing and tuning. */
 int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
-/* How a transform is launched.  0 (default) and 1: two launches, one per pass.  3: one workgroup carries a limb through
- * both passes in one launch (N >= 2^15; same residues, slower at large batches).  2: both passes in one launch with the
- * limb held in the XCD's L2 between them under a ticket scheduler - switched off in this build (its launches did not
- * complete on MI355X): transforms then return CKKS_E_UNAVAILABLE.
+/* How a transform is launched.  0 (default): chosen by the library; 1: two launches, one per pass, data in place between
+ * them; 2: chained - both passes in one launch, the second pass of a limb following its first pass on the same XCD so that
+ * the limb stays in that XCD's L2 in between (N >= 2^15; other rings take two launches), plus a small finishing launch;
+ * 3: one workgroup carries a limb through both passes (N >= 2^15).  All give the same residues.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
-/* Synchronises the context's stream and returns CKKS_E_UNAVAILABLE if a bounded scheduler wait of the one-launch transform
- * ran out (its outputs are then incomplete); clears the condition.  Plays the part of the reference's
+/* Synchronises the context's stream and returns what HIP reports for the launches so far.  Plays the part of the reference's
  * cudaDeviceSynchronize + cudaGetLastError checks (Utils.cuh CUDA_CHECK). */
 int ckks_ctx_check(ckks_ctx* ctx);
+/* Test / tuning hook of the chained transform (mode 2).  skew: limbs that a chain's first pass runs ahead of its second pass
+ * (0 = default); spin_max: polls that a second-pass workgroup spends waiting for its limb's first pass before it leaves its tile
+ * to the finishing launch (-1 = default; 0 sends every tile there).  Results do not depend on either. */
+int ckks_ctx_set_ntt_chain(ckks_ctx* ctx, int skew, int spin_max);
+/* Order of work of the chained transform, for tests: slot `slot` of a chain of `tiles` workgroups per pass -> pass (0 / 1),
+ * index k of the limb within the chain and tile; ckks_ntt_chain_slots = slots of a chain of kmax limbs.  Pure host functions. */
+int ckks_ntt_chain_slot(unsigned slot, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile);
+unsigned ckks_ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew);
 /* host copy of a constant table, flattened in the reference's device layout (names as in ckks_oracle.h /
  * Context_23.h: "pqt","psi","psi_table","psiinv_table","RiHatInv","QjHatModT",...). *count receives the length. */
 int ckks_ctx_table(const ckks_ctx* ctx, const char* name, uint64_t* host_out, size_t cap, size_t* count);

@@ -122,13 +122,11 @@ def test_reference_addressing_and_ext_variant():
     assert np.array_equal(from_dev(d2, e_h.shape), want) and np.array_equal(want, e_h)
 
 
-@pytest.mark.skip(reason="the one-launch transform is switched off: its launches did not complete on MI355X (ended by the "
-                         "test time-out twice, the second time with all scheduler waits bounded to 20 ms); cause not shown yet")
 @pytest.mark.parametrize("logN,polys,mode", [(16, 9, 0), (16, 5, 1), (15, 7, 0), (15, 3, 1)])
 def test_one_launch_transform_matches_two_launch_and_oracle(logN, polys, mode):
-    """The fused kernel (both passes in one launch, inter-pass data in L2, ticket scheduler) against the oracle and
-    against the two-launch path, both directions, both arithmetic back ends; two launches in a row reuse the
-    scheduler words the kernel restores at exit."""
+    """The chained transform (ntt_mode 2: both passes in one launch, the second pass of a limb behind its first pass on the
+    same XCD) against the oracle, both directions, both arithmetic back ends; launches in a row reuse the completion
+    words that the finishing launch returns to zero."""
     q = CFG2_Q[:5]
     pair = Pair(logN, [], q)
     N, L1 = pair.N, len(q)
@@ -186,17 +184,30 @@ def test_whole_limb_transform_matches_oracle(logN, polys, mode):
     buf.free()
 
 
-def test_one_launch_mode_reports_that_it_is_switched_off():
-    from ckks_llm_amd import CkksError
-    pair = Pair(15, [], CFG2_Q[:2])
-    d = to_dev(np.zeros((1, 2, pair.N), dtype=np.uint64))
+@pytest.mark.parametrize("skew,spin", [(1, 0), (3, 0), (2, -1), (64, -1)])
+def test_chained_transform_finishing_launch_and_skews(skew, spin):
+    """With a poll limit of zero every second-pass workgroup of the chained transform leaves its tile to the finishing launch,
+    which must then produce the whole second pass; any skew gives the same residues.  13 limbs: chains of unequal length."""
+    q = CFG2_Q[:13]
+    pair = Pair(16, [], q)
+    N, L1 = pair.N, len(q)
+    data = limbs_uniform(77, q, 1, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, 1, L1, L1)
     pair.dev.set_ntt_mode(2)
-    with pytest.raises(CkksError):
-        pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)
-    pair.dev.set_ntt_mode(0)
-    pair.dev.ToNTTInplace(d, 0, 0, 1, 2, 2)
+    pair.dev.set_ntt_chain(skew, spin)
+    buf = to_dev(data)
+    before = pair.dev.info("ntt_chain_deferred_tiles")
+    pair.dev.ToNTTInplace(buf, 0, 0, 1, L1, L1)
     pair.dev.check()
-    assert not from_dev(d, (2, pair.N)).any()
+    assert np.array_equal(from_dev(buf, data.shape), want)
+    pair.dev.FromNTTInplace(buf, 0, 0, 1, L1, L1)
+    pair.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), data)
+    left = pair.dev.info("ntt_chain_deferred_tiles") - before
+    if spin == 0:
+        assert left == 2 * 13 * 16          # every second-pass tile of both transforms
+    buf.free()
 
 
 def test_tables_match_oracle():
@@ -263,7 +274,7 @@ def test_full_size_properties_batch32():
     pair.dev.check()
     assert np.array_equal(from_dev(d, data.shape), data)
     # the two-launch path and the whole-limb path give the same residues on the whole batch
-    for m in (1, 3):
+    for m in (1, 2, 3):
         pair.dev.set_ntt_mode(m)
         pair.dev.ToNTTInplace(d, 0, 0, 2 * B, L1, L1)
         assert np.array_equal(from_dev(d, data.shape), got), m
