@@ -83,6 +83,8 @@ def _declare(L):
         "pcmm_ppmm_packed": (i, [vp, vp, vp, i, d]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
+        "pcmm_set_weight_cache": (i, [vp, i]),
+        "pcmm_weights_changed": (i, [vp, vp]),
     }
     missing = []
     for name, (res, args) in S.items():

@@ -607,6 +607,14 @@ class PCMM_Context:
         _check(self.L_.pcmm_info(self.h, name.encode(), C.byref(v)), "pcmm_info")
         return v.value
 
+    def set_weight_cache(self, enabled):
+        """Keep (default) or do not keep the digit planes of plaintext matrices between PPMM calls."""
+        _check(self.L_.pcmm_set_weight_cache(self.h, int(bool(enabled))), "pcmm_set_weight_cache")
+
+    def weights_changed(self, plain_mat=None):
+        """Say that a weight matrix was overwritten in place (None: all of them): its digit planes are built again."""
+        _check(self.L_.pcmm_weights_changed(self.h, _addr(plain_mat) if plain_mat is not None else None), "pcmm_weights_changed")
+
     # -- PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
     def decodeCoeffs(self, msg, vals):
         """PCMM_Context.cuh:165-178: vals = N1 device doubles."""

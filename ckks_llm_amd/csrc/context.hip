@@ -483,11 +483,21 @@ extern "C" int ckks_malloc(void** p, size_t bytes) {
     if (e != hipSuccess) return ckks::hip_fail(e, "hipMalloc");
     return CKKS_OK;
 }
-extern "C" int ckks_free(void* p) { if (p) CKKS_HIP_TRY(hipFree(p)); return CKKS_OK; }
-extern "C" int ckks_memcpy_h2d(void* d, const void* s, size_t n) { CKKS_HIP_TRY(hipMemcpy(d, s, n, hipMemcpyHostToDevice)); return CKKS_OK; }
+// Freeing or overwriting device memory through these calls also drops what the ring-pack handles had prepared from it (the digit
+// planes of a weight matrix are keyed by its address).
+extern "C" int ckks_free(void* p) {
+    if (!p) return CKKS_OK;
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) == hipSuccess && size) pcmm_forget_weights(base, size);
+    else { (void)hipGetLastError(); pcmm_forget_weights(p, 1); }
+    CKKS_HIP_TRY(hipFree(p));
+    return CKKS_OK;
+}
+extern "C" int ckks_memcpy_h2d(void* d, const void* s, size_t n) { pcmm_forget_weights(d, n); CKKS_HIP_TRY(hipMemcpy(d, s, n, hipMemcpyHostToDevice)); return CKKS_OK; }
 extern "C" int ckks_memcpy_d2h(void* d, const void* s, size_t n) { CKKS_HIP_TRY(hipMemcpy(d, s, n, hipMemcpyDeviceToHost)); return CKKS_OK; }
-extern "C" int ckks_memcpy_d2d(void* d, const void* s, size_t n) { CKKS_HIP_TRY(hipMemcpy(d, s, n, hipMemcpyDeviceToDevice)); return CKKS_OK; }
-extern "C" int ckks_memset(void* d, int v, size_t n) { CKKS_HIP_TRY(hipMemset(d, v, n)); return CKKS_OK; }
+extern "C" int ckks_memcpy_d2d(void* d, const void* s, size_t n) { pcmm_forget_weights(d, n); CKKS_HIP_TRY(hipMemcpy(d, s, n, hipMemcpyDeviceToDevice)); return CKKS_OK; }
+extern "C" int ckks_memset(void* d, int v, size_t n) { pcmm_forget_weights(d, n); CKKS_HIP_TRY(hipMemset(d, v, n)); return CKKS_OK; }
 extern "C" int ckks_sync(void) { CKKS_HIP_TRY(hipDeviceSynchronize()); return CKKS_OK; }
 extern "C" int ckks_device_count(int* n) { if (!n) return CKKS_E_INVALID; CKKS_HIP_TRY(hipGetDeviceCount(n)); return CKKS_OK; }
 extern "C" int ckks_timer_start(ckks_ctx* c) { if (!c) return CKKS_E_INVALID; CKKS_HIP_TRY(hipEventRecord(c->ev0, c->stream)); return CKKS_OK; }

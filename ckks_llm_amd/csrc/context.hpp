@@ -153,3 +153,7 @@ int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int star
 int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const uint64_t* keys, int rank, int prime0,
                               const NttEmbedSource& src, bool* done);
 }  // namespace ckks
+
+// Device memory [lo, lo + bytes) was freed or overwritten through the library's own plumbing: every ring-pack handle forgets the
+// plaintext matrices it had prepared from there (pcmm.hip).
+void pcmm_forget_weights(const void* lo, size_t bytes);

@@ -307,6 +307,13 @@ __device__ __forceinline__ u64 load_word(const u64* p) {
     if (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return *p;
 }
+// Final stores of such a second pass are not read again on the chip: marked non-temporal, the L2 gives their lines up first and
+// keeps the lines that are still between their two passes.
+template <bool STREAM>
+__device__ __forceinline__ void store_word(u64* p, u64 v) {
+    if (STREAM) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
 
 // ------------------------------------------------------------------------------------------------------------
 // strided pass (first SA forward stages / last SA inverse stages): one tile = CW adjacent columns, all N1 rows
@@ -409,8 +416,8 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
         for (int j = 0; j < R / 2; j++) {
             u64 ox, oy;
             ar.gs_last(v[j], v[j + R / 2], ox, oy);
-            col[(long)(g + j * G) * N2] = ox;
-            col[(long)(g + (j + R / 2) * G) * N2] = oy;
+            store_word<COHERENT>(col + (long)(g + j * G) * N2, ox);
+            store_word<COHERENT>(col + (long)(g + (j + R / 2) * G) * N2, oy);
         }
     }
 }
@@ -477,7 +484,7 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < R; j++) rp[u + j * U] = ar.to_canonical_fwd(lrow[padded(u + j * U)]);
+        for (int j = 0; j < R; j++) store_word<COHERENT>(rp + u + j * U, ar.to_canonical_fwd(lrow[padded(u + j * U)]));
     } else {
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = ar.from_canonical(load_word<COHERENT>(rp + u + j * U));

@@ -20,6 +20,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "pcmm.hpp"
@@ -281,6 +282,10 @@ __global__ __launch_bounds__(256) void ppmm_combine_kernel(PpmmCombineArgs a) {
 using namespace ckks;
 namespace H = ckks_host;
 
+// every live handle, for pcmm_forget_weights
+static std::mutex g_handles_mutex;
+static std::vector<pcmm_ctx*> g_handles;
+static void drop_weights(pcmm_ctx* h, pcmm_ctx::Weights* w);
 extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, const uint64_t* p, int np, const uint64_t* q, int nq) {
     if (!out || !ctx || N1 <= 0 || rank <= 0 || nq < 1 || np < 0 || (np > 0 && !p) || !q) { set_error("pcmm_ctx_create: bad argument"); return CKKS_E_INVALID; }
     if ((long)N1 * rank != ctx->N) { set_error("pcmm_ctx_create: N1 * mlwe_rank must equal N"); return CKKS_E_INVALID; }
@@ -302,20 +307,26 @@ extern "C" int pcmm_ctx_create(pcmm_ctx** out, ckks_ctx* ctx, int N1, int rank, 
     if (e == hipSuccess) e = hipMemcpy(h->d_pq, pc.data(), pc.size() * sizeof(PrimeConst), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMalloc((void**)&h->d_absmax, sizeof(unsigned long long) * (1 + PPMM_CONST_WORDS));
     if (e != hipSuccess) { pcmm_ctx_destroy(h); return hip_fail(e, "pcmm_ctx_create"); }
+    { std::lock_guard<std::mutex> lock(g_handles_mutex); g_handles.push_back(h); }
     *out = h;
     return CKKS_OK;
 }
 extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     if (!h) return CKKS_OK;
+    { std::lock_guard<std::mutex> lock(g_handles_mutex); g_handles.erase(std::remove(g_handles.begin(), g_handles.end(), h), g_handles.end()); }
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_A, h->d_Adig, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw, h->d_slices};
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw, h->d_slices};
     for (void* p : ptrs) if (p) (void)hipFree(p);
+    for (auto& w : h->weights) { if (w.d_A) (void)hipFree(w.d_A); if (w.d_Adig) (void)hipFree(w.d_Adig); }
+    if (h->pin) (void)hipHostFree(h->pin);
+    if (h->pin_ev) (void)hipEventDestroy(h->pin_ev);
     if (h->small) ckks_ctx_destroy(h->small);
     delete h;
     return CKKS_OK;
 }
 
 static int upload_ptrs(pcmm_ctx* h, const uint64_t* const* host_ptrs, int count) {
+    h->tab_sent.clear();                                                   // the table PPMM last sent is overwritten
     if (count > h->ptr_cap) {
         if (h->d_ptrs) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_ptrs); h->d_ptrs = nullptr; }
         int cap = std::max(count, 3072);                                   // PCMM_Scheme.cuh:16-18 sizes its table for 3072
@@ -624,6 +635,66 @@ extern "C" int pcmm_ntt_inv(pcmm_ctx* h, uint64_t* data, int poly_num, int mod_n
     return pcmm_small_ntt(h, data, poly_num, mod_num, start_mod_idx, mod_batch_size, true);
 }
 
+// Small host arrays (row-pointer table, epilogue constants) go to the device through a pinned staging area owned by the handle:
+// the copy is asynchronous for real and the caller's memory is free on return.  The area is reused, so a second upload first
+// waits for the first one's copy (an event, not the stream).
+static int stage_to_device(pcmm_ctx* h, void* dst, const void* src, size_t bytes) {
+    if (!h->pin_ev) CKKS_HIP_TRY(hipEventCreateWithFlags(&h->pin_ev, hipEventDisableTiming));
+    else CKKS_HIP_TRY(hipEventSynchronize(h->pin_ev));
+    if (bytes > h->pin_cap) {
+        if (h->pin) (void)hipHostFree(h->pin);
+        h->pin = nullptr; h->pin_cap = 0;
+        const size_t cap = std::max(bytes, (size_t)64 * 1024);
+        CKKS_HIP_TRY(hipHostMalloc(&h->pin, cap, hipHostMallocDefault));
+        h->pin_cap = cap;
+    }
+    memcpy(h->pin, src, bytes);
+    CKKS_HIP_TRY(hipMemcpyAsync(dst, h->pin, bytes, hipMemcpyHostToDevice, h->ctx->stream));
+    CKKS_HIP_TRY(hipEventRecord(h->pin_ev, h->ctx->stream));
+    return CKKS_OK;
+}
+uint64_t** pcmm_ctx::d_ptrs_slot(int count) {
+    if (count > ptr_cap) {
+        if (d_ptrs) { (void)hipDeviceSynchronize(); (void)hipFree(d_ptrs); d_ptrs = nullptr; ptr_cap = 0; }
+        const int cap = std::max(count, 3072);                             // PCMM_Scheme.cuh:16-18 sizes its table for 3072
+        if (hipMalloc((void**)&d_ptrs, (size_t)cap * sizeof(uint64_t*)) != hipSuccess) return nullptr;
+        ptr_cap = cap;
+        tab_sent.clear();
+    }
+    return d_ptrs;
+}
+// prepared plaintext matrices: at most WEIGHTS_MAX_BYTES of device memory, least recently used first out
+constexpr size_t WEIGHTS_MAX_BYTES = (size_t)4 << 30;
+static void drop_weights(pcmm_ctx* h, pcmm_ctx::Weights* w) {
+    (void)hipStreamSynchronize(h->ctx->stream);
+    if (w->d_A) (void)hipFree(w->d_A);
+    if (w->d_Adig) (void)hipFree(w->d_Adig);
+    const size_t idx = (size_t)(w - h->weights.data());
+    if (idx < h->weights.size()) {
+        h->weights_bytes -= w->bytes;
+        h->weights.erase(h->weights.begin() + (long)idx);
+    }
+}
+void pcmm_forget_weights(const void* lo, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_handles_mutex);
+    const uintptr_t a = (uintptr_t)lo, b = a + bytes;
+    for (pcmm_ctx* h : g_handles)
+        for (size_t i = h->weights.size(); i-- > 0;) {
+            const uintptr_t wa = (uintptr_t)h->weights[i].W, wb = wa + (size_t)h->weights[i].M * h->weights[i].Kin * sizeof(float);
+            if (wa < b && a < wb) drop_weights(h, &h->weights[i]);
+        }
+}
+static pcmm_ctx::Weights* keep_weights(pcmm_ctx* h, const pcmm_ctx::Weights& fresh) {
+    while (!h->weights.empty() && h->weights_bytes + fresh.bytes > WEIGHTS_MAX_BYTES) {
+        size_t old = 0;
+        for (size_t i = 1; i < h->weights.size(); i++) if (h->weights[i].stamp < h->weights[old].stamp) old = i;
+        drop_weights(h, &h->weights[old]);
+    }
+    h->weights.push_back(fresh);
+    h->weights_bytes += fresh.bytes;
+    return &h->weights.back();
+}
+
 static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_host, const uint64_t* strided, uint64_t* out,
                        int M, int Kin, int mod_num, double scaler, bool packed = false) {
     if (!h || !W || !out || (!ptrs_host && !strided && !packed)) return CKKS_E_INVALID;
@@ -647,73 +718,106 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         for (int n = 0; n < Kpad_tab; n++)
             tab[n] = n >= Kin ? h->d_zero : (ptrs_host ? ptrs_host[n] : strided + (size_t)n * mod_num * C);
         for (int n = 0; n < Kin; n++) aligned16 = aligned16 && (((uintptr_t)tab[n]) & 15) == 0;
-        if ((rc = upload_ptrs(h, tab.data(), Kpad_tab))) return rc;
-        CKKS_HIP_TRY(hipStreamSynchronize(c->stream));      // the table was copied from caller / stack memory
-    }
-    // workspace
-    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 191) / 192 * 192;   // K padded to a multiple of three 64-deep MFMA steps (LDS ring of three slots)
-    size_t needA = (size_t)M * Kin, needD = (size_t)9 * Mpad * Kpad;     // up to three slices of three digit planes
-    if (needA > h->A_cap) {
-        if (h->d_A) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_A); h->d_A = nullptr; }
-        CKKS_HIP_TRY(hipMalloc((void**)&h->d_A, needA * sizeof(long long)));
-        h->A_cap = needA;
-    }
-    if (needD > h->Adig_cap) {
-        if (h->d_Adig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Adig); h->d_Adig = nullptr; }
-        CKKS_HIP_TRY(hipMalloc((void**)&h->d_Adig, needD));
-        h->Adig_cap = needD;
-    }
-    // per-call epilogue constants, kept behind the |A| maximum word
-    std::vector<uint64_t> cst(PPMM_CONST_WORDS, 0);
-    const uint64_t qlast = h->pq[h->np + mod_num - 1];
-    uint64_t qmax = 0, qmin = ~0ull;
-    auto dbits = [](uint64_t x, uint64_t m) { double d = x > m / 2 ? -(double)(m - x) : (double)x; uint64_t b; memcpy(&b, &d, 8); return b; };
-    for (int i = 0; i < mod_num; i++) {
-        uint64_t qi = h->pq[h->np + i];
-        qmax = std::max(qmax, qi); qmin = std::min(qmin, qi);
-        if (i < mod_num - 1) {
-            cst[i] = H::invmod(qlast % qi, qi);
-            cst[PPMM_MAX_MODS + i] = H::shoup(cst[i], qi);
-            cst[4 * PPMM_MAX_MODS + i] = dbits(cst[i], qi);
+        if (tab != h->tab_sent) {                           // a layer calls with the same sample buffers again and again
+            uint64_t** slot = h->d_ptrs_slot(Kpad_tab);
+            if (!slot) { set_error("PPMM: cannot allocate the row-pointer table"); return CKKS_E_NOMEM; }
+            if ((rc = stage_to_device(h, slot, tab.data(), (size_t)Kpad_tab * sizeof(uint64_t*)))) return rc;
+            h->tab_sent = tab;
         }
-        cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 32, qi), qi);
-        cst[3 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 64, qi), qi);
     }
+    const int Mpad = (M + 127) / 128 * 128, Kpad = (Kin + 191) / 192 * 192;   // K padded to a multiple of three 64-deep MFMA steps (LDS ring of three slots)
+    // per-call epilogue constants, kept behind the |A| maximum word; they depend on mod_num only
+    uint64_t qmax = 0, qmin = ~0ull;
+    for (int i = 0; i < mod_num; i++) { qmax = std::max(qmax, h->pq[h->np + i]); qmin = std::min(qmin, h->pq[h->np + i]); }
     uint64_t* d_cst = (uint64_t*)(h->d_absmax + 1);
-    CKKS_HIP_TRY(hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream));
-    CKKS_HIP_TRY(hipMemcpyAsync(d_cst, cst.data(), PPMM_CONST_WORDS * sizeof(uint64_t), hipMemcpyHostToDevice, c->stream));
-    long count = (long)M * Kin;
-    hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 256 * QUANT_PER_LANE - 1) / (256 * QUANT_PER_LANE))), dim3(256), 0, c->stream, W, h->d_A,
-                       h->d_absmax, count, scaler);
-    unsigned long long absmax = 0;
-    CKKS_HIP_TRY(hipMemcpyAsync(&absmax, h->d_absmax, sizeof(absmax), hipMemcpyDeviceToHost, c->stream));
-    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
-
-    PpmmArgs a;
-    a.A = h->d_A; a.Adig = h->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
-    a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
-    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np; a.raw_all = 0;
+    if (h->cst_mods != mod_num) {
+        std::vector<uint64_t> cst(PPMM_CONST_WORDS, 0);
+        const uint64_t qlast = h->pq[h->np + mod_num - 1];
+        auto dbits = [](uint64_t x, uint64_t m) { double d = x > m / 2 ? -(double)(m - x) : (double)x; uint64_t b; memcpy(&b, &d, 8); return b; };
+        for (int i = 0; i < mod_num; i++) {
+            uint64_t qi = h->pq[h->np + i];
+            if (i < mod_num - 1) {
+                cst[i] = H::invmod(qlast % qi, qi);
+                cst[PPMM_MAX_MODS + i] = H::shoup(cst[i], qi);
+                cst[4 * PPMM_MAX_MODS + i] = dbits(cst[i], qi);
+            }
+            cst[2 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 32, qi), qi);
+            cst[3 * PPMM_MAX_MODS + i] = dbits(H::powmod(2, 64, qi), qi);
+        }
+        if ((rc = stage_to_device(h, d_cst, cst.data(), PPMM_CONST_WORDS * sizeof(uint64_t)))) return rc;
+        h->cst_mods = mod_num;
+    }
     // digit counts.  d balanced digits in [-128, 127] reach from -0x80..80 up to +0x7f..7f (d bytes each), NOT up to 2^(8d-1) - 1:
     // the bytes of x + 0x80..80 must not carry into byte d.  DW digits must hold +-|A|max, DC digits every residue 0 .. qmax - 1.
     auto top = [](int d) { unsigned long long v = 0; for (int i = 0; i < d; i++) v = (v << 8) | 0x7f; return v; };
-    int DW = 1; while (DW < 8 && absmax > top(DW)) DW++;
     int DC = 1; while (DC < 8 && qmax - 1 > top(DC)) DC++;
     static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
-    // residues in 5 digits (q < 2^39) with up to 4 plaintext digits, or in 7 digits (q < 2^50) with up to 3
-    // wider plaintext matrices (any int64) go through the same kernels in slices of three digits
-    const bool one_launch = (DC <= 5 && DW <= 4) || (DC <= 7 && qmax < (1ull << 50) && DW <= 3);
-    const int slices = one_launch ? 1 : (DW + 2) / 3;
-    const bool width_ok = (DC <= 5 || (DC <= 7 && qmax < (1ull << 50))) && slices <= 3;
-    const bool mfma_ok = !force_generic && aligned16 && (C % 64 == 0) && width_ok &&
-                         (long)Kpad * (slices == 1 && DW == 4 ? 4 : 3) <= 16384 && absmax < qmin && qmin > (1ull << 25);
+    // what the matrix of a given |A|max runs on.  Residues in 5 digits (q < 2^39) with up to 4 plaintext digits, or in 7 digits
+    // (q < 2^50) with up to 3; wider plaintext matrices (any int64) go through the same kernels in slices of three digits.
+    struct Plan { int DW, slices, planes; bool mfma; };
+    auto plan_for = [&](unsigned long long absmax) {
+        Plan pl;
+        pl.DW = 1; while (pl.DW < 8 && absmax > top(pl.DW)) pl.DW++;
+        const bool one_launch = (DC <= 5 && pl.DW <= 4) || (DC <= 7 && qmax < (1ull << 50) && pl.DW <= 3);
+        pl.slices = one_launch ? 1 : (pl.DW + 2) / 3;
+        const bool width_ok = (DC <= 5 || (DC <= 7 && qmax < (1ull << 50))) && pl.slices <= 3;
+        pl.mfma = !force_generic && aligned16 && (C % 64 == 0) && width_ok &&
+                  (long)Kpad * (pl.slices == 1 && pl.DW == 4 ? 4 : 3) <= 16384 && absmax < qmin && qmin > (1ull << 25);
+        // every plane the kernel instance reads is written (3 or 4: the instances are built for these widths), also those above the
+        // measured digit count, which are zero for this matrix
+        pl.planes = pl.slices > 1 ? 3 * pl.slices : pl.DW <= 3 ? 3 : 4;
+        return pl;
+    };
+    // the prepared matrix: found, or quantised, measured and split now
+    pcmm_ctx::Weights* we = nullptr;
+    for (auto& w : h->weights)
+        if (w.W == W && w.M == M && w.Kin == Kin && w.scaler == scaler) { we = &w; break; }
+    if (we) {
+        const Plan pl = plan_for(we->absmax);
+        if (pl.mfma ? !we->d_Adig || we->planes != pl.planes : !we->d_A) { drop_weights(h, we); we = nullptr; }   // prepared for the other kernel
+    }
+    pcmm_ctx::Weights fresh;
+    if (!we) {
+        const long count = (long)M * Kin;
+        fresh.W = W; fresh.M = M; fresh.Kin = Kin; fresh.scaler = scaler;
+        hipError_t e = hipMalloc((void**)&fresh.d_A, (size_t)count * sizeof(long long));
+        if (e != hipSuccess) { set_error("PPMM: cannot allocate the quantised plaintext matrix"); return CKKS_E_NOMEM; }
+        (void)hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream);
+        hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 256 * QUANT_PER_LANE - 1) / (256 * QUANT_PER_LANE))), dim3(256), 0, c->stream, W,
+                           fresh.d_A, h->d_absmax, count, scaler);
+        // the one host round trip of a matrix: its digit count selects the kernel instance
+        hipError_t e2 = hipMemcpyAsync(&fresh.absmax, h->d_absmax, sizeof(fresh.absmax), hipMemcpyDeviceToHost, c->stream);
+        if (e2 == hipSuccess) e2 = hipStreamSynchronize(c->stream);
+        if (e2 != hipSuccess) { (void)hipFree(fresh.d_A); return hip_fail(e2, "PPMM: |A| maximum"); }
+        const Plan pl = plan_for(fresh.absmax);
+        if (packed && !pl.mfma) { (void)hipFree(fresh.d_A); set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
+        fresh.bytes = (size_t)count * sizeof(long long);
+        if (pl.mfma) {
+            const size_t dbytes = (size_t)pl.planes * Mpad * Kpad;
+            e = hipMalloc((void**)&fresh.d_Adig, dbytes);
+            if (e != hipSuccess) { (void)hipFree(fresh.d_A); set_error("PPMM: cannot allocate the plaintext digit planes"); return CKKS_E_NOMEM; }
+            const long total = (long)Mpad * Kpad;
+            hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, fresh.d_A, fresh.d_Adig, M, Kin, Mpad, Kpad, pl.planes);
+            fresh.planes = pl.planes;
+            (void)hipFree(fresh.d_A);                       // waits for the kernel above; only the planes are kept
+            fresh.d_A = nullptr;
+            fresh.bytes = dbytes;
+        }
+        we = keep_weights(h, fresh);
+    }
+    we->stamp = ++h->weights_clock;
+    const Plan pl = plan_for(we->absmax);
+    const unsigned long long absmax = we->absmax;
+    const int DW = pl.DW, slices = pl.slices;
+    const bool mfma_ok = pl.mfma;
+
+    PpmmArgs a;
+    a.A = we->d_A; a.Adig = we->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
+    a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
+    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np; a.raw_all = 0;
     if (packed && !mfma_ok) { set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax; h->last_slices = mfma_ok ? slices : 0;
     if (mfma_ok) {
-        long total = (long)Mpad * Kpad;
-        // every plane the kernel instance reads is written (3 or 4: the instances are built for these widths), also those above the
-        // measured digit count, which are zero for this matrix but may hold an earlier call's digits
-        hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, h->d_A, h->d_Adig, M, Kin, Mpad, Kpad,
-                           slices > 1 ? 3 * slices : DW <= 3 ? 3 : 4);
         size_t need = ppmm_bdig_bytes(a, DC);
         if (packed && need > h->Bdig_cap) { set_error("PPMM on digit planes: planes not opened for this shape"); return CKKS_E_STATE; }
         if (need > h->Bdig_cap) {
@@ -737,7 +841,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             PpmmArgs sa = a;
             sa.raw_all = 1;
             for (int sl = 0; sl < slices; sl++) {
-                sa.Adig = h->d_Adig + (size_t)3 * sl * Mpad * Kpad;
+                sa.Adig = we->d_Adig + (size_t)3 * sl * Mpad * Kpad;
                 sa.out = sl == 0 ? out : h->d_slices + (size_t)(sl - 1) * per_slice;
                 rc = launch_ppmm_mfma_impl(c->stream, sa, 3, DC, h->d_Bdig, !packed && sl == 0);      // the residue planes are packed once
                 if (rc) return rc;
@@ -757,6 +861,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         hipLaunchKernelGGL(ppmm_generic_kernel, grid, block, 0, c->stream, a);
     }
     CKKS_HIP_TRY(hipGetLastError());
+    if (!h->weights_cached) drop_weights(h, we);            // the reference's behaviour: nothing survives the call (waits for it)
     return CKKS_OK;
 }
 
@@ -767,6 +872,18 @@ extern "C" int pcmm_info(const pcmm_ctx* h, const char* name, long* value) {
     else if (n == "last_slices") *value = h->last_slices;
     else if (n == "last_absmax") *value = (long)h->last_absmax; else if (n == "N1") *value = h->N1; else if (n == "mlwe_rank") *value = h->rank;
     else { set_error("pcmm_info: unknown name " + n); return CKKS_E_INVALID; }
+    return CKKS_OK;
+}
+extern "C" int pcmm_set_weight_cache(pcmm_ctx* h, int enabled) {
+    if (!h) return CKKS_E_INVALID;
+    h->weights_cached = enabled != 0;
+    if (!enabled) while (!h->weights.empty()) drop_weights(h, &h->weights.back());
+    return CKKS_OK;
+}
+extern "C" int pcmm_weights_changed(pcmm_ctx* h, const float* W) {
+    if (!h) return CKKS_E_INVALID;
+    for (size_t i = h->weights.size(); i-- > 0;)
+        if (!W || h->weights[i].W == W) drop_weights(h, &h->weights[i]);
     return CKKS_OK;
 }
 extern "C" int pcmm_ppmm(pcmm_ctx* h, const float* W, const uint64_t* const* mlwe_ptrs_host, uint64_t* out, int M, int Kin, int mod_num, double scaler) {

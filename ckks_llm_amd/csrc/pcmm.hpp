@@ -11,10 +11,6 @@ struct pcmm_ctx {
     ckks::PrimeConst* d_pq = nullptr;        // ring-pack primes [p_ringpack | q_ringpack]
     uint64_t** d_ptrs = nullptr;             // device copy of the caller's MLWE pointer table (PCMM_Scheme.cuh:16-18)
     int ptr_cap = 0;
-    // workspace of the quantised plaintext matrix
-    long long* d_A = nullptr;                // [M][Kin] int64
-    int8_t* d_Adig = nullptr;                // [DW][Mpad][Kpad] balanced digits
-    size_t A_cap = 0, Adig_cap = 0;
     int8_t* d_Bdig = nullptr;                // residue digit planes [prime][K step][digit][column][64]
     size_t Bdig_cap = 0;
     uint64_t* d_zero = nullptr;              // zero rows the K padding of the row-pointer table points to
@@ -29,6 +25,32 @@ struct pcmm_ctx {
     uint64_t* d_small_tw = nullptr;          // tables of the size-N1 transform when N1 < 256: [prime][forward | inverse][N1]
     uint64_t small_n_inv[8] = {};            // N1^-1 modulo each ring-pack prime (N1 < 256)
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
+    // Prepared plaintext matrices.  A weight matrix is static for the life of a layer: the first PPMM call with a given
+    // (device pointer, shape, scaler) quantises it, measures |A|max (the one host round trip) and splits it into digit planes;
+    // later calls with the same key reuse the planes and issue no host synchronisation at all.
+    struct Weights {
+        const float* W = nullptr;
+        int M = 0, Kin = 0;
+        double scaler = 0;
+        unsigned long long absmax = 0;
+        long long* d_A = nullptr;            // kept when the generic kernel runs this matrix
+        int8_t* d_Adig = nullptr;            // kept when the MFMA kernel runs it: `planes` planes of Mpad x Kpad
+        int planes = 0;
+        size_t bytes = 0;
+        uint64_t stamp = 0;
+    };
+    std::vector<Weights> weights;
+    bool weights_cached = true;
+    size_t weights_bytes = 0;
+    uint64_t weights_clock = 0;
+    // last row-pointer table and epilogue constants sent to the device (resent only when they change), and the pinned staging
+    // area they travel through, so that the copies need no stream synchronisation
+    std::vector<const uint64_t*> tab_sent;
+    int cst_mods = 0;
+    void* pin = nullptr;
+    size_t pin_cap = 0;
+    hipEvent_t pin_ev = nullptr;
+    uint64_t** d_ptrs_slot(int count);       // the device table, grown to `count` entries (nullptr: out of memory)
 };
 
 namespace ckks {

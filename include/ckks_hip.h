@@ -319,6 +319,15 @@ int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_
 /* same contraction with the MLWE operands in one contiguous device array [Kin][mod_num][(rank+1)*N1] */
 int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev, uint64_t* out_dev, int M, int Kin,
                       int mod_num, double scaler);
+/* Prepared plaintext matrices (no counterpart in the reference, which quantises W inside every call, PPMM_kernel.cuh:148).
+ * The weights of a layer do not change between calls, so the first PPMM call with a given (W_dev, M, Kin, scaler) quantises the
+ * matrix, measures |A|max (one stream synchronisation) and splits it into digit planes, and every later call with the same four
+ * values reuses them: such calls enqueue their kernels and return without waiting for the stream.  At most 4 GiB of planes are
+ * kept per handle, least recently used first out.  A caller that overwrites a weight matrix in place says so with
+ * pcmm_weights_changed(h, W_dev) (W_dev = NULL: every matrix); pcmm_set_weight_cache(h, 0) restores the reference's behaviour
+ * (every call reads W afresh and synchronises once), pcmm_set_weight_cache(h, 1) is the default. */
+int pcmm_set_weight_cache(pcmm_ctx* h, int enabled);
+int pcmm_weights_changed(pcmm_ctx* h, const float* W_dev);
 
 /* ---- the gather writing PPMM's operand directly.  No counterpart in the reference, where rlweCipherDecompose materialises every
  * MLWE sample as 8-byte words that PPMM reads back (PCMM_Scheme.cuh:90-125, PPMM_kernel.cuh:254-349); in a layer the two always

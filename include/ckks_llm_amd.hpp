@@ -710,6 +710,9 @@ public:
         check(pcmm_info(handle, name, &v), "pcmm_info");
         return v;
     }
+    // digit planes of plaintext matrices are kept between PPMM calls (default); a matrix overwritten in place is announced
+    void set_weight_cache(bool enabled) { check(pcmm_set_weight_cache(handle, enabled ? 1 : 0), "pcmm_set_weight_cache"); }
+    void weights_changed(const float* plain_mat = nullptr) { check(pcmm_weights_changed(handle, plain_mat), "pcmm_weights_changed"); }
     // PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
     void ToNTTInplace(uint64_tt* data, int poly_num, int mod_num, int start_poly_idx, int start_mod_idx, int mod_batch_size) {
         check(pcmm_ntt_fwd(handle, data, poly_num, mod_num, start_poly_idx, start_mod_idx, mod_batch_size), "PCMM_Context::ToNTTInplace");

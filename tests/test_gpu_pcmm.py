@@ -128,6 +128,57 @@ def test_ppmm_narrower_matrix_after_a_wider_one(wide):
         assert dev.pcmm_context.info("last_DW") == want_dw, (step, dev.pcmm_context.info("last_absmax"))
 
 
+def test_ppmm_prepared_weights_follow_the_buffer():
+    """The digit planes of a plaintext matrix are kept under (device address, shape, scaler).  A second call with the same matrix
+    reuses them; a matrix overwritten through the library's copy, a freed and reallocated buffer, an announced in-place change and
+    a switched-off cache must all give the product of what the buffer holds now."""
+    q = CFG2_Q[:2]
+    pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
+    C = (rank + 1) * 128
+    M, Kin, scaler = 32, 64, float(2 ** 26)
+    rng = np.random.default_rng(77)
+    mlwe = [limbs_uniform(900 + n, q, 1, C)[0] for n in range(Kin)]
+    bufs = [to_dev(m) for m in mlwe]
+
+    def want_for(W):
+        out = np.zeros((M, 2, C), dtype=np.uint64)
+        orc.PPMM(W, [m.reshape(-1) for m in mlwe], out.reshape(-1), M, Kin, 2, scaler)
+        return out
+
+    def run(dW):
+        dout = DeviceBuffer(8 * M * 2 * C)
+        dout.zero()
+        dev.PPMM(dW, bufs, dout, M, Kin, 128, Kin, 2, scaler)
+        return from_dev(dout, (M, 2, C))
+
+    W1 = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    W2 = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    W3 = rng.normal(0, 0.3, (M, Kin)).astype(np.float32)             # four plaintext digits: another kernel instance
+    dW = DeviceBuffer.from_numpy(W1)
+    assert np.array_equal(run(dW), want_for(W1))
+    assert np.array_equal(run(dW), want_for(W1))                      # prepared planes
+    dW.upload(W2)                                                     # overwritten in place through the library
+    assert np.array_equal(run(dW), want_for(W2))
+    dW.upload(W3)
+    assert np.array_equal(run(dW), want_for(W3)) and dev.pcmm_context.info("last_DW") == 4
+    addr = dW.ptr
+    dW.free()
+    dW = DeviceBuffer.from_numpy(W1)                                  # usually the same address again
+    assert np.array_equal(run(dW), want_for(W1)), ("reallocated at the same address", dW.ptr == addr)
+    # a change the library cannot see (another writer): announced by the caller
+    other = DeviceBuffer.from_numpy(W2)
+    import ctypes
+    hip = ctypes.CDLL("/opt/rocm/lib/libamdhip64.so")
+    assert hip.hipMemcpy(ctypes.c_void_p(dW.ptr), ctypes.c_void_p(other.ptr), ctypes.c_size_t(W2.nbytes), 3) == 0   # device to device
+    dev.pcmm_context.weights_changed(dW)
+    assert np.array_equal(run(dW), want_for(W2))
+    dev.pcmm_context.set_weight_cache(False)
+    first = DeviceBuffer.from_numpy(W1)
+    assert hip.hipMemcpy(ctypes.c_void_p(dW.ptr), ctypes.c_void_p(first.ptr), ctypes.c_size_t(W1.nbytes), 3) == 0
+    assert np.array_equal(run(dW), want_for(W1))                      # no cache: every call reads the matrix
+    dev.pcmm_context.set_weight_cache(True)
+
+
 @pytest.mark.parametrize("wide", [False, True])
 def test_ppmm_random_shapes_on_one_context(wide):
     """One context, a sequence of calls with random row counts, depths, modulus counts and plaintext magnitudes (1 to 4 digits),
