@@ -46,7 +46,7 @@ def _declare(L):
         "ckks_ntt_fwd_ext": (i, [vp, vp, i, i, i, i, i, i, i]), "ckks_ntt_inv_ext": (i, [vp, vp, i, i, i, i, i, i, i]),
         "ckks_modup_pq_to_t": (i, [vp, vp, vp, i, i]), "ckks_modup_qj_to_t": (i, [vp, vp, vp, i, i]),
         "ckks_modup_t_to_pql": (i, [vp, vp, vp, i, i]), "ckks_moddown_pql_to_ql": (i, [vp, vp, vp, i, i]),
-        "ckks_external_product_t": (i, [vp, vp, vp, vp, i]), "ckks_rescale": (i, [vp, vp, vp, i]),
+        "ckks_external_product_t": (i, [vp, vp, vp, vp, i]), "ckks_external_product_t_swk_reuse": (i, [vp, vp, vp, vp, i, i]), "ckks_rescale": (i, [vp, vp, vp, i]),
         "ckks_keyswitch_23": (i, [vp, vp, vp, vp, i, vp, vp, vp]),
         "ckks_hybrid_modup": (i, [vp, vp, vp, i]), "ckks_hybrid_inner_product": (i, [vp, vp, vp, vp, i]),
         "ckks_hybrid_moddown": (i, [vp, vp, vp, i]), "ckks_hybrid_keyswitch": (i, [vp, vp, vp, vp, i, vp]),

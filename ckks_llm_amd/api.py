@@ -3,6 +3,7 @@ Context_23 / PCMM_Context / PCMM_Scheme), calling the HIP library through its C 
 
 Polynomial arguments are DeviceBuffer objects or raw device addresses (ints, e.g. torch.Tensor.data_ptr()).
 """
+import os
 import ctypes as C
 
 import numpy as np
@@ -214,6 +215,11 @@ class Context_23:
     def external_product_T(self, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l):
         _check(self.L_.ckks_external_product_t(self.h, _addr(output), _addr(cipher_modUp_QjtoT), _addr(swk_modUp_RitoT), l), "ckks_external_product_t")
 
+    def external_product_T_swk_reuse(self, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l, batch_size):
+        """Context_23.h:62, ExternalProduct.cuh:151-162: one key against batch_size digit sets."""
+        _check(self.L_.ckks_external_product_t_swk_reuse(self.h, _addr(output), _addr(cipher_modUp_QjtoT), _addr(swk_modUp_RitoT), l, batch_size),
+               "ckks_external_product_t_swk_reuse")
+
     def rescaleAndEqual(self, cipher, scratch, l):
         _check(self.L_.ckks_rescale(self.h, _addr(cipher), _addr(scratch), l), "ckks_rescale")
 
@@ -320,9 +326,11 @@ class Ciphertext:
 class SecretKey:
     """SecretKey (SecretKey.cuh:9-31): sparse ternary secret of Hamming weight <= h over [P | Q], NTT domain, sampled from
     5*h bytes of the context's stream under (key, nonce).  h = None takes the context's Hamming weight, as the reference's
-    SecretKey(context) does (SecretKey.cuh:20-29)."""
+    SecretKey(context) does (SecretKey.cuh:20-29).  key = None (the default) draws 32 bytes from the operating system, so two
+    processes never share a secret; a fixed key is for runs that must repeat (the parity tests)."""
 
-    def __init__(self, context, h=None, key=bytes(32), nonce=0):
+    def __init__(self, context, h=None, key=None, nonce=0):
+        key = os.urandom(32) if key is None else bytes(key)
         if h is None:
             h = context.h_weight
         self.N, self.L, self.K = context.N, context.L, context.K
@@ -356,11 +364,12 @@ class Key_decomp:
 class Scheme_23:
     """The members of Scheme_23 on this path (Scheme_23.h:113-182): addEncKey, encryptZero, encryptMsg, decryptMsg,
     rescaleAndEqual, addMultKey_23, addConjKey_23, addLeftRotKey_23, mult_23, leftRotate_23, conjugate_23.
-    Randomness is the context's Salsa20 stream under this object's key with a nonce that counts calls."""
+    Randomness is the context's Salsa20 stream under this object's key with a nonce that counts calls; key = None (the
+    default) draws the key from the operating system, a fixed key makes a run repeatable."""
 
-    def __init__(self, context, key=bytes(32)):
+    def __init__(self, context, key=None):
         self.context = context
-        self.key = bytes(key)
+        self.key = os.urandom(32) if key is None else bytes(key)
         self.nonce = 1
         N, L = context.N, context.L
         self.publicKey = None
@@ -728,11 +737,12 @@ class PCMM_Scheme:
     """PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48): convertMLWESKfromRLWESK, addRepakcingKey, rlweCipherDecompose, PPMM,
     mlweCipherPacking, mlweDecrypt."""
 
-    def __init__(self, pcmm_context, key=bytes(32)):
+    def __init__(self, pcmm_context, key=None):
+        """key: 32 bytes of the random stream of the repacking keys; None (the default) draws them from the operating system."""
         self.L_ = load_library()
         self.pcmm_context = pcmm_context
         self.repackingKeys = None
-        self.key, self.nonce = bytes(key), 1 << 32
+        self.key, self.nonce = (os.urandom(32) if key is None else bytes(key)), 1 << 32
 
     def convertMLWESKfromRLWESK(self, mlwe_sk, rlwe_sk):
         """PCMM_Scheme.cuh:23-48."""
@@ -922,13 +932,35 @@ class Bert:
             parts = [(rlwe_cipher[0], 512, 0, 512), (rlwe_cipher[1], 256, 512, 512)]
         self.linear(plain_mat, 768, 768, parts, [(res_cipher[0], 256, 0), (res_cipher[1], 256, 256), (res_cipher[2], 256, 512)])
 
-    def mul_W_QKV(self, X, resQ, resK, resV, layer, do_s2c=1):
-        w = self.model_weights
+    def PCMM_Boot_768_768(self, plain_mat, rlwe_cipher, res_cipher, target_level, do_s2c):
+        """Bert.h:62 (Bert.cuh:379-498).  target_level is the level the reference raises the packed result to before its
+        coefficient-to-slot conversion and EvalMod (:472-497), a stage outside this library: accepted and not used."""
+        self.PCMM_768_768(plain_mat, rlwe_cipher, res_cipher, do_s2c)
+
+    test_PCMM_Boot_768_768 = PCMM_Boot_768_768                         # Bert.h:63
+
+    def mul_W_QKV(self, X, *args):
+        """Bert.h:51: mul_W_QKV(X, model_weights, resQ, resK, resV, layer), three inputs of 256 samples (do_s2c = 1) as the
+        reference calls it (Bert.cuh:155-169; its bias additions on slot-packed plaintexts are not part of this library).
+        Also mul_W_QKV(X, resQ, resK, resV, layer, do_s2c=1) on the object's own weights."""
+        if isinstance(args[0], Bert_model_weights):
+            w, resQ, resK, resV, layer = args
+            do_s2c = 1
+        else:
+            w = self.model_weights
+            resQ, resK, resV, layer = args[:4]
+            do_s2c = args[4] if len(args) > 4 else 1
         self.PCMM_768_768(w.attention_self_query_weight[layer], X, resQ, do_s2c)
         self.PCMM_768_768(w.attention_self_key_weight[layer], X, resK, do_s2c)
         self.PCMM_768_768(w.attention_self_value_weight[layer], X, resV, do_s2c)
 
-    def attn_output(self, O, res, layer, do_s2c=1):
+    def attn_output(self, O, *args):
+        """Bert.h:59: attn_output(O, layer), the dense product in place (Bert.cuh:204-211).  Also attn_output(O, res, layer, do_s2c=1)."""
+        if isinstance(args[0], int):
+            res, layer, do_s2c = O, args[0], 1
+        else:
+            res, layer = args[:2]
+            do_s2c = args[2] if len(args) > 2 else 1
         self.PCMM_768_768(self.model_weights.attention_output_dense_weight[layer], O, res, do_s2c)
 
     def intermediate(self, O, layer, res):
@@ -936,7 +968,8 @@ class Bert:
         self.linear(self.model_weights.intermediate_dense_weight[layer], 3072, 768, [(O[0], 512, 0, 512), (O[2], 256, 512, 256)],
                     [(res[2 * i], 512, 512 * i) for i in range(6)])
 
-    def layer_output(self, O, layer):
-        """Bert.cuh:290-302: 512 samples of each O[2 i]; 768 x 3072; rows 0..511 into O[0], 512..767 into O[2]."""
+    def layer_output(self, O, layer, layer_res=None):
+        """Bert.h:61, Bert.cuh:290-302: 512 samples of each O[2 i]; 768 x 3072; rows 0..511 into O[0], 512..767 into O[2].
+        layer_res is not touched: the reference's body does not use it either (Bert.cuh:333, 349-353 are commented out)."""
         self.linear(self.model_weights.output_dense_weight[layer], 768, 3072, [(O[2 * i], 512, 512 * i, 512) for i in range(6)],
                     [(O[0], 512, 0), (O[2], 256, 512)])

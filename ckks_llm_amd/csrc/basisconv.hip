@@ -254,6 +254,38 @@ __global__ __launch_bounds__(CONV_THREADS) void inner_product_kernel(InnerArgs a
     a.out[(a.out_z_stride + o) * a.N + x] = barrett128(acc2, pr.q, pr.mu_hi, pr.mu_lo);
 }
 
+// One switching key against `batch` digit sets (external_product_T_kernel_swk_reuse, ExternalProduct.cuh:103-149): every key word is
+// read once and multiplied into the accumulators of all the sets.  Set `it` lies c_set_stride limbs behind set it - 1; its two
+// result polynomials are polynomials 2 it and 2 it + 1 of the output (out_z_stride limbs each).
+constexpr int REUSE_MAX_BATCH = 8;                 // the reference's accumulator array holds eight sets
+__global__ __launch_bounds__(CONV_THREADS) void inner_product_reuse_kernel(InnerArgs a, int batch, long c_set_stride) {
+    const long x = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
+    const int o = blockIdx.y;
+    const int k = o % a.c_mod;
+    const PrimeConst& pr = a.primes[a.prime0 + k];
+    u128w acc1[REUSE_MAX_BATCH], acc2[REUSE_MAX_BATCH];
+#pragma unroll
+    for (int it = 0; it < REUSE_MAX_BATCH; it++) acc1[it] = acc2[it] = u128w{0, 0};
+    for (int d = 0; d < a.ndigits; d++) {
+        const long kidx = ((long)d * a.key_digit_stride + o) * a.N + x;
+        const u64 k1 = a.key[kidx], k2 = a.key[a.key_z_stride * a.N + kidx];
+        const u64* cp = a.c + ((long)d * a.c_digit_stride + k) * a.N + x;
+#pragma unroll
+        for (int it = 0; it < REUSE_MAX_BATCH; it++)
+            if (it < batch) {
+                const u64 ra = cp[(long)it * c_set_stride * a.N];
+                mac128(acc1[it], ra, k1);
+                mac128(acc2[it], ra, k2);
+            }
+    }
+#pragma unroll
+    for (int it = 0; it < REUSE_MAX_BATCH; it++)
+        if (it < batch) {
+            a.out[((long)(2 * it) * a.out_z_stride + o) * a.N + x] = barrett128(acc1[it], pr.q, pr.mu_hi, pr.mu_lo);
+            a.out[((long)(2 * it + 1) * a.out_z_stride + o) * a.N + x] = barrett128(acc2[it], pr.q, pr.mu_hi, pr.mu_lo);
+        }
+}
+
 // ---- rescale (Scheme_23.cuh:321-367) ----
 __global__ __launch_bounds__(CONV_THREADS) void mod_to_qi_kernel(u64* dst, const u64* src, const PrimeConst* primes, long N, int K, int q_num, int l) {
     const long x = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
@@ -309,6 +341,22 @@ extern "C" int ckks_external_product_t(ckks_ctx* c, uint64_t* out, const uint64_
     int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;         // :88
     dim3 grid((unsigned)(c->N / CONV_THREADS), blockNum * c->t_num), block(CONV_THREADS);
     hipLaunchKernelGGL(inner_product_kernel, grid, block, 0, c->stream, a);
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+extern "C" int ckks_external_product_t_swk_reuse(ckks_ctx* c, uint64_t* out, const uint64_t* cT, const uint64_t* swk, int l, int batch_size) {
+    if (!level_ok(c, l) || !out || !cT || !swk || c->t_num == 0 || c->gamma == 0 || c->p_num == 0) { set_error("external_product_T_swk_reuse: bad level or basis"); return CKKS_E_INVALID; }
+    if (batch_size < 1 || batch_size > REUSE_MAX_BATCH) { set_error("external_product_T_swk_reuse: batch_size must be 1 .. 8 (the reference's accumulator array)"); return CKKS_E_INVALID; }
+    InnerArgs a;
+    a.c = cT; a.key = swk; a.out = out; a.primes = c->d_primes; a.N = c->N;
+    a.ndigits = (l + 1 + c->p_num - 1) / c->p_num;                       // cipher_blockNum, ExternalProduct.cuh:153
+    if (a.ndigits > c->dnum) { set_error("external_product_T_swk_reuse: the level needs more digits than the key holds (q_num is no multiple of p_num)"); return CKKS_E_INVALID; }
+    a.c_mod = c->t_num; a.prime0 = c->p_num + c->q_num;
+    a.c_digit_stride = c->t_num; a.key_digit_stride = (long)c->t_num * c->Ri_blockNum;
+    a.key_z_stride = (long)c->Ri_blockNum * c->t_num * c->dnum; a.out_z_stride = (long)c->Ri_blockNum * c->t_num;
+    const int blockNum = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;   // :154
+    dim3 grid((unsigned)(c->N / CONV_THREADS), blockNum * c->t_num), block(CONV_THREADS);
+    hipLaunchKernelGGL(inner_product_reuse_kernel, grid, block, 0, c->stream, a, batch_size, (long)c->t_num * c->Qj_blockNum);   // :126
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }

@@ -124,6 +124,10 @@ int ckks_modup_t_to_pql(ckks_ctx* ctx, uint64_t* buf, const uint64_t* in, int l,
 int ckks_moddown_pql_to_ql(ckks_ctx* ctx, uint64_t* out, const uint64_t* buf, int l, int batch_size);
 /* Context_23::external_product_T (ExternalProduct.cuh:85-97); swk laid out as Key_decomp (Key_decomp.cuh:19-24) */
 int ckks_external_product_t(ckks_ctx* ctx, uint64_t* out, const uint64_t* c_T, const uint64_t* swk_T, int l);
+/* Context_23::external_product_T_swk_reuse (Context_23.h:62, ExternalProduct.cuh:103-162): one switching key against batch_size
+ * (1 .. 8) digit sets.  Set it of c_T starts Qj_blockNum * t_num limbs behind set it - 1 (the layout modUpQjtoT_23 writes for a
+ * batch); out holds 2 * batch_size polynomials of Ri_blockNum * t_num limbs: polynomials 2 it and 2 it + 1 are the pair of set it. */
+int ckks_external_product_t_swk_reuse(ckks_ctx* ctx, uint64_t* out, const uint64_t* c_T, const uint64_t* swk_T, int l, int batch_size);
 /* Scheme_23::rescaleAndEqual (Scheme_23.cuh:369-385): cipher = [a: L+1 limbs | b: L+1 limbs], level l -> l-1.
  * scratch: 2*(L+1)*N words (Scheme_23::rescale_buffer). */
 int ckks_rescale(ckks_ctx* ctx, uint64_t* cipher, uint64_t* scratch, int l);

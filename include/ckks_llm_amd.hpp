@@ -14,6 +14,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <iostream>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -132,6 +133,14 @@ public:
     Context_23(const Context_23&) = delete;
     Context_23& operator=(const Context_23&) = delete;
     ~Context_23() { if (handle) ckks_ctx_destroy(handle); }
+    void seed_rng_from_system() {
+        std::random_device rd;
+        for (int i = 0; i < 32; i += 4) {
+            const uint32_t w = rd();
+            for (int b = 0; b < 4; b++) rng_key[i + b] = (uint8_t)(w >> (8 * b));
+        }
+        rng_nonce = 0;
+    }
 
     long info(const char* name) const {
         long v = 0;
@@ -146,6 +155,7 @@ private:
         dnum = (int)info("dnum");
         Ri_blockNum = (int)info("Ri_blockNum");
         Qj_blockNum = (int)info("Qj_blockNum");
+        seed_rng_from_system();
     }
 public:
 
@@ -182,10 +192,16 @@ public:
     void external_product_T(uint64_tt* output, const uint64_tt* cipher_modUp_QjtoT, const uint64_tt* swk_modUp_RitoT, int l) {
         check(ckks_external_product_t(handle, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l), "external_product_T");
     }
+    // Context_23.h:62: one switching key against batch_size digit sets
+    void external_product_T_swk_reuse(uint64_tt* output, const uint64_tt* cipher_modUp_QjtoT, const uint64_tt* swk_modUp_RitoT, int l, int batch_size) {
+        check(ckks_external_product_t_swk_reuse(handle, output, cipher_modUp_QjtoT, swk_modUp_RitoT, l, batch_size), "external_product_T_swk_reuse");
+    }
 
     // RNG::generateRandom_device (RNG.cuh:18-56).  The reference draws a fresh key and nonce from rand() per call; here the
-    // context holds a key (settable) and a nonce that counts the calls, so a run can be repeated.
-    uint8_t rng_key[32] = {0};
+    // context holds a key and a nonce that counts the calls.  The key comes from std::random_device when the context is built, so
+    // no two processes share secrets or encryption randomness; a program that must repeat a run (the parity tests) overwrites
+    // rng_key with fixed bytes and resets rng_nonce before it draws anything.
+    uint8_t rng_key[32];
     uint64_t rng_nonce = 0;
     void generateRandom_device(uint8_t* a, uint64_tt n) {
         check(ckks_random_bytes(handle, a, (size_t)n, rng_key, ++rng_nonce), "generateRandom_device");

@@ -273,6 +273,40 @@ public:
         else in = {{rlwe_cipher[0], 512, 0, 512}, {rlwe_cipher[1], 256, 512, 512}};
         linear(plain_mat, 768, 768, in, {{res_cipher[0], 256, 0, 0}, {res_cipher[1], 256, 256, 0}, {res_cipher[2], 256, 512, 0}});
     }
+    // ---- the reference's own member signatures (Bert.h:51, 59-63), so that code written against Bert.h compiles.  What they do not
+    //      carry out of the reference's bodies is listed at each member. ----
+    // Bert::PCMM_Boot_768_768 (Bert.h:62, Bert.cuh:379-498).  target_level is the level the reference raises the packed result to
+    // before its coefficient-to-slot conversion and EvalMod (:472-497); that stage is outside this library, so the argument is
+    // accepted and not used: the results stay at level 0 in coefficient packing.
+    void PCMM_Boot_768_768(float* plain_mat, std::vector<Ciphertext*>& rlwe_cipher, std::vector<Ciphertext*>& res_cipher, int target_level, int do_s2c) {
+        (void)target_level;
+        PCMM_768_768(plain_mat, rlwe_cipher, res_cipher, do_s2c);
+    }
+    // Bert.h:63: the reference keeps a second copy of the member for its test program
+    void test_PCMM_Boot_768_768(float* plain_mat, std::vector<Ciphertext*>& rlwe_cipher, std::vector<Ciphertext*>& res_cipher, int target_level, int do_s2c) {
+        PCMM_Boot_768_768(plain_mat, rlwe_cipher, res_cipher, target_level, do_s2c);
+    }
+    // Bert::mul_W_QKV (Bert.h:51, Bert.cuh:155-169): the three products on the weights handed in, three input ciphertexts of 256
+    // samples (do_s2c = 1, as the reference calls it).  The bias additions of :158-168 act on slot-packed plaintexts after the
+    // bootstrapping and are not part of this library.
+    void mul_W_QKV(std::vector<Ciphertext*>& X, Bert_model_weights& weights, std::vector<Ciphertext*>& resQ, std::vector<Ciphertext*>& resK,
+                   std::vector<Ciphertext*>& resV, int layer) {
+        PCMM_Boot_768_768(weights.attention_self_query_weight[layer], X, resQ, X[0]->L - 2, 1);
+        PCMM_Boot_768_768(weights.attention_self_key_weight[layer], X, resK, X[0]->L - 2, 1);
+        PCMM_Boot_768_768(weights.attention_self_value_weight[layer], X, resV, 18, 1);
+    }
+    // Bert::attn_output (Bert.h:59, Bert.cuh:204-211): the dense product in place, O -> O; the LayerNorm behind it is not part of this library
+    void attn_output(std::vector<Ciphertext*>& O, int layer) {
+        PCMM_Boot_768_768(model_weights.attention_output_dense_weight[layer], O, O, O[0]->L, 1);
+    }
+    // Bert::layer_output (Bert.h:61, Bert.cuh:290-302).  layer_res is not touched: the reference's body does not use it either (every
+    // line that names it is commented out, Bert.cuh:333, 349-353).
+    void layer_output(std::vector<Ciphertext*>& O, int layer, std::vector<Ciphertext*>& layer_res) {
+        (void)layer_res;
+        layer_output(O, layer);
+    }
+
+    // ---- the same calls with the choices the reference hard-wires left to the caller ----
     // Bert::mul_W_QKV (Bert.cuh:155-169)
     void mul_W_QKV(std::vector<Ciphertext*>& X, std::vector<Ciphertext*>& resQ, std::vector<Ciphertext*>& resK, std::vector<Ciphertext*>& resV,
                    int layer, int do_s2c = 1) {

@@ -585,6 +585,32 @@ int orc_external_product_t(const orc_ctx* c, u64* out, const u64* cT, const u64*
     return 0;
 }
 
+// ExternalProduct.cuh:103-162: one key, batch_size digit sets; set `iter` of cT starts t_num * Qj_blockNum limbs behind the one
+// before (:126), its pair goes to polynomials 2 iter and 2 iter + 1 of out (:134, :155).  The reference holds eight accumulators.
+int orc_external_product_t_swk_reuse(const orc_ctx* c, u64* out, const u64* cT, const u64* swk, int l, int batch_size) {
+    const long N = c->N; const int g = c->gamma, P = c->p_num, Q = c->q_num, T = c->t_num, RB = c->Ri_blockNum, QB = c->Qj_blockNum, dnum = c->dnum;
+    if (g <= 0 || T <= 0 || P <= 0 || l < 0 || l > c->L || batch_size < 1 || batch_size > 8) return -1;
+    const int cipher_blockNum = ceil_div(l + 1, P), blockNum = ceil_div(P + l + 1, g);
+    if (cipher_blockNum > dnum) return -1;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int blk = 0; blk < blockNum; blk++)
+        for (int k = 0; k < T; k++)
+            for (long x = 0; x < N; x++) {
+                const long oidx = x + (long)blk * T * N + (long)k * N;
+                for (int half = 0; half < 2; half++)
+                    for (int iter = 0; iter < batch_size; iter++) {
+                        u128 acc = 0;
+                        for (int i = 0; i < cipher_blockNum; i++) {
+                            const u64 ra = cT[((long)i * T + k) * N + x + (long)iter * T * QB * N];
+                            const u64 rb = swk[(long)half * RB * T * dnum * N + ((long)i * T * RB + (long)blk * T + k) * N + x];
+                            acc += (u128)ra * rb;
+                        }
+                        out[(long)RB * T * N * (iter * 2 + half) + oidx] = barrett_idx(c, acc, P + Q + k);
+                    }
+            }
+    return 0;
+}
+
 // Scheme_23.cuh:321-385
 int orc_rescale(const orc_ctx* c, u64* cipher, int l) {
     const long N = c->N; const int K = c->K, L = c->L;

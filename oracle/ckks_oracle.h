@@ -94,6 +94,7 @@ int orc_modup_t_to_pql(const orc_ctx*, uint64_t* buf, const uint64_t* in, int l,
 int orc_moddown_pql_to_ql(const orc_ctx*, uint64_t* out, const uint64_t* buf, int l, int batch);
 /* ExternalProduct.cuh:7-97 */
 int orc_external_product_t(const orc_ctx*, uint64_t* out, const uint64_t* c_T, const uint64_t* swk_T, int l);
+int orc_external_product_t_swk_reuse(const orc_ctx*, uint64_t* out, const uint64_t* c_T, const uint64_t* swk_T, int l, int batch_size);
 /* Scheme_23.cuh:321-385 ; cipher = [a: L+1 limbs | b: L+1 limbs], NTT domain, level l -> l-1 */
 int orc_rescale(const orc_ctx*, uint64_t* cipher, int l);
 /* KeySwitch_23.cuh:216-231 (steps 2..9 of mult_23 without the tensor product):

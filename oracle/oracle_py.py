@@ -73,7 +73,7 @@ def lib():
             "orc_ntt_fwd_ext": (i, [vp, P64, i, i, i, i, i, i, i]), "orc_ntt_inv_ext": (i, [vp, P64, i, i, i, i, i, i, i]),
             "orc_modup_pq_to_t": (i, [vp, P64, P64, i, i]), "orc_modup_qj_to_t": (i, [vp, P64, P64, i, i]),
             "orc_modup_t_to_pql": (i, [vp, P64, P64, i, i]), "orc_moddown_pql_to_ql": (i, [vp, P64, P64, i, i]),
-            "orc_external_product_t": (i, [vp, P64, P64, P64, i]), "orc_rescale": (i, [vp, P64, i]),
+            "orc_external_product_t": (i, [vp, P64, P64, P64, i]), "orc_external_product_t_swk_reuse": (i, [vp, P64, P64, P64, i, i]), "orc_rescale": (i, [vp, P64, i]),
             "orc_keyswitch_23": (i, [vp, P64, P64, P64, i]),
             "orc_hybrid_modup": (i, [vp, P64, P64, i]), "orc_hybrid_inner_product": (i, [vp, P64, P64, P64, i]),
             "orc_hybrid_moddown": (i, [vp, P64, P64, i]), "orc_hybrid_keyswitch": (i, [vp, P64, P64, P64, i]),
@@ -178,6 +178,9 @@ class OracleContext:
 
     def external_product_T(self, out, cT, swk, l):
         self._ck(self.L_.orc_external_product_t(self.h, _ptr(out), _ptr(cT), _ptr(swk), l))
+
+    def external_product_T_swk_reuse(self, out, cT, swk, l, batch_size):
+        self._ck(self.L_.orc_external_product_t_swk_reuse(self.h, _ptr(out), _ptr(cT), _ptr(swk), l, batch_size))
 
     def rescaleAndEqual(self, cipher, l):
         self._ck(self.L_.orc_rescale(self.h, _ptr(cipher), l))

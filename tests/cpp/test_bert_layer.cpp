@@ -162,7 +162,7 @@ static int run(const std::string& catalog) {
             std::vector<double> Y = plain_product(W, X, tokens, 768, 768);
             std::vector<Ciphertext*> in = {hs.encrypt_part(X, 768, 0, 512, 512), hs.encrypt_part(X, 768, 512, 256, 512)};
             std::vector<Ciphertext*> out = {new Ciphertext(N, L, 0, N / 2, 1), new Ciphertext(N, L, 0, N / 2, 1), new Ciphertext(N, L, 0, N / 2, 1)};
-            bert.PCMM_768_768(bert.model_weights.attention_self_query_weight[0], in, out, 0);
+            bert.PCMM_Boot_768_768(bert.model_weights.attention_self_query_weight[0], in, out, L, 0);      // Bert.h:62
             double worst = 0;
             for (int j = 0; j < 3; j++) worst = std::max(worst, hs.worst_error(*out[j], Y, 768, 256 * j, 256));
             printf("768 x 768, 2 inputs (%s): worst error 2^%.1f, output scale 2^%.1f\n", how, std::log2(worst), (double)std::log2((double)out[0]->scale));
@@ -197,7 +197,7 @@ static int run(const std::string& catalog) {
             std::vector<Ciphertext*> in = {hs.encrypt_part(X, 768, 0, 256, 256), hs.encrypt_part(X, 768, 256, 256, 256), hs.encrypt_part(X, 768, 512, 256, 256)};
             std::vector<Ciphertext*> Q, K, V;
             for (int j = 0; j < 3; j++) { Q.push_back(new Ciphertext(N, L, 0, N / 2, 1)); K.push_back(new Ciphertext(N, L, 0, N / 2, 1)); V.push_back(new Ciphertext(N, L, 0, N / 2, 1)); }
-            bert.mul_W_QKV(in, Q, K, V, 0);
+            bert.mul_W_QKV(in, bert.model_weights, Q, K, V, 0);                    // the reference's signature (Bert.h:51)
             float* weights[3] = {bert.model_weights.attention_self_query_weight[0], bert.model_weights.attention_self_key_weight[0], bert.model_weights.attention_self_value_weight[0]};
             std::vector<Ciphertext*>* res[3] = {&Q, &K, &V};
             double worst = 0;
@@ -210,6 +210,19 @@ static int run(const std::string& catalog) {
             for (Ciphertext* c : in) delete c;
             for (int w = 0; w < 3; w++) for (Ciphertext* c : *res[w]) delete c;
         }
+        // ---- attn_output(O, layer) as Bert.h:59 declares it: the dense product in place, three ciphertexts of 256 samples ----
+        {
+            std::vector<double> X((size_t)tokens * 768);
+            for (double& v : X) v = act(rng);
+            std::vector<Ciphertext*> O = {hs.encrypt_part(X, 768, 0, 256, 256), hs.encrypt_part(X, 768, 256, 256, 256), hs.encrypt_part(X, 768, 512, 256, 256)};
+            bert.attn_output(O, 0);
+            std::vector<double> Y = plain_product(host_floats(bert.model_weights.attention_output_dense_weight[0], 768 * 768), X, tokens, 768, 768);
+            double worst = 0;
+            for (int j = 0; j < 3; j++) worst = std::max(worst, hs.worst_error(*O[j], Y, 768, 256 * j, 256));
+            printf("attn_output in place: worst error 2^%.1f\n", std::log2(worst));
+            EXPECT(worst < bound, "attn_output(O, layer) leaves W_o x in O");
+            for (Ciphertext* c : O) delete c;
+        }
         // ---- layer_output: 768 x 3072 on the previous product (scaled to unit size) ----
         {
             std::vector<double> X = H;
@@ -218,7 +231,8 @@ static int run(const std::string& catalog) {
             std::vector<double> Y = plain_product(W, X, tokens, 768, 3072);
             std::vector<Ciphertext*> O(12, nullptr);
             for (int i = 0; i < 6; i++) O[2 * i] = hs.encrypt_part(X, 3072, 512 * i, 512, 512);
-            bert.layer_output(O, 0);
+            std::vector<Ciphertext*> layer_res;
+            bert.layer_output(O, 0, layer_res);                                   // Bert.h:61
             const double worst = std::max(hs.worst_error(*O[0], Y, 768, 0, 512), hs.worst_error(*O[2], Y, 768, 512, 256));
             printf("layer_output 768 x 3072: worst error 2^%.1f\n", std::log2(worst));
             EXPECT(worst < bound, "layer_output decrypts to W x");

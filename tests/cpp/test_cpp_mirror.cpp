@@ -155,10 +155,11 @@ static int run() {
     EXPECT(threw, "mlweCipherPacking without keys throws std::invalid_argument");
 
     // ---- SecretKey, addEncKey, encode_coeffs, encryptMsg, decryptMsg, decode_coeffs: the context's stream is Salsa20 under its
-    //      key (zero here) with nonces 1, 2, 3 for the three draws, so the oracle can follow word for word ----
+    //      key (set to zero here; a fresh context holds random bytes) with nonces 1, 2, 3 for the three draws, so the oracle can follow word for word ----
     {
         const int h = 64, L1 = context.L + 1;
         const uint8_t zero_key[32] = {0};
+        for (int i = 0; i < 32; i++) context.rng_key[i] = 0;       // a fixed key, as a program that must repeat a run sets it
         context.rng_nonce = 0;
         SecretKey sk(context, h);
         std::vector<uint8_t> r1(5 * h), r2(8 * N * L1 + 4 * N), r3(9 * N);
@@ -212,6 +213,7 @@ static int run() {
         const int lg = 10, h = 64;
         const long n = 1l << lg;
         Context_23 c2(lg, p13, q13, t13, 3);
+        for (int i = 0; i < 32; i++) c2.rng_key[i] = 0;        // fixed key: the oracle follows the same stream
         orc_ctx* o2 = orc_ctx_create(lg, p13.data(), 1, q13.data(), 5, t13.data(), 3, 3);
         const int K = c2.K, L1 = c2.L + 1, KL = K + L1;
         const size_t keyw = (size_t)2 * c2.dnum * c2.Ri_blockNum * c2.t_num * n;

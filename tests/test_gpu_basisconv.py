@@ -63,6 +63,30 @@ def test_four_conversion_maps(params, logN):
 
 
 @pytest.mark.parametrize("params", [14, 15])
+def test_external_product_swk_reuse(params):
+    """Context_23::external_product_T_swk_reuse (ExternalProduct.cuh:103-162) against the oracle for 1, 3 and 8 digit sets."""
+    pair = ref_pair(params, 12)
+    o, d, N = pair.orc, pair.dev, pair.N
+    K, T, RB, QB, dnum, L = o.p_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum, o.dnum, o.L
+    swk = limbs_uniform(70, o.t, 2 * dnum * RB, N)
+    dswk = to_dev(swk)
+    for l, batch in ((L, 3), (L - 1, 8), (1, 1)):
+        cT = limbs_uniform(71 + l, o.t, batch * QB, N)
+        want = np.zeros((2 * batch, RB * T, N), dtype=np.uint64)
+        o.external_product_T_swk_reuse(want.reshape(-1), cT.reshape(-1), swk.reshape(-1), l, batch)
+        dout = to_dev(np.zeros_like(want))
+        d.external_product_T_swk_reuse(dout, to_dev(cT), dswk, l, batch)
+        nblk = -(-(K + l + 1) // o.gamma)
+        got = from_dev(dout, want.shape)
+        assert np.array_equal(got[:, :nblk * T], want[:, :nblk * T]), (l, batch)
+        assert not got[:, nblk * T:].any()                                    # blocks beyond the level stay untouched
+    with pytest.raises(Exception):
+        d.external_product_T_swk_reuse(dout, to_dev(cT), dswk, 1, 9)
+    with pytest.raises(Exception):
+        d.external_product_T_swk_reuse(dout, to_dev(cT), dswk, 1, 0)
+
+
+@pytest.mark.parametrize("params", [14, 15])
 def test_external_product_and_keyswitch_23(params):
     pair = ref_pair(params, 12)
     o, d, N = pair.orc, pair.dev, pair.N

@@ -162,6 +162,33 @@ def test_external_product_bruteforce():
                     assert int(out[z, blk, k, x]) == want
 
 
+def test_external_product_swk_reuse_bruteforce():
+    """One key against several digit sets (ExternalProduct.cuh:103-162): every output word against Python integers, with the
+    reference's addressing (set stride t_num * Qj_blockNum limbs, result pair of set i at polynomials 2i, 2i + 1), and equal to
+    the single-set product set by set."""
+    ctx = ref_ctx(14)
+    K, T, g, RB, QB, dnum = ctx.p_num, ctx.t_num, ctx.gamma, ctx.Ri_blockNum, ctx.Qj_blockNum, ctx.dnum
+    for l, batch in ((ctx.L - 1, 3), (1, 8), (ctx.L, 1)):
+        cb = -(-(l + 1) // K)
+        nblk = -(-(K + l + 1) // g)
+        cT = limbs_uniform(31 + l, ctx.t, batch * QB, N).reshape(batch, QB, T, N)
+        swk = limbs_uniform(32 + l, ctx.t, 2 * dnum * RB, N).reshape(2, dnum, RB, T, N)
+        out = np.zeros((batch, 2, RB, T, N), dtype=np.uint64)
+        ctx.external_product_T_swk_reuse(out.reshape(-1), cT.reshape(-1), swk.reshape(-1), l, batch)
+        for it in range(batch):
+            one = np.zeros((2, RB, T, N), dtype=np.uint64)
+            ctx.external_product_T(one.reshape(-1), np.ascontiguousarray(cT[it]).reshape(-1), swk.reshape(-1), l)
+            assert np.array_equal(out[it, :, :nblk], one[:, :nblk]), (l, it)
+            for z in range(2):
+                for blk in range(0, nblk, 2):
+                    for k in range(T):
+                        for x in range(0, N, 11):
+                            want = sum(int(cT[it, i, k, x]) * int(swk[z, i, blk, k, x]) for i in range(cb)) % ctx.t[k]
+                            assert int(out[it, z, blk, k, x]) == want
+    with pytest.raises(Exception):
+        ctx.external_product_T_swk_reuse(out.reshape(-1), cT.reshape(-1), swk.reshape(-1), 1, 9)
+
+
 def test_rescale_closed_form():
     ctx = ref_ctx(14, logN=5)
     n = 1 << 5
