@@ -11,7 +11,11 @@
 //     (KeySwitch_23.cuh:194-201, Scheme_23.cuh:192-194), std::runtime_error for everything the reference never checks.
 // Header-only, no HIP headers needed: any C++17 host compiler can build against it and link libckks_hip.so.
 #pragma once
+#include <algorithm>
+#include <cmath>
+#include <complex>
 #include <cstddef>
+#include <cstdio>
 #include <cstdint>
 #include <iostream>
 #include <random>
@@ -105,6 +109,70 @@ inline ReferenceParams reference_params(long logN) {
 }
 
 // Context_23 (Context_23.h:19-279): prime sets, tables, NTT and basis conversion.
+// PrecisionStats / GetPrecisionStats (precision.cuh:5-249): the table of log2(1 / |computed - wanted|) that the reference's test
+// programs print.  Kept as the reference computes it: MinDelta starts at 1, so the maximum precision is never reported below 0
+// bits; the median of an even number n of values is the mean of the sorted values n/2 and n/2 + 1 (counting from 0) unless
+// n/2 + 1 = n.  The cumulative distributions the reference fills and never prints are left out.
+struct Stats {
+    double Real, Imag, L2;
+};
+struct PrecisionStats {
+    Stats MaxDelta, MinDelta, MaxPrecision, MinPrecision, MeanDelta, MeanPrecision, MedianDelta, MedianPrecision;
+    std::string String() const {                                           // precision.cuh:29-44
+        char buffer[512];
+        snprintf(buffer, sizeof(buffer),
+                 "\n _________________________________\n"
+                 "|    Log2 | REAL  | IMAG  | L2    |\n"
+                 "|MIN Prec | %.2f | %.2f | %.2f |\n"
+                 "|MAX Prec | %.2f | %.2f | %.2f |\n"
+                 "|AVG Prec | %.2f | %.2f | %.2f |\n"
+                 "|MED Prec | %.2f | %.2f | %.2f |\n"
+                 "===================================\n",
+                 MinPrecision.Real, MinPrecision.Imag, MinPrecision.L2, MaxPrecision.Real, MaxPrecision.Imag, MaxPrecision.L2,
+                 MeanPrecision.Real, MeanPrecision.Imag, MeanPrecision.L2, MedianPrecision.Real, MedianPrecision.Imag, MedianPrecision.L2);
+        return std::string(buffer);
+    }
+};
+inline Stats deltaToPrecision(const Stats& c) { return {std::log2(1 / c.Real), std::log2(1 / c.Imag), std::log2(1 / c.L2)}; }
+inline PrecisionStats precision_from_deltas(std::vector<double> re, std::vector<double> im) {
+    const size_t n = re.size();
+    std::vector<double> l2(n);
+    PrecisionStats prec;
+    prec.MaxDelta = {0, 0, 0};
+    prec.MinDelta = {1, 1, 1};
+    prec.MeanDelta = {0, 0, 0};
+    for (size_t i = 0; i < n; i++) {
+        l2[i] = std::sqrt(re[i] * re[i] + im[i] * im[i]);
+        prec.MeanDelta.Real += re[i]; prec.MeanDelta.Imag += im[i]; prec.MeanDelta.L2 += l2[i];
+        prec.MaxDelta = {std::max(prec.MaxDelta.Real, re[i]), std::max(prec.MaxDelta.Imag, im[i]), std::max(prec.MaxDelta.L2, l2[i])};
+        prec.MinDelta = {std::min(prec.MinDelta.Real, re[i]), std::min(prec.MinDelta.Imag, im[i]), std::min(prec.MinDelta.L2, l2[i])};
+    }
+    prec.MeanDelta = {prec.MeanDelta.Real / n, prec.MeanDelta.Imag / n, prec.MeanDelta.L2 / n};
+    auto median = [n](std::vector<double>& v) {                            // calcMedian, precision.cuh:69-102
+        std::sort(v.begin(), v.end());
+        const size_t index = n / 2;
+        return (n % 2 == 1 || index + 1 == n) ? v[index] : (v[index] + v[index + 1]) / 2;
+    };
+    prec.MedianDelta = {median(re), median(im), median(l2)};
+    prec.MinPrecision = deltaToPrecision(prec.MaxDelta);
+    prec.MaxPrecision = deltaToPrecision(prec.MinDelta);
+    prec.MeanPrecision = deltaToPrecision(prec.MeanDelta);
+    prec.MedianPrecision = deltaToPrecision(prec.MedianDelta);
+    return prec;
+}
+inline PrecisionStats GetPrecisionStats(const std::vector<double>& valuesTest, const std::vector<double>& valuesWant) {      // precision.cuh:178-249
+    if (valuesTest.size() < valuesWant.size() || valuesWant.empty()) throw std::invalid_argument("GetPrecisionStats: vectors of the same positive length");
+    std::vector<double> re(valuesWant.size()), im(valuesWant.size(), 0.0);
+    for (size_t i = 0; i < re.size(); i++) re[i] = std::abs(valuesTest[i] - valuesWant[i]);
+    return precision_from_deltas(re, im);
+}
+inline PrecisionStats GetPrecisionStats(const std::vector<std::complex<double>>& valuesTest, const std::vector<std::complex<double>>& valuesWant) {  // :104-174
+    if (valuesTest.size() < valuesWant.size() || valuesWant.empty()) throw std::invalid_argument("GetPrecisionStats: vectors of the same positive length");
+    std::vector<double> re(valuesWant.size()), im(valuesWant.size());
+    for (size_t i = 0; i < re.size(); i++) { re[i] = std::abs(valuesTest[i].real() - valuesWant[i].real()); im[i] = std::abs(valuesTest[i].imag() - valuesWant[i].imag()); }
+    return precision_from_deltas(re, im);
+}
+
 class Context_23 {
 public:
     long logN, N;

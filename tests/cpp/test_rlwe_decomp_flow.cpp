@@ -33,12 +33,12 @@ static std::vector<double> host_doubles(const double* d, size_t n) {
     check(ckks_memcpy_d2h(h.data(), d, n * 8), "d2h");
     return h;
 }
-// worst and mean precision in bits, as GetPrecisionStats reports them (precision.cuh:104)
-static void precision_bits(const std::vector<double>& got, const std::vector<double>& want, double& worst, double& mean) {
-    double emax = 0, esum = 0;
-    for (size_t i = 0; i < got.size(); i++) { const double e = std::fabs(got[i] - want[i]); emax = std::max(emax, e); esum += e; }
-    worst = -std::log2(emax + 1e-300);
-    mean = -std::log2(esum / got.size() + 1e-300);
+// worst and mean precision in bits, from GetPrecisionStats as the reference's program calls it (test_rlwe_decomp.cu:195)
+static void precision_bits(const std::vector<double>& got, const std::vector<double>& want, double& worst, double& mean, bool print = false) {
+    const PrecisionStats st = GetPrecisionStats(got, want);
+    if (print) printf("%s", st.String().c_str());
+    worst = st.MinPrecision.Real;
+    mean = st.MeanPrecision.Real;
 }
 
 static int run() {
@@ -118,7 +118,7 @@ static int run() {
     scheme.decryptMsg(m2_dec, sk, c2);
     context.decode_coeffs(m2_dec, real_msg_dec);
     std::vector<double> real_values_computed = host_doubles(real_msg_dec, N);
-    precision_bits(real_values_computed, plain_gemm_host, worst, mean);
+    precision_bits(real_values_computed, plain_gemm_host, worst, mean, true);      // the table the reference prints (:195-196)
     printf("repacking decrypt vs plain gemm: worst %.1f bits, mean %.1f bits (scale 2^%.1f)\n", worst, mean, (double)std::log2((double)c2.scale));
     double biggest = 0;
     for (double v : plain_gemm_host) biggest = std::max(biggest, std::fabs(v));

@@ -50,3 +50,14 @@ def crt(residues, primes):
         Mi = M // p
         x += int(r) * Mi * pow(Mi, -1, p)
     return x % M, M
+
+
+def precision_table(got, want, label, min_bits, median_bits):
+    """The reference states the agreement of a decrypted result with its plaintext model as GetPrecisionStats' table of
+    log2(1 / |difference|) (precision.cuh:104-249; test programs print it).  Prints that table and asserts on its worst and median row."""
+    from ckks_llm_amd.precision import GetPrecisionStats
+    stats = GetPrecisionStats(np.asarray(got, dtype=np.float64).reshape(-1), np.asarray(want, dtype=np.float64).reshape(-1))
+    print("%s: precision in bits (log2 of 1 / |decrypted - plain product|)%s" % (label, stats.String()))
+    assert stats.MinPrecision.Real >= min_bits, (label, "worst coefficient", stats.MinPrecision.Real, "bits, wanted", min_bits)
+    assert stats.MedianPrecision.Real >= median_bits, (label, "median", stats.MedianPrecision.Real, "bits, wanted", median_bits)
+    return stats

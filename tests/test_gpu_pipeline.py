@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from ckks_llm_amd import Context_23, DeviceBuffer, PCMM_Context, PCMM_Scheme
-from tests.helpers import negacyclic_mul
+from tests.helpers import negacyclic_mul, precision_table
 from tests.params import CFG2_Q, CFG3_P
 
 pytestmark = pytest.mark.gpu
@@ -150,7 +150,7 @@ def test_bert_base_layer_on_encrypted_activations(activations):
     out_scale = x_scale * scaler / Q1
     embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
     dec, d_vals = Plaintext(N, L, 0, N // 2, 1), DeviceBuffer(8 * N)
-    worst = []
+    decrypted = np.zeros_like(want)
     for j in range(3):
         res = Ciphertext(N, L, 0, N // 2, out_scale)
         res.cipher_device.zero()
@@ -159,11 +159,11 @@ def test_bert_base_layer_on_encrypted_activations(activations):
         scheme.decryptMsg(dec, sk, res)
         ctx.decode_coeffs(dec, d_vals)
         got = d_vals.download(np.float64).reshape(tokens, k)                # coefficient n * k + 2 m = Y[n][256 j + m]
-        err = np.abs(got[:, 0:512:2] - want[:, 256 * j: 256 * (j + 1)])
-        worst.append(err.max())
+        decrypted[:, 256 * j: 256 * (j + 1)] = got[:, 0:512:2]
         assert np.abs(got[:, 1:512:2]).max() < 2.0 ** -9                    # the positions between the packed samples hold noise only
-        assert np.median(err) < 2.0 ** -13
-    assert np.abs(want).max() > 1.0 and max(worst) < 2.0 ** -10, worst
+    assert np.abs(want).max() > 1.0
+    # output scale 2^26: the floor is the repacking noise over that scale
+    precision_table(decrypted, want, "BERT-base 768 x 768 layer, %s activations" % activations, min_bits=12, median_bits=15)
 
 
 def test_layer_on_the_references_own_parameter_set():
@@ -213,7 +213,7 @@ def test_layer_on_the_references_own_parameter_set():
     out_scale = x_scale * scaler / q_rp[1]
     embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
     dec, d_vals = Plaintext(N, L, 0, N // 2, 1), DeviceBuffer(8 * N)
-    worst = []
+    decrypted = np.zeros_like(want)
     for j in range(3):
         res = Ciphertext(N, L, 0, N // 2, out_scale)
         res.cipher_device.zero()
@@ -222,10 +222,9 @@ def test_layer_on_the_references_own_parameter_set():
         scheme.decryptMsg(dec, sk, res)
         ctx.decode_coeffs(dec, d_vals)
         got = d_vals.download(np.float64).reshape(tokens, k)
-        err = np.abs(got[:, 0:512:2] - want[:, 256 * j: 256 * (j + 1)])
-        worst.append(err.max())
-        assert np.median(err) < 2.0 ** -20
-    assert np.abs(want).max() > 0.05 and np.abs(want).max() < 0.4 and max(worst) < 2.0 ** -16, worst
+        decrypted[:, 256 * j: 256 * (j + 1)] = got[:, 0:512:2]
+    assert np.abs(want).max() > 0.05 and np.abs(want).max() < 0.4
+    precision_table(decrypted, want, "768 x 768 layer on the reference's logN = 16 set, precision 2^49", min_bits=33, median_bits=36)
 
 
 def test_bert_mirror_layers_with_loaded_weights(tmp_path):
@@ -282,12 +281,69 @@ def test_bert_mirror_layers_with_loaded_weights(tmp_path):
     Y = X @ tensors[pre + "attention.self.query.weight"].astype(np.float64).T
     ins = [encrypt_part(X, 0, 512, 512), encrypt_part(X, 512, 256, 512)]
     outs = [Ciphertext(N, L, 0, N // 2, 1) for _ in range(3)]
-    bert.PCMM_768_768(w.attention_self_query_weight[0], ins, outs, 0)
+    bert.PCMM_Boot_768_768(w.attention_self_query_weight[0], ins, outs, L, 0)          # the reference's signature (Bert.h:62)
     assert max(worst_error(outs[j], Y, 256 * j, 256) for j in range(3)) < 2.0 ** -10
     X = rng.normal(0, 0.6, (N1, 3072))
     Y = X @ tensors[pre + "output.dense.weight"].astype(np.float64).T
     O = [None] * 12
     for i in range(6):
         O[2 * i] = encrypt_part(X, 512 * i, 512, 512)
-    bert.layer_output(O, 0)
+    bert.layer_output(O, 0, [])                                                         # Bert.h:61; layer_res is not touched
     assert O[0].l == 0 and max(worst_error(O[0], Y, 0, 512), worst_error(O[2], Y, 512, 256)) < 2.0 ** -10
+
+
+def test_llm_projection_4096_on_encrypted_activations():
+    """BASELINE config 5 from encryption to decryption: 128 tokens x 4096 activations ~ N(0, 1) in eight RLWE ciphertexts of 512 samples
+    at N = 2^16 (ternary secret of weight 192, Gaussian error 3.2, public-key encryption), times W 4096 x 4096 ~ N(0, 0.02) quantised at
+    2^26 (three balanced int8 digits against five residue digits on the matrix cores), the 4096 product rows ring-packed into sixteen
+    ciphertexts of 256 features, decrypted, decoded and compared with the plain fp64 product in the reference's unit.  Ring-pack moduli
+    [p0 | q0, q1], the shape the reference's packing supports."""
+    from ckks_llm_amd import Ciphertext, MLWESecretKey, Plaintext, Scheme_23, SecretKey
+    logN, N1 = 16, 128
+    P0, Q0, Q1 = CFG3_P[0], CFG2_Q[0], CFG2_Q[1]
+    ctx = Context_23(logN, [P0], [Q0, Q1])
+    N, L = ctx.N, ctx.L
+    k = N // N1
+    key = bytes(range(5, 37))
+    scheme = Scheme_23(ctx, key=key)
+    sk = SecretKey(ctx, h=192, key=key, nonce=1)
+    pc = PCMM_Context(N1, k, [P0], [Q0, Q1], ctx)
+    ps = PCMM_Scheme(pc, key=key)
+    mlwe_sk = MLWESecretKey(N1, pc.ringpack_pq_count - 1, k)
+    ps.convertMLWESKfromRLWESK(mlwe_sk, sk)
+    scheme.addEncKey(sk)
+    ps.addRepakcingKey(mlwe_sk, sk)
+    rng = np.random.default_rng(4096)
+    tokens, feat = N1, 4096
+    X = rng.normal(0, 1, (tokens, feat))
+    W = rng.normal(0, 0.02, (feat, feat)).astype(np.float32)
+    want = X @ W.astype(np.float64).T                                      # [token][output feature]
+    x_scale = 1 << 36
+    C = (k + 1) * N1
+    scaler = float(1 << 26)
+    ps.packed_begin(feat, 2)
+    for i in range(feat // 512):
+        msg = Plaintext(N, L, L, N // 2, x_scale)
+        ctx.encode_coeffs(DeviceBuffer.from_numpy(np.ascontiguousarray(X[:, 512 * i: 512 * (i + 1)]).reshape(-1)), msg)   # coefficient n * k + m = X[n][512 i + m]
+        ct = Ciphertext(N, L, L, N // 2, x_scale)
+        scheme.encryptMsg(ct, msg)
+        ps.rlweCipherDecompose_packed(ct.cipher_device, 512, 512 * i, 1)
+    out = DeviceBuffer(8 * feat * 2 * C)
+    ps.PPMM_packed(DeviceBuffer.from_numpy(W), out, feat, scaler)
+    assert pc.info("last_path") == 1 and pc.info("last_DW") == 3 and pc.info("last_DC") == 5
+    rows = [out.ptr + 8 * m * 2 * C for m in range(feat)]                   # row m, first modulus (PPMM_kernel.cuh:345-348)
+    out_scale = x_scale * scaler / Q1
+    embed, mult = DeviceBuffer(8 * (k + 1) * 2 * N), DeviceBuffer(8 * 4 * N)
+    dec, d_vals = Plaintext(N, L, 0, N // 2, 1), DeviceBuffer(8 * N)
+    decrypted = np.zeros_like(want)
+    res = Ciphertext(N, L, 0, N // 2, out_scale)
+    for j in range(feat // 256):
+        res.cipher_device.zero()
+        ps.mlweCipherPacking(res.cipher_device, rows[256 * j: 256 * (j + 1)], 256, 0, ps.repackingKeys, embed, mult)
+        res.l, res.scale = 0, out_scale
+        scheme.decryptMsg(dec, sk, res)
+        ctx.decode_coeffs(dec, d_vals)
+        got = d_vals.download(np.float64).reshape(tokens, k)                # coefficient n * k + 2 m = Y[n][256 j + m]
+        decrypted[:, 256 * j: 256 * (j + 1)] = got[:, 0:512:2]
+    assert np.abs(want).max() > 4.0
+    precision_table(decrypted, want, "Llama-7B-shaped projection 4096 x 4096", min_bits=12, median_bits=15)
