@@ -25,12 +25,47 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes moved by ONE forward row-pass launch of the default workload (1536 limbs), from the rocprofv3 counters FETCH_SIZE
-# and WRITE_SIZE of that launch, each scaled by what the same counter reads for a device-to-device copy of known size in the
-# same run (FETCH_SIZE reads 0.500 of the bytes copied, WRITE_SIZE 1.000): 480 MiB of 5-byte inter-pass values + 12 MiB of
-# twiddles read, 768 MiB written.  (The strided pass of the same transform moves 1.309e9: 768 MiB read, 480 MiB written.)
-NTT_PASS_TRAFFIC_BYTES_1536_LIMBS = 1.321e9
 MFMA_I8_PEAK_TMACS = 2516.6          # 5.033 POP/s dense int8 = 2.5166e15 MAC/s
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_per_call.txt")
+
+
+def kernel_sources_id():
+    """Short hash of the HIP sources: the traffic figures below are only quoted for the kernels they were measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "ckks_llm_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".hip", ".hpp")):
+            with open(os.path.join(src, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic():
+    """HBM bytes per call, from rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE, each scaled by what the same counter reads for a
+    device-to-device copy of known size in the same run) summarised in profiles/hbm_traffic_per_call.txt.  The file names the
+    kernel sources it was measured on; for other sources (or without the file) nothing is quoted."""
+    out = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            lines = f.read().splitlines()
+    except OSError:
+        return out, "no traffic summary"
+    measured_on = None
+    for ln in lines:
+        ln = ln.strip()
+        if ln.startswith("kernel_sources_id"):
+            measured_on = ln.split()[1]
+        elif ln and not ln.startswith("#"):
+            parts = ln.split()
+            if len(parts) >= 2:
+                try:
+                    out[parts[0]] = float(parts[1])
+                except ValueError:
+                    pass
+    if measured_on != kernel_sources_id():
+        return {}, "traffic summary is for kernel sources %s, these are %s: not quoted" % (measured_on, kernel_sources_id())
+    return out, "profiles/hbm_traffic_per_call.txt (kernel sources %s)" % measured_on
 
 
 def uniform_limbs(seed, primes, polys, N):
@@ -84,8 +119,10 @@ def bench_ntt(args, P):
     alg_bytes_launch = 16.0 * N * limbs / 2.0          # half a transform per launch
     dom_name, dom_ms = max([("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2)], key=lambda x: x[1])
     achieved = alg_bytes_launch / (dom_ms * 1e-3) / 1e9
+    traffic, traffic_note = measured_traffic()
+    key = "ntt_strided_pass_fwd_1536_limbs" if dom_name.startswith("ntt_strided") else "ntt_row_pass_fwd_1536_limbs"
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": NTT_PASS_TRAFFIC_BYTES_1536_LIMBS if limbs == 1536 else None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic.get(key) if limbs == 1536 else None, "traffic_source": traffic_note,
                 "kernel_ms": {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)},
                 "transform_algorithmic_GBps": {"fwd": round(16.0 * N * limbs / ((f1 + f2) * 1e-3) / 1e9, 1),
                                                "inv": round(16.0 * N * limbs / ((i1 + i2) * 1e-3) / 1e9, 1)},
@@ -176,11 +213,16 @@ def main():
     if not args.skip_extra:
         try:
             import bench_extra
-            line.update(bench_extra.run(P))
+            line.update(bench_extra.run(P, measured_traffic()))
         except ImportError:
             pass
     if not args.skip_cpu:
         line["cpu_baseline"] = bench_cpu_baseline(P)
+        if not args.skip_extra:
+            # the CPU oracle beside the other GPU figures of the line (bounded samples, a few seconds each)
+            import bench_extra
+            line["ppmm"]["cpu_baseline"] = bench_extra.cpu_ppmm(P)
+            line["keyswitch"]["cpu_baseline"] = bench_extra.cpu_keyswitch(P)
     print(json.dumps(line))
 
 

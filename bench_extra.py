@@ -42,7 +42,8 @@ def bench_ppmm(P, M=768, Kin=768, N1=128, L=12, reps=3, primes=None, label=None,
     DW, DC, path = sch.pcmm_context.info("last_DW"), sch.pcmm_context.info("last_DC"), sch.pcmm_context.info("last_path")
     word_macs = float(M) * Kin * C * L
     macs = word_macs * DW * DC
-    res = {"workload": label or "configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns" % (3 if M == 768 else 4, M, Kin, N1, L, C),
+    res = {"workload": label or ("configs[%d]: PPMM %dx%d, %d tokens (N1), N=2^16, %d primes <2^36, C=%d columns; the product alone - the ring packing behind it exists "
+                                "for two ring-pack moduli only (the reference's shape), so no packing stage follows this %d-prime product") % (3 if M == 768 else 4, M, Kin, N1, L, C, L),
            "ms": round(best, 3), "word_MAC_per_s": round(word_macs / (best * 1e-3), 1), "int8_MAC_per_s": round(macs / (best * 1e-3), 1),
            "D_w": DW, "D_c": DC, "plaintext_slices": sch.pcmm_context.info("last_slices"), "kernel": "int8 MFMA" if path == 1 else "generic u128",
            "roofline": {"bound": "mfma", "achieved": round(macs / (best * 1e-3) / 1e12, 2), "peak": round(MFMA_I8_PEAK_MACS / 1e12, 1),
@@ -307,10 +308,111 @@ def bench_hoisted_level(P, gs=16, bs=4, reps=3):
                          "frac": round(nbytes / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": nbytes}}
 
 
-def run(P):
+def cpu_ppmm(P, M=768, Kin=768, N1=128, L=12, seconds_target=8.0):
+    """The CPU oracle's PPMM (the reference's 128-bit accumulation, OpenMP over rows) at the configs[3] shape on a panel of the
+    C = 65,664 columns, sized to a few seconds and scaled to the whole product (every column costs the same)."""
+    import time
+    from oracle import oracle_py as O
+    primes = P.CFG2_Q[:L]
+    rank = (1 << 16) // N1
+    C = (rank + 1) * N1
+    octx = O.OracleContext(16, [], primes)
+    orc = O.OraclePCMM(octx, N1, rank, [], primes)
+    rng = np.random.default_rng(4)
+    W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+    rng5 = np.random.default_rng(5)
+    seeds = []
+    for s in range(16):
+        a = np.empty((L, C), dtype=np.uint64)
+        for j, q in enumerate(primes):
+            a[j] = rng5.integers(0, q, C, dtype=np.uint64)
+        seeds.append(a.reshape(-1))
+    mlwe = [seeds[n % 16] for n in range(Kin)]
+    out = np.zeros(M * L * C, dtype=np.uint64)
+    cols = 64
+    orc.PPMM(W, mlwe, out, M, Kin, L, float(2 ** 26), 0, cols)          # untimed: first touch of the output pages, thread start
+    t0 = time.perf_counter()
+    orc.PPMM(W, mlwe, out, M, Kin, L, float(2 ** 26), 0, cols)
+    once = time.perf_counter() - t0
+    cols = int(min(C, max(64, cols * seconds_target / max(once, 1e-3)))) // 64 * 64
+    t0 = time.perf_counter()
+    orc.PPMM(W, mlwe, out, M, Kin, L, float(2 ** 26), 0, cols)
+    dt = time.perf_counter() - t0
+    word_macs = float(M) * Kin * cols * L
+    return {"value": round(word_macs / dt, 1), "unit": "word_MAC_per_s", "cores": O.lib().orc_max_threads(), "kind": "port",
+            "ms_whole_product_extrapolated": round(dt * C / cols * 1e3, 1),
+            "sample": "oracle PPMM %dx%d, %d primes, columns 0..%d of %d (%.1f s), scaled by %d / %d to the whole product" % (M, Kin, L, cols - 1, C, dt, C, cols)}
+
+
+def cpu_keyswitch(P, seconds_target=8.0):
+    """The CPU oracle's hybrid key switch at the configs[2] shape (whole size), repeated for a few seconds."""
+    import time
+    from oracle import oracle_py as O
+    q, p = P.CFG2_Q, P.CFG3_P
+    octx = O.OracleContext(16, p, q)
+    N, Wd, nq, l, dn = 1 << 16, 30, 24, 23, 4
+    rng = np.random.default_rng(3)
+    evk = np.empty((2 * dn, Wd, N), dtype=np.uint64)
+    for j, m in enumerate(p + q):
+        evk[:, j, :] = rng.integers(0, m, size=(2 * dn, N), dtype=np.uint64)
+    inp = np.empty((nq, N), dtype=np.uint64)
+    for j, m in enumerate(q):
+        inp[j] = rng.integers(0, m, N, dtype=np.uint64)
+    out = np.zeros(2 * nq * N, dtype=np.uint64)
+    t0 = time.perf_counter()
+    octx.hybrid_keyswitch(out, inp.reshape(-1), evk.reshape(-1), l)
+    once = time.perf_counter() - t0
+    reps = max(1, min(50, int(seconds_target / max(once, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        octx.hybrid_keyswitch(out, inp.reshape(-1), evk.reshape(-1), l)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(1.0 / dt, 2), "unit": "keyswitch_per_s", "ms": round(dt * 1e3, 1), "cores": O.lib().orc_max_threads(), "kind": "port",
+            "sample": "%d x oracle hybrid key switch, N=2^16, 24 Q + 6 P primes, dnum=4 (whole size)" % reps}
+
+
+def with_traffic(entry, key, traffic, seconds):
+    """Beside the fraction on the stage sum (what the reference's unfused stages would move), the fraction on the bytes the
+    fused launches really move (rocprofv3 counters, summed over the call's launches)."""
+    moved = traffic.get(key)
+    r = entry["roofline"]
+    r["achieved_is"] = "stage-sum bytes of the reference's unfused stages / time"
+    r["traffic"] = moved
+    if moved:
+        r["traffic_GBps"] = round(moved / seconds / 1e9, 1)
+        r["traffic_frac"] = round(moved / seconds / HBM_PEAK, 4)
+    return entry
+
+
+def run(P, traffic_info=({}, "")):
+    traffic, note = traffic_info
     ref_label = "PPMM 768x768 on the reference's own two 49-bit ring-pack moduli (Params.cuh, logN = 16), N=2^16, 128 tokens, plaintext scaled by 2^26"
     ref_scale_label = ("PPMM 768x768 as the reference's BERT layer calls it: its two 49-bit ring-pack moduli and its scaler q1 * 2^49 / scale "
                        "with scale = 2^49 (PPMM_kernel.cuh:283-284), i.e. 46-bit plaintext entries, N=2^16, 128 tokens")
-    return {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label),
+    res = {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label),
             "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "mult_23_ref_params": bench_mult_23(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}
+    with_traffic(res["keyswitch"], "hybrid_keyswitch_config3", traffic, res["keyswitch"]["us"] * 1e-6)
+    with_traffic(res["rescale"], "rescale_one_ciphertext_level23", traffic, res["rescale"]["us"] * 1e-6)
+    with_traffic(res["mult_23_ref_params"], "mult_23_ref_params_level27", traffic, res["mult_23_ref_params"]["ms"] * 1e-3)
+    with_traffic(res["decompose"], "rlwe_decompose_512_samples", traffic, res["decompose"]["ms"] * 1e-3)
+    with_traffic(res["packing"], "mlwe_packing_512_samples", traffic, res["packing"]["ms"] * 1e-3)
+    with_traffic(res["hoisted_level"], "giant_rotate_gs16_bs4", traffic, res["hoisted_level"]["ms"] * 1e-3)
+    res["traffic_source"] = note
+    return res
+
+
+LEGS = {"ppmm": lambda P: bench_ppmm(P), "ppmm_4096": lambda P: bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused,
+        "keyswitch": bench_keyswitch, "rescale": bench_rescale, "mult_23_ref_params": bench_mult_23, "decompose": bench_decompose,
+        "packing": bench_packing, "hoisted_level": bench_hoisted_level, "cpu_ppmm": cpu_ppmm, "cpu_keyswitch": cpu_keyswitch}
+
+if __name__ == "__main__":
+    # one leg on its own, for profiling:  python3 bench_extra.py keyswitch
+    import json
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import ckks_llm_amd.params as params
+    if len(sys.argv) != 2 or sys.argv[1] not in LEGS:
+        sys.exit("usage: bench_extra.py <%s>" % " | ".join(LEGS))
+    print(json.dumps(LEGS[sys.argv[1]](params)))
