@@ -101,6 +101,43 @@ def bench_rescale(P, reps=20):
                          "frac": round(alg / (ms * 1e-3) / HBM_PEAK, 4), "algorithmic_bytes": alg}}
 
 
+def bench_ntt_ref_primes(P, cts=27, reps=10):
+    """The headline transform on the reference's own logN = 16 moduli: its 28 Q primes of 49 bits (Params.cuh:88-171), a batch of 27
+    ciphertexts (1512 limbs, 756 MiB).  These primes take the FP64 back end that balances after every register round, with the data
+    in place between the two launches (8-byte words; the 5-byte form is for primes below 2^39); the integer back end is timed beside it."""
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    primes = list(P.REF_PARAMS[16]["q"])
+    N, L1, polys = 1 << 16, len(primes), 2 * cts
+    limbs = polys * L1
+    ctx = Context_23(16, [], primes)
+    rng = np.random.default_rng(12)
+    one = np.empty((2, L1, N), dtype=np.uint64)
+    for j, q in enumerate(primes):
+        one[:, j] = rng.integers(0, q, (2, N), dtype=np.uint64)
+    buf = DeviceBuffer(8 * limbs * N)
+    for c in range(cts):
+        buf.L_.ckks_memcpy_h2d(buf.ptr + c * one.nbytes, one.ctypes.data, one.nbytes)
+    res = {"workload": "RNS NTT+iNTT, N=2^16, the reference's 28 Q primes of 49 bits, batch of %d ciphertexts (%d limbs, %d MiB) per step" % (cts, limbs, limbs * 8 * N >> 20)}
+    for name, mode in (("fp64_balanced", 0), ("integer", 1)):
+        ctx.set_arith_mode(mode)
+        for _ in range(3):
+            ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+            ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+        ctx.timer_start()
+        for _ in range(reps):
+            ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+            ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+        ms = ctx.timer_stop() / reps
+        rate = 2 * limbs / (ms * 1e-3)
+        res[name] = {"ms_per_step": round(ms, 4), "limb_transforms_per_s": round(rate, 1),
+                     "frac_of_hbm_roofline_whole_transform": round(rate * 16 * N / HBM_PEAK, 4)}
+    back = buf.download(np.uint64, one.size).reshape(one.shape)
+    assert np.array_equal(back, one), "NTT round trip changed the data"
+    ctx.set_arith_mode(0)
+    buf.free()
+    return res
+
+
 def bench_mult_23(P, reps=10):
     """Scheme_23::mult_23 (KeySwitch_23.cuh:192-236) on the reference's own logN = 16 parameter set at the top level: tensor product,
     key switch through the T basis with a relinearisation key generated on the device, the two additions."""
@@ -390,7 +427,7 @@ def run(P, traffic_info=({}, "")):
     ref_scale_label = ("PPMM 768x768 as the reference's BERT layer calls it: its two 49-bit ring-pack moduli and its scaler q1 * 2^49 / scale "
                        "with scale = 2^49 (PPMM_kernel.cuh:283-284), i.e. 46-bit plaintext entries, N=2^16, 128 tokens")
     res = {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label),
-            "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "mult_23_ref_params": bench_mult_23(P),
+            "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "ntt_ref_primes": bench_ntt_ref_primes(P), "mult_23_ref_params": bench_mult_23(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}
     with_traffic(res["keyswitch"], "hybrid_keyswitch_config3", traffic, res["keyswitch"]["us"] * 1e-6)
     with_traffic(res["rescale"], "rescale_one_ciphertext_level23", traffic, res["rescale"]["us"] * 1e-6)
@@ -403,7 +440,7 @@ def run(P, traffic_info=({}, "")):
 
 
 LEGS = {"ppmm": lambda P: bench_ppmm(P), "ppmm_4096": lambda P: bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused,
-        "keyswitch": bench_keyswitch, "rescale": bench_rescale, "mult_23_ref_params": bench_mult_23, "decompose": bench_decompose,
+        "keyswitch": bench_keyswitch, "rescale": bench_rescale, "ntt_ref_primes": bench_ntt_ref_primes, "mult_23_ref_params": bench_mult_23, "decompose": bench_decompose,
         "packing": bench_packing, "hoisted_level": bench_hoisted_level, "cpu_ppmm": cpu_ppmm, "cpu_keyswitch": cpu_keyswitch}
 
 if __name__ == "__main__":

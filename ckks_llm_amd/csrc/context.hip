@@ -151,7 +151,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         for (long k = 0; k < N; k++) {
             twf[(size_t)i * N + k] = make_ulonglong2(pt[k], H::shoup(pt[k], m));
             twi[(size_t)i * N + k] = make_ulonglong2(it[k], H::shoup(it[k], m));
-            if (c->f64_ok[i]) {
+            if (m < (1ull << 50)) {                                            // FP64 back ends: below 2^41, and the wide one below 2^50
                 twdf[(size_t)i * N + k] = balanced_double(pt[k], m);
                 twdi[(size_t)i * N + k] = balanced_double(it[k], m);
             }

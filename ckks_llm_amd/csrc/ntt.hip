@@ -52,6 +52,7 @@ struct IntArith {
     __device__ __forceinline__ u64 enc40_raw(V x) const { return x; }
     __device__ __forceinline__ V dec40(unsigned lo, unsigned) const { return lo; }
     __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return csub(csub(x, q2), q); }
+    template <int R> __device__ __forceinline__ void round_end(V (&)[R]) const {}          // lazy ranges hold for a whole pass
     // Harvey lazy butterflies; ranges as ntt_60bit.cuh:293-318
     __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
         x = x >= q2 ? x - q2 : x;
@@ -110,6 +111,7 @@ struct F64Arith {
         return __longlong_as_double((long long)(0x4330000000000000ull | ((u64)hi8 << 32) | lo)) - 4504149383184384.0;
     }
     __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon_any(x); }
+    template <int R> __device__ __forceinline__ void round_end(V (&)[R]) const {}          // q < 2^41: the ranges hold for a whole pass
     __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
         double t = mulmod(y, w);
         y = x - t;
@@ -124,6 +126,39 @@ struct F64Arith {
         double s = x + y, d = x - y;
         ox = canon_any(mulmod(s, n_inv));
         oy = canon_any(mulmod(d, w1n));
+    }
+};
+
+// FP64 back end for primes up to 2^50 (the reference's own 49-bit Q and P primes, Params.cuh:84-171).  Same exact-integer
+// arithmetic as F64Arith; what changes is how far a value may drift from zero before it is brought back, because every
+// integer involved must stay below 2^53 and the quotient estimate of mulmod loses accuracy as its operand grows:
+//   mulmod(y, w), |w| <= q/2, |y| <= b q: the estimate rint(fl(fl(y w) fl(1/q))) is off by at most 0.5 + 3 * 2^-53 * b q / 2
+//   < 0.5 + 0.19 b, so the result lies within (0.5 + 0.19 b) q of zero and h - c q, an integer below 2^53, is exact.
+//   forward (x +- t): from |x| <= q/2 four stages reach 1.2, 1.9, 2.8, 3.8 q; inverse (sums double): from q/2 four stages
+//   reach 8 q < 2^53.  So every value is balanced to (-q/2, q/2] when it is loaded, after each register round of at most four
+//   stages (round_end) and before it is stored between the passes; the last stage of an inverse transform multiplies sums
+//   of at most 8 q (results within 2 q of zero) and canonicalises by a balance and one conditional addition.
+struct F64WideArith : F64Arith {
+    double half;
+    __device__ __forceinline__ F64WideArith(const PrimeConst& pc) : F64Arith(pc), half(0.5 * pc.qd) {}
+    __device__ __forceinline__ V from_canonical(u64 x) const {
+        const double d = F64Arith::from_canonical(x);
+        return d > half ? d - q : d;
+    }
+    __device__ __forceinline__ u64 canon_wide(V x) const {            // any integer |x| < 2^53 -> [0, q)
+        const double r = balance(x);                                   // within (q + 1) / 2 of zero
+        return bits52(r < 0.0 ? r + q : r);
+    }
+    __device__ __forceinline__ u64 to_mid_fwd(V x) const { return (u64)__double_as_longlong(balance(x)); }
+    __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon_wide(x); }
+    template <int R> __device__ __forceinline__ void round_end(V (&v)[R]) const {
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = balance(v[j]);
+    }
+    __device__ __forceinline__ void gs_last(V& x, V& y, u64& ox, u64& oy) const {
+        double s = x + y, d = x - y;
+        ox = canon_wide(mulmod(s, n_inv));
+        oy = canon_wide(mulmod(d, w1n));
     }
 };
 
@@ -381,6 +416,7 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
             for (int j = 0; j < R; j++) v[j] = ar.from_canonical(load_word<COHERENT>(col + (long)(g + j * G) * N2));
         }
         fwd_spread<AR, SA, S1>(v, tw, 1u, ar);
+        ar.round_end(v);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
         __syncthreads();
@@ -405,6 +441,7 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
             for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(col + (long)(g * R + j) * N2));
         }
         inv_packed<AR, SA, S1>(v, tw, 1u, g, ar);
+        ar.round_end(v);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[(g * R + j) * CW + cl] = v[j];
         __syncthreads();
@@ -472,6 +509,7 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
             for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(rp + u + j * U));
         }
         fwd_spread<AR, SB, S1>(v, tw, tw_off, ar);
+        ar.round_end(v);
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];
         __syncthreads();
@@ -492,6 +530,7 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
         inv_packed<AR, SB, S1>(v, tw, tw_off, u, ar);
+        ar.round_end(v);
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
@@ -1447,10 +1486,33 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
     }
     long limbs = (long)poly_num * mod_num * batch;
     if (limbs > 65535) { set_error("NTT: more than 65535 limbs in one call"); return CKKS_E_INVALID; }
-    bool f64 = c->arith_mode == 0, compact_ok = true;
+    // back end per prime: 0 = FP64 (q < 2^41), 1 = FP64 with a balance per register round (q < 2^50), 2 = integer
+    auto klass = [&](int j) {
+        if (c->arith_mode != 0) return 2;
+        const u64 m = c->pqt[start_mod_idx + j];
+        return m < (1ull << 41) ? 0 : m < (1ull << 50) ? 1 : 2;
+    };
+    int back_end = klass(0);
+    bool mixed = false, compact_ok = true;
     for (int j = 0; j < mod_num; j++) {
-        f64 = f64 && c->f64_ok[start_mod_idx + j] != 0;
+        mixed = mixed || klass(j) != back_end;
         compact_ok = compact_ok && c->pqt[start_mod_idx + j] < (1ull << 39);
+    }
+    if (mixed) {
+        // a call that spans prime widths ([P | Q | T] of the reference's sets: 49-bit P and Q, 60-bit T) goes out as one launch
+        // sequence per run of primes of one back end; the timing hook and the gathering first pass take one back end for all
+        if (c->ev_mid_armed || src) back_end = 2;
+        else {
+            for (int j0 = 0; j0 < mod_num;) {
+                int j1 = j0 + 1;
+                while (j1 < mod_num && klass(j1) == klass(j0)) j1++;
+                const int rc = launch_ntt_from(c, dev, start_poly_idx + j0, start_mod_idx + j0, poly_num, j1 - j0, poly_mod_len, batch_stride_limbs,
+                                               batch, inverse, nullptr);
+                if (rc) return rc;
+                j0 = j1;
+            }
+            return CKKS_OK;
+        }
     }
     NttArgs args;
     args.data = (u64*)dev;
@@ -1467,9 +1529,13 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
         args.embed_logk = src->logk; args.embed_loggap = src->loggap; args.embed_n1 = src->n1;
         args.embed_no_wrap = src->q0 / 2 < src->p0 ? 1 : 0;
     }
-    if (f64) {
+    if (back_end == 0) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
         return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok);
+    }
+    if (back_end == 1) {
+        args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
+        return dispatch_logn<F64WideArith>(c, args, (int)limbs, inverse, false);
     }
     args.tw = inverse ? (const void*)c->d_tw_inv : (const void*)c->d_tw_fwd;
     return dispatch_logn<IntArith>(c, args, (int)limbs, inverse, false);

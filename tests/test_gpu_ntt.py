@@ -54,14 +54,56 @@ def test_config2_one_ciphertext_n65536_24primes():
 
 
 def test_n65536_integer_backend_and_large_primes():
-    """50-bit q/p and 60-bit t primes of the reference's logN = 16 set (Params.cuh:88-171) use the integer back end."""
+    """The reference's logN = 16 set (Params.cuh:88-171): its 49-bit q and p primes take the FP64 back end that balances after every
+    register round, its 60-bit t primes the integer back end; a call over [p | q | t] goes out as one launch sequence per run of
+    primes of one back end.  Both arithmetic modes against the oracle."""
     P = REF_PARAMS[16]
     p, q, t = P["p"][:1], P["q"][:2], P["t"][:2]
     pair = Pair(16, p, q, t, gamma=2)
-    check_fwd_inv(pair, 0, p + q + t, 1, seed=3)
+    for mode in (0, 1):
+        check_fwd_inv(pair, 0, p + q + t, 1, seed=3, mode=mode)
+        check_fwd_inv(pair, 0, p + q, 2, seed=5, mode=mode)
     # 36-bit primes through the integer back end as well
     pair2 = Pair(16, [], CFG2_Q[:2])
     check_fwd_inv(pair2, 0, CFG2_Q[:2], 2, seed=4, mode=1)
+
+
+@pytest.mark.parametrize("logN", [8, 11, 12, 14, 15, 16])
+def test_wide_fp64_backend_at_its_range_ends(logN):
+    """FP64 butterflies for primes of 41 to 50 bits: the two largest NTT-friendly primes below 2^50 (every bound of the range analysis
+    is tightest there), a 49-bit prime of the reference and the smallest prime the back end takes (just above 2^41), on uniform residues
+    and on the inputs that drive every butterfly to the ends of its range: all q - 1, alternating 0 / q - 1, alternating 1 / q - 1 in
+    blocks, all against the oracle in both directions."""
+    from ckks_llm_amd.params import small_primes
+    top = small_primes(50, 1 << 17, 2)
+    low = small_primes(42, 1 << 17, 1)
+    assert all((1 << 49) < m < (1 << 50) for m in top) and (1 << 41) <= low[0] < (1 << 42)
+    primes = top + [REF_PARAMS[16]["q"][0]] + low
+    pair = Pair(logN, [], primes)
+    pair.dev.set_arith_mode(0)
+    N = pair.N
+    check_fwd_inv(pair, 0, primes, 2, seed=40 + logN, mode=0)
+    pats = []
+    for kind in range(4):
+        d = np.empty((1, len(primes), N), dtype=np.uint64)
+        for j, m in enumerate(primes):
+            if kind == 0:
+                d[0, j] = m - 1
+            elif kind == 1:
+                d[0, j] = np.where(np.arange(N) % 2 == 0, 0, m - 1)
+            elif kind == 2:
+                d[0, j] = np.where((np.arange(N) // 16) % 2 == 0, 1, m - 1)
+            else:
+                d[0, j] = np.where(np.arange(N) % 3 == 0, m // 2, m // 2 + 1)
+        pats.append(d)
+    for d in pats:
+        for inverse in (False, True):
+            want = d.copy()
+            (pair.orc.FromNTTInplace if inverse else pair.orc.ToNTTInplace)(want.reshape(-1), 0, 0, 1, len(primes), len(primes))
+            buf = to_dev(d)
+            (pair.dev.FromNTTInplace if inverse else pair.dev.ToNTTInplace)(buf, 0, 0, 1, len(primes), len(primes))
+            assert np.array_equal(from_dev(buf, d.shape), want), (logN, inverse)
+            buf.free()
 
 
 def test_n65536_inter_pass_formats():
