@@ -207,29 +207,54 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
         bslot_t B_nxt = W == 0 ? lds_b0 : W == 1 ? lds_b1 : reinterpret_cast<bslot_t>(lds_b2);
         // operand reads in the order the MFMAs consume them (LDS reads return in order, so the first MFMA waits for its own two
         // operands only): plaintext chunks of the first 16 rows, residue chunks of the first 16 columns, then the rest
-        v4i bf[2][DC], af[2][DW];
+        if constexpr (DC > 5) {
+            // seven residue digits: 144 accumulator registers leave no room for both column halves' operands at once, so the
+            // residue chunks of one half are read just before its MFMAs (column half outer, row half inner)
+            v4i af[2][DW];
 #pragma unroll
-        for (int d = 0; d < DW; d++) af[0][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32][0] + frag_off);
+            for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
-#pragma unroll
-            for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16][0] + frag_off);
-#pragma unroll
-        for (int d = 0; d < DW; d++) af[1][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + 16][0] + frag_off);
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++)
+                for (int d = 0; d < DW; d++) af[mt][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + mt * 16][0] + frag_off);
 #pragma unroll
             for (int nt = 0; nt < 2; nt++) {
+                v4i bf[DC];
 #pragma unroll
-                for (int jj = 0; jj < DC; jj++)
+                for (int jj = 0; jj < DC; jj++) bf[jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16][0] + frag_off);
 #pragma unroll
-                    for (int d = 0; d < DW; d++)
-                        acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[mt][d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
-                // the refill of slot W (read one step ago, released by the barrier that ended that step) goes out behind the operand
-                // reads and the first quarter of the MFMAs, so that the matrix pipe starts as early as possible in a step; the loads
-                // are opaque assembly, the compiler adds no wait for them
-                if (mt == 0 && nt == 0) issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
+                for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+                    for (int jj = 0; jj < DC; jj++)
+#pragma unroll
+                        for (int d = 0; d < DW; d++)
+                            acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[mt][d], bf[jj], acc[d + jj][mt][nt], 0, 0, 0);
+                    if (mt == 0 && nt == 0) issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
+                }
             }
+        } else {
+            v4i bf[2][DC], af[2][DW];
+    #pragma unroll
+            for (int d = 0; d < DW; d++) af[0][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32][0] + frag_off);
+    #pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+    #pragma unroll
+                for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16][0] + frag_off);
+    #pragma unroll
+            for (int d = 0; d < DW; d++) af[1][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + 16][0] + frag_off);
+    #pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+    #pragma unroll
+                for (int nt = 0; nt < 2; nt++) {
+    #pragma unroll
+                    for (int jj = 0; jj < DC; jj++)
+    #pragma unroll
+                        for (int d = 0; d < DW; d++)
+                            acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[mt][d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
+                    // the refill of slot W (read one step ago, released by the barrier that ended that step) goes out behind the operand
+                    // reads and the first quarter of the MFMAs, so that the matrix pipe starts as early as possible in a step; the loads
+                    // are opaque assembly, the compiler adds no wait for them
+                    if (mt == 0 && nt == 0) issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, A_nxt, B_nxt);
+                }
+        }
         // the loads for step s+1 must have landed: with three slots those were issued one step ago and the ones just issued may
         // stay in flight; with two slots they are the ones just issued
         if (RING == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (A_PER_WAVE + B_PER_WAVE));      // vmcnt(loads of one step)
