@@ -12,6 +12,7 @@
 // Two residue widths are built: DC = 5 digits for q_i < 2^39 (the 36-bit sets of the benchmarks) and DC = 7 digits for
 // q_i < 2^50 (the reference's own 49-bit ring-pack primes), the latter with DW <= 3.
 //
+#include <cstdlib>
 #include <type_traits>
 
 #include "pcmm.hpp"
@@ -116,7 +117,8 @@ __global__ __launch_bounds__(256) void ppmm_pack_kernel(PpmmArgs a, int8_t* __re
 // The other shape that fits the LDS (NWAVES = 4, RING = 2: 64 x 64 tile, 64 KiB, two workgroups per CU that drift out of phase)
 // was measured and is no faster (its single step of load lead time costs what the overlap of the two workgroups gains).
 template <int DW, int NWAVES, int RING, int DC>
-__global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_block) {
+__global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, const int8_t* __restrict__ bdig, int c_tiles, int m_block,
+                                                                   int main_blocks, int tail_jobs) {
     constexpr int ND = DW + DC - 1, MT = 16 * NWAVES;
     constexpr bool WIDE = DC > 5;                                // residues of up to 50 bits: three groups of diagonals, wider r_last
     constexpr int A_SLABS = DW * (MT / 16), B_SLABS = DC * 4;    // 1 KiB slabs per step
@@ -136,11 +138,34 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
     // next m_block row tiles.  All workgroups of a patch advance through K at the same pace, so the L2 only has to hold a window of
     // their plaintext and residue slabs.  (With every row tile in one patch, 32 row tiles at M = 4096 re-read the plaintext digit
     // planes, which no longer fit the L2, for every column panel and prime: 40 times the algorithmic traffic.)
-    const unsigned id = blockIdx.x, xcd = id & 7, j = id >> 3;
-    const unsigned c_per_xcd = ((unsigned)c_tiles + 7) / 8;
-    const unsigned ml = j % m_block, t = j / m_block;
-    const unsigned m_tile = (t / c_per_xcd) * m_block + ml, c_tile = (t % c_per_xcd) * 8 + xcd;
+    //
+    // Tail.  The column panels do not divide among the XCDs in general, and a tile is a long job (all primes): with 1026 panels
+    // and six row tiles, six XCDs would sit idle for a whole round while two finish the last two panels.  With tail_jobs > 0 the
+    // ids from main_blocks on are those panels' tiles cut into tail_jobs jobs each: a job computes the last prime (every other
+    // prime's rescale needs its residues; job 0 stores them) and its share of the other primes, and the jobs spread over all XCDs.
+    const unsigned id = blockIdx.x;
+    unsigned m_tile, c_tile;
+    int prime_lo = 0, prime_hi = a.mod_num - 1;          // the other primes of this workgroup: prime_lo .. prime_hi - 1, after the last one
+    bool store_last = true;
+    if (tail_jobs > 0 && id >= (unsigned)main_blocks) {
+        const unsigned q = id - (unsigned)main_blocks, job = q % (unsigned)tail_jobs, tt = q / (unsigned)tail_jobs;
+        const unsigned m_tiles = (unsigned)a.Mpad / MT;
+        m_tile = tt % m_tiles;
+        c_tile = ((unsigned)c_tiles / 8) * 8 + tt / m_tiles;
+        const int others = a.mod_num - 1;
+        prime_lo = (int)((long)others * job / tail_jobs);
+        prime_hi = (int)((long)others * (job + 1) / tail_jobs);
+        store_last = job == 0;
+    } else {
+        const unsigned xcd = id & 7, j = id >> 3;
+        const unsigned c_per_xcd = tail_jobs > 0 ? (unsigned)c_tiles / 8 : ((unsigned)c_tiles + 7) / 8;
+        const unsigned ml = j % m_block, t = j / m_block;
+        m_tile = (t / c_per_xcd) * m_block + ml;
+        c_tile = (t % c_per_xcd) * 8 + xcd;
+    }
     if (c_tile >= (unsigned)c_tiles) return;
+    const int n_iters = 1 + prime_hi - prime_lo;          // the last prime, then prime_hi - 1 down to prime_lo
+    auto prime_of = [&](int it) { return it == 0 ? a.mod_num - 1 : prime_hi - it; };
     const int m0 = m_tile * MT;
     const unsigned c0 = c_tile * CT;
 
@@ -185,12 +210,14 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
 
     // (ks2, im2): K step and prime of global step s+AHEAD, advanced without divisions; past the end the loads re-fetch valid
     // data into slots nobody reads again, so that a step has no branches.
-    auto advance = [&](int& ks, int& im) { if (++ks == ksteps) { ks = 0; --im; } };
+    // it2 counts this workgroup's primes; im2 = prime of that iteration, or -1 past the end
+    int it2 = 0;
+    auto advance = [&](int& ks, int& im) { if (++ks == ksteps) { ks = 0; ++it2; im = it2 < n_iters ? prime_of(it2) : -1; } };
     int ks2 = 0, im2 = a.mod_num - 1;
     issue(ks2, im2, lds_a0, lds_b0);
     advance(ks2, im2);
     if (RING == 3) {
-        issue(ks2, im2 < 0 ? 0 : im2, lds_a1, lds_b1);
+        issue(im2 < 0 ? 0 : ks2, im2 < 0 ? 0 : im2, lds_a1, lds_b1);
         advance(ks2, im2);
     }
     wait_loads();
@@ -327,7 +354,8 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                         const double res = t[r] < 0.0 ? t[r] + q : t[r];
                         if (LAST) rl_wide[WIDE ? mt : 0][WIDE ? nt : 0][WIDE ? r : 0] = res;
                         const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
-                        if (FULL) orow[r][nt * 16] = ures;
+                        if (LAST && !store_last) {}                           // a tail job other than the first: the residues are only needed in registers
+                        else if (FULL) orow[r][nt * 16] = ures;
                         else if (mrow + mt * 16 + r < a.M) orow[r][nt * 16] = ures;
                     }
                     continue;
@@ -390,14 +418,16 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                         rl_lo[mt][r][nt] = (unsigned)ures;
                         rl_hi[mt][nt] = (r == 0 ? 0u : rl_hi[mt][nt]) | ((unsigned)(ures >> 32) << (8 * r));
                     }
-                    if (FULL) orow[r][nt * 16] = ures;
+                    if (LAST && !store_last) {}
+                    else if (FULL) orow[r][nt * 16] = ures;
                     else if (mrow + mt * 16 + r < a.M) orow[r][nt * 16] = ures;
                 }
             }
         }
     };
 
-    for (int im = a.mod_num - 1; im >= 0; im--) {
+    for (int it = 0; it < n_iters; it++) {
+        const int im = prime_of(it);
         q = a.pq[a.np + im].qd;
         qinv = a.pq[a.np + im].qinv_d;
         c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
@@ -434,8 +464,18 @@ static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool p
     const int m_tiles = a.Mpad / 128;
     int m_block = 1;                                   // row tiles per patch: the largest divisor of m_tiles up to 6
     for (int d = 2; d <= 6; d++) if (m_tiles % d == 0) m_block = d;
-    const unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
-    hipLaunchKernelGGL((ppmm_mfma_kernel<DW, 8, 3, DC>), dim3(blocks), dim3(512), 0, stream, a, (const int8_t*)bdig, c_tiles, m_block);
+    unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
+    // The column panels beyond the last full group of eight (one per XCD) are cut into jobs by prime where that pays: a single patch
+    // of row tiles (small M), enough primes to share, and the fused rescale (a job needs the last prime only then).
+    static const bool no_tail = getenv("CKKS_PPMM_NO_TAIL") != nullptr;        // test / tuning hook
+    int main_blocks = (int)blocks, tail_jobs = 0;
+    const int rest = c_tiles % 8;
+    if (!no_tail && rest != 0 && c_tiles >= 8 && m_block == m_tiles && a.mod_num >= 8 && !a.raw_all) {
+        tail_jobs = 4;
+        main_blocks = (c_tiles / 8) * 8 * m_tiles;
+        blocks = (unsigned)main_blocks + (unsigned)(rest * m_tiles * tail_jobs);
+    }
+    hipLaunchKernelGGL((ppmm_mfma_kernel<DW, 8, 3, DC>), dim3(blocks), dim3(512), 0, stream, a, (const int8_t*)bdig, c_tiles, m_block, main_blocks, tail_jobs);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }

@@ -349,8 +349,8 @@ def test_small_ring_ntt(N1):
 @pytest.mark.parametrize("M,Kin,wide", [(768, 768, False), (4096, 4096, False), (768, 768, True)])
 def test_ppmm_full_size_sampled_against_oracle(M, Kin, wide):
     """BASELINE configs 4 and 5 at their real shape (N = 2^16, N1 = 128, rank 512, C = 65,664 columns, 12 primes below 2^36, W ~ N(0, 0.02)
-    at scale 2^26): the whole product runs on the device; 24 rows of W over three column panels (the first columns, a panel inside the a
-    part that straddles a 64-column tile edge, the last columns of the b part) are recomputed by the oracle with the full contraction length
+    at scale 2^26): the whole product runs on the device; 24 rows of W over four column panels (the first columns, a panel inside the a
+    part that straddles a 64-column tile edge, a panel in the first and the last columns of the b part) are recomputed by the oracle with the full contraction length
     and compared on every modulus.  Operands: 16 distinct seeded samples, repeated."""
     L, N1 = (2, 128) if wide else (12, 128)
     primes = REF_PARAMS[16]["q"][:2] if wide else CFG2_Q[:L]          # wide: the reference's own two 49-bit ring-pack moduli
@@ -383,7 +383,7 @@ def test_ppmm_full_size_sampled_against_oracle(M, Kin, wide):
     Wsub = np.ascontiguousarray(W[rows])
     mlwe = [seeds[n % 16].reshape(-1) for n in range(Kin)]
     want = np.zeros((len(rows), L, C), dtype=np.uint64)             # only the panel columns get touched
-    panels = [(0, 8), (60, 8), (C - 8, 8)]
+    panels = [(0, 8), (60, 8), (1024 * 64 + 30, 8), (C - 8, 8)]     # the last two lie in the column panels whose tiles are cut into jobs by prime
     for c0, cnt in panels:
         orc.PPMM(Wsub, mlwe, want.reshape(-1), len(rows), Kin, L, scaler, c0, cnt)
     for r, m in enumerate(rows):
