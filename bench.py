@@ -82,6 +82,10 @@ def bench_ntt(args, P):
     N, L1, polys = 1 << logN, len(primes), 2 * cts
     limbs = polys * L1
     ctx = Context_23(logN, [], primes)
+    if args.ntt_mode:
+        ctx.set_ntt_mode(args.ntt_mode)                  # profiling aid: 2 = both passes chained in one launch, 3 = one workgroup per limb
+        if args.ntt_mode == 2 and args.chain_skew:
+            ctx.set_ntt_chain(args.chain_skew)
     # synthetic data: one ciphertext's worth of seeded residues, replicated over the batch (same distribution, bounded set-up time)
     one = uniform_limbs(2, primes, 2, N)
     buf = DeviceBuffer(8 * limbs * N)
@@ -108,9 +112,20 @@ def bench_ntt(args, P):
     value = 2 * limbs * args.steps / dt
 
     # per-kernel durations (HIP events between the two launches), averaged
-    reps = max(5, args.steps)
+    reps = max(5, args.steps) if not args.ntt_mode else 0       # the one-launch modes have no second launch to time
     f1 = f2 = i1 = i2 = 0.0
-    for _ in range(reps):
+    if not reps:
+        ctx.timer_start()
+        for _ in range(10):
+            ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+        f1 = f2 = ctx.timer_stop() / 20
+        ctx.timer_start()
+        for _ in range(10):
+            ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+        i1 = i2 = ctx.timer_stop() / 20
+        reps = 1
+        f1, f2, i1, i2 = [x * reps for x in (f1, f2, i1, i2)]
+    for _ in range(reps if not args.ntt_mode else 0):
         a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, True)
         i1 += a; i2 += b
         a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, False)
@@ -188,6 +203,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=32, help="ciphertexts per step (BASELINE configs[1]: 32)")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--ntt-mode", type=int, default=0, help="profiling aid: launch form of the transforms (ckks_ctx_set_ntt_mode); with a "
+                    "one-launch form the per-pass figures are half the transform's time")
+    ap.add_argument("--chain-skew", type=int, default=0, help="profiling aid with --ntt-mode 2: limbs the first pass runs ahead")
     ap.add_argument("--skip-extra", action="store_true", help="skip the PPMM / key-switch side measurements")
     ap.add_argument("--batch-only", action="store_true",
                     help="profiling aid: only the batched NTT launches (no one-ciphertext, PPMM, key-switch or CPU legs), plus one "
