@@ -7,5 +7,5 @@ Context_23 / PCMM_Context / PCMM_Scheme interface for that path; it has no CPU f
 """
 from ._lib import load_library, LibraryMissing  # noqa: F401
 from .api import (Context_23, PCMM_Context, PCMM_Scheme, DeviceBuffer, CkksError, Scheme_23, SecretKey, Key,  # noqa: F401
-                  Plaintext, Ciphertext, Key_decomp, MLWESecretKey, MLWEPlaintext, PlaintextT, EncodingMatrix, Bert_model_weights, Bert)
+                  Plaintext, Ciphertext, Key_decomp, MLWESecretKey, MLWEPlaintext, MLWECiphertext, PlaintextT, EncodingMatrix, Bert_model_weights, Bert)
 from .precision import GetPrecisionStats, PrecisionStats, Stats  # noqa: F401

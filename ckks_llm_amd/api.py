@@ -733,6 +733,14 @@ class MLWEPlaintext:
         self.mx_device = DeviceBuffer(8 * N1 * (L + 1))
 
 
+class MLWECiphertext:
+    """MLWECiphertext (pcmm/MLWECiphertext.cuh): [L+1 moduli][a_0 .. a_{k-1}, b][N1] words, level l, scale."""
+
+    def __init__(self, N1, L, l, k, scale):
+        self.N1, self.L, self.l, self.k, self.scale = N1, L, l, k, scale
+        self.cipher_device = DeviceBuffer(8 * N1 * (k + 1) * (L + 1))
+
+
 class PCMM_Scheme:
     """PCMM_Scheme (pcmm/PCMM_Scheme.h:12-48): convertMLWESKfromRLWESK, addRepakcingKey, rlweCipherDecompose, PPMM,
     mlweCipherPacking, mlweDecrypt."""
@@ -743,6 +751,9 @@ class PCMM_Scheme:
         self.pcmm_context = pcmm_context
         self.repackingKeys = None
         self.key, self.nonce = (os.urandom(32) if key is None else bytes(key)), 1 << 32
+        self.ppmm_output = None                       # the reference's ppmm_output buffer (PCMM_Scheme.h), grown on demand
+        self.ppmm_target_scale = float(1 << 49)       # PPMM_kernel.cuh:283 fixes 2^49, which suits its 50- to 60-bit ring-pack primes
+        self.last_scaler = 0
 
     def convertMLWESKfromRLWESK(self, mlwe_sk, rlwe_sk):
         """PCMM_Scheme.cuh:23-48."""
@@ -789,15 +800,39 @@ class PCMM_Scheme:
         _check(self.L_.pcmm_mlwe_pack(self.pcmm_context.h, _addr(rlwe_cipher), self._ptrs(bufs), mlwe_num, _addr(repacking_keys),
                                       _addr(embeded_mlwe_buffer), _addr(mult_key_output)), "pcmm_mlwe_pack")
 
-    def PPMM(self, plain_mat, mlwe_cipher_decomposed, out, mat_M, mat_N, mat_K, mlwe_num, mod_num, scaler):
-        """PPMM_kernel.cuh:254-349 (device part).  Shape errors are reported the way the reference does: a message and no
-        work (PPMM_kernel.cuh:256-263), here as ValueError."""
+    def PPMM(self, plain_mat, mlwe_cipher_decomposed, *args):
+        """Two forms.  The reference's (PCMM_Scheme.h, PPMM_kernel.cuh:254-349): PPMM(plain_mat, mlwe_cipher_decomposed, mat_M, mat_N, mat_K,
+        mlwe_num) on MLWECiphertext objects - the scaler is (long)(q_ringpack[1] * 2^49 / scale) (:283-284), all ring-pack moduli take
+        part, row i of the product (first modulus) is copied back into mlwe_cipher_decomposed[i] for i < min(mat_M, mlwe_num) and its
+        scale becomes scale * scaler / q_ringpack[1] (:345-348).  And the device part alone: PPMM(plain_mat, buffers, out, mat_M, mat_N,
+        mat_K, mlwe_num, mod_num, scaler).  Shape errors are reported the way the reference does: a message and no work
+        (PPMM_kernel.cuh:256-263), here as ValueError."""
+        if len(args) == 4:
+            return self._PPMM_reference(plain_mat, mlwe_cipher_decomposed, *args)
+        out, mat_M, mat_N, mat_K, mlwe_num, mod_num, scaler = args
         if mat_K != self.pcmm_context.N1:
             raise ValueError("matrix K should be equal to N1!")
         if mat_N != mlwe_num:
             raise ValueError("matrix N should be equal to mlwe number!")
         _check(self.L_.pcmm_ppmm(self.pcmm_context.h, _addr(plain_mat), self._ptrs(mlwe_cipher_decomposed[:mlwe_num]), _addr(out),
                                  mat_M, mat_N, mod_num, float(scaler)), "pcmm_ppmm")
+
+    def _PPMM_reference(self, plain_mat, mlwe, mat_M, mat_N, mat_K, mlwe_num):
+        pc = self.pcmm_context
+        if mat_K != pc.N1:
+            raise ValueError("matrix K should be equal to N1!")
+        if mat_N != mlwe_num:
+            raise ValueError("matrix N should be equal to mlwe number!")
+        mods, C = pc.ringpack_q_count, (pc.mlwe_rank + 1) * pc.N1
+        if self.ppmm_output is None or self.ppmm_output.nbytes < 8 * mat_M * mods * C:
+            self.ppmm_output = DeviceBuffer(8 * mat_M * mods * C)
+        scaler = int(pc.q_ringpack[1] * self.ppmm_target_scale / mlwe[0].scale)                 # PPMM_kernel.cuh:283-284
+        self.last_scaler = scaler
+        _check(self.L_.pcmm_ppmm(pc.h, _addr(plain_mat), self._ptrs([m.cipher_device for m in mlwe[:mlwe_num]]), _addr(self.ppmm_output),
+                                 mat_M, mat_N, mods, float(scaler)), "pcmm_ppmm")
+        for i in range(min(mat_M, mlwe_num)):                                                    # :345-348
+            mlwe[i].scale = mlwe[i].scale * scaler / pc.q_ringpack[1]
+            _check(self.L_.ckks_memcpy_d2d(mlwe[i].cipher_device.ptr, self.ppmm_output.ptr + 8 * i * C * mods, 8 * C), "ckks_memcpy_d2d")
 
     # -- the gather writing PPMM's operand directly (no counterpart in the reference: its layer runs rlweCipherDecompose and PPMM back
     #    to back through 8-byte MLWE samples, Bert.cuh:411-424)

@@ -128,6 +128,42 @@ def test_ppmm_narrower_matrix_after_a_wider_one(wide):
         assert dev.pcmm_context.info("last_DW") == want_dw, (step, dev.pcmm_context.info("last_absmax"))
 
 
+def test_ppmm_reference_form_on_mlwe_ciphertexts():
+    """PCMM_Scheme::PPMM as the reference declares it: the scaler from the first operand's scale (PPMM_kernel.cuh:283-284), every
+    ring-pack modulus, rows copied back into the MLWE ciphertexts and their scale updated (:345-348); fewer rows than operands and
+    more rows than operands."""
+    from ckks_llm_amd import MLWECiphertext
+    q = CFG2_Q[:2]
+    pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
+    dev.ppmm_target_scale = float(1 << 26)            # 36-bit moduli: rows must stay below q_ringpack[0] / 2
+    C = (rank + 1) * 128
+    rng = np.random.default_rng(5)
+    for M, Kin in ((24, 40), (48, 16)):
+        W = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
+        scale = float(1 << 30)
+        host = [limbs_uniform(50 + n, q, 1, C)[0] for n in range(Kin)]
+        mlwe = []
+        for n in range(Kin):
+            m = MLWECiphertext(128, 1, 1, rank, scale)
+            m.cipher_device.upload(host[n])
+            mlwe.append(m)
+        scaler = int(q[1] * float(1 << 26) / scale)
+        want = np.zeros((M, 2, C), dtype=np.uint64)
+        orc.PPMM(W, [h.reshape(-1) for h in host], want.reshape(-1), M, Kin, 2, float(scaler))
+        dev.PPMM(DeviceBuffer.from_numpy(W), mlwe, M, Kin, 128, Kin)
+        assert dev.last_scaler == scaler
+        assert np.array_equal(dev.ppmm_output.download(np.uint64, want.size).reshape(want.shape), want)
+        for i in range(Kin):
+            got = mlwe[i].cipher_device.download(np.uint64).reshape(2, C)
+            if i < min(M, Kin):
+                assert np.array_equal(got[0], want[i, 0]) and np.array_equal(got[1], host[i][1])      # first modulus replaced, second untouched
+                assert mlwe[i].scale == scale * scaler / q[1]
+            else:
+                assert np.array_equal(got, host[i]) and mlwe[i].scale == scale
+    with pytest.raises(ValueError):
+        dev.PPMM(DeviceBuffer.from_numpy(W), mlwe, M, Kin, 64, Kin)
+
+
 def test_ppmm_prepared_weights_follow_the_buffer():
     """The digit planes of a plaintext matrix are kept under (device address, shape, scaler).  A second call with the same matrix
     reuses them; a matrix overwritten through the library's copy, a freed and reallocated buffer, an announced in-place change and
