@@ -243,6 +243,7 @@ struct NttArgs {
     long batch_stride_limbs;
     unsigned limb_base, limbs_total;      // this launch covers limbs limb_base .. limb_base + gridDim.y - 1 of limbs_total
     char* mid;                            // compact inter-pass buffer (MID_LIMB_BYTES per limb of the launch) or nullptr
+    int reverse = 0;                      // take the limbs of the launch from the last to the first (see launch_passes)
     // Forward transforms of polynomials that exist only as scattered MLWE samples (the embedding of the ring packing): when
     // embed_mlwe is set the first pass takes coefficient pos of polynomial y from sample (pos mod k) / gap, coefficient
     // pos / k (zero where pos mod k is no multiple of gap), lifted around zero from q0 to p0 on the limbs of the first prime.
@@ -464,11 +465,12 @@ __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pas
     constexpr long N = 1l << (SA + SB);
     __shared__ typename AR::V lds[StridedCfg<SA, SB>::LDS_WORDS];
     int prime;
-    u64* limb = limb_ptr(a, blockIdx.y, N, prime);
+    const unsigned l = a.reverse ? gridDim.y - 1 - blockIdx.y : blockIdx.y;
+    u64* limb = limb_ptr(a, l, N, prime);
     const AR ar(a.primes[prime]);
     strided_tile<AR, SA, SB, INVERSE, false, COMPACT, EMBED>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
-                                                             COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr, &a,
-                                                             EMBED ? limb_poly(a, blockIdx.y) : 0u, EMBED && prime == a.start_mod_idx);
+                                                             COMPACT ? a.mid + l * MID_LIMB_BYTES : nullptr, &a,
+                                                             EMBED ? limb_poly(a, l) : 0u, EMBED && prime == a.start_mod_idx);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -554,10 +556,11 @@ __global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass(NttArg
     constexpr long N = 1l << (SA + SB);
     __shared__ typename AR::V lds[RowCfg<SA, SB>::LDS_WORDS];
     int prime;
-    u64* limb = limb_ptr(a, blockIdx.y, N, prime);
+    const unsigned l = a.reverse ? gridDim.y - 1 - blockIdx.y : blockIdx.y;
+    u64* limb = limb_ptr(a, l, N, prime);
     const AR ar(a.primes[prime]);
     row_tile<AR, SA, SB, INVERSE, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
-                                                  COMPACT ? a.mid + blockIdx.y * MID_LIMB_BYTES : nullptr);
+                                                  COMPACT ? a.mid + l * MID_LIMB_BYTES : nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -740,20 +743,25 @@ static int ensure_mid(ckks_ctx* c, size_t need);
 
 // launches of one chunk of limbs; COMPACT selects the 5-byte inter-pass buffer
 template <class AR, int SA, int SB, bool COMPACT>
-static void launch_passes(ckks_ctx* c, const NttArgs& args, int n, bool inverse) {
+static void launch_passes(ckks_ctx* c, const NttArgs& args_in, int n, bool inverse) {
     typedef StridedCfg<SA, SB> CS;
     typedef RowCfg<SA, SB> CR;
+    // The second launch walks the limbs backwards: what the first launch wrote last is still in the memory-side cache (256 MiB)
+    // when the second starts, and what the second writes last is what a following transform of the same data reads first.
+    static const bool rev_env = getenv("CKKS_NTT_NO_REVERSE") == nullptr;
+    NttArgs args = args_in, args2 = args_in;
+    args2.reverse = rev_env ? 1 : 0;
     dim3 gs(CS::TILES, n), bs(CS::THREADS);
     dim3 gr(CR::TILES, n), br(CR::THREADS);
     if (!inverse) {
         if (args.embed_mlwe) hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT, true>), gs, bs, 0, c->stream, args);
         else hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, false, COMPACT>), gs, bs, 0, c->stream, args);
         if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false, COMPACT>), gr, br, 0, c->stream, args);
+        hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, false, COMPACT>), gr, br, 0, c->stream, args2);
     } else {
         hipLaunchKernelGGL((ntt_row_pass<AR, SA, SB, true, COMPACT>), gr, br, 0, c->stream, args);
         if (c->ev_mid_armed) (void)hipEventRecord(c->ev_mid, c->stream);
-        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true, COMPACT>), gs, bs, 0, c->stream, args);
+        hipLaunchKernelGGL((ntt_strided_pass<AR, SA, SB, true, COMPACT>), gs, bs, 0, c->stream, args2);
     }
 }
 
