@@ -259,21 +259,21 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
             }
         } else {
             v4i bf[2][DC], af[2][DW];
-    #pragma unroll
+#pragma unroll
             for (int d = 0; d < DW; d++) af[0][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32][0] + frag_off);
-    #pragma unroll
+#pragma unroll
             for (int nt = 0; nt < 2; nt++)
-    #pragma unroll
+#pragma unroll
                 for (int jj = 0; jj < DC; jj++) bf[nt][jj] = *reinterpret_cast<const v4i*>(&B_cur[jj][wc * 32 + nt * 16][0] + frag_off);
-    #pragma unroll
+#pragma unroll
             for (int d = 0; d < DW; d++) af[1][d] = *reinterpret_cast<const v4i*>(&A_cur[d][wm * 32 + 16][0] + frag_off);
-    #pragma unroll
+#pragma unroll
             for (int mt = 0; mt < 2; mt++)
-    #pragma unroll
+#pragma unroll
                 for (int nt = 0; nt < 2; nt++) {
-    #pragma unroll
+#pragma unroll
                     for (int jj = 0; jj < DC; jj++)
-    #pragma unroll
+#pragma unroll
                         for (int d = 0; d < DW; d++)
                             acc[d + jj][mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[mt][d], bf[nt][jj], acc[d + jj][mt][nt], 0, 0, 0);
                     // the refill of slot W (read one step ago, released by the barrier that ended that step) goes out behind the operand
