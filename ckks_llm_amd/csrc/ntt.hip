@@ -309,6 +309,41 @@ __device__ __forceinline__ void mid_store_row_inverse(char* mid_limb, unsigned r
     }
 }
 
+// The two forms in which a stage-fused launch hands a forward transform's first pass to the kernel that runs its second:
+// the 5-byte pieces above (primes below 2^39) and, for wider primes, the limb itself as it lies between the passes of an
+// in-place transform (balanced doubles, row-major).  request() fetches lane (u, rl)'s sixteen words of row tile rb undecoded,
+// so that a caller can ask for them ahead of their use.
+struct MidPieces {
+    static constexpr long LIMB_BYTES = MID_LIMB_BYTES;
+    struct Raw { unsigned lo[16], hi[16]; };
+    template <class AR>
+    static __device__ __forceinline__ void store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const double (&v)[16], const AR& ar) {
+        mid_store_columns(mid_limb, cb, g, cl, v, ar);
+    }
+    static __device__ __forceinline__ void request(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, Raw& r) {
+        mid_load_row_raw(mid_limb, rb, rl, u, r.lo, r.hi);
+    }
+    template <class AR>
+    static __device__ __forceinline__ double decode(const AR& ar, const Raw& r, int j, unsigned rl) { return mid_decode_row(ar, r.lo[j], r.hi[j], rl); }
+};
+struct MidLimb {
+    static constexpr long LIMB_BYTES = 65536l * 8;
+    struct Raw { u64 w[16]; };
+    template <class AR>
+    static __device__ __forceinline__ void store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const double (&v)[16], const AR& ar) {
+        u64* col = reinterpret_cast<u64*>(mid_limb) + cb * 16 + cl;
+#pragma unroll
+        for (int j = 0; j < 16; j++) col[(long)(g * 16 + j) * 256] = ar.to_mid_fwd(v[j]);
+    }
+    static __device__ __forceinline__ void request(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, Raw& r) {
+        const u64* row = reinterpret_cast<const u64*>(mid_limb) + (long)(rb * 16 + rl) * 256 + u;
+#pragma unroll
+        for (int j = 0; j < 16; j++) r.w[j] = row[j * 16];
+    }
+    template <class AR>
+    static __device__ __forceinline__ double decode(const AR& ar, const Raw& r, int j, unsigned) { return ar.from_mid(r.w[j]); }
+};
+
 // limb index of this block -> base pointer and prime.  Limbs are ordered prime-major so that consecutive
 // workgroups reuse one prime's twiddle table while it is hot in L2.
 __device__ __forceinline__ u64* limb_ptr(const NttArgs& a, unsigned limb, long N, int& prime) {
@@ -1093,14 +1128,20 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 
 // The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
 // transform modes, every prime involved below 2^39.  CKKS_KS_SPLIT (any value) in the environment switches them off, for tuning.
-static bool stage_fusion_applies(const ckks_ctx* c, int first_prime, int prime_count) {
+// How the stage-fused launches can run on primes first_prime .. first_prime + prime_count - 1: 0 not at all, 1 with the 5-byte
+// inter-pass pieces (all primes below 2^39), 2 with whole limbs between the passes and the wide FP64 arithmetic (all below 2^50).
+static int stage_fusion_form(const ckks_ctx* c, int first_prime, int prime_count) {
     static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed) return false;
-    if (first_prime < 0 || prime_count < 1 || first_prime + prime_count > c->nprimes) return false;
-    for (int j = first_prime; j < first_prime + prime_count; j++)
-        if (!c->f64_ok[j] || c->pqt[j] >= (1ull << 39)) return false;
-    return true;
+    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed) return 0;
+    if (first_prime < 0 || prime_count < 1 || first_prime + prime_count > c->nprimes) return 0;
+    int form = 1;
+    for (int j = first_prime; j < first_prime + prime_count; j++) {
+        if (c->pqt[j] >= (1ull << 50)) return 0;
+        if (c->pqt[j] >= (1ull << 39)) form = 2;
+    }
+    return form;
 }
+static bool stage_fusion_applies(const ckks_ctx* c, int first_prime, int prime_count) { return stage_fusion_form(c, first_prime, prime_count) == 1; }
 
 static int ensure_mid(ckks_ctx* c, size_t need) {
     if (need <= c->ntt_mid_cap) return CKKS_OK;
@@ -1238,21 +1279,24 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
 // are never written: that is a write and a read of 2 * rank limbs less than the separate launches.
 // ------------------------------------------------------------------------------------------------------------
 struct RepackRowArgs {
-    const char* mid;             // inter-pass buffer of the embedded polynomials' forward transform, limb index im * rank + i
+    const char* mid;             // embedded polynomials after the first pass of their forward transform: limb (i, im) lies
+    long stride_i, stride_im;    //   at mid + i * stride_i + im * stride_im bytes, in the form MID
     const u64* keys;             // key i = [a: 2 limbs | b: 2 limbs], NTT domain
     u64* partial;                // [chunk][z][im][N]
     const PrimeConst* primes;
     const double* tw_fwd;
     int rank, chunk, prime0;     // limb im is modulo prime prime0 + im of the context
 };
+template <class AR, class MID>
 __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs a) {
     typedef RowCfg<8, 8> C;
+    constexpr bool WIDE = std::is_same<AR, F64WideArith>::value;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     constexpr long N = 1l << 16;
     __shared__ double lds[C::LDS_WORDS];
     const unsigned tile = blockIdx.x, im = blockIdx.y, tid = threadIdx.x;
     const int prime = a.prime0 + (int)im;
-    const F64Arith ar(a.primes[prime]);
+    const AR ar(a.primes[prime]);
     const double* twf = a.tw_fwd + (long)prime * N;
     const unsigned u = tid % U, rl = tid / U;
     const unsigned row = tile * ROWS + rl;
@@ -1262,8 +1306,8 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
     double acc[2][R];
 #pragma unroll
     for (int j = 0; j < R; j++) acc[0][j] = acc[1][j] = 0.0;
-    unsigned raw_lo[R], raw_hi[R];
-    auto request = [&](int i) { mid_load_row_raw(a.mid + ((long)im * a.rank + i) * MID_LIMB_BYTES, tile, rl, u, raw_lo, raw_hi); };
+    typename MID::Raw raw;
+    auto request = [&](int i) { MID::request(a.mid + i * a.stride_i + im * a.stride_im, tile, rl, u, raw); };
     if (i0 < i1) request(i0);
     for (int i = i0; i < i1; i++) {
         const u64* ka = a.keys + ((long)i * 4 + im) * N + (long)row * N2 + u;
@@ -1272,14 +1316,15 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
         unsigned two = tw_off;                              // opaque per polynomial: the twiddle loads stay inside the loop
         asm volatile("" : "+v"(two));
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, raw_lo[j], raw_hi[j], rl);
-        fwd_spread<F64Arith, 8, S1>(v, twf, two, ar);
+        for (int j = 0; j < R; j++) v[j] = MID::decode(ar, raw, j, rl);
+        fwd_spread<AR, 8, S1>(v, twf, two, ar);
+        ar.round_end(v);
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];           // the words this lane read last: no barrier before
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
-        fwd_packed<F64Arith, 8, S1>(v, twf, two, u, ar);
+        fwd_packed<AR, 8, S1>(v, twf, two, u, ar);
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
@@ -1291,8 +1336,19 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
 #pragma unroll
         for (int j = 0; j < R; j++) {
             const double x = ar.balance(lrow[padded(u + j * U)]);
-            acc[0][j] += ar.mulmod(x, (double)(long long)k0[j]);              // each term in (-0.51 q, 0.51 q): exact over any chunk
-            acc[1][j] += ar.mulmod(x, (double)(long long)k1[j]);              // of fewer than 2^13 polynomials
+            if constexpr (WIDE) {                                             // key words balanced: each term within 0.6 q of zero
+                acc[0][j] += ar.mulmod(x, ar.from_canonical(k0[j]));
+                acc[1][j] += ar.mulmod(x, ar.from_canonical(k1[j]));
+            } else {
+                acc[0][j] += ar.mulmod(x, (double)(long long)k0[j]);          // each term in (-0.51 q, 0.51 q): exact over any chunk
+                acc[1][j] += ar.mulmod(x, (double)(long long)k1[j]);          // of fewer than 2^13 polynomials
+            }
+        }
+        if constexpr (WIDE) {
+            if (((i - i0) & 3) == 3) {                                        // four terms on a balanced sum: below 3 q < 2^52
+#pragma unroll
+                for (int j = 0; j < R; j++) { acc[0][j] = ar.balance(acc[0][j]); acc[1][j] = ar.balance(acc[1][j]); }
+            }
         }
     }
 #pragma unroll
@@ -1302,13 +1358,14 @@ __global__ __launch_bounds__(256, 2) void repack_row_fused_kernel(RepackRowArgs 
         for (int j = 0; j < R; j++) out[j * U] = ar.canon(ar.balance(acc[z][j]));
     }
 }
+template <class AR>
 __global__ __launch_bounds__(256) void repack_reduce_kernel(const u64* partial, u64* acc, const PrimeConst* primes, int prime0, int chunks) {
     constexpr long N = 1l << 16;
     const long x = (long)blockIdx.x * 256 + threadIdx.x;
     const int zi = blockIdx.y;                               // z * 2 + im
-    const F64Arith ar(primes[prime0 + (zi & 1)]);
+    const AR ar(primes[prime0 + (zi & 1)]);
     double s = 0.0;
-    for (int ch = 0; ch < chunks; ch++) s += exact_u2d(partial[((long)ch * 4 + zi) * N + x]);      // < chunks * q: exact
+    for (int ch = 0; ch < chunks; ch++) s += ar.from_canonical(partial[((long)ch * 4 + zi) * N + x]);      // at most 16 terms below q (q / 2 for wide primes): exact
     acc[(long)zi * N + x] = ar.canon(ar.balance(s));
 }
 
@@ -1317,33 +1374,48 @@ __global__ __launch_bounds__(256) void repack_reduce_kernel(const u64* partial, 
 int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const uint64_t* keys, int rank, int prime0,
                               const NttEmbedSource& src, bool* done) {
     *done = false;
-    if (rank < 1 || !stage_fusion_applies(c, prime0, 2)) return CKKS_OK;
+    const int form = rank < 1 ? 0 : stage_fusion_form(c, prime0, 2);
+    if (form == 0) return CKKS_OK;
     if (!src.mlwe || src.logk < 0 || src.loggap < 0 || src.loggap > src.logk || src.n1 <= 0 || ((long)src.n1 << src.logk) != c->N ||
         (1 << src.logk) != rank) return CKKS_OK;
     int chunks = 16;
     while (chunks > 1 && (chunks * 4 > 2 * rank || chunks > rank)) chunks >>= 1;
     const int chunk = (rank + chunks - 1) / chunks;
     if (chunks * 4 > 2 * rank || chunk >= (1 << 13)) return CKKS_OK;
-    const size_t mid_bytes = (size_t)2 * rank * MID_LIMB_BYTES;
+    // form 1: first pass into the inter-pass pieces, partial sums into `work`; form 2: first pass into `work` as whole limbs
+    // (polynomial i, limb im at limb index 2 i + im), partial sums into the inter-pass area
+    const size_t mid_bytes = form == 1 ? (size_t)2 * rank * MidPieces::LIMB_BYTES : (size_t)chunks * 4 * c->N * sizeof(u64);
     if (mid_bytes > (1ul << 30)) return CKKS_OK;
     int rc = ensure_mid(c, mid_bytes);
     if (rc) return rc;
     typedef StridedCfg<8, 8> CS;
     NttArgs args;
-    args.data = (u64*)work; args.primes = c->d_primes; args.tw = c->d_twd_fwd; args.mid = (char*)c->d_ntt_mid;
+    args.data = (u64*)work; args.primes = c->d_primes; args.tw = c->d_twd_fwd; args.mid = form == 1 ? (char*)c->d_ntt_mid : nullptr;
     args.start_poly_idx = 0; args.start_mod_idx = prime0; args.poly_num = rank; args.mod_num = 2; args.poly_mod_len = 2;
     args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)(2 * rank);
     args.embed_mlwe = (const u64* const*)src.mlwe;
     args.embed_p0 = src.p0; args.embed_q0 = src.q0;
     args.embed_logk = src.logk; args.embed_loggap = src.loggap; args.embed_n1 = src.n1;
     args.embed_no_wrap = src.q0 / 2 < src.p0 ? 1 : 0;
-    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, false, true, true>), dim3(CS::TILES, 2 * rank), dim3(CS::THREADS), 0, c->stream, args);
     RepackRowArgs r;
-    r.mid = (const char*)c->d_ntt_mid; r.keys = (const u64*)keys; r.partial = (u64*)work; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd;
+    r.keys = (const u64*)keys; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd;
     r.rank = rank; r.chunk = chunk; r.prime0 = prime0;
-    hipLaunchKernelGGL(repack_row_fused_kernel, dim3(RowCfg<8, 8>::TILES, 2, chunks), dim3(256), 0, c->stream, r);
-    hipLaunchKernelGGL(repack_reduce_kernel, dim3((unsigned)(c->N / 256), 4), dim3(256), 0, c->stream, (const u64*)work, (u64*)acc,
-                       (const PrimeConst*)c->d_primes, prime0, chunks);
+    const dim3 gs(CS::TILES, 2 * rank), gr(RowCfg<8, 8>::TILES, 2, chunks), gd((unsigned)(c->N / 256), 4);
+    if (form == 1) {
+        r.mid = (const char*)c->d_ntt_mid; r.stride_i = MidPieces::LIMB_BYTES; r.stride_im = (long)rank * MidPieces::LIMB_BYTES;
+        r.partial = (u64*)work;
+        hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, false, true, true>), gs, dim3(CS::THREADS), 0, c->stream, args);
+        hipLaunchKernelGGL((repack_row_fused_kernel<F64Arith, MidPieces>), gr, dim3(256), 0, c->stream, r);
+        hipLaunchKernelGGL(repack_reduce_kernel<F64Arith>, gd, dim3(256), 0, c->stream, (const u64*)r.partial, (u64*)acc,
+                           (const PrimeConst*)c->d_primes, prime0, chunks);
+    } else {
+        r.mid = (const char*)work; r.stride_i = 2 * MidLimb::LIMB_BYTES; r.stride_im = MidLimb::LIMB_BYTES;
+        r.partial = (u64*)c->d_ntt_mid;
+        hipLaunchKernelGGL((ntt_strided_pass<F64WideArith, 8, 8, false, false, true>), gs, dim3(CS::THREADS), 0, c->stream, args);
+        hipLaunchKernelGGL((repack_row_fused_kernel<F64WideArith, MidLimb>), gr, dim3(256), 0, c->stream, r);
+        hipLaunchKernelGGL(repack_reduce_kernel<F64WideArith>, gd, dim3(256), 0, c->stream, (const u64*)r.partial, (u64*)acc,
+                           (const PrimeConst*)c->d_primes, prime0, chunks);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
     return CKKS_OK;
@@ -1362,6 +1434,7 @@ struct RescaleArgs {
     const u64* inv;              // q_l^-1 mod q_i, i < l
     int l, poly_mod_len, prime0; // limb i is modulo prime prime0 + i
 };
+template <class AR, class MID>
 __global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
@@ -1370,21 +1443,23 @@ __global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
     const unsigned tile = blockIdx.y, limb = blockIdx.x, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const unsigned cl = tid % CW, g = tid / CW;
     const int prime = a.prime0 + (int)i;
-    const F64Arith ar(a.primes[prime]);
+    const AR ar(a.primes[prime]);
     const u64* col = a.cipher + ((long)z * a.poly_mod_len + a.l) * N + tile * CW + cl;
     double v[R];
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = ar.balance(exact_u2d(col[(long)(g + j * G) * N2]));      // x mod q_i, |.| <= q_i / 2
     const double* tw = a.tw_fwd + (long)prime * N;
-    fwd_spread<F64Arith, 8, S1>(v, tw, 1u, ar);
+    fwd_spread<AR, 8, S1>(v, tw, 1u, ar);
+    ar.round_end(v);
 #pragma unroll
     for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
-    fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
-    mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
+    fwd_packed<AR, 8, S1>(v, tw, 1u, g, ar);
+    MID::store_columns(a.mid + (long)limb * MID::LIMB_BYTES, tile, g, cl, v, ar);
 }
+template <class AR, class MID>
 __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
     typedef RowCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
@@ -1392,33 +1467,34 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
     __shared__ double lds[C::LDS_WORDS];
     const unsigned tile = blockIdx.x, limb = blockIdx.y, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const int prime = a.prime0 + (int)i;
-    const F64Arith ar(a.primes[prime]);
+    const AR ar(a.primes[prime]);
     const double* tw = a.tw_fwd + (long)prime * N;
     const unsigned u = tid % U, rl = tid / U;
     const unsigned row = tile * ROWS + rl;
     double* lrow = lds + rl * C::PITCH;
     const unsigned tw_off = N1 + row;
     u64* rp = a.cipher + ((long)z * a.poly_mod_len + i) * N + (long)row * N2 + u;
-    unsigned lo[R], hi[R];
-    mid_load_row_raw(a.mid + (long)limb * MID_LIMB_BYTES, tile, rl, u, lo, hi);
+    typename MID::Raw raw;
+    MID::request(a.mid + (long)limb * MID::LIMB_BYTES, tile, rl, u, raw);
     u64 c[R];                                            // the limb's own words, needed after the butterflies
 #pragma unroll
     for (int j = 0; j < R; j++) c[j] = rp[j * U];
     double v[R];
 #pragma unroll
-    for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, lo[j], hi[j], rl);
-    fwd_spread<F64Arith, 8, S1>(v, tw, tw_off, ar);
+    for (int j = 0; j < R; j++) v[j] = MID::decode(ar, raw, j, rl);
+    fwd_spread<AR, 8, S1>(v, tw, tw_off, ar);
+    ar.round_end(v);
 #pragma unroll
     for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = v[j];
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
-    fwd_packed<F64Arith, 8, S1>(v, tw, tw_off, u, ar);
+    fwd_packed<AR, 8, S1>(v, tw, tw_off, u, ar);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
     __syncthreads();
-    const double inv = exact_u2d(a.inv[i]);
+    const double inv = ar.from_canonical(a.inv[i]);     // balanced for wide primes: the product's quotient estimate needs |inv| <= q / 2
 #pragma unroll
     for (int j = 0; j < R; j++) {
         const double x = ar.balance(lrow[padded(u + j * U)]);
@@ -1429,15 +1505,22 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
 // *done = false (nothing launched) where it does not apply.
 int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done) {
     *done = false;
-    if (l < 1 || l > c->L || !stage_fusion_applies(c, c->K, l + 1)) return CKKS_OK;
+    const int form = l < 1 || l > c->L ? 0 : stage_fusion_form(c, c->K, l + 1);
+    if (form == 0) return CKKS_OK;
     const int limbs = 2 * l;
-    int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
+    int rc = ensure_mid(c, (size_t)limbs * (form == 1 ? MidPieces::LIMB_BYTES : MidLimb::LIMB_BYTES));
     if (rc) return rc;
     RescaleArgs r;
     r.cipher = (u64*)cipher; r.mid = (char*)c->d_ntt_mid; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd; r.inv = (const u64*)inv;
     r.l = l; r.poly_mod_len = c->L + 1; r.prime0 = c->K;
-    hipLaunchKernelGGL(rescale_strided_kernel, dim3(limbs, StridedCfg<8, 8>::TILES), dim3(256), 0, c->stream, r);
-    hipLaunchKernelGGL(rescale_row_kernel, dim3(RowCfg<8, 8>::TILES, limbs), dim3(256), 0, c->stream, r);
+    const dim3 gs(limbs, StridedCfg<8, 8>::TILES), gr(RowCfg<8, 8>::TILES, limbs);
+    if (form == 1) {
+        hipLaunchKernelGGL((rescale_strided_kernel<F64Arith, MidPieces>), gs, dim3(256), 0, c->stream, r);
+        hipLaunchKernelGGL((rescale_row_kernel<F64Arith, MidPieces>), gr, dim3(256), 0, c->stream, r);
+    } else {
+        hipLaunchKernelGGL((rescale_strided_kernel<F64WideArith, MidLimb>), gs, dim3(256), 0, c->stream, r);
+        hipLaunchKernelGGL((rescale_row_kernel<F64WideArith, MidLimb>), gr, dim3(256), 0, c->stream, r);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
     return CKKS_OK;

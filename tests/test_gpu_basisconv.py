@@ -163,11 +163,17 @@ def test_rescale():
         d.rescaleAndEqual(dc, scratch, 0)                   # level-0 operand (Scheme_23.cuh:192-194 behaviour)
 
 
-def test_rescale_full_ring():
-    """rescaleAndEqual at N = 2^16 on 36-bit primes with a special prime in front (limb i is modulo prime K + i): there the
-    reduction of the last limb and the final subtraction run inside the two passes of the forward transform; same words as the
-    oracle and as the device's separate steps (ntt mode 1), the last limb left in coefficient form, higher limbs untouched."""
+@pytest.mark.parametrize("primes", ["36", "49", "mixed"])
+def test_rescale_full_ring(primes):
+    """rescaleAndEqual at N = 2^16 with a special prime in front (limb i is modulo prime K + i): there the reduction of the last
+    limb and the final subtraction run inside the two passes of the forward transform; same words as the oracle and as the
+    device's separate steps (ntt mode 1), the last limb left in coefficient form, higher limbs untouched.  On 36-bit primes (5-byte
+    form between the passes), on the reference's 49-bit primes and on a chain that mixes both (whole limbs between the passes)."""
     q, p = CFG2_Q[:7], CFG3_P[:1]
+    if primes == "49":
+        q, p = REF_PARAMS[16]["q"][:7], REF_PARAMS[16]["p"][:1]
+    elif primes == "mixed":
+        q = CFG2_Q[:2] + REF_PARAMS[16]["q"][:2] + CFG2_Q[2:4] + REF_PARAMS[16]["q"][2:3]
     pair = Pair(16, p, q)
     o, d, N = pair.orc, pair.dev, pair.N
     for l in (6, 3, 1):

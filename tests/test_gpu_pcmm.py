@@ -313,13 +313,18 @@ def test_ppmm_shape_errors():
         dev.PPMM(0, [], 0, 4, 4, 128, 5, 2, 1.0)           # mat_N != mlwe_num (:260-263)
 
 
-@pytest.mark.parametrize("logN,N1,mlwe_num", [(12, 128, 32), (12, 128, 8), (10, 64, 16), (16, 128, 512), (16, 128, 64), (16, 256, 256),
-                                              (16, 64, 1024), (16, 4096, 16)])
-def test_mlwe_packing(logN, N1, mlwe_num):
+@pytest.mark.parametrize("logN,N1,mlwe_num,primes", [(12, 128, 32, "36"), (12, 128, 8, "36"), (10, 64, 16, "36"), (16, 128, 512, "36"),
+                                                     (16, 128, 64, "36"), (16, 256, 256, "36"), (16, 64, 1024, "36"), (16, 4096, 16, "36"),
+                                                     (16, 128, 512, "49"), (16, 128, 128, "49"), (16, 256, 256, "36/49"), (16, 64, 1024, "49"),
+                                                     (12, 128, 32, "49")])
+def test_mlwe_packing(logN, N1, mlwe_num, primes):
     """mlweCipherPacking through the C ABI against the oracle: embedding, lift to the special prime, NTT, inner product with the
     repacking keys, iNTT, division by the special prime, + (0, b), NTT - bit-exact on random samples and random keys (the
-    oracle itself is pinned by a decrypt identity with real keys)."""
-    p0, q = CFG3_P[0], CFG2_Q[:2]
+    oracle itself is pinned by a decrypt identity with real keys).  On 36-bit primes, on the reference's own 49-bit special prime
+    and moduli (at N = 2^16 the stage-fused launches then hand whole limbs over instead of the 5-byte form and balance their sums
+    every few terms), and on a 36-bit special prime under 49-bit moduli."""
+    p0 = REF_PARAMS[16]["p"][0] if primes == "49" else CFG3_P[0]
+    q = CFG2_Q[:2] if primes == "36" else REF_PARAMS[16]["q"][:2]
     pair, dev, orc, rank = make(logN, N1, q, [p0], [p0], q)
     N = pair.N
     assert rank % mlwe_num == 0
