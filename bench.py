@@ -166,6 +166,19 @@ def bench_ntt(args, P):
     iv = ctx.timer_stop() / R
     one_ct = {"fwd_us": round(fw * 1e3, 2), "inv_us": round(iv * 1e3, 2),
               "fwd_limb_transforms_per_s": round(2 * L1 / (fw * 1e-3)), "inv_limb_transforms_per_s": round(2 * L1 / (iv * 1e-3))}
+    # a ciphertext at level 15 (32 limbs): below 41 limbs the library takes the paired one-launch form; two launches beside it
+    if not args.ntt_mode:
+        lv = {}
+        for label, mode in (("fwd_us", 0), ("two_launch_fwd_us", 1)):
+            ctx.set_ntt_mode(mode)
+            for _ in range(5):
+                ctx.ToNTTInplace(small, 0, 0, 2, 16, L1)
+            ctx.timer_start()
+            for _ in range(R):
+                ctx.ToNTTInplace(small, 0, 0, 2, 16, L1)
+            lv[label] = round(ctx.timer_stop() / R * 1e3, 2)
+        ctx.set_ntt_mode(0)
+        one_ct["level15_32_limbs"] = lv
     buf.free(); small.free()
     return value, ms_per_step, roofline, one_ct, limbs
 

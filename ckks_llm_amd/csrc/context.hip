@@ -370,6 +370,7 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) c->cu_count = cus;
         c->device = dev;
         if (rc == CKKS_OK) rc = ckks::ntt_noalloc_init(nullptr);
+        if (rc == CKKS_OK && c->logN == 16) rc = ckks::ntt_pair_init(c);
     }
     if (rc == CKKS_OK && hipEventCreate(&c->ev0) != hipSuccess) rc = CKKS_E_HIP;
     if (rc == CKKS_OK && hipEventCreate(&c->ev1) != hipSuccess) rc = CKKS_E_HIP;
@@ -385,6 +386,8 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     void* ptrs[] = {c->d_primes, c->d_primes_moddown, c->d_primes_modup, c->d_tw_fwd, c->d_tw_inv, c->d_twd_fwd, c->d_twd_inv, c->d_conv, c->d_pHatVecModq,
                     c->d_pHatInvVecModp, c->d_PinvModq, c->d_qiInvModql, c->d_ntt_chain, c->d_ntt_mid};
     for (void* p : ptrs) if (p) (void)hipFree(p);
+    if (c->d_ntt_pair) (void)hipFree(c->d_ntt_pair);
+    if (c->h_pair_fail) (void)hipHostFree(c->h_pair_fail);
     for (auto& e : c->decode_tabs) (void)hipFree(e.dev);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
@@ -420,9 +423,10 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
 }
 
 // test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = chained one-launch transform wherever that kernel exists
-// (N >= 2^15), 3 = one workgroup per limb wherever that kernel exists (N >= 2^15)
+// (N >= 2^15), 3 = one workgroup per limb wherever that kernel exists (N >= 2^15), 4 = paired one-launch transform at every batch
+// size (N = 2^16; the automatic mode takes it for small batches), 5 = the same with the tiles of a limb spread over all XCDs
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
-    if (!c || mode < 0 || mode > 3) return CKKS_E_INVALID;
+    if (!c || mode < 0 || mode > 5) return CKKS_E_INVALID;
     c->ntt_mode = mode;
     return CKKS_OK;
 }
@@ -442,6 +446,7 @@ extern "C" int ckks_ctx_check(ckks_ctx* c) {
     if (!c) return CKKS_E_INVALID;
     CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
     CKKS_HIP_TRY(hipGetLastError());
+    if (ckks::ntt_pair_failed(c)) { ckks::set_error("NTT: a one-launch transform gave up waiting for its first pass; its output is incomplete"); return CKKS_E_UNAVAILABLE; }
     return CKKS_OK;
 }
 

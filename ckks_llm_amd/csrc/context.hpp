@@ -84,7 +84,8 @@ struct ckks_ctx {
     size_t qiInv_count = 0;
 
     int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
-    int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: chained one-launch transform, 3: one workgroup per limb
+    int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: chained one-launch transform, 3: one workgroup per limb,
+                                          // 4: paired one-launch transform at every batch size, 5: the same with a limb's tiles spread over the XCDs
     int cu_count = 256;
     void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
     size_t ntt_mid_cap = 0;
@@ -94,6 +95,8 @@ struct ckks_ctx {
     struct DecodeTab { int level, words; void* dev; };
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     int chain_skew = 0, chain_spin = -1;  // chained transform: limbs a chain's first pass runs ahead of its second (0: default), poll limit of a wait (-1: default)
+    void* d_ntt_pair = nullptr;           // completion words of the paired (one-launch, small-batch) transform, one per 128-byte line
+    unsigned* h_pair_fail = nullptr;      // pinned host word that a paired transform raises when one of its waits ran out
     void* d_ntt_chain = nullptr;          // completion words of the chained (one-launch) transform, allocated on its first use; zero between transforms
 };
 
@@ -109,6 +112,9 @@ int hip_fail(hipError_t e, const char* what);
 // launchers (ntt.hip, basisconv.hip)
 // chained (one-launch) transform: tiles left to its finishing launch so far, and the host view of its slot order (for tests)
 int ntt_chain_deferred(ckks_ctx* c, long* tiles);
+// 1 once a paired (one-launch) transform of the context has given up a wait: its output is incomplete and the context unusable
+int ntt_pair_failed(const ckks_ctx* c);
+int ntt_pair_init(ckks_ctx* c);
 void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile);
 unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew);
 // Address, on the current device, of the file-scope inter-pass area of the transform that allocates nothing (looked up once per

@@ -259,11 +259,23 @@ struct NttArgs {
 //   hi bytes  forward transforms: [r_local / 4][c_local] dwords, byte r_local % 4; inverse transforms: [r_local][c_local]   256 B
 // The strided pass (tile = cb) touches pieces (cb, 0..15), the row pass (tile = rb) pieces (0..15, rb); in all four access
 // patterns 16 lanes cover 64 contiguous bytes.
+// Accesses to data that another workgroup of the SAME launch writes or reads (the paired transform): relaxed atomics at agent
+// scope, i.e. ordinary loads and stores that are carried out at the level of the memory hierarchy all compute units share.
+template <bool SHARED, class T>
+__device__ __forceinline__ void put(T* p, T v) {
+    if (SHARED) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+template <bool SHARED, class T>
+__device__ __forceinline__ T get(const T* p) {
+    if (SHARED) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
 constexpr int MID_PIECE_BYTES = 1280;
 constexpr long MID_LIMB_BYTES = 256l * MID_PIECE_BYTES;
 __device__ __forceinline__ char* mid_piece(char* mid_limb, unsigned cb, unsigned rb) { return mid_limb + (cb * 16 + rb) * MID_PIECE_BYTES; }
 // Forward first pass, lane (cl, g) holding rows 16g .. 16g+15 of column cl of tile cb: writes its 16 values into piece (cb, g).
-template <class AR>
+template <class AR, bool SHARED = false>
 __device__ __forceinline__ void mid_store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const typename AR::V (&v)[16], const AR& ar) {
     char* piece = mid_piece(mid_limb, cb, g);
     unsigned hi[4] = {0, 0, 0, 0};
@@ -277,20 +289,21 @@ __device__ __forceinline__ void mid_store_columns(char* mid_limb, unsigned cb, u
     }
 #pragma unroll
     for (int j = 0; j < 16; j++) {
-        *reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4) = (unsigned)e[j];
+        put<SHARED>(reinterpret_cast<unsigned*>(piece + (j * 16 + cl) * 4), (unsigned)e[j]);
         hi[j >> 2] |= (unsigned)(e[j] >> 32) << (8 * (j & 3));
     }
 #pragma unroll
-    for (int jg = 0; jg < 4; jg++) *reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4) = hi[jg];
+    for (int jg = 0; jg < 4; jg++) put<SHARED>(reinterpret_cast<unsigned*>(piece + 1024 + (jg * 16 + cl) * 4), hi[jg]);
 }
 // Forward second pass, lane (u, rl) of row tile rb taking columns u + 16j of row 16 rb + rl: element (rl, u) of piece (j, rb).
 // The raw words are returned undecoded so that a caller can request them ahead of their use.
+template <bool SHARED = false>
 __device__ __forceinline__ void mid_load_row_raw(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, unsigned (&lo)[16], unsigned (&hi)[16]) {
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const char* piece = mid_piece(const_cast<char*>(mid_limb), j, rb);
-        lo[j] = *reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4);
-        hi[j] = *reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4);
+        lo[j] = get<SHARED>(reinterpret_cast<const unsigned*>(piece + (rl * 16 + u) * 4));
+        hi[j] = get<SHARED>(reinterpret_cast<const unsigned*>(piece + 1024 + ((rl >> 2) * 16 + u) * 4));
     }
 }
 template <class AR>
@@ -298,14 +311,14 @@ __device__ __forceinline__ typename AR::V mid_decode_row(const AR& ar, unsigned 
     return ar.dec40(lo, (hi >> (8 * (rl & 3))) & 0xffu);
 }
 // Inverse first pass (row pass) output in the inverse layout of the high bytes: bytes [r_local][c_local].
-template <class AR>
+template <class AR, bool SHARED = false>
 __device__ __forceinline__ void mid_store_row_inverse(char* mid_limb, unsigned rb, unsigned rl, unsigned u, const typename AR::V (&v)[16], const AR& ar) {
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         char* piece = mid_piece(mid_limb, j, rb);
         const u64 e = ar.enc40(v[j]);
-        *reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4) = (unsigned)e;
-        *reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u) = (unsigned char)(e >> 32);
+        put<SHARED>(reinterpret_cast<unsigned*>(piece + (rl * 16 + u) * 4), (unsigned)e);
+        put<SHARED>(reinterpret_cast<unsigned char*>(piece + 1024 + rl * 16 + u), (unsigned char)(e >> 32));
     }
 }
 
@@ -396,7 +409,8 @@ struct StridedCfg {
     static constexpr int THREADS = G * CW, TILES = N2 / CW, LDS_WORDS = N1 * CW;
 };
 
-template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool EMBED = false>
+// PAIRED: the tile is one half of a paired transform - what it hands to or takes from the other pass moves as shared accesses
+template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool EMBED = false, bool PAIRED = false>
 __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
                                              typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const NttArgs* ea = nullptr,
                                              unsigned poly = 0, bool lift = false) {
@@ -460,21 +474,21 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
         for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
         fwd_packed<AR, SA, S1>(v, tw, 1u, g, ar);
         if constexpr (COMPACT) {
-            if constexpr (R == 16) mid_store_columns(mid_limb, tile, g, cl, v, ar);      // the 5-byte form exists for 256 x 256 only
+            if constexpr (R == 16) mid_store_columns<AR, PAIRED>(mid_limb, tile, g, cl, v, ar);      // the 5-byte form exists for 256 x 256 only
         } else {
 #pragma unroll
-            for (int j = 0; j < R; j++) col[(long)(g * R + j) * N2] = ar.to_mid_fwd(v[j]);
+            for (int j = 0; j < R; j++) put<PAIRED>(col + (long)(g * R + j) * N2, ar.to_mid_fwd(v[j]));
         }
     } else {
         if constexpr (COMPACT) {
             const char* piece = mid_piece(mid_limb, tile, g);
 #pragma unroll
             for (int j = 0; j < R; j++)
-                v[j] = ar.dec40(*reinterpret_cast<const unsigned*>(piece + (j * 16 + cl) * 4),
-                                *reinterpret_cast<const unsigned char*>(piece + 1024 + j * 16 + cl));
+                v[j] = ar.dec40(get<PAIRED>(reinterpret_cast<const unsigned*>(piece + (j * 16 + cl) * 4)),
+                                get<PAIRED>(reinterpret_cast<const unsigned char*>(piece + 1024 + j * 16 + cl)));
         } else {
 #pragma unroll
-            for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(col + (long)(g * R + j) * N2));
+            for (int j = 0; j < R; j++) v[j] = ar.from_mid(PAIRED ? get<true>(col + (long)(g * R + j) * N2) : load_word<COHERENT>(col + (long)(g * R + j) * N2));
         }
         inv_packed<AR, SA, S1>(v, tw, 1u, g, ar);
         ar.round_end(v);
@@ -521,7 +535,7 @@ struct RowCfg {
 };
 __device__ __forceinline__ int padded(int pos) { return pos + (pos >> 4); }
 
-template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false>
+template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool PAIRED = false>
 __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
                                          typename AR::V* lds, unsigned tid, char* mid_limb = nullptr) {
     typedef RowCfg<SA, SB> C;
@@ -537,13 +551,13 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         if constexpr (COMPACT) {
             if constexpr (R == 16) {
                 unsigned lo[16], hi[16];
-                mid_load_row_raw(mid_limb, tile, rl, u, lo, hi);
+                mid_load_row_raw<PAIRED>(mid_limb, tile, rl, u, lo, hi);
 #pragma unroll
                 for (int j = 0; j < R; j++) v[j] = mid_decode_row(ar, lo[j], hi[j], rl);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < R; j++) v[j] = ar.from_mid(load_word<COHERENT>(rp + u + j * U));
+            for (int j = 0; j < R; j++) v[j] = ar.from_mid(PAIRED ? get<true>(rp + u + j * U) : load_word<COHERENT>(rp + u + j * U));
         }
         fwd_spread<AR, SB, S1>(v, tw, tw_off, ar);
         ar.round_end(v);
@@ -578,10 +592,10 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         if constexpr (COMPACT) {
             // inverse transforms keep the hi bytes as bytes [r_local][c_local]: a wave (16 columns x 4 rows of a piece) stores
             // 64 contiguous bytes per instruction and needs no cross-lane packing
-            if constexpr (R == 16) mid_store_row_inverse(mid_limb, tile, rl, u, v, ar);
+            if constexpr (R == 16) mid_store_row_inverse<AR, PAIRED>(mid_limb, tile, rl, u, v, ar);
         } else {
 #pragma unroll
-            for (int j = 0; j < R; j++) rp[u + j * U] = ar.to_mid_inv(v[j]);
+            for (int j = 0; j < R; j++) put<PAIRED>(rp + u + j * U, ar.to_mid_inv(v[j]));
         }
     }
 }
@@ -774,7 +788,124 @@ __global__ __launch_bounds__(256) void ntt_chain_finish_kernel(NttArgs a, ChainA
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Paired transform for small batches: both passes in one launch, one workgroup per (limb, tile) that runs the tile of the
+// first pass, waits until the limb's other first-pass tiles are done, and runs the same-numbered tile of the second pass.
+// A launch of a few hundred workgroups is over before the chip has ramped up, so for one ciphertext the second launch's
+// ramp and the drain between the launches cost as much as the work; here they fall away.
+//
+// Synchronisation is that of the programming model, with no assumption about where a workgroup runs: every wave releases its
+// first-pass stores at agent scope, the workgroup adds 1 to the limb's completion word, polls it (agent-scope loads) until
+// it reads a multiple of TILES, and every wave acquires at agent scope before the second pass loads.  The word is a
+// multiple of TILES between launches (launches of one context are ordered on its stream and each adds TILES to the words of
+// its limbs), so nothing has to be cleared; a workgroup has added its own 1 before it polls, so a multiple of TILES can only
+// be the completed count.
+// Progress: a waiting workgroup waits for workgroups that wait for nothing.  Workgroups start in the order of their index and
+// the sixteen of a limb lie within 128 consecutive indices, so at most 128 resident workgroups can be waiting for one that has not
+// started; the launcher only uses this kernel where the chip holds more than that many at once.  The wait is bounded all the
+// same (about two seconds of polls): a workgroup that runs out of polls leaves its tile undone and raises the context's
+// host-visible failure word, which fails the next call or synchronisation on the context.
+// Blocks are numbered so that the tiles of a limb go to one XCD (workgroup b of a grid goes to XCD b mod 8): the inter-pass
+// data then stays in that XCD's L2.  Placement only matters for speed.
+// ------------------------------------------------------------------------------------------------------------
+constexpr unsigned PAIR_XCDS = 8;
+constexpr int PAIR_MAX_LIMBS = 4096;               // completion words per context
+constexpr int PAIR_WORD_STRIDE = 32;               // one completion word per 128-byte line: atomics on one line are carried out one after the other
+constexpr int PAIR_AUTO_LIMBS = 40;                // automatic mode: batches up to this many limbs take the paired kernel
+struct PairArgs {
+    unsigned* done;            // [limb * PAIR_WORD_STRIDE] first-pass completion count, a multiple of TILES between launches
+    unsigned* fail;            // host-visible word: nonzero once a wait has run out
+    unsigned limbs, spin_max;
+    unsigned spread;           // test setting: the tiles of a limb go to consecutive workgroups, i.e. to all XCDs
+};
+template <class AR, int SA, int SB, bool INVERSE, bool COMPACT>
+__global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
+    typedef StridedCfg<SA, SB> CS;
+    typedef RowCfg<SA, SB> CR;
+    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES && CS::TILES == 16, "paired kernel: tile shapes");
+    constexpr unsigned TILES = CS::TILES;
+    constexpr long N = 1l << (SA + SB);
+    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
+    typedef typename AR::TW TW;
+    __shared__ typename AR::V lds[LDS_WORDS];
+    __shared__ unsigned go;
+    const unsigned idx = blockIdx.x / PAIR_XCDS;
+    const unsigned limb_id = p.spread ? blockIdx.x / TILES : blockIdx.x % PAIR_XCDS + PAIR_XCDS * (idx / TILES);
+    const unsigned tile = p.spread ? blockIdx.x % TILES : idx % TILES;
+    if (limb_id >= p.limbs) return;                                             // uniform over the workgroup
+    int prime;
+    u64* limb = limb_ptr(a, limb_id, N, prime);
+    const AR ar(a.primes[prime]);
+    const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
+    char* mid_limb = COMPACT ? a.mid + (long)limb_id * MID_LIMB_BYTES : nullptr;
+    if (!INVERSE) strided_tile<AR, SA, SB, false, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
+    else row_tile<AR, SA, SB, true, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);                                              // every shared store of this wave has been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned* word = p.done + (size_t)limb_id * PAIR_WORD_STRIDE;
+        (void)__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned ok = 0;
+        for (unsigned n = 0; n < p.spin_max; n++) {
+            if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) % TILES == 0) { ok = 1; break; }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (!ok) __hip_atomic_store(p.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        go = ok;
+    }
+    __syncthreads();
+    if (!go) return;
+    if (!INVERSE) row_tile<AR, SA, SB, false, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
+    else strided_tile<AR, SA, SB, true, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
+}
+
 static int ensure_mid(ckks_ctx* c, size_t need);
+
+// Completion words and failure word of the paired transform, once per context (at its creation, so that no transform allocates).
+int ntt_pair_init(ckks_ctx* c) {
+    if (c->d_ntt_pair) return CKKS_OK;
+    if (hipHostMalloc((void**)&c->h_pair_fail, sizeof(unsigned), hipHostMallocMapped) != hipSuccess) { set_error("NTT: cannot allocate the failure word of the paired transform"); return CKKS_E_NOMEM; }
+    *c->h_pair_fail = 0;
+    const size_t bytes = (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE * sizeof(unsigned);
+    if (hipMalloc(&c->d_ntt_pair, bytes) != hipSuccess) { set_error("NTT: cannot allocate the completion words of the paired transform"); return CKKS_E_NOMEM; }
+    CKKS_HIP_TRY(hipMemsetAsync(c->d_ntt_pair, 0, bytes, c->stream));
+    return CKKS_OK;
+}
+int ntt_pair_failed(const ckks_ctx* c) { return c->h_pair_fail && *(volatile unsigned*)c->h_pair_fail ? 1 : 0; }
+
+template <class AR, int SA, int SB>
+static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok) {
+    constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
+    int rc = ntt_pair_init(c);
+    if (rc) return rc;
+    const bool compact = CAN_COMPACT && compact_ok;
+    args.limb_base = 0;
+    args.limbs_total = (unsigned)limbs;
+    args.mid = nullptr;
+    if (compact) {
+        if ((rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES))) return rc;
+        args.mid = (char*)c->d_ntt_mid;
+    }
+    PairArgs p;
+    p.done = (unsigned*)c->d_ntt_pair; p.fail = c->h_pair_fail; p.limbs = (unsigned)limbs;
+    p.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
+    p.spread = c->ntt_mode == 5 ? 1u : 0u;
+    const unsigned blocks = ((unsigned)limbs + PAIR_XCDS - 1) / PAIR_XCDS * PAIR_XCDS * StridedCfg<SA, SB>::TILES;
+    const dim3 g(blocks), b(256);
+    if constexpr (CAN_COMPACT) {
+        if (compact) {
+            if (!inverse) hipLaunchKernelGGL((ntt_pair_kernel<AR, SA, SB, false, true>), g, b, 0, c->stream, args, p);
+            else hipLaunchKernelGGL((ntt_pair_kernel<AR, SA, SB, true, true>), g, b, 0, c->stream, args, p);
+            CKKS_HIP_TRY(hipGetLastError());
+            return CKKS_OK;
+        }
+    }
+    if (!inverse) hipLaunchKernelGGL((ntt_pair_kernel<AR, SA, SB, false, false>), g, b, 0, c->stream, args, p);
+    else hipLaunchKernelGGL((ntt_pair_kernel<AR, SA, SB, true, false>), g, b, 0, c->stream, args, p);
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
 
 // launches of one chunk of limbs; COMPACT selects the 5-byte inter-pass buffer
 template <class AR, int SA, int SB, bool COMPACT>
@@ -910,6 +1041,16 @@ static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse)
     return CKKS_OK;
 }
 
+// Whether a transform of `limbs` limbs runs as the paired kernel: always in modes 4 and 5 while its completion words suffice, in
+// the automatic mode up to the batch at which two launches are as fast (measured: 15 us against 22 us at 32 limbs, level at 48;
+// CKKS_NTT_PAIR_MAX overrides that limit).
+static bool pair_applies(const ckks_ctx* c, int limbs) {
+    static const int max_env = getenv("CKKS_NTT_PAIR_MAX") ? atoi(getenv("CKKS_NTT_PAIR_MAX")) : -1;
+    if (limbs > PAIR_MAX_LIMBS || c->cu_count < 64) return false;            // the progress argument needs more than 128 resident workgroups
+    if (c->ntt_mode == 4 || c->ntt_mode == 5) return true;
+    return c->ntt_mode == 0 && limbs <= (max_env >= 0 ? max_env : PAIR_AUTO_LIMBS);
+}
+
 template <class AR>
 static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok) {
     // mode 2: both passes in one launch, the limb held in the XCD's L2 between them (N >= 2^15)
@@ -917,6 +1058,8 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
         if (c->logN == 16) return launch_chain<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_chain<AR, 8, 7>(c, args, limbs, inverse);
     }
+    // mode 4, and the automatic mode for small batches: both passes in one launch of one workgroup per (limb, tile)
+    if (!c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs)) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
     // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
     // (the limbs in flight, 0.5 MiB per resident workgroup, exceed the L2 by far), so the automatic mode does not pick it.
     if (!c->ev_mid_armed && c->ntt_mode == 3) {
@@ -1570,6 +1713,7 @@ int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int star
 static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                            int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src) {
     if (!c || !dev) { set_error("NTT: null argument"); return CKKS_E_INVALID; }
+    if (ntt_pair_failed(c)) { set_error("NTT: an earlier one-launch transform of this context gave up waiting for its first pass"); return CKKS_E_UNAVAILABLE; }
     if (poly_num <= 0 || mod_num <= 0 || batch <= 0) return CKKS_OK;      // empty batch: nothing to do
     if (start_mod_idx < 0 || start_mod_idx + mod_num > c->nprimes || start_poly_idx < 0 || poly_mod_len < 0) {
         set_error("NTT: prime range outside the context");

@@ -67,7 +67,11 @@ int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
 /* How a transform is launched.  0 (default): chosen by the library; 1: two launches, one per pass, data in place between
  * them; 2: chained - both passes in one launch, the second pass of a limb following its first pass on the same XCD so that
  * the limb stays in that XCD's L2 in between (N >= 2^15; other rings take two launches), plus a small finishing launch;
- * 3: one workgroup carries a limb through both passes (N >= 2^15).  All give the same residues.
+ * 3: one workgroup carries a limb through both passes (N >= 2^15); 4: paired - both passes in one launch of one workgroup per
+ * (limb, tile), which waits between its two tiles until the limb's first pass is complete (N = 2^16, up to 4096 limbs; mode 0
+ * takes this form for batches of up to 40 limbs, where it is faster than two launches); 5: as 4 with the tiles of a limb spread
+ * over all XCDs (a test setting).  All give the same residues.  Should a wait of the paired form ever run out (about two
+ * seconds), the transform's output is incomplete, ckks_ctx_check and every later transform of the context return CKKS_E_UNAVAILABLE.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
 /* Synchronises the context's stream and returns what HIP reports for the launches so far.  Plays the part of the reference's
@@ -75,7 +79,8 @@ int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
 int ckks_ctx_check(ckks_ctx* ctx);
 /* Test / tuning hook of the chained transform (mode 2).  skew: limbs that a chain's first pass runs ahead of its second pass
  * (0 = default); spin_max: polls that a second-pass workgroup spends waiting for its limb's first pass before it leaves its tile
- * to the finishing launch (-1 = default; 0 sends every tile there).  Results do not depend on either. */
+ * to the finishing launch (-1 = default; 0 sends every tile there).  Results do not depend on either.  spin_max also bounds
+ * the wait of the paired transform (modes 0, 4, 5), which has no finishing launch: there a wait that runs out is an error. */
 int ckks_ctx_set_ntt_chain(ckks_ctx* ctx, int skew, int spin_max);
 /* Order of work of the chained transform, for tests: slot `slot` of a chain of `tiles` workgroups per pass -> pass (0 / 1),
  * index k of the limb within the chain and tile; ckks_ntt_chain_slots = slots of a chain of kmax limbs.  Pure host functions. */

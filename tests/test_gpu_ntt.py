@@ -226,6 +226,69 @@ def test_whole_limb_transform_matches_oracle(logN, polys, mode):
     buf.free()
 
 
+@pytest.mark.parametrize("primes,polys,arith,mode", [("36", 9, 0, 4), ("36", 5, 1, 4), ("49", 3, 0, 4), ("mixed", 2, 0, 4), ("36", 1, 0, 4),
+                                                    ("36", 7, 0, 5), ("49", 2, 0, 5), ("36", 3, 1, 5), ("36", 8, 0, 0)])
+def test_paired_transform_matches_oracle(primes, polys, arith, mode):
+    """The paired transform (both passes in one launch, a workgroup per (limb, tile) that waits between its two tiles for the
+    limb's first pass) against the oracle: 5-byte and in-place inter-pass forms, all three arithmetic back ends, limb counts
+    that are no multiple of eight, several launches in a row on the same completion words, the reference's sub-range
+    addressing.  Mode 5 spreads the tiles of a limb over all XCDs, so that what one pass hands to the other really crosses
+    from one L2 to another; mode 0 with 40 limbs is the automatic choice of this form."""
+    q = {"36": CFG2_Q[:5], "49": REF_PARAMS[16]["q"][:5], "mixed": CFG2_Q[:2] + REF_PARAMS[16]["q"][:2] + REF_PARAMS[16]["t"][:1]}[primes]
+    pair = Pair(16, [], q)
+    N, L1 = pair.N, len(q)
+    pair.dev.set_arith_mode(arith)
+    data = limbs_uniform(140 + polys, q, polys, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, L1, L1)
+    want_inv = data.copy()
+    pair.orc.FromNTTInplace(want_inv.reshape(-1), 0, 0, polys, L1, L1)
+    pair.dev.set_ntt_mode(mode)
+    buf = to_dev(data)
+    for _ in range(3):
+        pair.dev.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), want)
+        pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), data)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    pair.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), want_inv)
+    buf.upload(data)
+    pair.dev.ToNTTInplace(buf, 1, 1, polys, 3, L1)
+    pair.dev.check()
+    got = from_dev(buf, data.shape)
+    assert np.array_equal(got[:, 1:4], want[:, 1:4]) and np.array_equal(got[:, 0], data[:, 0]) and np.array_equal(got[:, 4], data[:, 4])
+    buf.free()
+
+
+def test_paired_transform_reports_a_wait_that_ran_out():
+    """With a poll limit of zero no second-pass tile of the paired transform may start unless its limb is already complete at the
+    first look; every workgroup still ends normally, the context's failure word is raised, check() and every later transform of
+    the context report it.  Another context is not affected."""
+    from ckks_llm_amd import CkksError
+    q = CFG2_Q[:3]
+    pair = Pair(16, [], q)
+    data = limbs_uniform(5, q, 2, pair.N)
+    buf = to_dev(data)
+    pair.dev.set_ntt_mode(4)
+    pair.dev.set_ntt_chain(0, 0)
+    pair.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
+    with pytest.raises(CkksError):
+        pair.dev.check()
+    with pytest.raises(CkksError):
+        pair.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
+    other = Pair(16, [], q)
+    want = data.copy()
+    other.orc.ToNTTInplace(want.reshape(-1), 0, 0, 2, 3, 3)
+    buf.upload(data)
+    other.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
+    other.dev.check()
+    assert np.array_equal(from_dev(buf, data.shape), want)
+    buf.free()
+
+
 @pytest.mark.parametrize("skew,spin", [(1, 0), (3, 0), (2, -1), (64, -1)])
 def test_chained_transform_finishing_launch_and_skews(skew, spin):
     """With a poll limit of zero every second-pass workgroup of the chained transform leaves its tile to the finishing launch,
