@@ -116,6 +116,60 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel_f64(ConvArgs a) {
     }
 }
 
+// ---- sources of any width, targets below 2^50 (the reference's 60-bit T basis back into its 49-bit P and Q primes) ----
+// The scaled residues y_j are formed in integers as in conv_kernel (they are residues of the source primes), so v is the same
+// number.  The sums modulo the targets are the FP64 ones: y_j = yh 2^31 + yl with both parts below 2^31, each multiplied by its
+// own constant ((D/d_j) and (D/d_j) 2^31 mod r_k, balanced) in the two-product form; every term lies within 0.51 r_k of zero and
+// the running sum is balanced after every four sources, so all integers stay below 2^53.  A 64 x 64 -> 128-bit product costs
+// more than ten quarter-rate 32-bit multiplies on this part, the two FP64 products ten full-rate instructions.
+// The targets of a block are shared out over `parts` workgroups, each of which forms the y_j again: one part per eight targets
+// (reading and scaling the sources is two thirds of a part's time, so the 8 x 8 blocks of the T basis run unsplit: 53 us against
+// 71 us in two parts and 114 us in four).
+template <int MAXS>
+__global__ __launch_bounds__(CONV_THREADS) void conv_kernel_split(ConvArgs a, int parts) {
+    const int blk = blockIdx.y / parts, part = blockIdx.y % parts;
+    const ConvBlock& __restrict__ b = a.blocks[blk];
+    const long x = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
+    const u64* in = a.in + (long)blockIdx.z * a.in_batch_stride;
+    u64* out = a.out + (long)blockIdx.z * a.out_batch_stride + (long)blk * a.out_block_stride;
+    const int nsrc = b.nsrc;
+    double yl[MAXS], yh[MAXS];
+    double vv = 0.0;
+#pragma unroll
+    for (int j = 0; j < MAXS; j++) {
+        yl[j] = yh[j] = 0.0;
+        if (j < nsrc) {
+            const u64 d = a.primes[b.src_prime[j]].q;
+            u64 xin = in[(long)b.src_limb[j] * a.N + x];
+            if (j < b.ncopy && part == 0) out[(long)b.copy_limb[j] * a.N + x] = xin;
+            xin += b.add_in[j];
+            const u64 y = mul_shoup(xin, b.hatinv[j], b.hatinv_s[j], d);
+            vv += (double)y / (double)d;
+            yl[j] = u2d(y & 0x7fffffffull);
+            yh[j] = u2d(y >> 31);
+        }
+    }
+    const double v = (double)(int)vv;
+    const int per = (b.ntgt + parts - 1) / parts, k_end = min(b.ntgt, (part + 1) * per);
+    for (int k = part * per; k < k_end; k++) {
+        const PrimeConst& pr = a.primes[b.tgt_prime[k]];
+        const double q = pr.qd, qinv = pr.qinv_d;
+        double acc = -mulmod_d(v, b.dmod_d[k], q, qinv);
+#pragma unroll
+        for (int j = 0; j < MAXS; j++)
+            if (j < nsrc) {
+                acc += mulmod_d(yl[j], b.hat_d[k][j], q, qinv) + mulmod_d(yh[j], b.hat31_d[k][j], q, qinv);
+                if ((j & 3) == 3) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
+            }
+        double r = canon_d(acc, q, qinv);
+        if (a.centred) {
+            r -= u2d(b.sub_out[k]);
+            r = r < 0.0 ? r + q : r;
+        }
+        out[(long)b.tgt_limb[k] * a.N + x] = d2u(r);
+    }
+}
+
 static int launch_conv(ckks_ctx* c, const ConvPlan& plan, u64* out, const u64* in, int batch, long in_bs, long out_bs,
                        long out_block_stride, int centred, int max_src) {
     if (plan.count == 0 || batch <= 0) return CKKS_OK;
@@ -129,6 +183,16 @@ static int launch_conv(ckks_ctx* c, const ConvPlan& plan, u64* out, const u64* i
         if (max_src <= 4) hipLaunchKernelGGL(conv_kernel_f64<4>, grid, block, 0, c->stream, a);
         else if (max_src <= 8) hipLaunchKernelGGL(conv_kernel_f64<8>, grid, block, 0, c->stream, a);
         else hipLaunchKernelGGL(conv_kernel_f64<CONV_MAX_SRC>, grid, block, 0, c->stream, a);
+        CKKS_HIP_TRY(hipGetLastError());
+        return CKKS_OK;
+    }
+    static const bool no_split = getenv("CKKS_CONV_INT") != nullptr;
+    if (plan.split_ok && c->arith_mode == 0 && !no_split) {
+        const int parts = plan.max_tgt <= 8 ? 1 : plan.max_tgt <= 16 ? 2 : 4;
+        grid.y *= parts;
+        if (max_src <= 4) hipLaunchKernelGGL(conv_kernel_split<4>, grid, block, 0, c->stream, a, parts);
+        else if (max_src <= 8) hipLaunchKernelGGL(conv_kernel_split<8>, grid, block, 0, c->stream, a, parts);
+        else hipLaunchKernelGGL(conv_kernel_split<CONV_MAX_SRC>, grid, block, 0, c->stream, a, parts);
         CKKS_HIP_TRY(hipGetLastError());
         return CKKS_OK;
     }

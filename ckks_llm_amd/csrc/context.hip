@@ -69,11 +69,17 @@ static void fill_conv_block(ckks::ConvBlock& b, const std::vector<u64>& pqt, con
     b.f64_ok = 1;
     for (int i : src) if (pqt[i] >= (1ull << 41)) b.f64_ok = 0;
     for (int i : tgt) if (pqt[i] >= (1ull << 41)) b.f64_ok = 0;
-    if (b.f64_ok) {
+    b.split_ok = 1;
+    for (int i : tgt) if (pqt[i] >= (1ull << 50)) b.split_ok = 0;
+    if (b.f64_ok)
         for (int j = 0; j < b.nsrc; j++) b.hatinv_d[j] = balanced_double(b.hatinv[j], sp[j]);
+    if (b.f64_ok || b.split_ok) {
         for (int k = 0; k < b.ntgt; k++) {
             const u64 r = pqt[tgt[k]];
-            for (int j = 0; j < b.nsrc; j++) b.hat_d[k][j] = balanced_double(b.hat[k][j], r);
+            for (int j = 0; j < b.nsrc; j++) {
+                b.hat_d[k][j] = balanced_double(b.hat[k][j], r);
+                b.hat31_d[k][j] = balanced_double(H::mulmod(b.hat[k][j], (1ull << 31) % r, r), r);
+            }
             b.dmod_d[k] = balanced_double(b.dmod[k], r);
         }
     }
@@ -314,6 +320,9 @@ extern "C" int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int 
         for (ckks::ConvPlan& pl : *plans) {
             pl.f64_ok = pl.count > 0;
             for (int b = 0; b < pl.count; b++) pl.f64_ok = pl.f64_ok && blocks[pl.first + b].f64_ok;
+            pl.split_ok = pl.count > 0;
+            for (int b = 0; b < pl.count; b++) pl.split_ok = pl.split_ok && blocks[pl.first + b].split_ok;
+            for (int b = 0; b < pl.count; b++) pl.max_tgt = std::max(pl.max_tgt, blocks[pl.first + b].ntgt);
         }
 
     // ---- upload ----

@@ -35,15 +35,19 @@ struct ConvBlock {
     u64 sub_out[CONV_MAX_TGT];                          // subtracted from the output residue (T -> PQ centring)
     short copy_prime[CONV_MAX_SRC], copy_limb[CONV_MAX_SRC];  // ncopy source limbs passed through unchanged
     int ncopy;
-    int f64_ok;                                         // every prime of the block is below 2^41: the FP64 tables below are filled
+    int f64_ok;                                         // every prime of the block is below 2^41: all FP64 tables below are filled
+    int split_ok;                                       // every TARGET prime is below 2^50: hat_d, hat31_d and dmod_d are filled
     double hatinv_d[CONV_MAX_SRC];                      // balanced representatives as doubles
     double hat_d[CONV_MAX_TGT][CONV_MAX_SRC];
+    double hat31_d[CONV_MAX_TGT][CONV_MAX_SRC];         // (D/d_j) 2^31 mod r_k: the factor of the upper part of a scaled residue split at bit 31
     double dmod_d[CONV_MAX_TGT];
 };
 
 struct ConvPlan {          // blocks of one map at one level, contiguous in device memory
     int first = 0, count = 0;
     bool f64_ok = false;   // all blocks can take the FP64 kernel
+    bool split_ok = false; // all blocks can take the kernel that scales in integers and sums in FP64
+    int max_tgt = 0;       // largest number of targets of a block
 };
 
 }  // namespace ckks

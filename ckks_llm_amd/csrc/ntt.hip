@@ -1204,7 +1204,8 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
 struct KsModDownArgs {
     const u64* in;               // two extended polynomials, coefficient domain: limb i < K modulo p_i, limb K + i modulo q_i
     long in_z_stride;            // words between the two polynomials
-    char* mid;                   // inter-pass buffer of the forward transform of the results, limb index i * 2 + z
+    char* mid;                   // where the first pass of the results' forward transform goes, in the form MID: limb (i, z) lies
+    long mid_stride_i, mid_stride_z;   //   at mid + i * mid_stride_i + z * mid_stride_z bytes
     const PrimeConst* primes;
     const double* tw_fwd;
     const u64* pHatVecModq;      // [q index][K]
@@ -1216,10 +1217,14 @@ struct KsModDownArgs {
 __device__ __forceinline__ double exact_u2d(u64 x) {                  // x < 2^52
     return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0;
 }
-__device__ __forceinline__ double canon_f(const F64Arith& ar, double r) {       // any |r| < 2^52 -> [0, q)
+template <class AR>
+__device__ __forceinline__ double canon_f(const AR& ar, double r) {               // any |r| < 2^52 -> [0, q)
     r = ar.balance(r);
     return r < 0.0 ? r + ar.q : r;
 }
+// With the wide arithmetic every constant enters balanced and at most 8 special primes are admitted: a term of the sum lies within
+// 0.88 q of zero (its operand, a residue modulo p_i, may be up to twice q), so eight of them stay below 2^53.
+template <class AR, class MID>
 __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
@@ -1229,7 +1234,7 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
     const unsigned tile = blockIdx.y, limb = blockIdx.x, iq = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const unsigned cl = tid % CW, g = tid / CW;
     const int prime = a.K + (int)iq;
-    const F64Arith ar(a.primes[prime]);
+    const AR ar(a.primes[prime]);
     const u64* col = a.in + (long)z * a.in_z_stride + tile * CW + cl;
     double acc[R];
 #pragma unroll
@@ -1239,8 +1244,8 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 #pragma unroll
     for (int j = 0; j < R; j++) x[j] = col[(long)(g + j * G) * N2];
     for (int i = 0; i < a.K; i++) {
-        const F64Arith ap(a.primes[i]);
-        const double hinv = exact_u2d(a.pHatInv[i]), hat = exact_u2d(a.pHatVecModq[(long)iq * a.K + i]);
+        const AR ap(a.primes[i]);
+        const double hinv = ap.from_canonical(a.pHatInv[i]), hat = ar.from_canonical(a.pHatVecModq[(long)iq * a.K + i]);
         const u64* nl = col + (long)(i + 1 < a.K ? i + 1 : prime) * N;
 #pragma unroll
         for (int j = 0; j < R; j++) xn[j] = nl[(long)(g + j * G) * N2];
@@ -1254,19 +1259,21 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 #pragma unroll
         for (int j = 0; j < R; j++) x[j] = xn[j];
     }
-    const double pinv = exact_u2d(a.PinvModq[iq]);
+    const double pinv = ar.from_canonical(a.PinvModq[iq]);
     double v[R];
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = ar.mulmod(ar.q - canon_f(ar, acc[j]) + exact_u2d(x[j]), pinv);      // in (-0.51 q, 0.51 q)
     const double* tw = a.tw_fwd + (long)prime * N;
-    fwd_spread<F64Arith, 8, S1>(v, tw, 1u, ar);
+    ar.round_end(v);
+    fwd_spread<AR, 8, S1>(v, tw, 1u, ar);
+    ar.round_end(v);
 #pragma unroll
     for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
-    fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
-    mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
+    fwd_packed<AR, 8, S1>(v, tw, 1u, g, ar);
+    MID::store_columns(a.mid + iq * a.mid_stride_i + z * a.mid_stride_z, tile, g, cl, v, ar);
 }
 
 // The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
@@ -1674,19 +1681,32 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
                             bool* done) {
     *done = false;
-    if (c->p_num <= 0 || l < 0 || l > c->L || !stage_fusion_applies(c, 0, c->K + l + 1)) return CKKS_OK;
+    const int form = c->p_num <= 0 || l < 0 || l > c->L ? 0 : stage_fusion_form(c, 0, c->K + l + 1);
+    if (form == 0 || (form == 2 && c->K > 8)) return CKKS_OK;
     const int limbs = 2 * (l + 1);
-    int rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES);
-    if (rc) return rc;
+    const long N = c->N;
     KsModDownArgs m;
-    m.in = (const u64*)in; m.in_z_stride = in_z_stride; m.mid = (char*)c->d_ntt_mid; m.primes = c->d_primes; m.tw_fwd = c->d_twd_fwd;
+    m.in = (const u64*)in; m.in_z_stride = in_z_stride; m.primes = c->d_primes; m.tw_fwd = c->d_twd_fwd;
     m.pHatVecModq = c->d_pHatVecModq; m.pHatInv = c->d_pHatInvVecModp; m.PinvModq = c->d_PinvModq; m.K = c->K; m.pre_scaled = pre_scaled ? 1 : 0;
-    hipLaunchKernelGGL(ks_moddown_strided_kernel, dim3(limbs, StridedCfg<8, 8>::TILES), dim3(256), 0, c->stream, m);
     NttArgs args;
     args.data = (u64*)out; args.primes = c->d_primes; args.tw = c->d_twd_fwd;
     args.start_poly_idx = 0; args.start_mod_idx = c->K; args.poly_num = 2; args.mod_num = l + 1; args.poly_mod_len = out_poly_mod_len;
-    args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)limbs; args.mid = (char*)c->d_ntt_mid;
-    hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), dim3(RowCfg<8, 8>::TILES, limbs), dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+    args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)limbs;
+    const dim3 gs(limbs, StridedCfg<8, 8>::TILES), gr(RowCfg<8, 8>::TILES, limbs);
+    if (form == 1) {
+        int rc = ensure_mid(c, (size_t)limbs * MidPieces::LIMB_BYTES);
+        if (rc) return rc;
+        m.mid = (char*)c->d_ntt_mid; m.mid_stride_i = 2 * MidPieces::LIMB_BYTES; m.mid_stride_z = MidPieces::LIMB_BYTES;
+        args.mid = (char*)c->d_ntt_mid;
+        hipLaunchKernelGGL((ks_moddown_strided_kernel<F64Arith, MidPieces>), gs, dim3(256), 0, c->stream, m);
+        hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+    } else {
+        // wide primes: the first pass writes the output limbs themselves, as an in-place transform leaves them between its passes
+        m.mid = (char*)out; m.mid_stride_i = N * (long)sizeof(u64); m.mid_stride_z = (long)out_poly_mod_len * N * (long)sizeof(u64);
+        args.mid = nullptr;
+        hipLaunchKernelGGL((ks_moddown_strided_kernel<F64WideArith, MidLimb>), gs, dim3(256), 0, c->stream, m);
+        hipLaunchKernelGGL((ntt_row_pass<F64WideArith, 8, 8, false, false>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+    }
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
     return CKKS_OK;

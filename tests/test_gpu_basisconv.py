@@ -116,11 +116,15 @@ def test_external_product_and_keyswitch_23(params):
         assert np.array_equal(from_dev(do, wout.shape)[:, :l + 1], wout[:, :l + 1]), ("keyswitch_23", l)
 
 
-def test_keyswitch_23_full_ring_small_special_primes():
-    """The T-basis switch at N = 2^16 with P and Q primes below 2^39 (36- and 37-bit primes, the reference's 60-bit T primes): at this
-    size its ModDown runs inside the first pass of the final transform; same words as the oracle's separate steps, and as the
-    device's own separate steps (ntt mode 1)."""
+@pytest.mark.parametrize("primes", ["36", "49"])
+def test_keyswitch_23_full_ring(primes):
+    """The T-basis switch at N = 2^16 with the reference's 60-bit T primes over P and Q primes below 2^39 (36- and 37-bit) and over
+    the reference's own 49- and 50-bit P and Q primes: at this size its ModDown runs inside the first pass of the final transform
+    (handing over 5-byte values below 2^39, whole limbs on the wide FP64 arithmetic above); same words as the oracle's separate
+    steps, and as the device's own separate steps (ntt mode 1)."""
     q, p, t = CFG2_Q[:6], CFG3_P[:2], REF_PARAMS[16]["t"][:3]      # q_num a multiple of p_num, as in every set of the reference
+    if primes == "49":
+        q, p = REF_PARAMS[16]["q"][:6], REF_PARAMS[16]["p"][:2]
     pair = Pair(16, p, q, t, 3)
     o, d, N = pair.orc, pair.dev, pair.N
     Q, T, RB, QB, dnum, L = o.q_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum, o.dnum, o.L
@@ -235,15 +239,22 @@ def test_hybrid_keyswitch_stages(logN, nq, np_, arith_mode):
         assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), ("keyswitch", l)
 
 
-@pytest.mark.parametrize("nq,np_,l", [(24, 6, 23), (24, 6, 9), (5, 2, 4), (3, 1, 2), (3, 1, 0), (7, 3, 3)])
-def test_config3_full_size_keyswitch(nq, np_, l):
+@pytest.mark.parametrize("nq,np_,l,primes", [(24, 6, 23, "36"), (24, 6, 9, "36"), (5, 2, 4, "36"), (3, 1, 2, "36"), (3, 1, 0, "36"), (7, 3, 3, "36"),
+                                             (5, 2, 4, "49"), (3, 1, 2, "49"), (8, 4, 7, "49"), (4, 2, 3, "mixed")])
+def test_config3_full_size_keyswitch(nq, np_, l, primes):
     """BASELINE config 3 at full size: N = 2^16, 24 Q + 6 P primes, dnum = 4, seed 3; parity with the oracle on the
     whole switch output (every residue), at the top level and at a level whose last digit is partial (10 limbs in digits of 6);
     then smaller prime sets at the same ring size: a partial last digit at the top level, one special prime (digits of one prime, the
     ModDown's single-prime branch), level 0, and a level that leaves whole digits unused.
     At this ring size the middle of the switch (row passes of both transforms around the inner product) is one launch; the
-    same call with the transforms forced to two launches each (ntt mode 1) takes the separate steps and must give the same words."""
+    same call with the transforms forced to two launches each (ntt mode 1) takes the separate steps and must give the same words.
+    On the reference's 49- and 50-bit primes (and on a chain that mixes widths) only the end of the switch is fused: the ModDown
+    inside the first pass of the last transform, on the wide FP64 arithmetic."""
     q, p = CFG2_Q[:nq], CFG3_P[:np_]
+    if primes == "49":
+        q, p = REF_PARAMS[16]["q"][:nq], REF_PARAMS[16]["p"][:np_]
+    elif primes == "mixed":
+        q, p = CFG2_Q[:2] + REF_PARAMS[16]["q"][:nq - 2], [CFG3_P[0]] + REF_PARAMS[16]["p"][:np_ - 1]
     pair = Pair(16, p, q)
     o, d, N = pair.orc, pair.dev, pair.N
     W = nq + np_
