@@ -142,7 +142,7 @@ class Context_23:
     def set_ntt_mode(self, mode):
         """0: automatic, 1: two launches per transform (data in place between them), 2: chained one-launch transform
         (N >= 2^15), 3: one workgroup per limb (N >= 2^15), 4: paired one-launch transform (N = 2^16; what mode 0 takes for
-        batches of up to 40 limbs), 5: as 4 with a limb's tiles spread over all XCDs.  All give the same residues."""
+        batches of up to 128 limbs), 5: as 4 with a limb's tiles spread over all XCDs (mode 0 above 40 limbs).  All give the same residues."""
         _check(self.L_.ckks_ctx_set_ntt_mode(self.h, mode), "ckks_ctx_set_ntt_mode")
 
     def set_ntt_chain(self, skew=0, spin_max=-1):

@@ -434,6 +434,7 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
 // test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = chained one-launch transform wherever that kernel exists
 // (N >= 2^15), 3 = one workgroup per limb wherever that kernel exists (N >= 2^15), 4 = paired one-launch transform at every batch
 // size (N = 2^16; the automatic mode takes it for small batches), 5 = the same with the tiles of a limb spread over all XCDs
+// (the automatic mode's choice between 41 and 128 limbs)
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
     if (!c || mode < 0 || mode > 5) return CKKS_E_INVALID;
     c->ntt_mode = mode;

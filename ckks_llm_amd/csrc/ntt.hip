@@ -810,13 +810,14 @@ __global__ __launch_bounds__(256) void ntt_chain_finish_kernel(NttArgs a, ChainA
 // ------------------------------------------------------------------------------------------------------------
 constexpr unsigned PAIR_XCDS = 8;
 constexpr int PAIR_MAX_LIMBS = 4096;               // completion words per context
+constexpr int PAIR_GROUPED_LIMBS = 40;             // ... and up to this many with a limb's tiles on one XCD, above it spread over all
 constexpr int PAIR_WORD_STRIDE = 32;               // one completion word per 128-byte line: atomics on one line are carried out one after the other
-constexpr int PAIR_AUTO_LIMBS = 40;                // automatic mode: batches up to this many limbs take the paired kernel
+constexpr int PAIR_AUTO_LIMBS = 128;                // automatic mode: batches up to this many limbs take the paired kernel
 struct PairArgs {
     unsigned* done;            // [limb * PAIR_WORD_STRIDE] first-pass completion count, a multiple of TILES between launches
     unsigned* fail;            // host-visible word: nonzero once a wait has run out
     unsigned limbs, spin_max;
-    unsigned spread;           // test setting: the tiles of a limb go to consecutive workgroups, i.e. to all XCDs
+    unsigned spread;           // the tiles of a limb go to consecutive workgroups, i.e. to all XCDs (larger batches, and a test setting)
 };
 template <class AR, int SA, int SB, bool INVERSE, bool COMPACT>
 __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
@@ -890,7 +891,7 @@ static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool 
     PairArgs p;
     p.done = (unsigned*)c->d_ntt_pair; p.fail = c->h_pair_fail; p.limbs = (unsigned)limbs;
     p.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
-    p.spread = c->ntt_mode == 5 ? 1u : 0u;
+    p.spread = c->ntt_mode == 5 || (c->ntt_mode == 0 && limbs > PAIR_GROUPED_LIMBS) ? 1u : 0u;
     const unsigned blocks = ((unsigned)limbs + PAIR_XCDS - 1) / PAIR_XCDS * PAIR_XCDS * StridedCfg<SA, SB>::TILES;
     const dim3 g(blocks), b(256);
     if constexpr (CAN_COMPACT) {
@@ -1042,8 +1043,10 @@ static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse)
 }
 
 // Whether a transform of `limbs` limbs runs as the paired kernel: always in modes 4 and 5 while its completion words suffice, in
-// the automatic mode up to the batch at which two launches are as fast (measured: 15 us against 22 us at 32 limbs, level at 48;
-// CKKS_NTT_PAIR_MAX overrides that limit).
+// the automatic mode up to the batch at which two launches are as fast (CKKS_NTT_PAIR_MAX overrides that limit).  Measured
+// against two launches: with a limb's tiles on one XCD 9.5 us against 15.7 us at 16 limbs, 15 against 22.5 at 32, level at 48 and
+// behind above; with the tiles spread over the XCDs 14.4 us at 16 limbs, 20.5 against 22.5 at 48, 34.8 against 36 at 96,
+// 49.5 against 48 at 144.  Hence: one XCD per limb up to 40 limbs, spread from there to 128.
 static bool pair_applies(const ckks_ctx* c, int limbs) {
     static const int max_env = getenv("CKKS_NTT_PAIR_MAX") ? atoi(getenv("CKKS_NTT_PAIR_MAX")) : -1;
     if (limbs > PAIR_MAX_LIMBS || c->cu_count < 64) return false;            // the progress argument needs more than 128 resident workgroups

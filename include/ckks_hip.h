@@ -69,8 +69,8 @@ int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
  * the limb stays in that XCD's L2 in between (N >= 2^15; other rings take two launches), plus a small finishing launch;
  * 3: one workgroup carries a limb through both passes (N >= 2^15); 4: paired - both passes in one launch of one workgroup per
  * (limb, tile), which waits between its two tiles until the limb's first pass is complete (N = 2^16, up to 4096 limbs; mode 0
- * takes this form for batches of up to 40 limbs, where it is faster than two launches); 5: as 4 with the tiles of a limb spread
- * over all XCDs (a test setting).  All give the same residues.  Should a wait of the paired form ever run out (about two
+ * takes this form for batches of up to 128 limbs, where it is faster than two launches); 5: as 4 with the tiles of a limb spread
+ * over all XCDs (what mode 0 does above 40 limbs).  All give the same residues.  Should a wait of the paired form ever run out (about two
  * seconds), the transform's output is incomplete, ckks_ctx_check and every later transform of the context return CKKS_E_UNAVAILABLE.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);

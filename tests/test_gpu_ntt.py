@@ -227,13 +227,13 @@ def test_whole_limb_transform_matches_oracle(logN, polys, mode):
 
 
 @pytest.mark.parametrize("primes,polys,arith,mode", [("36", 9, 0, 4), ("36", 5, 1, 4), ("49", 3, 0, 4), ("mixed", 2, 0, 4), ("36", 1, 0, 4),
-                                                    ("36", 7, 0, 5), ("49", 2, 0, 5), ("36", 3, 1, 5), ("36", 8, 0, 0)])
+                                                    ("36", 7, 0, 5), ("49", 2, 0, 5), ("36", 3, 1, 5), ("36", 8, 0, 0), ("36", 11, 0, 0)])
 def test_paired_transform_matches_oracle(primes, polys, arith, mode):
     """The paired transform (both passes in one launch, a workgroup per (limb, tile) that waits between its two tiles for the
     limb's first pass) against the oracle: 5-byte and in-place inter-pass forms, all three arithmetic back ends, limb counts
     that are no multiple of eight, several launches in a row on the same completion words, the reference's sub-range
     addressing.  Mode 5 spreads the tiles of a limb over all XCDs, so that what one pass hands to the other really crosses
-    from one L2 to another; mode 0 with 40 limbs is the automatic choice of this form."""
+    from one L2 to another; mode 0 with 40 and with 55 limbs is the automatic choice of the two numberings."""
     q = {"36": CFG2_Q[:5], "49": REF_PARAMS[16]["q"][:5], "mixed": CFG2_Q[:2] + REF_PARAMS[16]["q"][:2] + REF_PARAMS[16]["t"][:1]}[primes]
     pair = Pair(16, [], q)
     N, L1 = pair.N, len(q)
