@@ -138,6 +138,35 @@ def bench_ntt_ref_primes(P, cts=27, reps=10):
     return res
 
 
+def bench_small_batches(P, reps=100):
+    """Forward transform of small batches at N = 2^16 (24 primes below 2^36): the automatic launch form (the paired one-launch
+    kernel up to 128 limbs), the paired kernel with a limb's tiles on one XCD and spread over the XCDs, and two launches.
+    Times are per call from HIP events around `reps` calls in a row; the 8-limb line is bound by the host's launch rate."""
+    from ckks_llm_amd import Context_23, DeviceBuffer
+    q = list(P.CFG2_Q[:8])
+    N, L1 = 1 << 16, len(q)
+    ctx = Context_23(16, [], q)
+    rng = np.random.default_rng(7)
+    one = np.stack([rng.integers(0, m, N, dtype=np.uint64) for m in q])
+    rows = []
+    for polys in (1, 2, 3, 4, 5, 6, 8, 12, 18):
+        buf = DeviceBuffer.from_numpy(np.tile(one, (polys, 1)))
+        row = {"limbs": polys * L1}
+        for name, mode in (("automatic_us", 0), ("paired_one_xcd_us", 4), ("paired_spread_us", 5), ("two_launches_us", 1)):
+            ctx.set_ntt_mode(mode)
+            for _ in range(5):
+                ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+            ctx.timer_start()
+            for _ in range(reps):
+                ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+            row[name] = round(ctx.timer_stop() / reps * 1e3, 1)
+        ctx.check()
+        rows.append(row)
+        buf.free()
+    ctx.set_ntt_mode(0)
+    return {"workload": "forward NTT of small batches, N=2^16, 8 primes <2^36 x 1..18 polynomials", "rows": rows}
+
+
 def bench_mult_23(P, reps=10):
     """Scheme_23::mult_23 (KeySwitch_23.cuh:192-236) on the reference's own logN = 16 parameter set at the top level: tensor product,
     key switch through the T basis with a relinearisation key generated on the device, the two additions."""
@@ -427,7 +456,7 @@ def run(P, traffic_info=({}, "")):
     ref_scale_label = ("PPMM 768x768 as the reference's BERT layer calls it: its two 49-bit ring-pack moduli and its scaler q1 * 2^49 / scale "
                        "with scale = 2^49 (PPMM_kernel.cuh:283-284), i.e. 46-bit plaintext entries, N=2^16, 128 tokens")
     res = {"ppmm": bench_ppmm(P), "ppmm_ref_primes": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_label),
-            "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "ntt_ref_primes": bench_ntt_ref_primes(P), "mult_23_ref_params": bench_mult_23(P),
+            "ppmm_ref_primes_ref_scaler": bench_ppmm(P, L=2, primes=P.REF_PARAMS[16]["q"], label=ref_scale_label, scaler=float(P.REF_PARAMS[16]["q"][1])), "ppmm_4096": bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused(P), "keyswitch": bench_keyswitch(P), "rescale": bench_rescale(P), "ntt_ref_primes": bench_ntt_ref_primes(P), "small_batches": bench_small_batches(P), "mult_23_ref_params": bench_mult_23(P),
             "decompose": bench_decompose(P), "packing": bench_packing(P), "hoisted_level": bench_hoisted_level(P)}
     with_traffic(res["keyswitch"], "hybrid_keyswitch_config3", traffic, res["keyswitch"]["us"] * 1e-6)
     with_traffic(res["rescale"], "rescale_one_ciphertext_level23", traffic, res["rescale"]["us"] * 1e-6)
@@ -441,7 +470,8 @@ def run(P, traffic_info=({}, "")):
 
 LEGS = {"ppmm": lambda P: bench_ppmm(P), "ppmm_4096": lambda P: bench_ppmm(P, M=4096, Kin=4096, reps=2), "pcmm_layer": bench_pcmm_fused,
         "keyswitch": bench_keyswitch, "rescale": bench_rescale, "ntt_ref_primes": bench_ntt_ref_primes, "mult_23_ref_params": bench_mult_23, "decompose": bench_decompose,
-        "packing": bench_packing, "hoisted_level": bench_hoisted_level, "cpu_ppmm": cpu_ppmm, "cpu_keyswitch": cpu_keyswitch}
+        "packing": bench_packing, "hoisted_level": bench_hoisted_level, "cpu_ppmm": cpu_ppmm, "cpu_keyswitch": cpu_keyswitch,
+        "small_batches": bench_small_batches}
 
 if __name__ == "__main__":
     # one leg on its own, for profiling:  python3 bench_extra.py keyswitch

@@ -244,6 +244,7 @@ struct NttArgs {
     unsigned limb_base, limbs_total;      // this launch covers limbs limb_base .. limb_base + gridDim.y - 1 of limbs_total
     char* mid;                            // compact inter-pass buffer (MID_LIMB_BYTES per limb of the launch) or nullptr
     int reverse = 0;                      // take the limbs of the launch from the last to the first (see launch_passes)
+    long out_delta = 0;                   // paired transform with the 5-byte inter-pass form: its second pass writes out_delta words behind data
     // Forward transforms of polynomials that exist only as scattered MLWE samples (the embedding of the ring packing): when
     // embed_mlwe is set the first pass takes coefficient pos of polynomial y from sample (pos mod k) / gap, coefficient
     // pos / k (zero where pos mod k is no multiple of gap), lifted around zero from q0 to p0 on the limbs of the first prime.
@@ -857,6 +858,7 @@ __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     }
     __syncthreads();
     if (!go) return;
+    if (COMPACT) limb += a.out_delta;
     if (!INVERSE) row_tile<AR, SA, SB, false, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
     else strided_tile<AR, SA, SB, true, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
 }
@@ -876,7 +878,7 @@ int ntt_pair_init(ckks_ctx* c) {
 int ntt_pair_failed(const ckks_ctx* c) { return c->h_pair_fail && *(volatile unsigned*)c->h_pair_fail ? 1 : 0; }
 
 template <class AR, int SA, int SB>
-static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok) {
+static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, char* mid = nullptr) {
     constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
     int rc = ntt_pair_init(c);
     if (rc) return rc;
@@ -884,7 +886,9 @@ static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool 
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
     args.mid = nullptr;
-    if (compact) {
+    if (compact && mid) {
+        args.mid = mid;                                   // the caller's inter-pass area
+    } else if (compact) {
         if ((rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES))) return rc;
         args.mid = (char*)c->d_ntt_mid;
     }
@@ -1400,9 +1404,17 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     args.start_poly_idx = 0; args.start_mod_idx = P; args.poly_num = 1; args.mod_num = l + 1; args.poly_mod_len = Q;
     args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)(l + 1);
     args.data = (u64*)in_ntt;
-    hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, true, true>), dim3(CR::TILES, l + 1), dim3(CR::THREADS), 0, c->stream, args);
-    args.data = (u64*)work; args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
-    hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, l + 1), dim3(CS::THREADS), 0, c->stream, args);
+    if (pair_applies(c, l + 1)) {
+        // one launch: the constants that differ between the two tables (N^-1 and the last twiddle) only enter the second pass
+        args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
+        args.out_delta = (long)((u64*)work - (u64*)in_ntt);
+        if ((rc = launch_pair<F64Arith, 8, 8>(c, args, l + 1, true, true, mid))) return rc;
+        args.out_delta = 0;
+    } else {
+        hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, true, true>), dim3(CR::TILES, l + 1), dim3(CR::THREADS), 0, c->stream, args);
+        args.data = (u64*)work; args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
+        hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, l + 1), dim3(CS::THREADS), 0, c->stream, args);
+    }
     // quotient estimates, then the conversion inside the first pass of the digits' forward transform
     KsModUpArgs u;
     u.y = (const u64*)work; u.v = (signed char*)(work + (size_t)(l + 1) * N); u.mid = mid; u.blocks = c->d_conv + plan.first;
