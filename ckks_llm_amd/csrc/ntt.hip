@@ -330,12 +330,13 @@ __device__ __forceinline__ void mid_store_row_inverse(char* mid_limb, unsigned r
 struct MidPieces {
     static constexpr long LIMB_BYTES = MID_LIMB_BYTES;
     struct Raw { unsigned lo[16], hi[16]; };
-    template <class AR>
+    template <class AR, bool SHARED = false>
     static __device__ __forceinline__ void store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const double (&v)[16], const AR& ar) {
-        mid_store_columns(mid_limb, cb, g, cl, v, ar);
+        mid_store_columns<AR, SHARED>(mid_limb, cb, g, cl, v, ar);
     }
+    template <bool SHARED = false>
     static __device__ __forceinline__ void request(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, Raw& r) {
-        mid_load_row_raw(mid_limb, rb, rl, u, r.lo, r.hi);
+        mid_load_row_raw<SHARED>(mid_limb, rb, rl, u, r.lo, r.hi);
     }
     template <class AR>
     static __device__ __forceinline__ double decode(const AR& ar, const Raw& r, int j, unsigned rl) { return mid_decode_row(ar, r.lo[j], r.hi[j], rl); }
@@ -343,16 +344,17 @@ struct MidPieces {
 struct MidLimb {
     static constexpr long LIMB_BYTES = 65536l * 8;
     struct Raw { u64 w[16]; };
-    template <class AR>
+    template <class AR, bool SHARED = false>
     static __device__ __forceinline__ void store_columns(char* mid_limb, unsigned cb, unsigned g, unsigned cl, const double (&v)[16], const AR& ar) {
         u64* col = reinterpret_cast<u64*>(mid_limb) + cb * 16 + cl;
 #pragma unroll
-        for (int j = 0; j < 16; j++) col[(long)(g * 16 + j) * 256] = ar.to_mid_fwd(v[j]);
+        for (int j = 0; j < 16; j++) put<SHARED>(col + (long)(g * 16 + j) * 256, ar.to_mid_fwd(v[j]));
     }
+    template <bool SHARED = false>
     static __device__ __forceinline__ void request(const char* mid_limb, unsigned rb, unsigned rl, unsigned u, Raw& r) {
         const u64* row = reinterpret_cast<const u64*>(mid_limb) + (long)(rb * 16 + rl) * 256 + u;
 #pragma unroll
-        for (int j = 0; j < 16; j++) r.w[j] = row[j * 16];
+        for (int j = 0; j < 16; j++) r.w[j] = get<SHARED>(row + j * 16);
     }
     template <class AR>
     static __device__ __forceinline__ double decode(const AR& ar, const Raw& r, int j, unsigned) { return ar.from_mid(r.w[j]); }
@@ -820,6 +822,32 @@ struct PairArgs {
     unsigned limbs, spin_max;
     unsigned spread;           // the tiles of a limb go to consecutive workgroups, i.e. to all XCDs (larger batches, and a test setting)
 };
+// (limb, tile) of workgroup b of a paired launch
+__device__ __forceinline__ void pair_block(const PairArgs& p, unsigned b, unsigned tiles, unsigned& limb_id, unsigned& tile) {
+    const unsigned idx = b / PAIR_XCDS;
+    limb_id = p.spread ? b / tiles : b % PAIR_XCDS + PAIR_XCDS * (idx / tiles);
+    tile = p.spread ? b % tiles : idx % tiles;
+}
+// Between the two tiles of a workgroup: this workgroup's shared stores are complete, the limb's count moves, and the workgroup
+// waits for the count to read a multiple of `tiles`.  false: the wait ran out (the failure word is raised), the caller leaves.
+__device__ __forceinline__ bool pair_hand_over(const PairArgs& p, unsigned limb_id, unsigned tiles, unsigned* go) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);                                              // every shared store of this wave has been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned* word = p.done + (size_t)limb_id * PAIR_WORD_STRIDE;
+        (void)__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned ok = 0;
+        for (unsigned n = 0; n < p.spin_max; n++) {
+            if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) % tiles == 0) { ok = 1; break; }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (!ok) __hip_atomic_store(p.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        *go = ok;
+    }
+    __syncthreads();
+    return *go != 0;
+}
 template <class AR, int SA, int SB, bool INVERSE, bool COMPACT>
 __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     typedef StridedCfg<SA, SB> CS;
@@ -831,9 +859,8 @@ __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     typedef typename AR::TW TW;
     __shared__ typename AR::V lds[LDS_WORDS];
     __shared__ unsigned go;
-    const unsigned idx = blockIdx.x / PAIR_XCDS;
-    const unsigned limb_id = p.spread ? blockIdx.x / TILES : blockIdx.x % PAIR_XCDS + PAIR_XCDS * (idx / TILES);
-    const unsigned tile = p.spread ? blockIdx.x % TILES : idx % TILES;
+    unsigned limb_id, tile;
+    pair_block(p, blockIdx.x, TILES, limb_id, tile);
     if (limb_id >= p.limbs) return;                                             // uniform over the workgroup
     int prime;
     u64* limb = limb_ptr(a, limb_id, N, prime);
@@ -842,22 +869,7 @@ __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     char* mid_limb = COMPACT ? a.mid + (long)limb_id * MID_LIMB_BYTES : nullptr;
     if (!INVERSE) strided_tile<AR, SA, SB, false, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
     else row_tile<AR, SA, SB, true, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);                                              // every shared store of this wave has been acknowledged
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned* word = p.done + (size_t)limb_id * PAIR_WORD_STRIDE;
-        (void)__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned ok = 0;
-        for (unsigned n = 0; n < p.spin_max; n++) {
-            if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) % TILES == 0) { ok = 1; break; }
-            __builtin_amdgcn_s_sleep(4);
-        }
-        if (!ok) __hip_atomic_store(p.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        go = ok;
-    }
-    __syncthreads();
-    if (!go) return;
+    if (!pair_hand_over(p, limb_id, TILES, &go)) return;
     if (COMPACT) limb += a.out_delta;
     if (!INVERSE) row_tile<AR, SA, SB, false, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
     else strided_tile<AR, SA, SB, true, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
@@ -877,6 +889,15 @@ int ntt_pair_init(ckks_ctx* c) {
 }
 int ntt_pair_failed(const ckks_ctx* c) { return c->h_pair_fail && *(volatile unsigned*)c->h_pair_fail ? 1 : 0; }
 
+static PairArgs pair_args(const ckks_ctx* c, int limbs) {
+    PairArgs p;
+    p.done = (unsigned*)c->d_ntt_pair; p.fail = c->h_pair_fail; p.limbs = (unsigned)limbs;
+    p.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
+    p.spread = c->ntt_mode == 5 || (c->ntt_mode == 0 && limbs > PAIR_GROUPED_LIMBS) ? 1u : 0u;
+    return p;
+}
+static unsigned pair_blocks(int limbs, unsigned tiles) { return ((unsigned)limbs + PAIR_XCDS - 1) / PAIR_XCDS * PAIR_XCDS * tiles; }
+
 template <class AR, int SA, int SB>
 static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, char* mid = nullptr) {
     constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
@@ -892,11 +913,8 @@ static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool 
         if ((rc = ensure_mid(c, (size_t)limbs * MID_LIMB_BYTES))) return rc;
         args.mid = (char*)c->d_ntt_mid;
     }
-    PairArgs p;
-    p.done = (unsigned*)c->d_ntt_pair; p.fail = c->h_pair_fail; p.limbs = (unsigned)limbs;
-    p.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
-    p.spread = c->ntt_mode == 5 || (c->ntt_mode == 0 && limbs > PAIR_GROUPED_LIMBS) ? 1u : 0u;
-    const unsigned blocks = ((unsigned)limbs + PAIR_XCDS - 1) / PAIR_XCDS * PAIR_XCDS * StridedCfg<SA, SB>::TILES;
+    const PairArgs p = pair_args(c, limbs);
+    const unsigned blocks = pair_blocks(limbs, StridedCfg<SA, SB>::TILES);
     const dim3 g(blocks), b(256);
     if constexpr (CAN_COMPACT) {
         if (compact) {
@@ -1599,13 +1617,13 @@ struct RescaleArgs {
     const u64* inv;              // q_l^-1 mod q_i, i < l
     int l, poly_mod_len, prime0; // limb i is modulo prime prime0 + i
 };
-template <class AR, class MID>
-__global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
+// SHARED: the two tiles are the halves of one paired launch (what the first hands to the second moves as shared accesses)
+template <class AR, class MID, bool SHARED>
+__device__ __forceinline__ void rescale_strided_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     constexpr long N = 1l << 16;
-    __shared__ double lds[C::LDS_WORDS];
-    const unsigned tile = blockIdx.y, limb = blockIdx.x, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
+    const unsigned i = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const unsigned cl = tid % CW, g = tid / CW;
     const int prime = a.prime0 + (int)i;
     const AR ar(a.primes[prime]);
@@ -1622,15 +1640,14 @@ __global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<AR, 8, S1>(v, tw, 1u, g, ar);
-    MID::store_columns(a.mid + (long)limb * MID::LIMB_BYTES, tile, g, cl, v, ar);
+    MID::template store_columns<AR, SHARED>(a.mid + (long)limb * MID::LIMB_BYTES, tile, g, cl, v, ar);
 }
-template <class AR, class MID>
-__global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
+template <class AR, class MID, bool SHARED>
+__device__ __forceinline__ void rescale_row_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds) {
     typedef RowCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     constexpr long N = 1l << 16;
-    __shared__ double lds[C::LDS_WORDS];
-    const unsigned tile = blockIdx.x, limb = blockIdx.y, i = limb >> 1, z = limb & 1, tid = threadIdx.x;
+    const unsigned i = limb >> 1, z = limb & 1, tid = threadIdx.x;
     const int prime = a.prime0 + (int)i;
     const AR ar(a.primes[prime]);
     const double* tw = a.tw_fwd + (long)prime * N;
@@ -1640,7 +1657,7 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
     const unsigned tw_off = N1 + row;
     u64* rp = a.cipher + ((long)z * a.poly_mod_len + i) * N + (long)row * N2 + u;
     typename MID::Raw raw;
-    MID::request(a.mid + (long)limb * MID::LIMB_BYTES, tile, rl, u, raw);
+    MID::template request<SHARED>(a.mid + (long)limb * MID::LIMB_BYTES, tile, rl, u, raw);
     u64 c[R];                                            // the limb's own words, needed after the butterflies
 #pragma unroll
     for (int j = 0; j < R; j++) c[j] = rp[j * U];
@@ -1666,6 +1683,31 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
         rp[j * U] = ar.canon(ar.mulmod(exact_u2d(c[j]) - x, inv));          // |c - x| < 1.5 q
     }
 }
+template <class AR, class MID>
+__global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
+    __shared__ double lds[StridedCfg<8, 8>::LDS_WORDS];
+    rescale_strided_tile<AR, MID, false>(a, blockIdx.x, blockIdx.y, lds);
+}
+template <class AR, class MID>
+__global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
+    __shared__ double lds[RowCfg<8, 8>::LDS_WORDS];
+    rescale_row_tile<AR, MID, false>(a, blockIdx.y, blockIdx.x, lds);
+}
+// both in one launch, paired like ntt_pair_kernel
+template <class AR, class MID>
+__global__ __launch_bounds__(256) void rescale_pair_kernel(RescaleArgs a, PairArgs p) {
+    constexpr int LDS_WORDS = StridedCfg<8, 8>::LDS_WORDS > RowCfg<8, 8>::LDS_WORDS ? StridedCfg<8, 8>::LDS_WORDS : RowCfg<8, 8>::LDS_WORDS;
+    constexpr unsigned TILES = StridedCfg<8, 8>::TILES;
+    static_assert(TILES == RowCfg<8, 8>::TILES, "tile counts");
+    __shared__ double lds[LDS_WORDS];
+    __shared__ unsigned go;
+    unsigned limb, tile;
+    pair_block(p, blockIdx.x, TILES, limb, tile);
+    if (limb >= p.limbs) return;
+    rescale_strided_tile<AR, MID, true>(a, limb, tile, lds);
+    if (!pair_hand_over(p, limb, TILES, &go)) return;
+    rescale_row_tile<AR, MID, true>(a, limb, tile, lds);
+}
 // cipher: [2][poly_mod_len] limbs over q_0 .. (prime indices K + i); limb l already in the coefficient domain.
 // *done = false (nothing launched) where it does not apply.
 int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done) {
@@ -1679,7 +1721,12 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
     r.cipher = (u64*)cipher; r.mid = (char*)c->d_ntt_mid; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd; r.inv = (const u64*)inv;
     r.l = l; r.poly_mod_len = c->L + 1; r.prime0 = c->K;
     const dim3 gs(limbs, StridedCfg<8, 8>::TILES), gr(RowCfg<8, 8>::TILES, limbs);
-    if (form == 1) {
+    if (pair_applies(c, limbs) && c->d_ntt_pair) {
+        const PairArgs p = pair_args(c, limbs);
+        const dim3 gp(pair_blocks(limbs, StridedCfg<8, 8>::TILES));
+        if (form == 1) hipLaunchKernelGGL((rescale_pair_kernel<F64Arith, MidPieces>), gp, dim3(256), 0, c->stream, r, p);
+        else hipLaunchKernelGGL((rescale_pair_kernel<F64WideArith, MidLimb>), gp, dim3(256), 0, c->stream, r, p);
+    } else if (form == 1) {
         hipLaunchKernelGGL((rescale_strided_kernel<F64Arith, MidPieces>), gs, dim3(256), 0, c->stream, r);
         hipLaunchKernelGGL((rescale_row_kernel<F64Arith, MidPieces>), gr, dim3(256), 0, c->stream, r);
     } else {
