@@ -493,7 +493,9 @@ extern "C" int ckks_hybrid_keyswitch(ckks_ctx* c, uint64_t* out, uint64_t* in_nt
     bool fused = false;
     // Where it applies (N = 2^16, primes below 2^39): five launches up to the sums in the coefficient domain, the digit area of the
     // scratch serving as work space, the input left as it is; the sums' special-prime limbs come out scaled for the ModDown below.
-    if ((rc = launch_hybrid_front_fused(c, in_ntt, dig, ip, evk, l, &fused))) return rc;
+    bool finished = false;
+    if ((rc = launch_hybrid_front_fused(c, in_ntt, dig, ip, evk, l, &fused, out, Q, &finished))) return rc;
+    if (finished) return CKKS_OK;
     if (!fused) {
         if ((rc = launch_ntt(c, in_ntt, 0, P, 1, l + 1, Q, 0, 1, true))) return rc;
         if ((rc = ckks_hybrid_modup(c, dig, in_ntt, l))) return rc;

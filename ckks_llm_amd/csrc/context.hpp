@@ -100,6 +100,7 @@ struct ckks_ctx {
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     int chain_skew = 0, chain_spin = -1;  // chained transform: limbs a chain's first pass runs ahead of its second (0: default), poll limit of a wait (-1: default)
     void* d_ntt_pair = nullptr;           // completion words of the paired (one-launch, small-batch) transform, one per 128-byte line
+    unsigned ks_back_epoch = 0;           // what the counters of the key switch's last fused launch have reached (they are never cleared)
     unsigned* h_pair_fail = nullptr;      // pinned host word that a paired transform raises when one of its waits ran out
     void* d_ntt_chain = nullptr;          // completion words of the chained (one-launch) transform, allocated on its first use; zero between transforms
 };
@@ -137,7 +138,11 @@ int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx
 //   transform.  in_ntt: l + 1 limbs of a polynomial of q_num limbs, NTT domain, left untouched; work: at least l + 2 limbs;
 //   sums: two polynomials of poly_mod_len limbs, coefficient domain on return, their first p_num limbs multiplied by (P/p_i)^-1 mod p_i
 //   (ready for launch_ks_moddown_fused(..., pre_scaled = true)).  *done = false where it does not apply (nothing launched).
-int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done);
+// With `out` and `finished` given the call may also finish the switch (the last pass of the sums' inverse transform, the ModDown
+// and the results' forward transform, written to two polynomials of out_poly_mod_len limbs): then *finished = true and `sums`
+// holds the special-prime limbs only.
+int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done,
+                              uint64_t* out = nullptr, int out_poly_mod_len = 0, bool* finished = nullptr);
 // Rescale after the inverse transform of limb l (cipher: [2][L+1] limbs, inv: q_l^-1 mod q_i for i < l): the reduction of limb l
 // modulo each remaining prime, its forward transform and the final subtraction and scaling in two launches; *done = false where
 // it does not apply.

@@ -882,7 +882,7 @@ int ntt_pair_init(ckks_ctx* c) {
     if (c->d_ntt_pair) return CKKS_OK;
     if (hipHostMalloc((void**)&c->h_pair_fail, sizeof(unsigned), hipHostMallocMapped) != hipSuccess) { set_error("NTT: cannot allocate the failure word of the paired transform"); return CKKS_E_NOMEM; }
     *c->h_pair_fail = 0;
-    const size_t bytes = (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE * sizeof(unsigned);
+    const size_t bytes = ((size_t)PAIR_MAX_LIMBS + 64) * PAIR_WORD_STRIDE * sizeof(unsigned);      // the last 64: counters of ks_back_kernel
     if (hipMalloc(&c->d_ntt_pair, bytes) != hipSuccess) { set_error("NTT: cannot allocate the completion words of the paired transform"); return CKKS_E_NOMEM; }
     CKKS_HIP_TRY(hipMemsetAsync(c->d_ntt_pair, 0, bytes, c->stream));
     return CKKS_OK;
@@ -1301,6 +1301,124 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
     MID::store_columns(a.mid + iq * a.mid_stride_i + z * a.mid_stride_z, tile, g, cl, v, ar);
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// End of the hybrid key switch in one launch less: the strided (last) pass of the sums' inverse transform and the ModDown
+// pass above share their column tiling, so a ModDown workgroup (q limb, polynomial z, 16 columns) needs from that inverse
+// pass exactly the same 16 columns of its own limb and of the K special-prime limbs.  Here it runs the inverse pass of its own
+// limb itself and keeps the coefficients in registers (they come out in the lane layout the ModDown reads them in), and the
+// special-prime limbs' passes are 2 K 16 workgroups at the front of the grid that write their (scaled) coefficients as shared
+// stores and count themselves done per (z, tile).  The coefficients of the q limbs are never written: a write and a read of
+// 2 (l + 1) limbs and one launch less.  A waiting workgroup waits only for workgroups of lower index that wait for nothing;
+// the counters grow by K per launch and the launcher hands in the value they must reach, so nothing is cleared.
+// ------------------------------------------------------------------------------------------------------------
+struct KsBackArgs {
+    const char* mid_in;          // sums after the row pass of their inverse transform: limb o * 2 + z, 5-byte form
+    u64* sums;                   // [2][z_stride]: only the K special-prime limbs of each polynomial are written
+    long z_stride;               // words between the two polynomials
+    char* mid_out;               // first pass of the results' forward transform: limb iq * 2 + z, 5-byte form
+    const PrimeConst* primes;    // constants whose special-prime entries carry (P/p_i)^-1 in N^-1 and the last twiddle
+    const double* tw_inv;
+    const double* tw_fwd;
+    const u64* pHatVecModq;      // [q index][K]
+    const u64* PinvModq;         // [q index]
+    unsigned* count;             // [2 * 16] counters, one per 128-byte line
+    unsigned* fail;
+    unsigned target, spin_max;
+    int K, nq;
+};
+__global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
+    typedef StridedCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
+    constexpr long N = 1l << 16;
+    __shared__ double lds[C::LDS_WORDS];
+    __shared__ unsigned go;
+    const unsigned tid = threadIdx.x, cl = tid % CW, g = tid / CW;
+    const unsigned producers = (unsigned)a.K * 32u;
+    const bool special = blockIdx.x < producers;
+    const unsigned b = special ? blockIdx.x : blockIdx.x - producers;
+    const unsigned li = b / 32u, z = (b / 16u) & 1u, tile = b % 16u;       // li: special prime i, or q index iq
+    const int prime = special ? (int)li : a.K + (int)li;
+    const F64Arith ar(a.primes[prime]);
+    // last pass of the inverse transform of limb `prime` of polynomial z, columns of `tile`
+    double v[R];
+    {
+        const char* piece = mid_piece(const_cast<char*>(a.mid_in) + ((long)prime * 2 + z) * MID_LIMB_BYTES, tile, g);
+#pragma unroll
+        for (int j = 0; j < R; j++)
+            v[j] = ar.dec40(*reinterpret_cast<const unsigned*>(piece + (j * 16 + cl) * 4), *reinterpret_cast<const unsigned char*>(piece + 1024 + j * 16 + cl));
+    }
+    const double* twi = a.tw_inv + (long)prime * N;
+    inv_packed<F64Arith, 8, S1>(v, twi, 1u, g, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lds[(g * R + j) * CW + cl] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lds[(g + j * G) * CW + cl];
+    inv_spread<F64Arith, 8, S1, 1>(v, twi, 1u, ar);
+    u64 own[R];                                                       // coefficient of row g + j G, canonical
+#pragma unroll
+    for (int j = 0; j < R / 2; j++) ar.gs_last(v[j], v[j + R / 2], own[j], own[j + R / 2]);
+    unsigned* word = a.count + (size_t)(z * 16u + tile) * PAIR_WORD_STRIDE;
+    if (special) {
+        u64* col = a.sums + (long)z * a.z_stride + (long)li * N + tile * CW + cl;
+#pragma unroll
+        for (int j = 0; j < R; j++) put<true>(col + (long)(g + j * G) * N2, own[j]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);                                // this wave's shared stores have been acknowledged
+        __syncthreads();
+        if (tid == 0) (void)__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    if (tid == 0) {
+        unsigned ok = 0;
+        for (unsigned n = 0; n < a.spin_max; n++) {
+            if ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - a.target) >= 0) { ok = 1; break; }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (!ok) __hip_atomic_store(a.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        go = ok;
+    }
+    __syncthreads();                                                  // also: every lane is done with the LDS tile of the inverse pass
+    if (!go) return;
+    // ModDown (BasisConv.cuh:257-326) on the scaled special-prime coefficients, as in ks_moddown_strided_kernel with pre_scaled
+    const u64* col = a.sums + (long)z * a.z_stride + tile * CW + cl;
+    double acc[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[j] = 0.0;
+    u64 x[R], xn[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) x[j] = get<true>(col + (long)(g + j * G) * N2);
+    for (int i = 0; i < a.K; i++) {
+        const double hat = exact_u2d(a.pHatVecModq[(long)li * a.K + i]);
+        if (i + 1 < a.K) {
+            const u64* nl = col + (long)(i + 1) * N;
+#pragma unroll
+            for (int j = 0; j < R; j++) xn[j] = get<true>(nl + (long)(g + j * G) * N2);
+        }
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            if (a.K == 1) acc[j] = exact_u2d(x[j]);                                                  // BasisConv.cuh:274
+            else acc[j] += ar.mulmod(exact_u2d(x[j]), hat);
+        }
+        if (i + 1 < a.K) {
+#pragma unroll
+            for (int j = 0; j < R; j++) x[j] = xn[j];
+        }
+    }
+    const double pinv = exact_u2d(a.PinvModq[li]);
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = ar.mulmod(ar.q - canon_f(ar, acc[j]) + exact_u2d(own[j]), pinv);      // in (-0.51 q, 0.51 q)
+    const double* twf = a.tw_fwd + (long)prime * N;
+    fwd_spread<F64Arith, 8, S1>(v, twf, 1u, ar);
+#pragma unroll
+    for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
+    fwd_packed<F64Arith, 8, S1>(v, twf, 1u, g, ar);
+    mid_store_columns(a.mid_out + ((long)li * 2 + z) * MID_LIMB_BYTES, tile, g, cl, v, ar);
+}
+
 // The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
 // transform modes, every prime involved below 2^39.  CKKS_KS_SPLIT (any value) in the environment switches them off, for tuning.
 // How the stage-fused launches can run on primes first_prime .. first_prime + prime_count - 1: 0 not at all, 1 with the 5-byte
@@ -1400,9 +1518,10 @@ __global__ __launch_bounds__(256) void ks_modup_strided_kernel(KsModUpArgs a) {
     fwd_packed<F64Arith, 8, S1>(v, tw, 1u, g, ar);
     mid_store_columns(a.mid + (long)limb * MID_LIMB_BYTES, tile, g, cl, v, ar);
 }
-
-int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done) {
+int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* work, uint64_t* sums, const uint64_t* key, int l, bool* done,
+                              uint64_t* out, int out_poly_mod_len, bool* finished) {
     *done = false;
+    if (finished) *finished = false;
     const int P = c->p_num, Q = c->q_num, W = P + Q;
     if (P <= 0 || l < 0 || l > c->L || !stage_fusion_applies(c, 0, P + l + 1)) return CKKS_OK;
     const int mod_num = P + l + 1, ndigits = (l + 1 + P - 1) / P, dnum = (Q + P - 1) / P;
@@ -1422,6 +1541,9 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     args.start_poly_idx = 0; args.start_mod_idx = P; args.poly_num = 1; args.mod_num = l + 1; args.poly_mod_len = Q;
     args.batch_stride_limbs = 0; args.limb_base = 0; args.limbs_total = (unsigned)(l + 1);
     args.data = (u64*)in_ntt;
+    KsModUpArgs u;
+    u.y = (const u64*)work; u.v = (signed char*)(work + (size_t)(l + 1) * N); u.mid = mid; u.blocks = c->d_conv + plan.first;
+    u.primes = c->d_primes; u.tw_fwd = c->d_twd_fwd; u.ndigits = ndigits; u.p_num = P;
     if (pair_applies(c, l + 1)) {
         // one launch: the constants that differ between the two tables (N^-1 and the last twiddle) only enter the second pass
         args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
@@ -1434,9 +1556,6 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
         hipLaunchKernelGGL((ntt_strided_pass<F64Arith, 8, 8, true, true>), dim3(CS::TILES, l + 1), dim3(CS::THREADS), 0, c->stream, args);
     }
     // quotient estimates, then the conversion inside the first pass of the digits' forward transform
-    KsModUpArgs u;
-    u.y = (const u64*)work; u.v = (signed char*)(work + (size_t)(l + 1) * N); u.mid = mid; u.blocks = c->d_conv + plan.first;
-    u.primes = c->d_primes; u.tw_fwd = c->d_twd_fwd; u.ndigits = ndigits; u.p_num = P;
     hipLaunchKernelGGL(ks_modup_quotient_kernel, dim3((unsigned)(N / 256), ndigits), dim3(256), 0, c->stream, u);
     hipLaunchKernelGGL(ks_modup_strided_kernel, dim3(ndigits * mod_num, CS::TILES), dim3(256), 0, c->stream, u);
     // row passes of both transforms around the inner product
@@ -1445,6 +1564,30 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     k.tw_fwd = c->d_twd_fwd; k.tw_inv = c->d_twd_inv; k.ndigits = ndigits; k.key_digit_stride = W; k.key_z_stride = (long)dnum * W;
     k.in_ntt = (const u64*)in_ntt; k.p_num = P;
     hipLaunchKernelGGL(ks_row_fused_kernel, dim3(CR::TILES, mod_num), dim3(256), 0, c->stream, k);
+    static const bool back_split = getenv("CKKS_KS_BACK_SPLIT") != nullptr;
+    if (out && finished && !back_split && c->d_ntt_pair && pair_applies(c, 2 * mod_num)) {
+        // last pass of the sums' inverse transform, ModDown and first pass of the results' forward transform in one launch, then
+        // the row pass of the results
+        KsBackArgs bk;
+        bk.mid_in = k.mid_out; bk.sums = (u64*)sums; bk.z_stride = (long)W * N; bk.mid_out = mid;
+        bk.primes = c->d_primes_moddown; bk.tw_inv = c->d_twd_inv; bk.tw_fwd = c->d_twd_fwd;
+        bk.pHatVecModq = c->d_pHatVecModq; bk.PinvModq = c->d_PinvModq;
+        bk.count = (unsigned*)c->d_ntt_pair + (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE; bk.fail = c->h_pair_fail;
+        c->ks_back_epoch += (unsigned)P;
+        bk.target = c->ks_back_epoch;
+        bk.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
+        bk.K = P; bk.nq = l + 1;
+        hipLaunchKernelGGL(ks_back_kernel, dim3((unsigned)(P + l + 1) * 32u), dim3(256), 0, c->stream, bk);
+        NttArgs fin;
+        fin.data = (u64*)out; fin.primes = c->d_primes; fin.tw = c->d_twd_fwd;
+        fin.start_poly_idx = 0; fin.start_mod_idx = P; fin.poly_num = 2; fin.mod_num = l + 1; fin.poly_mod_len = out_poly_mod_len;
+        fin.batch_stride_limbs = 0; fin.limb_base = 0; fin.limbs_total = (unsigned)(2 * (l + 1)); fin.mid = mid;
+        hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), dim3(CR::TILES, 2 * (l + 1)), dim3(CR::THREADS), 0, c->stream, fin);
+        CKKS_HIP_TRY(hipGetLastError());
+        *done = true;
+        *finished = true;
+        return CKKS_OK;
+    }
     // second pass of the sums' inverse transform, special-prime limbs scaled for the ModDown that follows
     args.data = (u64*)sums; args.primes = c->d_primes_moddown; args.tw = c->d_twd_inv; args.mid = k.mid_out;
     args.start_mod_idx = 0; args.poly_num = 2; args.mod_num = mod_num; args.poly_mod_len = W; args.limbs_total = (unsigned)(2 * mod_num);
