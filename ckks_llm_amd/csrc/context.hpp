@@ -131,7 +131,7 @@ int launch_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
 // Hybrid key switch up to the inverse transform of the two sums, in five launches (four where the input's transform runs as one
-// paired launch) where the separate steps take nine:
+// paired launch; with `out` given the whole switch is five) where the separate steps take nine:
 //   inverse transform of the input (two passes; the second leaves the residues scaled for the exact conversion, in `work`),
 //   the conversion's quotient estimate per digit and coefficient, the conversion inside the first pass of every digit limb's
 //   forward transform, the row passes of both transforms around the inner product with the key, the last pass of the sums' inverse

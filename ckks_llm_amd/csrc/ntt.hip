@@ -1310,27 +1310,32 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 // stores and count themselves done per (z, tile).  The coefficients of the q limbs are never written: a write and a read of
 // 2 (l + 1) limbs and one launch less.  A waiting workgroup waits only for workgroups of lower index that wait for nothing;
 // the counters grow by K per launch and the launcher hands in the value they must reach, so nothing is cleared.
+// The row pass of the results follows in the same workgroup after the hand-over of the paired transform (the sixteen tiles of
+// a limb are consecutive workgroups).
 // ------------------------------------------------------------------------------------------------------------
 struct KsBackArgs {
     const char* mid_in;          // sums after the row pass of their inverse transform: limb o * 2 + z, 5-byte form
     u64* sums;                   // [2][z_stride]: only the K special-prime limbs of each polynomial are written
     long z_stride;               // words between the two polynomials
-    char* mid_out;               // first pass of the results' forward transform: limb iq * 2 + z, 5-byte form
+    char* mid_out;               // between the passes of the results' forward transform: limb iq * 2 + z, 5-byte form
+    u64* out;                    // results: limb iq of polynomial z at out + (z * out_z_stride + iq * N) words, NTT domain
+    long out_z_stride;
+    PairArgs pair;               // completion words of the hand-over between those two passes, limb index iq * 2 + z
     const PrimeConst* primes;    // constants whose special-prime entries carry (P/p_i)^-1 in N^-1 and the last twiddle
     const double* tw_inv;
     const double* tw_fwd;
     const u64* pHatVecModq;      // [q index][K]
     const u64* PinvModq;         // [q index]
     unsigned* count;             // [2 * 16] counters, one per 128-byte line
-    unsigned* fail;
-    unsigned target, spin_max;
-    int K, nq;
+    unsigned target;
+    int K;
 };
 __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     constexpr long N = 1l << 16;
-    __shared__ double lds[C::LDS_WORDS];
+    constexpr int LDS_WORDS = C::LDS_WORDS > RowCfg<8, 8>::LDS_WORDS ? C::LDS_WORDS : RowCfg<8, 8>::LDS_WORDS;
+    __shared__ double lds[LDS_WORDS];
     __shared__ unsigned go;
     const unsigned tid = threadIdx.x, cl = tid % CW, g = tid / CW;
     const unsigned producers = (unsigned)a.K * 32u;
@@ -1371,11 +1376,11 @@ __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
     }
     if (tid == 0) {
         unsigned ok = 0;
-        for (unsigned n = 0; n < a.spin_max; n++) {
+        for (unsigned n = 0; n < a.pair.spin_max; n++) {
             if ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - a.target) >= 0) { ok = 1; break; }
             __builtin_amdgcn_s_sleep(4);
         }
-        if (!ok) __hip_atomic_store(a.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (!ok) __hip_atomic_store(a.pair.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         go = ok;
     }
     __syncthreads();                                                  // also: every lane is done with the LDS tile of the inverse pass
@@ -1416,7 +1421,11 @@ __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<F64Arith, 8, S1>(v, twf, 1u, g, ar);
-    mid_store_columns(a.mid_out + ((long)li * 2 + z) * MID_LIMB_BYTES, tile, g, cl, v, ar);
+    char* mid_limb = a.mid_out + ((long)li * 2 + z) * MID_LIMB_BYTES;
+    mid_store_columns<F64Arith, true>(mid_limb, tile, g, cl, v, ar);
+    // second pass of the result's forward transform, once the limb's sixteen first-pass tiles are there
+    if (!pair_hand_over(a.pair, li * 2u + z, 16u, &go)) return;
+    row_tile<F64Arith, 8, 8, false, false, true, true>(a.out + (long)z * a.out_z_stride + (long)li * N, tile, twf, ar, lds, tid, mid_limb);
 }
 
 // The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
@@ -1566,23 +1575,18 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     hipLaunchKernelGGL(ks_row_fused_kernel, dim3(CR::TILES, mod_num), dim3(256), 0, c->stream, k);
     static const bool back_split = getenv("CKKS_KS_BACK_SPLIT") != nullptr;
     if (out && finished && !back_split && c->d_ntt_pair && pair_applies(c, 2 * mod_num)) {
-        // last pass of the sums' inverse transform, ModDown and first pass of the results' forward transform in one launch, then
-        // the row pass of the results
+        // last pass of the sums' inverse transform, ModDown and both passes of the results' forward transform in one launch
         KsBackArgs bk;
         bk.mid_in = k.mid_out; bk.sums = (u64*)sums; bk.z_stride = (long)W * N; bk.mid_out = mid;
         bk.primes = c->d_primes_moddown; bk.tw_inv = c->d_twd_inv; bk.tw_fwd = c->d_twd_fwd;
         bk.pHatVecModq = c->d_pHatVecModq; bk.PinvModq = c->d_PinvModq;
-        bk.count = (unsigned*)c->d_ntt_pair + (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE; bk.fail = c->h_pair_fail;
+        bk.count = (unsigned*)c->d_ntt_pair + (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE;
+        bk.pair = pair_args(c, 2 * (l + 1));
+        bk.out = (u64*)out; bk.out_z_stride = (long)out_poly_mod_len * N;
         c->ks_back_epoch += (unsigned)P;
         bk.target = c->ks_back_epoch;
-        bk.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
-        bk.K = P; bk.nq = l + 1;
+        bk.K = P;
         hipLaunchKernelGGL(ks_back_kernel, dim3((unsigned)(P + l + 1) * 32u), dim3(256), 0, c->stream, bk);
-        NttArgs fin;
-        fin.data = (u64*)out; fin.primes = c->d_primes; fin.tw = c->d_twd_fwd;
-        fin.start_poly_idx = 0; fin.start_mod_idx = P; fin.poly_num = 2; fin.mod_num = l + 1; fin.poly_mod_len = out_poly_mod_len;
-        fin.batch_stride_limbs = 0; fin.limb_base = 0; fin.limbs_total = (unsigned)(2 * (l + 1)); fin.mid = mid;
-        hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), dim3(CR::TILES, 2 * (l + 1)), dim3(CR::THREADS), 0, c->stream, fin);
         CKKS_HIP_TRY(hipGetLastError());
         *done = true;
         *finished = true;
