@@ -289,6 +289,46 @@ def test_paired_transform_reports_a_wait_that_ran_out():
     buf.free()
 
 
+def test_paired_transforms_of_two_contexts_on_two_streams():
+    """Two contexts, each on a stream of its own, run paired transforms at the same time (each context has its own completion
+    words); twenty rounds in flight without a synchronisation, then both results against the oracle."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    q = CFG2_Q[:4]
+    pairs = [Pair(16, [], q), Pair(16, [], q)]
+    streams = []
+    for p_ in pairs:
+        s = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(s)) == 0
+        p_.dev.set_stream(s)
+        streams.append(s)
+    N, L1 = pairs[0].N, len(q)
+    datas = [limbs_uniform(300 + i, q, 2 + i, N) for i in range(2)]
+    wants = []
+    for p_, d in zip(pairs, datas):
+        w = d.copy()
+        p_.orc.ToNTTInplace(w.reshape(-1), 0, 0, d.shape[0], L1, L1)
+        wants.append(w)
+    bufs = [to_dev(d) for d in datas]
+    for p_ in pairs:
+        p_.dev.check()                       # uploads done before the streams start
+    for _ in range(10):
+        for p_, b, d in zip(pairs, bufs, datas):
+            p_.dev.ToNTTInplace(b, 0, 0, d.shape[0], L1, L1)
+        for p_, b, d in zip(pairs, bufs, datas):
+            p_.dev.FromNTTInplace(b, 0, 0, d.shape[0], L1, L1)
+    for p_, b, d in zip(pairs, bufs, datas):
+        p_.dev.ToNTTInplace(b, 0, 0, d.shape[0], L1, L1)
+    for p_ in pairs:
+        p_.dev.check()
+    for b, d, w in zip(bufs, datas, wants):
+        assert np.array_equal(from_dev(b, d.shape), w)
+        b.free()
+    for p_, s in zip(pairs, streams):
+        p_.dev.set_stream(None)
+        assert hip.hipStreamDestroy(s) == 0
+
+
 @pytest.mark.parametrize("skew,spin", [(1, 0), (3, 0), (2, -1), (64, -1)])
 def test_chained_transform_finishing_launch_and_skews(skew, spin):
     """With a poll limit of zero every second-pass workgroup of the chained transform leaves its tile to the finishing launch,
