@@ -100,7 +100,6 @@ struct ckks_ctx {
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     int chain_skew = 0, chain_spin = -1;  // chained transform: limbs a chain's first pass runs ahead of its second (0: default), poll limit of a wait (-1: default)
     void* d_ntt_pair = nullptr;           // completion words of the paired (one-launch, small-batch) transform, one per 128-byte line
-    unsigned ks_back_epoch = 0;           // what the counters of the key switch's last fused launch have reached (they are never cleared)
     unsigned* h_pair_fail = nullptr;      // pinned host word that a paired transform raises when one of its waits ran out
     void* d_ntt_chain = nullptr;          // completion words of the chained (one-launch) transform, allocated on its first use; zero between transforms
 };

@@ -1308,8 +1308,10 @@ __global__ __launch_bounds__(256) void ks_moddown_strided_kernel(KsModDownArgs a
 // limb itself and keeps the coefficients in registers (they come out in the lane layout the ModDown reads them in), and the
 // special-prime limbs' passes are 2 K 16 workgroups at the front of the grid that write their (scaled) coefficients as shared
 // stores and count themselves done per (z, tile).  The coefficients of the q limbs are never written: a write and a read of
-// 2 (l + 1) limbs and one launch less.  A waiting workgroup waits only for workgroups of lower index that wait for nothing;
-// the counters grow by K per launch and the launcher hands in the value they must reach, so nothing is cleared.
+// 2 (l + 1) limbs and one launch less.  A waiting workgroup waits only for workgroups of lower index that wait for nothing.
+// Each (z, tile) has two counters: the special-prime workgroups that are done (waited for until it reads K) and the ModDown
+// workgroups that have seen that; the last of those returns both to zero, so a launch leaves the counters as it found them
+// and needs nothing from the host (it can be replayed from a captured graph).
 // The row pass of the results follows in the same workgroup after the hand-over of the paired transform (the sixteen tiles of
 // a limb are consecutive workgroups).
 // ------------------------------------------------------------------------------------------------------------
@@ -1326,9 +1328,8 @@ struct KsBackArgs {
     const double* tw_fwd;
     const u64* pHatVecModq;      // [q index][K]
     const u64* PinvModq;         // [q index]
-    unsigned* count;             // [2 * 16] counters, one per 128-byte line
-    unsigned target;
-    int K;
+    unsigned* count;             // [2 * 16] pairs (done, seen), one pair per 128-byte line; zero between launches
+    int K, nq;
 };
 __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
     typedef StridedCfg<8, 8> C;
@@ -1377,10 +1378,15 @@ __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
     if (tid == 0) {
         unsigned ok = 0;
         for (unsigned n = 0; n < a.pair.spin_max; n++) {
-            if ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - a.target) >= 0) { ok = 1; break; }
+            if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (unsigned)a.K) { ok = 1; break; }
             __builtin_amdgcn_s_sleep(4);
         }
         if (!ok) __hip_atomic_store(a.pair.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        else if (__hip_atomic_fetch_add(word + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == (unsigned)a.nq) {
+            // every ModDown workgroup of this (z, tile) has seen the count: back to zero for the next launch
+            __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(word + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         go = ok;
     }
     __syncthreads();                                                  // also: every lane is done with the LDS tile of the inverse pass
@@ -1583,9 +1589,7 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
         bk.count = (unsigned*)c->d_ntt_pair + (size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE;
         bk.pair = pair_args(c, 2 * (l + 1));
         bk.out = (u64*)out; bk.out_z_stride = (long)out_poly_mod_len * N;
-        c->ks_back_epoch += (unsigned)P;
-        bk.target = c->ks_back_epoch;
-        bk.K = P;
+        bk.K = P; bk.nq = l + 1;
         hipLaunchKernelGGL(ks_back_kernel, dim3((unsigned)(P + l + 1) * 32u), dim3(256), 0, c->stream, bk);
         CKKS_HIP_TRY(hipGetLastError());
         *done = true;

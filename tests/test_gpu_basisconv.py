@@ -271,3 +271,46 @@ def test_config3_full_size_keyswitch(nq, np_, l, primes):
         scratch = DeviceBuffer(8 * (dn + 2) * W * N)
         d.hybrid_keyswitch(dks, to_dev(inp), devk, l, scratch)
         assert np.array_equal(from_dev(dks, wks.shape)[:, :l + 1], wks[:, :l + 1]), mode
+
+
+def test_hybrid_keyswitch_and_paired_transform_replayed_from_a_graph():
+    """The fused key switch (five launches with waits between workgroups of one launch) and a paired transform captured into a HIP
+    graph and replayed: no launch depends on host-side state, so every replay on fresh inputs gives the oracle's words.  Eager work
+    and synchronisations lie between the replays."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    nq, np_, l = 6, 2, 5
+    q, p = CFG2_Q[:nq], CFG3_P[:np_]
+    pair = Pair(16, p, q)
+    o, d, N = pair.orc, pair.dev, pair.N
+    W, dn = nq + np_, -(-(l + 1) // np_)
+    evk = limbs_uniform(3, p + q, 2 * -(-nq // np_), N)
+    devk = to_dev(evk)
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+    d.set_stream(stream)
+    dks, dinp, scratch = to_dev(np.zeros((2, nq, N), dtype=np.uint64)), to_dev(np.zeros((nq, N), dtype=np.uint64)), DeviceBuffer(8 * (dn + 2) * W * N)
+    d.hybrid_keyswitch(dks, dinp, devk, l, scratch)              # eager once: the inter-pass area is allocated before the capture
+    d.FromNTTInplace(dinp, 0, np_, 1, l + 1, nq)
+    d.check()
+    graph, gexec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0
+    d.hybrid_keyswitch(dks, dinp, devk, l, scratch)
+    d.FromNTTInplace(dks, 0, np_, 2, l + 1, nq)                   # a paired transform of the result, 12 limbs
+    assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, ctypes.c_size_t(0)) == 0
+    for rep in range(3):
+        inp = np.zeros((nq, N), dtype=np.uint64)
+        inp[:l + 1] = limbs_uniform(70 + rep, q[:l + 1], 1, N)[0]
+        want = np.zeros((2, nq, N), dtype=np.uint64)
+        o.hybrid_keyswitch(want.reshape(-1), inp.copy().reshape(-1), evk.reshape(-1), l)
+        o.FromNTTInplace(want.reshape(-1), 0, np_, 2, l + 1, nq)
+        dinp.upload(inp)
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        d.check()
+        assert np.array_equal(from_dev(dks, want.shape)[:, :l + 1], want[:, :l + 1]), rep
+        d.ToNTTInplace(dks, 0, np_, 2, l + 1, nq)                  # eager work between the replays
+        d.check()
+    assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
+    d.set_stream(None)
+    assert hip.hipStreamDestroy(stream) == 0
