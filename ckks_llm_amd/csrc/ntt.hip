@@ -1537,6 +1537,7 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
                               uint64_t* out, int out_poly_mod_len, bool* finished) {
     *done = false;
     if (finished) *finished = false;
+    if (ntt_pair_failed(c)) { set_error("an earlier one-launch transform of this context gave up a wait: the context is unusable"); return CKKS_E_UNAVAILABLE; }
     const int P = c->p_num, Q = c->q_num, W = P + Q;
     if (P <= 0 || l < 0 || l > c->L || !stage_fusion_applies(c, 0, P + l + 1)) return CKKS_OK;
     const int mod_num = P + l + 1, ndigits = (l + 1 + P - 1) / P, dnum = (Q + P - 1) / P;
@@ -1863,6 +1864,7 @@ __global__ __launch_bounds__(256) void rescale_pair_kernel(RescaleArgs a, PairAr
 // *done = false (nothing launched) where it does not apply.
 int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done) {
     *done = false;
+    if (ntt_pair_failed(c)) { set_error("an earlier one-launch transform of this context gave up a wait: the context is unusable"); return CKKS_E_UNAVAILABLE; }
     const int form = l < 1 || l > c->L ? 0 : stage_fusion_form(c, c->K, l + 1);
     if (form == 0) return CKKS_OK;
     const int limbs = 2 * l;
