@@ -227,6 +227,12 @@ private:
     }
 public:
 
+    // Where the reference's programs call cudaDeviceSynchronize and check the last error (Utils.cuh CUDA_CHECK): waits for the
+    // context's stream and throws on anything the launches so far have reported, including a one-launch transform that gave up a wait.
+    void synchronize() { check(ckks_ctx_check(handle), "synchronize"); }
+    // launch form of the transforms (0 = chosen by the library); no counterpart in the reference
+    void set_ntt_mode(int mode) { check(ckks_ctx_set_ntt_mode(handle, mode), "set_ntt_mode"); }
+
     // Context_23.h:42-45
     void ToNTTInplace(uint64_tt* device_a, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len) {
         check(ckks_ntt_fwd(handle, device_a, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len), "ToNTTInplace");
