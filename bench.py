@@ -232,7 +232,7 @@ def main():
     line = {
         "metric": "NTT limb-transforms/s @N=2^16", "value": round(value, 1), "unit": "limb-transforms/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u64 residues (f64 butterflies for q < 2^41)", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": "u64 residues (exact-integer f64 butterflies for q < 2^50, u64 butterflies above)", "data": "synthetic",
         "config": {"workload": "configs[1]: RNS NTT+iNTT, N=2^16, 24 primes <2^36, batch of %d ciphertexts (%d limbs, %d MiB) per step"
                                % (args.batch, limbs, limbs * 8 * 65536 >> 20), "limb_transforms_per_step": 2 * limbs},
         "roofline": roofline, "one_ciphertext": one_ct,
