@@ -436,7 +436,7 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
 // size (N = 2^16; the automatic mode takes it for small batches), 5 = the same with the tiles of a limb spread over all XCDs
 // (the automatic mode's choice between 41 and 128 limbs)
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
-    if (!c || mode < 0 || mode > 5) return CKKS_E_INVALID;
+    if (!c || mode < 0 || mode > 6) return CKKS_E_INVALID;
     c->ntt_mode = mode;
     return CKKS_OK;
 }

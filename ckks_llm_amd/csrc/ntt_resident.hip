@@ -1,0 +1,384 @@
+// Resident transform at N = 2^16: both passes of a limb in one workgroup, the limb held in registers between them.
+//
+// Same transform as the two launches of ntt.hip (Context_23::ToNTTInplace / FromNTTInplace, Context_23.cuh:847-930,
+// ntt_60bit.cuh:421-1318), same tiles, same butterflies; what changes is where a limb is between its two passes.  The
+// two-launch form writes it to memory and reads it back (26 bytes per value through HBM); here a workgroup of 512 lanes keeps
+// all 65536 values of its limb in its own registers - 128 values per lane in the 5-byte form of ntt.hip's inter-pass buffer,
+// 160 of the 256 registers a lane has - so HBM sees the limb once in and once out: 16 bytes per value.
+//
+// One persistent workgroup per compute unit (its registers and its LDS leave room for exactly one) walks through its share of
+// the limbs.  The workgroup is two groups of 256 lanes; a step handles two tiles, one per group:
+//   pass 1, step s: tiles 2s and 2s+1 of the first pass (forward: 16 columns x 256 rows; inverse: 16 rows x 256 columns).
+//                   The tile arrives in LDS by asynchronous loads (global_load_lds) requested during the step before, every
+//                   wave fetching exactly what its own lanes read, so the only synchronisation is the wave's own counter.
+//                   Of its 16 results a lane keeps the 8 that its own group's tiles of pass 2 need and hands the other 8 to
+//                   the same lane of the other group (through LDS, in the 5-byte form), receiving 8 of the other tile.
+//   pass 2, step s: every lane decodes the 16 values it holds of tile 2s + group and runs the tile; nothing is exchanged
+//                   between the groups.
+// For that the 16 x 256 tiles are interleaved: tile k of the row pass is the rows 16 m + k (m = 0..15), lane group m taking
+// row 16 m + k, which is exactly the set of rows (forward: that a lane of the column pass ends with; inverse: that a lane of
+// the column pass starts from).
+//
+// Vector memory operations complete in the order of their issue and share one counter.  The asynchronous loads are issued
+// from inline assembly, invisible to the compiler's own bookkeeping, so a step is written such that no load the compiler
+// waits for is older than an asynchronous load still in flight: the twiddles of a step are in registers (drain()) before the
+// next tile is requested.
+#include <cstdlib>
+#include <type_traits>
+
+#include "context.hpp"
+#include "ntt_core.hpp"
+
+namespace ckks {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+constexpr int RES_LANES = 512;
+constexpr long RES_N = 65536;
+constexpr int RES_PITCH = RowCfg<8, 8>::PITCH;                       // 272: padded row of the row pass
+constexpr int RES_P_BYTES = 65536;                                   // staging of the tiles that arrive: 8 KiB per wave
+constexpr int RES_R_BYTES = 2 * 16 * RES_PITCH * 8;                  // exchange area of a step: one tile per group (69632 bytes)
+constexpr int RES_S_BYTES = 9 * RES_LANES * 4;                       // hand-over between the groups: 9 words per lane
+constexpr int RES_T_BYTES = 2 * 8 * 512;                             // inverse transforms: row twiddles of a step, 512 bytes per wave, two parities
+
+// limb of workgroup b in round `it`: consecutive workgroups of a grid go to the eight XCDs in turn, and the workgroups of one
+// XCD take consecutive limbs - limbs are ordered prime-major, so one XCD's compute units read one prime's twiddles from its L2.
+__device__ __forceinline__ unsigned resident_limb(unsigned b, unsigned grid, unsigned it) {
+    const unsigned per_x = grid / 8;
+    return ((b % 8) + 8 * it) * per_x + b / 8;
+}
+
+// 16 bytes per lane from global memory into LDS at lds_addr + 16 * lane (lds_addr wave-uniform)
+__device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
+    const unsigned base = __builtin_amdgcn_readfirstlane(lds_addr);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void wait_all_vmem() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
+
+// The fifteen twiddles of the last four stages of an axis (packed layout, lane group g: stage 4 + d, butterfly group k),
+// fetched together ahead of their use.
+template <class AR>
+struct PackedTwiddles {
+    typename AR::TW t[15];
+    __device__ __forceinline__ void load(const typename AR::TW* __restrict__ tw, unsigned off, unsigned g) {
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+#pragma unroll
+            for (int k = 0; k < (1 << d); k++) t[(1 << d) - 1 + k] = tw[(off << (4 + d)) + (g << d) + k];
+    }
+    // all fifteen are in registers after this (the compiler waits for them here, where no asynchronous load is in flight)
+    __device__ __forceinline__ void drain() {
+        asm volatile("" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]));
+        asm volatile("" : "+v"(t[8]), "+v"(t[9]), "+v"(t[10]), "+v"(t[11]), "+v"(t[12]), "+v"(t[13]), "+v"(t[14]));
+    }
+};
+// Four stages on sixteen register values (the first four of an axis in the spread layout, the last four in the packed layout: the
+// same butterfly pattern), the twiddles of a stage fetched while the stage before runs: fetch(s, k) gives the twiddle of the
+// round's stage s, butterfly group k = j >> (4 - s).
+template <class AR, class F>
+__device__ __forceinline__ void fwd_round(typename AR::V (&v)[16], const AR& ar, F fetch) {
+    typename AR::TW cur[8], nxt[8];
+    cur[0] = fetch(0, 0);
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (s < 3) {
+#pragma unroll
+            for (int k = 0; k < (2 << s); k++) nxt[k] = fetch(s + 1, k);
+        }
+        const int half = 8 >> s;
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if ((j & half) == 0) ar.ct(v[j], v[j + half], cur[j >> (4 - s)]);
+        if (s < 3) {
+#pragma unroll
+            for (int k = 0; k < (2 << s); k++) cur[k] = nxt[k];
+        }
+    }
+}
+template <class AR, int S_STOP, class F>
+__device__ __forceinline__ void inv_round(typename AR::V (&v)[16], const AR& ar, F fetch) {                           // the round's stages 3 .. S_STOP
+    typename AR::TW cur[8], nxt[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) cur[k] = fetch(3, k);
+#pragma unroll
+    for (int s = 3; s >= S_STOP; s--) {
+        if (s > S_STOP) {
+#pragma unroll
+            for (int k = 0; k < (1 << (s - 1)); k++) nxt[k] = fetch(s - 1, k);
+        }
+        const int half = 8 >> s;
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if ((j & half) == 0) ar.gs(v[j], v[j + half], cur[j >> (4 - s)]);
+        if (s > S_STOP) {
+#pragma unroll
+            for (int k = 0; k < (1 << (s - 1)); k++) cur[k] = nxt[k];
+        }
+    }
+}
+
+// The low words of the limb live in the accumulation registers, which only these two moves reach: the register allocator has
+// the other half of the lane's registers for a step's working set and cannot be tempted to spill the limb to memory.
+__device__ __forceinline__ unsigned to_acc(unsigned x) {
+    unsigned a;
+    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(a) : "v"(x));
+    return a;
+}
+__device__ __forceinline__ unsigned from_acc(unsigned a) {
+    unsigned x;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(a));
+    return x;
+}
+
+// What a lane keeps of its limb between the passes: per step of pass 1 and per tile of that step, eight 5-byte values
+// (low words, and the high bytes four to a register).
+struct Stash {
+    unsigned lo[8][2][8];
+    unsigned hi[8][2];
+};
+
+template <bool INVERSE>
+__global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsigned limbs) {
+    typedef F64Arith AR;
+    typedef double V;
+    typedef double TW;
+    __shared__ __align__(16) unsigned char lds_p[RES_P_BYTES];
+    __shared__ __align__(16) unsigned char lds_r[RES_R_BYTES];
+    __shared__ __align__(16) unsigned lds_s[RES_S_BYTES / 4];
+    __shared__ __align__(16) unsigned char lds_t[INVERSE ? RES_T_BYTES : 16];
+    __shared__ TW lds_w[256];                            // twiddles 1 .. 255 of the limb's prime: the column pass's, the same for every column
+    const unsigned grp = threadIdx.x >> 8, tid0 = threadIdx.x & 255;
+    unsigned tid = tid0, cl = tid & 15, g = tid >> 4;    // column pass: column within the tile, group of rows; row pass: lane within the row (u = cl), row group (rl = g)
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wq = wave & 3;
+    unsigned lane = threadIdx.x & 63;
+    // this wave's part of the staging area, and where this lane reads its sixteen words from (word j at + 512 j)
+    const unsigned p_wave = (unsigned)(size_t)(lptr_t)lds_p + wave * 8192;
+    const u64* p_lane;
+    // asynchronous load m (0..7) of a tile moves 1 KiB: words 2m and 2m+1 of every lane of the wave
+    unsigned d_chunk, d_i, d_jl;
+    V* col_area;                                         // column pass: [row][16 columns]
+    V* row_area;                                         // row pass: this lane's row
+    Stash st;
+    // The lane's coordinates and LDS addresses are formed anew in every step from a value the compiler cannot see through:
+    // shared across the 32 unrolled steps they would sit in registers for the whole limb, and the 160 registers of the
+    // limb leave no room for that.
+    auto coordinates = [&]() __attribute__((always_inline)) {
+        unsigned x = threadIdx.x;
+        asm volatile("" : "+v"(x));
+        tid = x & 255; cl = x & 15; g = tid >> 4; lane = x & 63;
+        d_chunk = lane & 7; d_i = (lane >> 3) & 3; d_jl = lane >> 5;
+        p_lane = reinterpret_cast<const u64*>(lds_p + wave * 8192 + lane * 8);
+        col_area = reinterpret_cast<V*>(lds_r) + grp * 4096;
+        row_area = reinterpret_cast<V*>(lds_r) + grp * (16 * RES_PITCH) + g * RES_PITCH;
+    };
+    coordinates();
+
+    // Requests tile (2 s + grp) of the first pass of `limb`.  Inverse transforms: with it the twiddles of the tile's last four
+    // stages, which depend on the row only: 15 per row = 8 chunks of 16 bytes (stage 3: 4, stage 2: 2, stage 1: 1, stage 0: the
+    // chunk that holds its one twiddle), 4 rows per wave, into this wave's 512 bytes of the twiddle staging of the step's parity.
+    auto request = [&](const u64* limb, const TW* tw, int s) __attribute__((always_inline)) {
+        const unsigned tile = 2 * s + grp;
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");       // this wave has read everything it wanted from its staging area
+#pragma unroll
+        for (int m = 0; m < 8; m++) {
+            const u64* src;
+            if (!INVERSE) src = limb + (long)(4 * wq + d_i + 16 * (2 * m + d_jl)) * 256 + tile * 16 + 2 * d_chunk;      // rows g + 16 j of 16 columns
+            else src = limb + (long)(16 * (4 * wq + d_i) + tile) * 256 + 16 * (2 * m + d_jl) + 2 * d_chunk;             // columns u + 16 j of row 16 rl + tile
+            dma16(src, p_wave + m * 1024);
+        }
+        if (INVERSE) {
+            if (lane < 32) {
+                const unsigned i = lane >> 3, c = lane & 7;
+                const unsigned off = 256 + 16 * (4 * wq + i) + tile;
+                const TW* src = c < 4 ? tw + (off << 3) + 2 * c : c < 6 ? tw + (off << 2) + 2 * (c - 4) : c == 6 ? tw + (off << 1) : tw + (off & ~1u);
+                dma16(src, (unsigned)(size_t)(lptr_t)lds_t + ((s & 1) * 8 + wave) * 512);
+            }
+        }
+    };
+    // end of a pass-1 step: v[j] (forward: row 16 g + j of the group's column tile; inverse: column tile j of the group's row) ->
+    // keep the eight values of the parity of this group, hand the other eight to the partner lane, take its eight
+    auto hand_over = [&](const V (&v)[16], const AR& ar, int s) __attribute__((always_inline)) {
+        unsigned klo[8], khi = 0, shi = 0;
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const V keep = grp ? v[2 * jj + 1] : v[2 * jj], send = grp ? v[2 * jj] : v[2 * jj + 1];
+            const u64 ek = ar.enc36(keep), es = ar.enc36(send);
+            klo[jj] = (unsigned)ek;
+            lds_s[(jj * 2 + grp) * 256 + tid] = (unsigned)es;
+            khi |= (unsigned)(ek >> 32) << (4 * jj);
+            shi |= (unsigned)(es >> 32) << (4 * jj);
+        }
+        lds_s[(8 * 2 + grp) * 256 + tid] = shi;
+        __syncthreads();
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const unsigned r = lds_s[(jj * 2 + (1 - grp)) * 256 + tid];
+            st.lo[s][0][jj] = to_acc(grp ? r : klo[jj]);
+            st.lo[s][1][jj] = to_acc(grp ? klo[jj] : r);
+        }
+        const unsigned r = lds_s[(8 * 2 + (1 - grp)) * 256 + tid];
+        st.hi[s][0] = grp ? r : khi;
+        st.hi[s][1] = grp ? khi : r;
+    };
+    // start of a pass-2 step: the sixteen values this lane holds of tile 2 s + grp
+    auto take = [&](V (&v)[16], const AR& ar, int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = ar.dec36(from_acc(st.lo[j >> 1][j & 1][s]), (st.hi[j >> 1][j & 1] >> (4 * s)) & 0xfu);
+    };
+
+    unsigned it = 0;
+    unsigned limb_id = resident_limb(blockIdx.x, gridDim.x, it);
+    if (limb_id >= limbs) return;
+    int prime;
+    u64* limb = limb_ptr(a, limb_id, RES_N, prime);
+    request(limb, (const TW*)a.tw + (long)prime * RES_N, 0);
+    TW w_col = 0.0;                                      // this lane's entry of the column pass's twiddle table, fetched ahead
+    if (!INVERSE && threadIdx.x < 256) w_col = ((const TW*)a.tw + (long)prime * RES_N)[threadIdx.x];
+    for (;;) {
+        const AR ar(a.primes[prime]);
+        const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * RES_N;
+        const unsigned next_id = resident_limb(blockIdx.x, gridDim.x, it + 1);
+        const bool more = next_id < limbs;
+        int next_prime = prime;
+        u64* next_limb = more ? limb_ptr(a, next_id, RES_N, next_prime) : limb;
+        const TW* next_tw = (const TW*)a.tw + (long)next_prime * RES_N;
+
+        if (!INVERSE) {
+            // ---------------- pass 1: columns (first eight stages) ----------------
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                coordinates();
+                wait_all_vmem();                        // this wave's part of the tile has arrived
+                V v[16];
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = ar.from_canonical(p_lane[j * 64]);
+                if (s < 7) request(limb, tw, s + 1);
+                if (s == 0 && threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
+                fwd_round(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; });        // the same for every lane: scalar loads
+#pragma unroll
+                for (int j = 0; j < 16; j++) col_area[(g + 16 * j) * 16 + cl] = v[j];
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = col_area[(g * 16 + j) * 16 + cl];
+                fwd_round(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; });
+                hand_over(v, ar, s);
+            }
+            // ---------------- pass 2: rows (last eight stages), tile k = rows 16 m + k ----------------
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                coordinates();
+                const unsigned row = 16 * g + 2 * s + grp;
+                const unsigned tw_off = 256 + row;
+                V v[16];
+                take(v, ar, s);
+                fwd_round(v, ar, [&](int d, int k) { return tw[(tw_off << d) + k]; });
+                PackedTwiddles<AR> wp;
+                wp.load(tw, tw_off, cl);
+                if (s == 6 && more && threadIdx.x < 256) w_col = next_tw[threadIdx.x];
+                __syncthreads();                        // the exchange area is free: every lane has read what the step before left there
+#pragma unroll
+                for (int j = 0; j < 16; j++) row_area[padded(cl + 16 * j)] = v[j];
+                if (s == 7 && more) {
+                    wp.drain();
+                    request(next_limb, next_tw, 0);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl * 16 + j)];
+                fwd_round(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; });
+#pragma unroll
+                for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
+                __syncthreads();
+                u64* rp = limb + (long)row * 256;
+#pragma unroll
+                for (int j = 0; j < 16; j++) rp[cl + 16 * j] = ar.to_canonical_fwd(row_area[padded(cl + 16 * j)]);
+            }
+        } else {
+            // ---------------- pass 1: rows (stages 15 .. 8), tile k = rows 16 m + k ----------------
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                coordinates();
+                const unsigned row = 16 * g + 2 * s + grp;
+                const unsigned tw_off = 256 + row;
+                wait_all_vmem();                        // this wave's part of the tile and its row twiddles have arrived
+                PackedTwiddles<AR> wp;
+                wp.load(tw, tw_off, cl);
+#pragma unroll
+                for (int j = 0; j < 16; j++) row_area[padded(cl + 16 * j)] = ar.from_canonical(p_lane[j * 64]);
+                // the row's fifteen twiddles of the last four stages, before the staging of this parity is requested again (two steps on)
+                const TW* trow = reinterpret_cast<const TW*>(lds_t + ((s & 1) * 8 + wave) * 512 + (lane >> 4) * 128);
+                wp.drain();
+                if (s < 7) request(limb, tw, s + 1);
+                __syncthreads();
+                V v[16];
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl * 16 + j)];
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; });
+#pragma unroll
+                for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
+                if (s == 7 && threadIdx.x < 256) w_col = tw[threadIdx.x];
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl + 16 * j)];
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return d == 3 ? trow[k] : d == 2 ? trow[8 + k] : d == 1 ? trow[12 + k] : trow[14 + (tw_off & 1u)]; });
+                hand_over(v, ar, s);                    // balanced to (-q/2, q/2] between the passes, as in the two-launch form
+            }
+            if (threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
+            __syncthreads();
+            // ---------------- pass 2: columns (stages 7 .. 0) ----------------
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                coordinates();
+                V v[16];
+                take(v, ar, s);
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; });
+                __syncthreads();                        // the exchange area is free
+#pragma unroll
+                for (int j = 0; j < 16; j++) col_area[(g * 16 + j) * 16 + cl] = v[j];
+                if (s == 7 && more) request(next_limb, next_tw, 0);
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = col_area[(g + 16 * j) * 16 + cl];
+                inv_round<AR, 1>(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; });       // scalar loads
+                u64* col = limb + (2 * s + grp) * 16 + cl;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    u64 ox, oy;
+                    ar.gs_last(v[j], v[j + 8], ox, oy);
+                    col[(long)(g + 16 * j) * 256] = ox;
+                    col[(long)(g + 16 * (j + 8)) * 256] = oy;
+                }
+            }
+        }
+        if (!more) break;
+        __syncthreads();                                // the exchange area is free for the next limb's first step
+        it++;
+        limb = next_limb;
+        prime = next_prime;
+    }
+}
+
+}  // namespace
+
+// Whether the resident transform takes a call: N = 2^16 and enough limbs to give every compute unit work.
+bool ntt_resident_applies(const ckks_ctx* c, int limbs) { return c->logN == 16 && limbs >= c->cu_count; }
+
+// args: as for the two-launch transform.  FP64 back end, every prime of the call below 2^39 (the 5-byte form).
+int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, bool inverse) {
+    NttArgs args = args_in;
+    args.limb_base = 0;
+    args.limbs_total = (unsigned)limbs;
+    args.mid = nullptr;
+    // one workgroup per compute unit, a multiple of eight so that the XCDs get equal shares
+    unsigned grid = (unsigned)c->cu_count / 8 * 8;
+    if (grid == 0) grid = 8;
+    const dim3 g(grid), b(RES_LANES);
+    if (!inverse) hipLaunchKernelGGL((ntt_resident_kernel<false>), g, b, 0, c->stream, args, (unsigned)limbs);
+    else hipLaunchKernelGGL((ntt_resident_kernel<true>), g, b, 0, c->stream, args, (unsigned)limbs);
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+
+}  // namespace ckks
