@@ -33,6 +33,13 @@ namespace ckks {
 
 namespace {
 
+#ifdef CKKS_RES_TIMING
+__device__ unsigned long long g_res_ticks[8][136];
+#define RES_TICK(n) do { if (it == 1 && blockIdx.x < 8 && threadIdx.x == 0) g_res_ticks[blockIdx.x][(n)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define RES_TICK(n) do { } while (0)
+#endif
+
 typedef __attribute__((address_space(3))) void* lptr_t;
 
 constexpr int RES_LANES = 512;
@@ -41,7 +48,7 @@ constexpr int RES_PITCH = RowCfg<8, 8>::PITCH;                       // 272: pad
 constexpr int RES_P_BYTES = 65536;                                   // staging of the tiles that arrive: 8 KiB per wave
 constexpr int RES_R_BYTES = 2 * 16 * RES_PITCH * 8;                  // exchange area of a step: one tile per group (69632 bytes)
 constexpr int RES_S_BYTES = 9 * RES_LANES * 4;                       // hand-over between the groups: 9 words per lane
-constexpr int RES_T_BYTES = 2 * 8 * 512;                             // inverse transforms: row twiddles of a step, 512 bytes per wave, two parities
+constexpr int RES_T_BYTES = 8 * 1024;                                // inverse transforms: row twiddles of a step, 512 bytes per wave (written twice over by the wave's 64 lanes)
 
 // limb of workgroup b in round `it`: consecutive workgroups of a grid go to the eight XCDs in turn, and the workgroups of one
 // XCD take consecutive limbs - limbs are ordered prime-major, so one XCD's compute units read one prime's twiddles from its L2.
@@ -55,6 +62,9 @@ __device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
     const unsigned base = __builtin_amdgcn_readfirstlane(lds_addr);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory", "m0");
 }
+// Ordering point for what a wave exchanges with itself through LDS (the hardware carries out a wave's LDS accesses in order; this
+// keeps the compiler from reordering them: as one thread sees it, the lane that writes and the lane that reads are unrelated).
+__device__ __forceinline__ void wave_sync() { __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); __builtin_amdgcn_wave_barrier(); }
 __device__ __forceinline__ void wait_all_vmem() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 
 // The fifteen twiddles of the last four stages of an axis (packed layout, lane group g: stage 4 + d, butterfly group k),
@@ -68,6 +78,16 @@ struct PackedTwiddles {
 #pragma unroll
             for (int k = 0; k < (1 << d); k++) t[(1 << d) - 1 + k] = tw[(off << (4 + d)) + (g << d) + k];
     }
+    // The same, as accesses the compiler keeps in program order (it would otherwise sink them towards their use, behind the
+    // stores in between - and loads and stores complete in the order of their issue): relaxed atomic loads at wavefront scope
+    // are ordinary load instructions that the scheduler does not move across other memory accesses.
+    __device__ __forceinline__ void load_ordered(const typename AR::TW* tw, unsigned off, unsigned g) {
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+#pragma unroll
+            for (int k = 0; k < (1 << d); k++)
+                t[(1 << d) - 1 + k] = __hip_atomic_load(tw + (off << (4 + d)) + (g << d) + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    }
     // all fifteen are in registers after this (the compiler waits for them here, where no asynchronous load is in flight)
     __device__ __forceinline__ void drain() {
         asm volatile("" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]));
@@ -77,8 +97,21 @@ struct PackedTwiddles {
 // Four stages on sixteen register values (the first four of an axis in the spread layout, the last four in the packed layout: the
 // same butterfly pattern), the twiddles of a stage fetched while the stage before runs: fetch(s, k) gives the twiddle of the
 // round's stage s, butterfly group k = j >> (4 - s).
-template <class AR, class F>
-__device__ __forceinline__ void fwd_round(typename AR::V (&v)[16], const AR& ar, F fetch) {
+// The fifteen twiddles of the first four stages of an axis (spread layout: stage s, butterfly group k), fetched together.
+template <class AR>
+struct SpreadTwiddles {
+    typename AR::TW t[15];
+    __device__ __forceinline__ void load(const typename AR::TW* __restrict__ tw, unsigned off) {
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int k = 0; k < (1 << s); k++) t[(1 << s) - 1 + k] = tw[(off << s) + k];
+    }
+};
+struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
+// after(s) runs behind the butterflies of the round's stage s (the asynchronous loads of the next tile go out there, one per stage)
+template <class AR, class F, class H = NoHook>
+__device__ __forceinline__ void fwd_round(typename AR::V (&v)[16], const AR& ar, F fetch, H after = H()) {
     typename AR::TW cur[8], nxt[8];
     cur[0] = fetch(0, 0);
 #pragma unroll
@@ -91,14 +124,15 @@ __device__ __forceinline__ void fwd_round(typename AR::V (&v)[16], const AR& ar,
 #pragma unroll
         for (int j = 0; j < 16; j++)
             if ((j & half) == 0) ar.ct(v[j], v[j + half], cur[j >> (4 - s)]);
+        after(s);
         if (s < 3) {
 #pragma unroll
             for (int k = 0; k < (2 << s); k++) cur[k] = nxt[k];
         }
     }
 }
-template <class AR, int S_STOP, class F>
-__device__ __forceinline__ void inv_round(typename AR::V (&v)[16], const AR& ar, F fetch) {                           // the round's stages 3 .. S_STOP
+template <class AR, int S_STOP, class F, class H = NoHook>
+__device__ __forceinline__ void inv_round(typename AR::V (&v)[16], const AR& ar, F fetch, H after = H()) {                          // the round's stages 3 .. S_STOP
     typename AR::TW cur[8], nxt[8];
 #pragma unroll
     for (int k = 0; k < 8; k++) cur[k] = fetch(3, k);
@@ -112,6 +146,7 @@ __device__ __forceinline__ void inv_round(typename AR::V (&v)[16], const AR& ar,
 #pragma unroll
         for (int j = 0; j < 16; j++)
             if ((j & half) == 0) ar.gs(v[j], v[j + half], cur[j >> (4 - s)]);
+        after(s);
         if (s > S_STOP) {
 #pragma unroll
             for (int k = 0; k < (1 << (s - 1)); k++) cur[k] = nxt[k];
@@ -128,7 +163,7 @@ __device__ __forceinline__ unsigned to_acc(unsigned x) {
 }
 __device__ __forceinline__ unsigned from_acc(unsigned a) {
     unsigned x;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(a));
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(a) : "memory");      // "memory": stays behind the barrier in front of its step
     return x;
 }
 
@@ -147,10 +182,10 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     __shared__ __align__(16) unsigned char lds_p[RES_P_BYTES];
     __shared__ __align__(16) unsigned char lds_r[RES_R_BYTES];
     __shared__ __align__(16) unsigned lds_s[RES_S_BYTES / 4];
-    __shared__ __align__(16) unsigned char lds_t[INVERSE ? RES_T_BYTES : 16];
+    __shared__ __align__(16) unsigned char lds_t[RES_T_BYTES];
     __shared__ TW lds_w[256];                            // twiddles 1 .. 255 of the limb's prime: the column pass's, the same for every column
-    const unsigned grp = threadIdx.x >> 8, tid0 = threadIdx.x & 255;
-    unsigned tid = tid0, cl = tid & 15, g = tid >> 4;    // column pass: column within the tile, group of rows; row pass: lane within the row (u = cl), row group (rl = g)
+    unsigned grp = threadIdx.x >> 8;
+    unsigned tid = threadIdx.x & 255, cl = tid & 15, g = tid >> 4;    // column pass: column within the tile, group of rows; row pass: lane within the row (u = cl), row group (rl = g)
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wq = wave & 3;
     unsigned lane = threadIdx.x & 63;
     // this wave's part of the staging area, and where this lane reads its sixteen words from (word j at + 512 j)
@@ -167,7 +202,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     auto coordinates = [&]() __attribute__((always_inline)) {
         unsigned x = threadIdx.x;
         asm volatile("" : "+v"(x));
-        tid = x & 255; cl = x & 15; g = tid >> 4; lane = x & 63;
+        grp = x >> 8; tid = x & 255; cl = x & 15; g = tid >> 4; lane = x & 63;
         d_chunk = lane & 7; d_i = (lane >> 3) & 3; d_jl = lane >> 5;
         p_lane = reinterpret_cast<const u64*>(lds_p + wave * 8192 + lane * 8);
         col_area = reinterpret_cast<V*>(lds_r) + grp * 4096;
@@ -178,29 +213,38 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     // Requests tile (2 s + grp) of the first pass of `limb`.  Inverse transforms: with it the twiddles of the tile's last four
     // stages, which depend on the row only: 15 per row = 8 chunks of 16 bytes (stage 3: 4, stage 2: 2, stage 1: 1, stage 0: the
     // chunk that holds its one twiddle), 4 rows per wave, into this wave's 512 bytes of the twiddle staging of the step's parity.
-    auto request = [&](const u64* limb, const TW* tw, int s) __attribute__((always_inline)) {
+    // part m (0..7: 1 KiB of the tile; 8: the row twiddles) of the request; part 0 first
+    auto request_part = [&](const u64* limb, const TW* tw, int s, int m) __attribute__((always_inline)) {
         const unsigned tile = 2 * s + grp;
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");       // this wave has read everything it wanted from its staging area
-#pragma unroll
-        for (int m = 0; m < 8; m++) {
+        if (m == 0) asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");       // this wave has read everything it wanted from its staging area
+        if (m < 8) {
             const u64* src;
             if (!INVERSE) src = limb + (long)(4 * wq + d_i + 16 * (2 * m + d_jl)) * 256 + tile * 16 + 2 * d_chunk;      // rows g + 16 j of 16 columns
             else src = limb + (long)(16 * (4 * wq + d_i) + tile) * 256 + 16 * (2 * m + d_jl) + 2 * d_chunk;             // columns u + 16 j of row 16 rl + tile
             dma16(src, p_wave + m * 1024);
+        } else {
+            // every lane takes part (the upper half of the wave repeats the lower half's chunks into the second half of the wave's
+            // 1 KiB): no branch; the staging is single: the step's own reads of it are over (they come before this in the last round)
+            const unsigned i = (lane >> 3) & 3, c = lane & 7;
+            const unsigned off = 256 + 16 * (4 * wq + i) + tile;
+            // chunk c: 0..3 stage 3 (twiddles 8 off + 2 c ..), 4..5 stage 2 (4 off + 2 (c - 4) ..), 6 stage 1 (2 off ..), 7 the pair that holds stage 0's (off)
+            const unsigned sh = (0x01223333u >> (4 * c)) & 15u, add = (0x00206420u >> (4 * c)) & 15u;
+            const TW* src = tw + (((off << sh) + add) & ~1u);
+            asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+            dma16(src, (unsigned)(size_t)(lptr_t)lds_t + wave * 1024);
         }
-        if (INVERSE) {
-            if (lane < 32) {
-                const unsigned i = lane >> 3, c = lane & 7;
-                const unsigned off = 256 + 16 * (4 * wq + i) + tile;
-                const TW* src = c < 4 ? tw + (off << 3) + 2 * c : c < 6 ? tw + (off << 2) + 2 * (c - 4) : c == 6 ? tw + (off << 1) : tw + (off & ~1u);
-                dma16(src, (unsigned)(size_t)(lptr_t)lds_t + ((s & 1) * 8 + wave) * 512);
-            }
-        }
+    };
+    auto request = [&](const u64* limb, const TW* tw, int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int m = 0; m < (INVERSE ? 9 : 8); m++) request_part(limb, tw, s, m);
     };
     // end of a pass-1 step: v[j] (forward: row 16 g + j of the group's column tile; inverse: column tile j of the group's row) ->
     // keep the eight values of the parity of this group, hand the other eight to the partner lane, take its eight
     auto hand_over = [&](const V (&v)[16], const AR& ar, int s) __attribute__((always_inline)) {
         unsigned klo[8], khi = 0, shi = 0;
+        // Inverse transforms have no other barrier in a step of pass 1: this one says that the partner has taken what the step
+        // before handed over (the waves are about to meet at the next barrier anyway).
+        if (INVERSE) __syncthreads();
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) {
             const V keep = grp ? v[2 * jj + 1] : v[2 * jj], send = grp ? v[2 * jj] : v[2 * jj + 1];
@@ -219,13 +263,21 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             st.lo[s][1][jj] = to_acc(grp ? klo[jj] : r);
         }
         const unsigned r = lds_s[(8 * 2 + (1 - grp)) * 256 + tid];
-        st.hi[s][0] = grp ? r : khi;
-        st.hi[s][1] = grp ? khi : r;
+        unsigned h0 = grp ? r : khi, h1 = grp ? khi : r;
+        asm volatile("" : "+v"(h0), "+v"(h1));          // formed here, not left in pieces until pass 2 asks for them
+        st.hi[s][0] = h0;
+        st.hi[s][1] = h1;
     };
     // start of a pass-2 step: the sixteen values this lane holds of tile 2 s + grp
     auto take = [&](V (&v)[16], const AR& ar, int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = ar.dec36(from_acc(st.lo[j >> 1][j & 1][s]), (st.hi[j >> 1][j & 1] >> (4 * s)) & 0xfu);
+        for (int j = 0; j < 16; j++) {
+            // the nibble is cut out here and not ahead of time: seen through, the shifts of all eight steps would be formed where
+            // the word is made, and their results kept for the whole limb
+            unsigned h = st.hi[j >> 1][j & 1];
+            asm volatile("" : "+v"(h) : : "memory");
+            v[j] = ar.dec36(from_acc(st.lo[j >> 1][j & 1][s]), (h >> (4 * s)) & 0xfu);
+        }
     };
 
     unsigned it = 0;
@@ -233,9 +285,14 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     if (limb_id >= limbs) return;
     int prime;
     u64* limb = limb_ptr(a, limb_id, RES_N, prime);
+#ifdef CKKS_RES_EXP_STAGGER
+    if ((blockIdx.x >> 3) & 1) { for (int z = 0; z < CKKS_RES_EXP_STAGGER; z++) __builtin_amdgcn_s_sleep(127); }
+#endif
     request(limb, (const TW*)a.tw + (long)prime * RES_N, 0);
+    PackedTwiddles<AR> wp;                               // second-round twiddles of a row-pass step, fetched a step ahead
     TW w_col = 0.0;                                      // this lane's entry of the column pass's twiddle table, fetched ahead
     if (!INVERSE && threadIdx.x < 256) w_col = ((const TW*)a.tw + (long)prime * RES_N)[threadIdx.x];
+    if (INVERSE) wp.load_ordered((const TW*)a.tw + (long)prime * RES_N, 256 + 16 * g + grp, cl);
     for (;;) {
         const AR ar(a.primes[prime]);
         const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * RES_N;
@@ -250,79 +307,110 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
 #pragma unroll
             for (int s = 0; s < 8; s++) {
                 coordinates();
+                RES_TICK(8 * s);
                 wait_all_vmem();                        // this wave's part of the tile has arrived
+                RES_TICK(8 * s + 1);
                 V v[16];
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = ar.from_canonical(p_lane[j * 64]);
-                if (s < 7) request(limb, tw, s + 1);
                 if (s == 0 && threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
-                fwd_round(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; });        // the same for every lane: scalar loads
+                // the same twiddles for every lane: scalar loads; behind each stage one eighth of the next tile is requested
+                fwd_round(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, d); });
 #pragma unroll
                 for (int j = 0; j < 16; j++) col_area[(g + 16 * j) * 16 + cl] = v[j];
+                RES_TICK(8 * s + 5);
                 __syncthreads();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = col_area[(g * 16 + j) * 16 + cl];
-                fwd_round(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; });
+                if (s == 7) {                           // for the first step of pass 2: its row twiddles, both rounds
+                    wp.load_ordered(tw, 256 + 16 * g + grp, cl);
+                    request_part(limb, tw, 0, 8);
+                }
+                fwd_round(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, 4 + d); });
+                RES_TICK(8 * s + 6);
                 hand_over(v, ar, s);
             }
             // ---------------- pass 2: rows (last eight stages), tile k = rows 16 m + k ----------------
+            // Loads and stores complete in the order of their issue, so a load issued behind a step's stores would be waited for
+            // until those stores are done.  Both sets of twiddles of a step are therefore requested before the stores of the step
+            // before: the fifteen of the first round (the same for the sixteen lanes of a row) into the wave's twiddle staging, the
+            // fifteen of the second round into registers.
+            // No barrier in this pass: the sixteen lanes of a row are in one wave, so what a wave exchanges through the row area it
+            // exchanges with itself, and a wave's LDS accesses are carried out in order.
 #pragma unroll
             for (int s = 0; s < 8; s++) {
                 coordinates();
                 const unsigned row = 16 * g + 2 * s + grp;
                 const unsigned tw_off = 256 + row;
+                // the staging has arrived: everything but the sixteen stores behind it is complete
+                RES_TICK(64 + 8 * s);
+                if (s == 0) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+                else asm volatile("s_waitcnt vmcnt(16)" : : : "memory");
+                RES_TICK(64 + 8 * s + 1);
+                const TW* trow = reinterpret_cast<const TW*>(lds_t + wave * 1024 + (lane >> 4) * 128);
                 V v[16];
                 take(v, ar, s);
-                fwd_round(v, ar, [&](int d, int k) { return tw[(tw_off << d) + k]; });
-                PackedTwiddles<AR> wp;
-                wp.load(tw, tw_off, cl);
-                if (s == 6 && more && threadIdx.x < 256) w_col = next_tw[threadIdx.x];
-                __syncthreads();                        // the exchange area is free: every lane has read what the step before left there
+                RES_TICK(64 + 8 * s + 2);
+                fwd_round(v, ar, [&](int d, int k) { return d == 3 ? trow[k] : d == 2 ? trow[8 + k] : d == 1 ? trow[12 + k] : trow[14 + (tw_off & 1u)]; });
+                RES_TICK(64 + 8 * s + 3);
+                RES_TICK(64 + 8 * s + 4);
+                wave_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl + 16 * j)] = v[j];
-                if (s == 7 && more) {
-                    wp.drain();
-                    request(next_limb, next_tw, 0);
-                }
-                __syncthreads();
+                if (s == 7 && more) wp.drain();         // no load of the compiler's is pending when the next limb's tile is requested
+                wave_sync();
+                RES_TICK(64 + 8 * s + 5);
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl * 16 + j)];
-                fwd_round(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; });
+                fwd_round(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; },
+                          [&](int d) { if (s == 7 && more) { request_part(next_limb, next_tw, 0, 2 * d); request_part(next_limb, next_tw, 0, 2 * d + 1); } });
+                RES_TICK(64 + 8 * s + 6);
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
-                __syncthreads();
+                wave_sync();
+                RES_TICK(64 + 8 * s + 7);
+                if (s == 6 && more && threadIdx.x < 256) w_col = next_tw[threadIdx.x];
+                if (s < 7) {
+                    wp.load_ordered(tw, tw_off + 2, cl);
+                    request_part(limb, tw, s + 1, 8);
+                }
                 u64* rp = limb + (long)row * 256;
 #pragma unroll
-                for (int j = 0; j < 16; j++) rp[cl + 16 * j] = ar.to_canonical_fwd(row_area[padded(cl + 16 * j)]);
+                for (int j = 0; j < 16; j++) {
+                    const u64 o = ar.to_canonical_fwd(row_area[padded(cl + 16 * j)]);
+#ifdef CKKS_RES_EXP_NOSTORE
+                    if (o == 0x123456789abcull) rp[cl + 16 * j] = o;
+#else
+                    rp[cl + 16 * j] = o;
+#endif
+                }
             }
         } else {
             // ---------------- pass 1: rows (stages 15 .. 8), tile k = rows 16 m + k ----------------
+            // the row area is exchanged within a wave (the sixteen lanes of a row): no barrier but the hand-over's
 #pragma unroll
             for (int s = 0; s < 8; s++) {
                 coordinates();
                 const unsigned row = 16 * g + 2 * s + grp;
                 const unsigned tw_off = 256 + row;
-                wait_all_vmem();                        // this wave's part of the tile and its row twiddles have arrived
-                PackedTwiddles<AR> wp;
-                wp.load(tw, tw_off, cl);
+                wait_all_vmem();                        // this wave's part of the tile, its row twiddles and the lane's twiddles have arrived
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl + 16 * j)] = ar.from_canonical(p_lane[j * 64]);
-                // the row's fifteen twiddles of the last four stages, before the staging of this parity is requested again (two steps on)
-                const TW* trow = reinterpret_cast<const TW*>(lds_t + ((s & 1) * 8 + wave) * 512 + (lane >> 4) * 128);
-                wp.drain();
-                if (s < 7) request(limb, tw, s + 1);
-                __syncthreads();
+                const TW* trow = reinterpret_cast<const TW*>(lds_t + wave * 1024 + (lane >> 4) * 128);
+                wave_sync();
                 V v[16];
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl * 16 + j)];
-                inv_round<AR, 0>(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; });
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, 3 - d); });
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
                 if (s == 7 && threadIdx.x < 256) w_col = tw[threadIdx.x];
-                __syncthreads();
+                wave_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl + 16 * j)];
-                inv_round<AR, 0>(v, ar, [&](int d, int k) { return d == 3 ? trow[k] : d == 2 ? trow[8 + k] : d == 1 ? trow[12 + k] : trow[14 + (tw_off & 1u)]; });
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return d == 3 ? trow[k] : d == 2 ? trow[8 + k] : d == 1 ? trow[12 + k] : trow[14 + (tw_off & 1u)]; },
+                                 [&](int d) { if (s < 7) { request_part(limb, tw, s + 1, 7 - d); if (d == 0) request_part(limb, tw, s + 1, 8); } });
+                if (s < 7) wp.load_ordered(tw, tw_off + 2, cl);         // the next step's, behind the requests: they arrive together
                 hand_over(v, ar, s);                    // balanced to (-q/2, q/2] between the passes, as in the two-launch form
             }
             if (threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
@@ -337,11 +425,12 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 __syncthreads();                        // the exchange area is free
 #pragma unroll
                 for (int j = 0; j < 16; j++) col_area[(g * 16 + j) * 16 + cl] = v[j];
-                if (s == 7 && more) request(next_limb, next_tw, 0);
                 __syncthreads();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = col_area[(g + 16 * j) * 16 + cl];
-                inv_round<AR, 1>(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; });       // scalar loads
+                inv_round<AR, 1>(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; },        // scalar loads
+                                 [&](int d) { if (s == 7 && more) { request_part(next_limb, next_tw, 0, 9 - 3 * d); request_part(next_limb, next_tw, 0, 10 - 3 * d); request_part(next_limb, next_tw, 0, 11 - 3 * d); } });
+                if (s == 7 && more) wp.load_ordered(next_tw, 256 + 16 * g + grp, cl);
                 u64* col = limb + (2 * s + grp) * 16 + cl;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -352,6 +441,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 }
             }
         }
+        RES_TICK(128);
         if (!more) break;
         __syncthreads();                                // the exchange area is free for the next limb's first step
         it++;
@@ -380,5 +470,11 @@ int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, bool inv
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
+
+#ifdef CKKS_RES_TIMING
+extern "C" int ckks_debug_resident_ticks(unsigned long long* out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_res_ticks), sizeof(unsigned long long) * 8 * 136) == hipSuccess ? 0 : 1;
+}
+#endif
 
 }  // namespace ckks
