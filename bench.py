@@ -7,8 +7,9 @@ One step = inverse transform then forward transform of the whole batch (the orde
 = 2 * 1536 limb-transforms.  value = limb-transforms per second.
 
 Also measured and reported in the same JSON line:
-  roofline      - the slower of the two kernel launches of a forward transform, HIP events on the launch stream;
-                  algorithmic bytes = 16*N per limb-transform, half of it credited to each of the two launches
+  roofline      - the slowest kernel launch of the step, HIP events on the launch stream; algorithmic bytes = 16*N per
+                  limb-transform (all of it in one launch where the library takes the resident transform, half of it credited to
+                  each launch of the two-launch form); beside the published peak the ceiling measured in the same run
   ppmm          - the ring-packed PPMM at the BERT-base shape (configs[3]), int8-MAC/s against the int8 MFMA peak
   keyswitch     - one textbook hybrid key switch at configs[2]
   cpu_baseline  - the CPU oracle (a port of the reference arithmetic, OpenMP) on a bounded sample of the same workload
@@ -111,42 +112,76 @@ def bench_ntt(args, P):
     ms_per_step = dt / args.steps * 1e3
     value = 2 * limbs * args.steps / dt
 
-    # per-kernel durations (HIP events between the two launches), averaged
-    reps = max(5, args.steps) if not args.ntt_mode else 0       # the one-launch modes have no second launch to time
+    # Per-kernel durations, HIP events on the launch stream.  Where the library takes the resident transform (one launch per
+    # transform: N = 2^16, primes below 2^36, at least a limb per compute unit) the launch is the transform; otherwise a transform
+    # is two launches and the events sit between them.
+    reps = max(5, args.steps)
+    per_round = ctx.info("ntt_resident_round")
+    resident = args.ntt_mode in (0, 6) and per_round > 0 and limbs >= per_round and max(primes) < (1 << 36)
+    one_launch = resident or args.ntt_mode in (2, 3, 4, 5)
+    alg_bytes_transform = 16.0 * N * limbs
+    traffic, traffic_note = measured_traffic()
+
+    def timed(f, n):
+        for _ in range(2):
+            f(buf, 0, 0, polys, L1, L1)
+        ctx.timer_start()
+        for _ in range(n):
+            f(buf, 0, 0, polys, L1, L1)
+        return ctx.timer_stop() / n
+
+    # the two-launch form, pass by pass (what the library falls back to, and the reference point of the one-launch forms)
+    ctx.set_ntt_mode(0 if one_launch else args.ntt_mode)      # the timed entry point always takes two launches (5-byte form between them)
     f1 = f2 = i1 = i2 = 0.0
-    if not reps:
-        ctx.timer_start()
-        for _ in range(10):
-            ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
-        f1 = f2 = ctx.timer_stop() / 20
-        ctx.timer_start()
-        for _ in range(10):
-            ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
-        i1 = i2 = ctx.timer_stop() / 20
-        reps = 1
-        f1, f2, i1, i2 = [x * reps for x in (f1, f2, i1, i2)]
-    for _ in range(reps if not args.ntt_mode else 0):
+    for _ in range(reps):
         a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, True)
         i1 += a; i2 += b
         a, b = ctx.ntt_timed(buf, 0, 0, polys, L1, L1, False)
         f1 += a; f2 += b
     f1, f2, i1, i2 = [x / reps for x in (f1, f2, i1, i2)]
-    alg_bytes_launch = 16.0 * N * limbs / 2.0          # half a transform per launch
-    dom_name, dom_ms = max([("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2)], key=lambda x: x[1])
+    ctx.set_ntt_mode(args.ntt_mode)
+    passes = [("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2), ("ntt_row_pass(inv)", i1), ("ntt_strided_pass(inv)", i2)]
+    pass_ms = {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)}
+    if one_launch:
+        fwd_ms, inv_ms = timed(ctx.ToNTTInplace, 2 * reps), timed(ctx.FromNTTInplace, 2 * reps)
+        name = "ntt_resident_kernel" if resident else "one-launch transform (ntt_mode %d)" % args.ntt_mode
+        dom_name, dom_ms = max([(name + "(fwd)", fwd_ms), (name + "(inv)", inv_ms)], key=lambda x: x[1])
+        alg_bytes_launch = alg_bytes_transform
+        key = "ntt_resident_fwd_1536_limbs" if dom_name.endswith("(fwd)") else "ntt_resident_inv_1536_limbs"
+        kernel_ms = {"fwd": round(fwd_ms, 4), "inv": round(inv_ms, 4)}
+    else:
+        fwd_ms, inv_ms = f1 + f2, i1 + i2
+        dom_name, dom_ms = max(passes, key=lambda x: x[1])          # the slowest of all four passes
+        alg_bytes_launch = alg_bytes_transform / 2.0                # half a transform per launch
+        key = {"ntt_strided_pass(fwd)": "ntt_strided_pass_fwd_1536_limbs", "ntt_row_pass(fwd)": "ntt_row_pass_fwd_1536_limbs",
+               "ntt_row_pass(inv)": "ntt_row_pass_inv_1536_limbs", "ntt_strided_pass(inv)": "ntt_strided_pass_inv_1536_limbs"}[dom_name]
+        kernel_ms = pass_ms
     achieved = alg_bytes_launch / (dom_ms * 1e-3) / 1e9
-    traffic, traffic_note = measured_traffic()
-    key = "ntt_strided_pass_fwd_1536_limbs" if dom_name.startswith("ntt_strided") else "ntt_row_pass_fwd_1536_limbs"
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic.get(key) if limbs == 1536 else None, "traffic_source": traffic_note,
-                "kernel_ms": {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)},
-                "transform_algorithmic_GBps": {"fwd": round(16.0 * N * limbs / ((f1 + f2) * 1e-3) / 1e9, 1),
-                                               "inv": round(16.0 * N * limbs / ((i1 + i2) * 1e-3) / 1e9, 1)},
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic.get(key) if limbs == 1536 and resident == (args.ntt_mode in (0, 6)) else None,
+                "traffic_source": traffic_note, "launches_per_transform": 1 if one_launch else 2, "kernel_ms": kernel_ms,
+                "two_launch_form_pass_ms": pass_ms,
+                "transform_algorithmic_GBps": {"fwd": round(alg_bytes_transform / (fwd_ms * 1e-3) / 1e9, 1),
+                                               "inv": round(alg_bytes_transform / (inv_ms * 1e-3) / 1e9, 1)},
                 "algorithmic_bytes_per_launch": alg_bytes_launch}
-    if args.batch_only:
-        # reference point for the traffic counters: one device-to-device copy of known size in the same process
-        half = 4 * limbs * N
+    # measured ceiling of the same run: a device-to-device copy of half the batch onto the other half (reads and writes %d MiB each)
+    half = 4 * limbs * N
+    for _ in range(2):
         buf.L_.ckks_memcpy_d2d(buf.ptr + half, buf.ptr, half)
-        ctx.sync()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        buf.L_.ckks_memcpy_d2d(buf.ptr + half, buf.ptr, half)
+    ctx.sync()
+    copy_gbs = 2.0 * half * 5 / (time.perf_counter() - t0) / 1e9
+    roofline["peak_measured"] = round(copy_gbs, 1)
+    roofline["peak_measured_how"] = "device-to-device copy of %d MiB in the same run, bytes read + bytes written per second" % (half >> 20)
+    roofline["frac_of_measured"] = round(achieved / copy_gbs, 4)
+    # the copy overwrote half of the batch: put the seeded data back for what follows
+    for c in range(cts):
+        buf.L_.ckks_memcpy_h2d(buf.ptr + c * one.nbytes, one.ctypes.data, one.nbytes)
+    ctx.sync()
+    if args.batch_only:
         buf.free()
         return value, ms_per_step, roofline, None, limbs
     # one ciphertext (48 limbs, 24 MiB): the latency-oriented half of configs[1]
@@ -221,8 +256,8 @@ def main():
     ap.add_argument("--chain-skew", type=int, default=0, help="profiling aid with --ntt-mode 2: limbs the first pass runs ahead")
     ap.add_argument("--skip-extra", action="store_true", help="skip the PPMM / key-switch side measurements")
     ap.add_argument("--batch-only", action="store_true",
-                    help="profiling aid: only the batched NTT launches (no one-ciphertext, PPMM, key-switch or CPU legs), plus one "
-                         "device-to-device copy of half the batch as the reference point of the traffic counters")
+                    help="profiling aid: only the batched NTT launches (no one-ciphertext, PPMM, key-switch or CPU legs); the "
+                         "device-to-device copies of half the batch in it are the reference point of the traffic counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)

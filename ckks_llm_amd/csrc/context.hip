@@ -419,6 +419,7 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
     else if (n == "gamma") *value = c->gamma; else if (n == "dnum") *value = c->dnum;
     else if (n == "Ri_blockNum") *value = c->Ri_blockNum; else if (n == "Qj_blockNum") *value = c->Qj_blockNum;
     else if (n == "arith_mode") *value = c->arith_mode; else if (n == "ntt_mode") *value = c->ntt_mode;
+    else if (n == "ntt_resident_round") *value = c->logN == 16 ? ckks::ntt_resident_round(c) : 0;      // limbs per round of the resident transform (0: it never applies)
     else if (n == "ntt_chain_deferred_tiles") return ckks::ntt_chain_deferred(const_cast<ckks_ctx*>(c), value);
     else { ckks::set_error("ckks_ctx_info: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
@@ -434,7 +435,8 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
 // test / tuning hook: 0 = automatic, 1 = two launches per transform, 2 = chained one-launch transform wherever that kernel exists
 // (N >= 2^15), 3 = one workgroup per limb wherever that kernel exists (N >= 2^15), 4 = paired one-launch transform at every batch
 // size (N = 2^16; the automatic mode takes it for small batches), 5 = the same with the tiles of a limb spread over all XCDs
-// (the automatic mode's choice between 41 and 128 limbs)
+// (the automatic mode's choice between 41 and 128 limbs), 6 = the resident transform wherever it applies (N = 2^16, primes below
+// 2^36, at least one limb per compute unit; the automatic mode takes it there too)
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
     if (!c || mode < 0 || mode > 6) return CKKS_E_INVALID;
     c->ntt_mode = mode;

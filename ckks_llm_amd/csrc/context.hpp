@@ -127,10 +127,12 @@ int ntt_noalloc_init(char** ptr_out);
 int ntt_noalloc_max_limbs();
 int launch_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num, int poly_mod_len,
                        bool inverse);
-// Resident transform (ntt_resident.hip): whether it takes a call of `limbs` limbs, and its launch (FP64 back end, primes below 2^39).
+// Resident transform (ntt_resident.hip): whether it takes a call of `limbs` limbs, and its launch (FP64 back end, primes below 2^36).
 struct NttArgs;
 bool ntt_resident_applies(const ckks_ctx* c, int limbs);
-int launch_ntt_resident(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse);
+int ntt_resident_round(const ckks_ctx* c);              // limbs per round: one per workgroup of its grid
+// transforms the first `count` of the call's `limbs` limbs (limb order of the two-launch form)
+int launch_ntt_resident(ckks_ctx* c, const NttArgs& args, int limbs, int count, bool inverse);
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse);
 // Hybrid key switch up to the inverse transform of the two sums, in five launches (four where the input's transform runs as one

@@ -573,17 +573,18 @@ static void launch_passes(ckks_ctx* c, const NttArgs& args_in, int n, bool inver
 }
 
 template <class AR, int SA, int SB>
-static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok) {
+static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, int first = 0) {
+    // first: the limbs before it have been taken by another launch form (the resident transform takes whole rounds of a batch)
     constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
     static const int chunk_env = getenv("CKKS_NTT_CHUNK") ? atoi(getenv("CKKS_NTT_CHUNK")) : 0;
-    int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs;
+    int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs - first;
     const bool compact = CAN_COMPACT && compact_ok && c->ntt_mode != 1;
     if (compact) {
         // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
         if (c->mid_fixed) {
             // caller-provided inter-pass area (the entry point that allocates nothing): the batch must fit it whole
-            if ((size_t)limbs * MID_LIMB_BYTES > c->mid_fixed_cap) { set_error("NTT: batch larger than the fixed inter-pass area"); return CKKS_E_INVALID; }
-            chunk = limbs;
+            if ((size_t)(limbs - first) * MID_LIMB_BYTES > c->mid_fixed_cap) { set_error("NTT: batch larger than the fixed inter-pass area"); return CKKS_E_INVALID; }
+            chunk = limbs - first;
             args.mid = c->mid_fixed;
         } else {
             const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
@@ -596,7 +597,7 @@ static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, b
         args.mid = nullptr;
     }
     args.limbs_total = (unsigned)limbs;
-    for (int base = 0; base < limbs; base += chunk) {
+    for (int base = first; base < limbs; base += chunk) {
         const int n = limbs - base < chunk ? limbs - base : chunk;
         args.limb_base = (unsigned)base;
         if constexpr (CAN_COMPACT) {
@@ -695,15 +696,25 @@ static bool pair_applies(const ckks_ctx* c, int limbs) {
 }
 
 template <class AR>
-static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok) {
+static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok, bool res36_ok = false) {
     // mode 2: both passes in one launch, the limb held in the XCD's L2 between them (N >= 2^15)
     if (!c->ev_mid_armed && c->ntt_mode == 2 && !args.embed_mlwe) {
         if (c->logN == 16) return launch_chain<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_chain<AR, 8, 7>(c, args, limbs, inverse);
     }
-    // mode 6: the resident transform - one persistent workgroup per compute unit carries whole limbs through both passes in its registers
-    if (!c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && c->ntt_mode == 6 && std::is_same<AR, F64Arith>::value && compact_ok && ntt_resident_applies(c, limbs))
-        return launch_ntt_resident(c, args, limbs, inverse);
+    // The resident transform - one persistent workgroup per compute unit carries whole limbs through both passes in its registers
+    // (N = 2^16, primes below 2^36) - takes the whole rounds of a batch (one limb per compute unit and round) and a last round that is
+    // at least three quarters full; what is left goes out as two launches behind it.  Mode 6 asks for it wherever it applies, the
+    // automatic mode takes it too, mode 1 never.
+    if (std::is_same<AR, F64Arith>::value && !c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && (c->ntt_mode == 0 || c->ntt_mode == 6) && res36_ok &&
+        ntt_resident_applies(c, limbs)) {
+        const int per_round = ntt_resident_round(c);
+        int whole = limbs / per_round * per_round;
+        if (limbs - whole >= per_round * 3 / 4) whole = limbs;
+        int rc = launch_ntt_resident(c, args, limbs, whole, inverse);
+        if (rc || whole == limbs) return rc;
+        return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok, whole);
+    }
     // mode 4, and the automatic mode for small batches: both passes in one launch of one workgroup per (limb, tile)
     if (!c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs)) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
     // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
@@ -1584,10 +1595,11 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
         return m < (1ull << 41) ? 0 : m < (1ull << 50) ? 1 : 2;
     };
     int back_end = klass(0);
-    bool mixed = false, compact_ok = true;
+    bool mixed = false, compact_ok = true, res36_ok = true;
     for (int j = 0; j < mod_num; j++) {
         mixed = mixed || klass(j) != back_end;
         compact_ok = compact_ok && c->pqt[start_mod_idx + j] < (1ull << 39);
+        res36_ok = res36_ok && c->pqt[start_mod_idx + j] < (1ull << 36);
     }
     if (mixed) {
         // a call that spans prime widths ([P | Q | T] of the reference's sets: 49-bit P and Q, 60-bit T) goes out as one launch
@@ -1622,7 +1634,7 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
     }
     if (back_end == 0) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
-        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok);
+        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok, res36_ok);
     }
     if (back_end == 1) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;

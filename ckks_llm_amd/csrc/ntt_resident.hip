@@ -65,6 +65,16 @@ __device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
 // Ordering point for what a wave exchanges with itself through LDS (the hardware carries out a wave's LDS accesses in order; this
 // keeps the compiler from reordering them: as one thread sees it, the lane that writes and the lane that reads are unrelated).
 __device__ __forceinline__ void wave_sync() { __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); __builtin_amdgcn_wave_barrier(); }
+#ifdef CKKS_RES_EXP_NOCOLBAR
+__device__ __forceinline__ void col_sync() { wave_sync(); }
+#else
+__device__ __forceinline__ void col_sync() { __syncthreads(); }
+#endif
+#ifdef CKKS_RES_EXP_NOHANDBAR
+__device__ __forceinline__ void hand_sync() { wave_sync(); }
+#else
+__device__ __forceinline__ void hand_sync() { __syncthreads(); }
+#endif
 __device__ __forceinline__ void wait_all_vmem() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 
 // The fifteen twiddles of the last four stages of an axis (packed layout, lane group g: stage 4 + d, butterfly group k),
@@ -244,7 +254,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
         unsigned klo[8], khi = 0, shi = 0;
         // Inverse transforms have no other barrier in a step of pass 1: this one says that the partner has taken what the step
         // before handed over (the waves are about to meet at the next barrier anyway).
-        if (INVERSE) __syncthreads();
+        if (INVERSE) hand_sync();
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) {
             const V keep = grp ? v[2 * jj + 1] : v[2 * jj], send = grp ? v[2 * jj] : v[2 * jj + 1];
@@ -255,7 +265,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             shi |= (unsigned)(es >> 32) << (4 * jj);
         }
         lds_s[(8 * 2 + grp) * 256 + tid] = shi;
-        __syncthreads();
+        hand_sync();
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) {
             const unsigned r = lds_s[(jj * 2 + (1 - grp)) * 256 + tid];
@@ -319,7 +329,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
 #pragma unroll
                 for (int j = 0; j < 16; j++) col_area[(g + 16 * j) * 16 + cl] = v[j];
                 RES_TICK(8 * s + 5);
-                __syncthreads();
+                col_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = col_area[(g * 16 + j) * 16 + cl];
                 if (s == 7) {                           // for the first step of pass 2: its row twiddles, both rounds
@@ -422,10 +432,10 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 V v[16];
                 take(v, ar, s);
                 inv_round<AR, 0>(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; });
-                __syncthreads();                        // the exchange area is free
+                col_sync();                             // the exchange area is free
 #pragma unroll
                 for (int j = 0; j < 16; j++) col_area[(g * 16 + j) * 16 + cl] = v[j];
-                __syncthreads();
+                col_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = col_area[(g + 16 * j) * 16 + cl];
                 inv_round<AR, 1>(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; },        // scalar loads
@@ -452,21 +462,24 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
 
 }  // namespace
 
-// Whether the resident transform takes a call: N = 2^16 and enough limbs to give every compute unit work.
-bool ntt_resident_applies(const ckks_ctx* c, int limbs) { return c->logN == 16 && limbs >= c->cu_count; }
+// Whether the resident transform takes a call: N = 2^16 and enough limbs to give every compute unit one.
+static unsigned resident_grid(const ckks_ctx* c) {
+    // one workgroup per compute unit, a multiple of eight so that the XCDs get equal shares
+    const unsigned grid = (unsigned)c->cu_count / 8 * 8;
+    return grid ? grid : 8;
+}
+bool ntt_resident_applies(const ckks_ctx* c, int limbs) { return c->logN == 16 && limbs >= (int)resident_grid(c); }
+int ntt_resident_round(const ckks_ctx* c) { return (int)resident_grid(c); }
 
-// args: as for the two-launch transform.  FP64 back end, every prime of the call below 2^39 (the 5-byte form).
-int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, bool inverse) {
+// args: as for the two-launch transform.  FP64 back end, every prime of the call below 2^36 (the 36-bit form of the values between the passes).
+int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, int count, bool inverse) {
     NttArgs args = args_in;
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
     args.mid = nullptr;
-    // one workgroup per compute unit, a multiple of eight so that the XCDs get equal shares
-    unsigned grid = (unsigned)c->cu_count / 8 * 8;
-    if (grid == 0) grid = 8;
-    const dim3 g(grid), b(RES_LANES);
-    if (!inverse) hipLaunchKernelGGL((ntt_resident_kernel<false>), g, b, 0, c->stream, args, (unsigned)limbs);
-    else hipLaunchKernelGGL((ntt_resident_kernel<true>), g, b, 0, c->stream, args, (unsigned)limbs);
+    const dim3 g(resident_grid(c)), b(RES_LANES);
+    if (!inverse) hipLaunchKernelGGL((ntt_resident_kernel<false>), g, b, 0, c->stream, args, (unsigned)count);
+    else hipLaunchKernelGGL((ntt_resident_kernel<true>), g, b, 0, c->stream, args, (unsigned)count);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }

@@ -59,7 +59,8 @@ int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int p_num, cons
 int ckks_ctx_destroy(ckks_ctx* ctx);
 int ckks_set_stream(ckks_ctx* ctx, void* hip_stream);
 /* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum","arith_mode","ntt_mode";
- * "ntt_chain_deferred_tiles" (synchronises): second-pass tiles that chained transforms have left to their finishing launch */
+ * "ntt_chain_deferred_tiles" (synchronises): second-pass tiles that chained transforms have left to their finishing launch;
+ * "ntt_resident_round": limbs that one round of the resident transform takes (one per compute unit; 0 where it never applies) */
 int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
 /* 0 (default): FP64 butterflies for primes < 2^41, integer butterflies otherwise; 1: integer butterflies everywhere.
  * Both give the same residues; the switch exists for testing and tuning. */
@@ -70,7 +71,9 @@ int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
  * 3: one workgroup carries a limb through both passes (N >= 2^15); 4: paired - both passes in one launch of one workgroup per
  * (limb, tile), which waits between its two tiles until the limb's first pass is complete (N = 2^16, up to 4096 limbs; mode 0
  * takes this form for batches of up to 128 limbs, where it is faster than two launches); 5: as 4 with the tiles of a limb spread
- * over all XCDs (what mode 0 does above 40 limbs).  All give the same residues.  Should a wait of the paired form ever run out (about two
+ * over all XCDs (what mode 0 does above 40 limbs); 6: resident - one persistent workgroup per compute unit carries whole limbs
+ * through both passes in its registers, so that a limb crosses HBM once in and once out (N = 2^16, primes below 2^36, at least one
+ * limb per compute unit; mode 0 takes it there too, for the whole rounds of a batch).  All give the same residues.  Should a wait of the paired form ever run out (about two
  * seconds), the transform's output is incomplete, ckks_ctx_check and every later transform of the context return CKKS_E_UNAVAILABLE.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);

@@ -226,6 +226,37 @@ def test_whole_limb_transform_matches_oracle(logN, polys, mode):
     buf.free()
 
 
+@pytest.mark.parametrize("polys,mode", [(11, 6), (19, 0), (12, 0), (53, 0)])
+def test_resident_transform_matches_oracle(polys, mode):
+    """The resident transform (one persistent workgroup per compute unit carries whole limbs through both passes in its registers;
+    N = 2^16, primes below 2^36, at least 256 limbs) against the oracle, both directions and the reference's sub-range addressing:
+    264 limbs (a full round and a few), 456 (a second round three quarters full: all resident), 288 (the 32 limbs beyond the first
+    round go out as two launches), 1272 (five rounds less eight limbs)."""
+    q = CFG2_Q
+    pair = Pair(16, [], q)
+    N, L1 = pair.N, len(q)
+    data = limbs_uniform(600 + polys, q, polys, N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, L1, L1)
+    want_inv = data.copy()
+    pair.orc.FromNTTInplace(want_inv.reshape(-1), 0, 0, polys, L1, L1)
+    pair.dev.set_ntt_mode(mode)
+    buf = to_dev(data)
+    for _ in range(2):
+        pair.dev.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+        assert np.array_equal(from_dev(buf, data.shape), want)
+        pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+        assert np.array_equal(from_dev(buf, data.shape), data)
+    pair.dev.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+    assert np.array_equal(from_dev(buf, data.shape), want_inv)
+    # limbs 1 .. 22 of every polynomial (the first and the last stay as they are)
+    buf.upload(data)
+    pair.dev.ToNTTInplace(buf, 1, 1, polys, L1 - 2, L1)
+    got = from_dev(buf, data.shape)
+    assert np.array_equal(got[:, 1:L1 - 1], want[:, 1:L1 - 1]) and np.array_equal(got[:, 0], data[:, 0]) and np.array_equal(got[:, L1 - 1], data[:, L1 - 1])
+    buf.free()
+
+
 @pytest.mark.parametrize("primes,polys,arith,mode", [("36", 9, 0, 4), ("36", 5, 1, 4), ("49", 3, 0, 4), ("mixed", 2, 0, 4), ("36", 1, 0, 4),
                                                     ("36", 7, 0, 5), ("49", 2, 0, 5), ("36", 3, 1, 5), ("36", 8, 0, 0), ("36", 11, 0, 0)])
 def test_paired_transform_matches_oracle(primes, polys, arith, mode):
