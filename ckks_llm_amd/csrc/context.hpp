@@ -88,6 +88,7 @@ struct ckks_ctx {
     size_t qiInv_count = 0;
 
     int arith_mode = 0;                   // 0: automatic (FP64 where valid), 1: force integer back end
+    unsigned res_backwards = 0;           // resident transform: direction in which the next launch walks its rounds (alternates)
     int ntt_mode = 0;                     // 0: automatic, 1: two launches per transform, 2: chained one-launch transform, 3: one workgroup per limb,
                                           // 4: paired one-launch transform at every batch size, 5: the same with a limb's tiles spread over the XCDs
     int cu_count = 256;

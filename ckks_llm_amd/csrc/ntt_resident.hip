@@ -185,7 +185,7 @@ struct Stash {
 };
 
 template <bool INVERSE>
-__global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsigned limbs) {
+__global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsigned limbs, unsigned backwards) {
     typedef F64Arith AR;
     typedef double V;
     typedef double TW;
@@ -290,9 +290,14 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
         }
     };
 
+    // Rounds of this workgroup (its limbs lie `gridDim.x` apart, so they are the rounds 0 .. rounds - 1), walked upwards or
+    // downwards: a launch that starts where the launch before it ended finds the last-written limbs in the memory-side cache.
+    const unsigned first_id = resident_limb(blockIdx.x, gridDim.x, 0);
+    if (first_id >= limbs) return;
+    const unsigned rounds = (limbs - first_id + gridDim.x - 1) / gridDim.x;
+    auto round_limb = [&](unsigned i) { return resident_limb(blockIdx.x, gridDim.x, backwards ? rounds - 1 - i : i); };
     unsigned it = 0;
-    unsigned limb_id = resident_limb(blockIdx.x, gridDim.x, it);
-    if (limb_id >= limbs) return;
+    unsigned limb_id = round_limb(0);
     int prime;
     u64* limb = limb_ptr(a, limb_id, RES_N, prime);
 #ifdef CKKS_RES_EXP_STAGGER
@@ -306,8 +311,8 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     for (;;) {
         const AR ar(a.primes[prime]);
         const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * RES_N;
-        const unsigned next_id = resident_limb(blockIdx.x, gridDim.x, it + 1);
-        const bool more = next_id < limbs;
+        const bool more = it + 1 < rounds;
+        const unsigned next_id = more ? round_limb(it + 1) : limb_id;
         int next_prime = prime;
         u64* next_limb = more ? limb_ptr(a, next_id, RES_N, next_prime) : limb;
         const TW* next_tw = (const TW*)a.tw + (long)next_prime * RES_N;
@@ -478,8 +483,13 @@ int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, int coun
     args.limbs_total = (unsigned)limbs;
     args.mid = nullptr;
     const dim3 g(resident_grid(c)), b(RES_LANES);
-    if (!inverse) hipLaunchKernelGGL((ntt_resident_kernel<false>), g, b, 0, c->stream, args, (unsigned)count);
-    else hipLaunchKernelGGL((ntt_resident_kernel<true>), g, b, 0, c->stream, args, (unsigned)count);
+    // Successive launches of a context walk the rounds in opposite directions: where the same batch goes through several
+    // transforms in a row, each starts on the limbs that the one before wrote last.  The order of the limbs has no effect
+    // on the results.
+    const unsigned backwards = c->res_backwards;
+    c->res_backwards ^= 1u;
+    if (!inverse) hipLaunchKernelGGL((ntt_resident_kernel<false>), g, b, 0, c->stream, args, (unsigned)count, backwards);
+    else hipLaunchKernelGGL((ntt_resident_kernel<true>), g, b, 0, c->stream, args, (unsigned)count, backwards);
     CKKS_HIP_TRY(hipGetLastError());
     return CKKS_OK;
 }
