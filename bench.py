@@ -279,7 +279,7 @@ def main():
     if not args.skip_extra:
         try:
             import bench_extra
-            line.update(bench_extra.run(P, measured_traffic()))
+            line.update(bench_extra.run(P, measured_traffic(), roofline.get("peak_measured")))
         except ImportError:
             pass
     if not args.skip_cpu:

@@ -33,6 +33,7 @@ def _declare(L):
         "ckks_malloc": (i, [C.POINTER(vp), sz]), "ckks_free": (i, [vp]),
         "ckks_memcpy_h2d": (i, [vp, vp, sz]), "ckks_memcpy_d2h": (i, [vp, vp, sz]), "ckks_memcpy_d2d": (i, [vp, vp, sz]),
         "ckks_memset": (i, [vp, i, sz]), "ckks_sync": (i, []), "ckks_device_count": (i, [C.POINTER(i)]),
+        "ckks_measure_mfma_i8_peak": (i, [vp, C.POINTER(d)]),
         "ckks_timer_start": (i, [vp]), "ckks_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
         "ckks_ctx_create": (i, [C.POINTER(vp), i, u64p, i, u64p, i, u64p, i, i]), "ckks_ctx_destroy": (i, [vp]),
         "ckks_set_stream": (i, [vp, vp]), "ckks_ctx_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
@@ -83,7 +84,7 @@ def _declare(L):
         "pcmm_ppmm_packed": (i, [vp, vp, vp, i, d]),
         "pcmm_ppmm": (i, [vp, vp, C.POINTER(vp), vp, i, i, i, d]),
         "pcmm_ppmm_strided": (i, [vp, vp, vp, vp, i, i, i, d]),
-        "pcmm_set_weight_cache": (i, [vp, i]),
+        "pcmm_set_weight_cache": (i, [vp, i]), "pcmm_weights_static": (i, [vp, vp, sz, i]),
         "pcmm_weights_changed": (i, [vp, vp]),
     }
     missing = []

@@ -617,8 +617,14 @@ class PCMM_Context:
         _check(self.L_.pcmm_info(self.h, name.encode(), C.byref(v)), "pcmm_info")
         return v.value
 
+    def weights_static(self, plain_mat, nbytes=None, is_static=True):
+        """Declare a weight matrix static (it changes only through this library's copies): its digit planes are kept between PPMM
+        calls.  By default every call reads its matrix afresh, as the reference does (PPMM_kernel.cuh:148)."""
+        n = nbytes if nbytes is not None else plain_mat.nbytes
+        _check(self.L_.pcmm_weights_static(self.h, _addr(plain_mat), n, int(bool(is_static))), "pcmm_weights_static")
+
     def set_weight_cache(self, enabled):
-        """Keep (default) or do not keep the digit planes of plaintext matrices between PPMM calls."""
+        """Declare every plaintext matrix given to this context static (True), or take that back (False, the default)."""
         _check(self.L_.pcmm_set_weight_cache(self.h, int(bool(enabled))), "pcmm_set_weight_cache")
 
     def weights_changed(self, plain_mat=None):
@@ -922,6 +928,13 @@ class Bert_model_weights:
                 for leaf in self.LAYER:
                     getattr(self, leaf.replace(".", "_"))[i] = load("bert.encoder.layer.%d.%s" % (i, leaf))
 
+    def buffers(self):
+        """Every device buffer that was loaded."""
+        out = [getattr(self, m) for m in self.GLOBAL]
+        for leaf in self.LAYER:
+            out += getattr(self, leaf.replace(".", "_"))
+        return [b for b in out if b is not None]
+
 
 class Bert:
     """The PCMM calls of the linear layers of Bert (src/bert/Bert.h:15-66; Bert.cuh:155-169, 204-211, 249-257, 296-302, 404-489):
@@ -942,6 +955,9 @@ class Bert:
         self.ppmm_output = None
         self.embeded_mlwe_buffer = DeviceBuffer(8 * (self.mlwe_rank + 1) * 2 * self.N)
         self.mult_key_output = DeviceBuffer(8 * 4 * self.N)
+        # the model's tensors were uploaded by this object and are not written again: their digit planes are kept between calls
+        for buf in self.model_weights.buffers():
+            pc.weights_static(buf)
 
     def linear(self, plain_mat, M, Nin, parts_in, parts_out):
         """parts_in: (ciphertext, count, offset, extract); parts_out: (ciphertext, count, offset)."""

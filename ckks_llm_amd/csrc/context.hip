@@ -419,6 +419,7 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
     else if (n == "gamma") *value = c->gamma; else if (n == "dnum") *value = c->dnum;
     else if (n == "Ri_blockNum") *value = c->Ri_blockNum; else if (n == "Qj_blockNum") *value = c->Qj_blockNum;
     else if (n == "arith_mode") *value = c->arith_mode; else if (n == "ntt_mode") *value = c->ntt_mode;
+    else if (n == "ntt_mid_bytes") *value = (long)c->ntt_mid_cap;      // size of the inter-pass buffer the ordinary entry points have grown so far
     else if (n == "ntt_resident_round") *value = c->logN == 16 ? ckks::ntt_resident_round(c) : 0;      // limbs per round of the resident transform (0: it never applies)
     else if (n == "ntt_chain_deferred_tiles") return ckks::ntt_chain_deferred(const_cast<ckks_ctx*>(c), value);
     else { ckks::set_error("ckks_ctx_info: unknown name " + n); return CKKS_E_INVALID; }
@@ -506,8 +507,8 @@ extern "C" int ckks_free(void* p) {
     if (!p) return CKKS_OK;
     hipDeviceptr_t base = nullptr;
     size_t size = 0;
-    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) == hipSuccess && size) pcmm_forget_weights(base, size);
-    else { (void)hipGetLastError(); pcmm_forget_weights(p, 1); }
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) == hipSuccess && size) pcmm_forget_weights(base, size, true);
+    else { (void)hipGetLastError(); pcmm_forget_weights(p, 1, true); }
     CKKS_HIP_TRY(hipFree(p));
     return CKKS_OK;
 }

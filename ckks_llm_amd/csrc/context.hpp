@@ -94,8 +94,6 @@ struct ckks_ctx {
     int cu_count = 256;
     void* d_ntt_mid = nullptr;            // compact inter-pass buffer of the two-launch transform, grown on demand
     size_t ntt_mid_cap = 0;
-    char* mid_fixed = nullptr;            // set for the duration of a call that must not allocate: inter-pass area to use instead
-    size_t mid_fixed_cap = 0;
     int device = 0;                       // the device that was current when the context was created
     struct DecodeTab { int level, words; void* dev; };
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
@@ -178,4 +176,4 @@ int launch_repack_front_fused(ckks_ctx* c, uint64_t* work, uint64_t* acc, const 
 
 // Device memory [lo, lo + bytes) was freed or overwritten through the library's own plumbing: every ring-pack handle forgets the
 // plaintext matrices it had prepared from there (pcmm.hip).
-void pcmm_forget_weights(const void* lo, size_t bytes);
+void pcmm_forget_weights(const void* lo, size_t bytes, bool freed = false);

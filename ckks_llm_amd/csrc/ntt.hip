@@ -548,6 +548,9 @@ static int launch_pair(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool 
     return CKKS_OK;
 }
 
+// inter-pass area that a call brings with it (the entry point that allocates nothing) instead of the context's buffer
+struct NttFixedArea { char* mid; size_t cap; };
+
 // launches of one chunk of limbs; COMPACT selects the 5-byte inter-pass buffer
 template <class AR, int SA, int SB, bool COMPACT>
 static void launch_passes(ckks_ctx* c, const NttArgs& args_in, int n, bool inverse) {
@@ -573,19 +576,19 @@ static void launch_passes(ckks_ctx* c, const NttArgs& args_in, int n, bool inver
 }
 
 template <class AR, int SA, int SB>
-static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, int first = 0) {
+static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, int first = 0, const NttFixedArea* fixed = nullptr) {
     // first: the limbs before it have been taken by another launch form (the resident transform takes whole rounds of a batch)
     constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
     static const int chunk_env = getenv("CKKS_NTT_CHUNK") ? atoi(getenv("CKKS_NTT_CHUNK")) : 0;
     int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs - first;
-    const bool compact = CAN_COMPACT && compact_ok && c->ntt_mode != 1;
+    const bool compact = CAN_COMPACT && compact_ok && (fixed || c->ntt_mode != 1);
     if (compact) {
         // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
-        if (c->mid_fixed) {
-            // caller-provided inter-pass area (the entry point that allocates nothing): the batch must fit it whole
-            if ((size_t)(limbs - first) * MID_LIMB_BYTES > c->mid_fixed_cap) { set_error("NTT: batch larger than the fixed inter-pass area"); return CKKS_E_INVALID; }
+        if (fixed) {
+            // inter-pass area given with the call (the entry point that allocates nothing): the batch must fit it whole
+            if ((size_t)(limbs - first) * MID_LIMB_BYTES > fixed->cap) { set_error("NTT: batch larger than the fixed inter-pass area"); return CKKS_E_INVALID; }
             chunk = limbs - first;
-            args.mid = c->mid_fixed;
+            args.mid = fixed->mid;
         } else {
             const int max_limbs = (int)((1l << 30) / MID_LIMB_BYTES);
             if (chunk > max_limbs) chunk = max_limbs;
@@ -696,9 +699,13 @@ static bool pair_applies(const ckks_ctx* c, int limbs) {
 }
 
 template <class AR>
-static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok, bool res36_ok = false) {
+static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok, bool res36_ok = false,
+                         const NttFixedArea* fixed = nullptr) {
+    // A call that brings its inter-pass area runs as two launches whatever the context's mode (nothing of the context is
+    // changed for it: other threads' calls on the same context see the mode they set).
+    const int mode = fixed ? 1 : c->ntt_mode;
     // mode 2: both passes in one launch, the limb held in the XCD's L2 between them (N >= 2^15)
-    if (!c->ev_mid_armed && c->ntt_mode == 2 && !args.embed_mlwe) {
+    if (!c->ev_mid_armed && mode == 2 && !args.embed_mlwe) {
         if (c->logN == 16) return launch_chain<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_chain<AR, 8, 7>(c, args, limbs, inverse);
     }
@@ -706,7 +713,7 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
     // (N = 2^16, primes below 2^36) - takes the whole rounds of a batch (one limb per compute unit and round) and a last round that is
     // at least three quarters full; what is left goes out as two launches behind it.  Mode 6 asks for it wherever it applies, the
     // automatic mode takes it too, mode 1 never.
-    if (std::is_same<AR, F64Arith>::value && !c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && (c->ntt_mode == 0 || c->ntt_mode == 6) && res36_ok &&
+    if (std::is_same<AR, F64Arith>::value && !c->ev_mid_armed && !args.embed_mlwe && (mode == 0 || mode == 6) && res36_ok &&
         ntt_resident_applies(c, limbs)) {
         const int per_round = ntt_resident_round(c);
         int whole = limbs / per_round * per_round;
@@ -716,23 +723,23 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
         return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok, whole);
     }
     // mode 4, and the automatic mode for small batches: both passes in one launch of one workgroup per (limb, tile)
-    if (!c->ev_mid_armed && !c->mid_fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs)) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
+    if (!c->ev_mid_armed && !fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs)) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
     // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
     // (the limbs in flight, 0.5 MiB per resident workgroup, exceed the L2 by far), so the automatic mode does not pick it.
-    if (!c->ev_mid_armed && c->ntt_mode == 3) {
+    if (!c->ev_mid_armed && mode == 3) {
         if (c->logN == 16) return launch_whole_limb<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_whole_limb<AR, 8, 7>(c, args, limbs, inverse);
     }
     switch (c->logN) {
-        case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse, compact_ok);
-        case 9:  return launch_two_pass<AR, 5, 4>(c, args, limbs, inverse, compact_ok);
-        case 10: return launch_two_pass<AR, 5, 5>(c, args, limbs, inverse, compact_ok);
-        case 11: return launch_two_pass<AR, 6, 5>(c, args, limbs, inverse, compact_ok);
-        case 12: return launch_two_pass<AR, 6, 6>(c, args, limbs, inverse, compact_ok);
-        case 13: return launch_two_pass<AR, 7, 6>(c, args, limbs, inverse, compact_ok);
-        case 14: return launch_two_pass<AR, 7, 7>(c, args, limbs, inverse, compact_ok);
-        case 15: return launch_two_pass<AR, 8, 7>(c, args, limbs, inverse, compact_ok);
-        case 16: return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
+        case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 9:  return launch_two_pass<AR, 5, 4>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 10: return launch_two_pass<AR, 5, 5>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 11: return launch_two_pass<AR, 6, 5>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 12: return launch_two_pass<AR, 6, 6>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 13: return launch_two_pass<AR, 7, 6>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 14: return launch_two_pass<AR, 7, 7>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 15: return launch_two_pass<AR, 8, 7>(c, args, limbs, inverse, compact_ok, 0, fixed);
+        case 16: return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok, 0, fixed);
         default: set_error("NTT: logN must be in [8, 16]"); return CKKS_E_INVALID;
     }
 }
@@ -1560,7 +1567,8 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
 }
 
 static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
-                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src);
+                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src,
+                           const NttFixedArea* fixed = nullptr);
 
 int launch_ntt(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                int poly_mod_len, long batch_stride_limbs, int batch, bool inverse) {
@@ -1578,7 +1586,8 @@ int launch_ntt_embedded(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int star
 }
 
 static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
-                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src) {
+                           int poly_mod_len, long batch_stride_limbs, int batch, bool inverse, const NttEmbedSource* src,
+                           const NttFixedArea* fixed) {
     if (!c || !dev) { set_error("NTT: null argument"); return CKKS_E_INVALID; }
     if (ntt_pair_failed(c)) { set_error("NTT: an earlier one-launch transform of this context gave up waiting for its first pass"); return CKKS_E_UNAVAILABLE; }
     if (poly_num <= 0 || mod_num <= 0 || batch <= 0) return CKKS_OK;      // empty batch: nothing to do
@@ -1610,7 +1619,7 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
                 int j1 = j0 + 1;
                 while (j1 < mod_num && klass(j1) == klass(j0)) j1++;
                 const int rc = launch_ntt_from(c, dev, start_poly_idx + j0, start_mod_idx + j0, poly_num, j1 - j0, poly_mod_len, batch_stride_limbs,
-                                               batch, inverse, nullptr);
+                                               batch, inverse, nullptr, fixed);
                 if (rc) return rc;
                 j0 = j1;
             }
@@ -1634,14 +1643,14 @@ static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int s
     }
     if (back_end == 0) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
-        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok, res36_ok);
+        return dispatch_logn<F64Arith>(c, args, (int)limbs, inverse, compact_ok, res36_ok, fixed);
     }
     if (back_end == 1) {
         args.tw = inverse ? (const void*)c->d_twd_inv : (const void*)c->d_twd_fwd;
-        return dispatch_logn<F64WideArith>(c, args, (int)limbs, inverse, false);
+        return dispatch_logn<F64WideArith>(c, args, (int)limbs, inverse, false, false, fixed);
     }
     args.tw = inverse ? (const void*)c->d_tw_inv : (const void*)c->d_tw_fwd;
-    return dispatch_logn<IntArith>(c, args, (int)limbs, inverse, false);
+    return dispatch_logn<IntArith>(c, args, (int)limbs, inverse, false, false, fixed);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -1690,16 +1699,10 @@ int launch_ntt_noalloc(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start
     char* ptr = nullptr;
     int rc = ntt_noalloc_init(&ptr);
     if (rc) return rc;
-    // two launches, inter-pass data in the fixed area where the 5-byte form applies and in place otherwise
-    const int mode = c->ntt_mode;
-    c->ntt_mode = 0;
-    c->mid_fixed = ptr;
-    c->mid_fixed_cap = (size_t)NOALLOC_MAX_LIMBS * MID_LIMB_BYTES;
-    rc = launch_ntt_from(c, dev, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, 0, 1, inverse, nullptr);
-    c->mid_fixed = nullptr;
-    c->mid_fixed_cap = 0;
-    c->ntt_mode = mode;
-    return rc;
+    // two launches, inter-pass data in the fixed area where the 5-byte form applies and in place otherwise; the area travels
+    // with the call, nothing of the context is changed
+    const NttFixedArea fixed = {ptr, (size_t)NOALLOC_MAX_LIMBS * MID_LIMB_BYTES};
+    return launch_ntt_from(c, dev, start_poly_idx, start_mod_idx, poly_num, mod_num, poly_mod_len, 0, 1, inverse, nullptr, &fixed);
 }
 
 }  // namespace ckks

@@ -315,7 +315,7 @@ extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     if (!h) return CKKS_OK;
     { std::lock_guard<std::mutex> lock(g_handles_mutex); g_handles.erase(std::remove(g_handles.begin(), g_handles.end(), h), g_handles.end()); }
     (void)hipDeviceSynchronize();
-    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw, h->d_slices};
+    void* ptrs[] = {h->d_pq, h->d_ptrs, h->d_absmax, h->d_zero, h->d_Bdig, h->d_small_tw, h->d_slices, h->d_workA, h->d_workAdig};
     for (void* p : ptrs) if (p) (void)hipFree(p);
     for (auto& w : h->weights) { if (w.d_A) (void)hipFree(w.d_A); if (w.d_Adig) (void)hipFree(w.d_Adig); }
     if (h->pin) (void)hipHostFree(h->pin);
@@ -675,14 +675,26 @@ static void drop_weights(pcmm_ctx* h, pcmm_ctx::Weights* w) {
         h->weights.erase(h->weights.begin() + (long)idx);
     }
 }
-void pcmm_forget_weights(const void* lo, size_t bytes) {
+void pcmm_forget_weights(const void* lo, size_t bytes, bool freed) {
     std::lock_guard<std::mutex> lock(g_handles_mutex);
     const uintptr_t a = (uintptr_t)lo, b = a + bytes;
-    for (pcmm_ctx* h : g_handles)
+    for (pcmm_ctx* h : g_handles) {
+        if (freed)                                        // memory that goes back to the allocator is nobody's static matrix any more
+            for (size_t i = h->static_ranges.size(); i-- > 0;)
+                if (h->static_ranges[i].first < b && a < h->static_ranges[i].first + h->static_ranges[i].second)
+                    h->static_ranges.erase(h->static_ranges.begin() + (long)i);
         for (size_t i = h->weights.size(); i-- > 0;) {
             const uintptr_t wa = (uintptr_t)h->weights[i].W, wb = wa + (size_t)h->weights[i].M * h->weights[i].Kin * sizeof(float);
             if (wa < b && a < wb) drop_weights(h, &h->weights[i]);
         }
+    }
+}
+// whether the prepared form of the matrix at W is kept between calls
+static bool weights_kept(const pcmm_ctx* h, const float* W) {
+    if (h->weights_cached) return true;
+    const uintptr_t a = (uintptr_t)W;
+    for (const auto& r : h->static_ranges) if (a >= r.first && a < r.first + r.second) return true;
+    return false;
 }
 static pcmm_ctx::Weights* keep_weights(pcmm_ctx* h, const pcmm_ctx::Weights& fresh) {
     while (!h->weights.empty() && h->weights_bytes + fresh.bytes > WEIGHTS_MAX_BYTES) {
@@ -768,10 +780,17 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         pl.planes = pl.slices > 1 ? 3 * pl.slices : pl.DW <= 3 ? 3 : 4;
         return pl;
     };
-    // the prepared matrix: found, or quantised, measured and split now
+    // The plaintext matrix as the kernels take it (quantised; for the MFMA kernel split into digit planes).  By default it is made
+    // anew in every call, in work space of the handle - the reference quantises W inside every call (PPMM_kernel.cuh:148), so
+    // whatever the caller has written to W since the last call is what this call multiplies by.  For a matrix the caller has
+    // declared static (pcmm_weights_static), or every matrix with pcmm_set_weight_cache(h, 1) - the caller's promise that W changes
+    // only through this library's copies or with pcmm_weights_changed - the prepared form is kept under (device address, shape,
+    // scaler) and found again here.
     pcmm_ctx::Weights* we = nullptr;
-    for (auto& w : h->weights)
-        if (w.W == W && w.M == M && w.Kin == Kin && w.scaler == scaler) { we = &w; break; }
+    const bool keep = weights_kept(h, W);
+    if (keep)
+        for (auto& w : h->weights)
+            if (w.W == W && w.M == M && w.Kin == Kin && w.scaler == scaler) { we = &w; break; }
     if (we) {
         const Plan pl = plan_for(we->absmax);
         if (pl.mfma ? !we->d_Adig || we->planes != pl.planes : !we->d_A) { drop_weights(h, we); we = nullptr; }   // prepared for the other kernel
@@ -780,30 +799,47 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     if (!we) {
         const long count = (long)M * Kin;
         fresh.W = W; fresh.M = M; fresh.Kin = Kin; fresh.scaler = scaler;
-        hipError_t e = hipMalloc((void**)&fresh.d_A, (size_t)count * sizeof(long long));
+        // work space of a call that keeps nothing: grown when a call needs more, reused in stream order otherwise (a call on another
+        // stream than the last waits for the device first)
+        auto work = [&](void** slot, size_t* cap, size_t need) -> hipError_t {
+            if (need <= *cap) return hipSuccess;
+            if (*slot) { (void)hipDeviceSynchronize(); (void)hipFree(*slot); *slot = nullptr; *cap = 0; }
+            hipError_t e = hipMalloc(slot, need);
+            if (e == hipSuccess) *cap = need;
+            return e;
+        };
+        if (!keep && h->work_stream_known && h->work_stream != c->stream) (void)hipDeviceSynchronize();
+        h->work_stream = c->stream; h->work_stream_known = true;
+        hipError_t e = keep ? hipMalloc((void**)&fresh.d_A, (size_t)count * sizeof(long long))
+                            : work((void**)&h->d_workA, &h->workA_cap, (size_t)count * sizeof(long long));
         if (e != hipSuccess) { set_error("PPMM: cannot allocate the quantised plaintext matrix"); return CKKS_E_NOMEM; }
+        if (!keep) fresh.d_A = h->d_workA;
+        auto release = [&]() { if (keep && fresh.d_A) (void)hipFree(fresh.d_A); };
         (void)hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream);
         hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 256 * QUANT_PER_LANE - 1) / (256 * QUANT_PER_LANE))), dim3(256), 0, c->stream, W,
                            fresh.d_A, h->d_absmax, count, scaler);
         // the one host round trip of a matrix: its digit count selects the kernel instance
         hipError_t e2 = hipMemcpyAsync(&fresh.absmax, h->d_absmax, sizeof(fresh.absmax), hipMemcpyDeviceToHost, c->stream);
         if (e2 == hipSuccess) e2 = hipStreamSynchronize(c->stream);
-        if (e2 != hipSuccess) { (void)hipFree(fresh.d_A); return hip_fail(e2, "PPMM: |A| maximum"); }
+        if (e2 != hipSuccess) { release(); return hip_fail(e2, "PPMM: |A| maximum"); }
         const Plan pl = plan_for(fresh.absmax);
-        if (packed && !pl.mfma) { (void)hipFree(fresh.d_A); set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
+        if (packed && !pl.mfma) { release(); set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
         fresh.bytes = (size_t)count * sizeof(long long);
         if (pl.mfma) {
             const size_t dbytes = (size_t)pl.planes * Mpad * Kpad;
-            e = hipMalloc((void**)&fresh.d_Adig, dbytes);
-            if (e != hipSuccess) { (void)hipFree(fresh.d_A); set_error("PPMM: cannot allocate the plaintext digit planes"); return CKKS_E_NOMEM; }
+            e = keep ? hipMalloc((void**)&fresh.d_Adig, dbytes) : work((void**)&h->d_workAdig, &h->workAdig_cap, dbytes);
+            if (e != hipSuccess) { release(); set_error("PPMM: cannot allocate the plaintext digit planes"); return CKKS_E_NOMEM; }
+            if (!keep) fresh.d_Adig = h->d_workAdig;
             const long total = (long)Mpad * Kpad;
             hipLaunchKernelGGL(digits_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, fresh.d_A, fresh.d_Adig, M, Kin, Mpad, Kpad, pl.planes);
             fresh.planes = pl.planes;
-            (void)hipFree(fresh.d_A);                       // waits for the kernel above; only the planes are kept
-            fresh.d_A = nullptr;
+            if (keep) {
+                (void)hipFree(fresh.d_A);                   // waits for the kernel above; only the planes are kept
+                fresh.d_A = nullptr;
+            }
             fresh.bytes = dbytes;
         }
-        we = keep_weights(h, fresh);
+        we = keep ? keep_weights(h, fresh) : &fresh;
     }
     we->stamp = ++h->weights_clock;
     const Plan pl = plan_for(we->absmax);
@@ -861,7 +897,6 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         hipLaunchKernelGGL(ppmm_generic_kernel, grid, block, 0, c->stream, a);
     }
     CKKS_HIP_TRY(hipGetLastError());
-    if (!h->weights_cached) drop_weights(h, we);            // the reference's behaviour: nothing survives the call (waits for it)
     return CKKS_OK;
 }
 
@@ -877,7 +912,24 @@ extern "C" int pcmm_info(const pcmm_ctx* h, const char* name, long* value) {
 extern "C" int pcmm_set_weight_cache(pcmm_ctx* h, int enabled) {
     if (!h) return CKKS_E_INVALID;
     h->weights_cached = enabled != 0;
-    if (!enabled) while (!h->weights.empty()) drop_weights(h, &h->weights.back());
+    if (!enabled)                                         // what is kept from now on: the matrices declared static
+        for (size_t i = h->weights.size(); i-- > 0;)
+            if (!weights_kept(h, h->weights[i].W)) drop_weights(h, &h->weights[i]);
+    return CKKS_OK;
+}
+extern "C" int pcmm_weights_static(pcmm_ctx* h, const float* W, size_t bytes, int is_static) {
+    if (!h || !W || !bytes) return CKKS_E_INVALID;
+    std::lock_guard<std::mutex> lock(g_handles_mutex);
+    const uintptr_t a = (uintptr_t)W, b = a + bytes;
+    for (size_t i = h->static_ranges.size(); i-- > 0;)
+        if (h->static_ranges[i].first < b && a < h->static_ranges[i].first + h->static_ranges[i].second)
+            h->static_ranges.erase(h->static_ranges.begin() + (long)i);
+    if (is_static) h->static_ranges.emplace_back(a, bytes);
+    else if (!h->weights_cached)
+        for (size_t i = h->weights.size(); i-- > 0;) {
+            const uintptr_t wa = (uintptr_t)h->weights[i].W;
+            if (wa >= a && wa < b) drop_weights(h, &h->weights[i]);
+        }
     return CKKS_OK;
 }
 extern "C" int pcmm_weights_changed(pcmm_ctx* h, const float* W) {

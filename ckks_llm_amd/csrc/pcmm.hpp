@@ -1,5 +1,6 @@
 // Internal types shared by the PCMM launchers and kernels.
 #pragma once
+#include <utility>
 #include <vector>
 
 #include "context.hpp"
@@ -25,9 +26,9 @@ struct pcmm_ctx {
     uint64_t* d_small_tw = nullptr;          // tables of the size-N1 transform when N1 < 256: [prime][forward | inverse][N1]
     uint64_t small_n_inv[8] = {};            // N1^-1 modulo each ring-pack prime (N1 < 256)
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
-    // Prepared plaintext matrices.  A weight matrix is static for the life of a layer: the first PPMM call with a given
-    // (device pointer, shape, scaler) quantises it, measures |A|max (the one host round trip) and splits it into digit planes;
-    // later calls with the same key reuse the planes and issue no host synchronisation at all.
+    // Prepared plaintext matrices (only while the caller has switched the cache on: pcmm_set_weight_cache).  The first PPMM call
+    // with a given (device pointer, shape, scaler) quantises the matrix, measures |A|max (the one host round trip) and splits it
+    // into digit planes; later calls with the same key reuse the planes and issue no host synchronisation at all.
     struct Weights {
         const float* W = nullptr;
         int M = 0, Kin = 0;
@@ -40,7 +41,15 @@ struct pcmm_ctx {
         uint64_t stamp = 0;
     };
     std::vector<Weights> weights;
-    bool weights_cached = true;
+    bool weights_cached = false;
+    std::vector<std::pair<uintptr_t, size_t>> static_ranges;    // device address ranges whose matrices the caller has declared static
+    // work space of the calls that keep nothing: the quantised matrix and its digit planes of the call in flight
+    long long* d_workA = nullptr;
+    size_t workA_cap = 0;
+    int8_t* d_workAdig = nullptr;
+    size_t workAdig_cap = 0;
+    hipStream_t work_stream = nullptr;
+    bool work_stream_known = false;
     size_t weights_bytes = 0;
     uint64_t weights_clock = 0;
     // last row-pointer table and epilogue constants sent to the device (resent only when they change), and the pinned staging

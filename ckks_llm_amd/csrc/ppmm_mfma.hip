@@ -491,3 +491,61 @@ int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC,
 }
 
 }  // namespace ckks
+
+// ------------------------------------------------------------------------------------------------------------
+// Measured ceiling of the matrix pipe: v_mfma_i32_16x16x64_i8 from registers only, eight independent accumulators per wave
+// (no LDS, no memory), two workgroups of 512 lanes per compute unit as the contraction kernel runs.  What this loop reaches is
+// what the clock under matrix load allows; the contraction's fraction of it says how much of the time its matrix pipe is busy.
+// ------------------------------------------------------------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(512, 2) void mfma_i8_peak_kernel(int* sink, int iters, int seed) {
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    v4i a = {seed + (int)threadIdx.x, seed, 1, 2}, b = {seed, 3, (int)threadIdx.x, 4};
+    v4i acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = v4i{i, 0, 0, 0};
+    for (int n = 0; n < iters; n++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i], 0, 0, 0);
+    }
+    v4i s = acc[0];
+#pragma unroll
+    for (int i = 1; i < 8; i++) s += acc[i];
+    if (s[0] + s[1] + s[2] + s[3] == 0x7fffffff) sink[0] = 1;      // never true in practice: keeps the loop alive
+}
+}  // namespace
+
+// int8 MAC/s of the loop above on the current device (timed with HIP events on `stream` over `reps` launches)
+extern "C" int ckks_measure_mfma_i8_peak(void* stream_v, double* macs_per_s) {
+    using namespace ckks;
+    if (!macs_per_s) return CKKS_E_INVALID;
+    hipStream_t stream = (hipStream_t)stream_v;
+    int dev = 0, cus = 0;
+    CKKS_HIP_TRY(hipGetDevice(&dev));
+    CKKS_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    int* sink = nullptr;
+    CKKS_HIP_TRY(hipMalloc((void**)&sink, sizeof(int)));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const int iters = 4096, reps = 5;
+    const unsigned blocks = (unsigned)cus * 2u;
+    float ms = 0.f;
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(mfma_i8_peak_kernel, dim3(blocks), dim3(512), 0, stream, sink, iters, 1);      // warm-up
+        e = hipEventRecord(e0, stream);
+        for (int r = 0; r < reps; r++) hipLaunchKernelGGL(mfma_i8_peak_kernel, dim3(blocks), dim3(512), 0, stream, sink, iters, r + 2);
+        if (e == hipSuccess) e = hipEventRecord(e1, stream);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    if (e != hipSuccess) return hip_fail(e, "ckks_measure_mfma_i8_peak");
+    // per wave and iteration: 8 instructions of 16 x 16 x 64 multiply-accumulates
+    const double macs = (double)reps * blocks * 8.0 /* waves */ * iters * 8.0 * (16.0 * 16.0 * 64.0);
+    *macs_per_s = macs / (ms * 1e-3);
+    return CKKS_OK;
+}
+

@@ -114,10 +114,18 @@ int ckks_ntt_inv_ext(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start
  * and grow on demand; this one keeps it in a fixed device array inside the library (ckks_ntt_noalloc_max_limbs() limbs of
  * 320 KiB = 20 MiB per GPU, held until the process ends) and calls no allocating routine.  poly_num * mod_num above that limit
  * returns CKKS_E_INVALID.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two host threads)
- * race.  The context must have been created on the current device.  Results are those of ckks_ntt_fwd / ckks_ntt_inv. */
+ * race.  The call runs as two launches whatever launch form the context is set to and changes nothing in the context, so it
+ * may run beside other host threads' calls on the same context (on data of their own).  The context must have been created on
+ * the current device.  Results are those of ckks_ntt_fwd / ckks_ntt_inv. */
 int ckks_ntt_noalloc(ckks_ctx* ctx, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,
                      int poly_mod_len, int inverse);
 int ckks_ntt_noalloc_max_limbs(void);
+
+/* Measurement aid of the benchmark (no counterpart in the reference): int8 multiply-accumulates per second that a loop of
+ * v_mfma_i32_16x16x64_i8 on registers alone reaches on the current device, two workgroups of 512 lanes per compute unit, timed
+ * with HIP events on `stream` (NULL: the default stream).  The ceiling that the PPMM contraction is set against beside the
+ * published peak. */
+int ckks_measure_mfma_i8_peak(void* stream, double* macs_per_s);
 
 /* One transform with HIP-event timing of its two kernel launches (strided pass and row pass; the forward transform
  * runs the strided pass first, the inverse the row pass first).  Replaces the cudaEvent pairs of ntt_throughput.cu:51-60. */
@@ -332,12 +340,19 @@ int pcmm_ppmm(pcmm_ctx* h, const float* W_dev, const uint64_t* const* mlwe_ptrs_
 int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev, uint64_t* out_dev, int M, int Kin,
                       int mod_num, double scaler);
 /* Prepared plaintext matrices (no counterpart in the reference, which quantises W inside every call, PPMM_kernel.cuh:148).
- * The weights of a layer do not change between calls, so the first PPMM call with a given (W_dev, M, Kin, scaler) quantises the
- * matrix, measures |A|max (one stream synchronisation) and splits it into digit planes, and every later call with the same four
- * values reuses them: such calls enqueue their kernels and return without waiting for the stream.  At most 4 GiB of planes are
- * kept per handle, least recently used first out.  A caller that overwrites a weight matrix in place says so with
- * pcmm_weights_changed(h, W_dev) (W_dev = NULL: every matrix); pcmm_set_weight_cache(h, 0) restores the reference's behaviour
- * (every call reads W afresh and synchronises once), pcmm_set_weight_cache(h, 1) is the default. */
+ * By default every PPMM call reads W afresh, as the reference does: it quantises the matrix, measures |A|max (one stream
+ * synchronisation) and splits it into digit planes in work space of the handle, so a call always multiplies by what W_dev
+ * holds when it is made, whoever wrote it.
+ * pcmm_weights_static(h, W_dev, bytes, 1) declares the device memory [W_dev, W_dev + bytes) static: the caller's promise that a
+ * weight matrix in it changes only through this library's own copies (ckks_memcpy_h2d / _d2d, ckks_memset, ckks_free - the last
+ * also ends the declaration) or is announced with pcmm_weights_changed(h, W_dev) (W_dev = NULL: every matrix).
+ * pcmm_set_weight_cache(h, 1) makes the same promise for every matrix the handle is given.  The planes of a static
+ * (W_dev, M, Kin, scaler) are kept after the first call (at most 4 GiB per handle, least recently used first out) and later
+ * calls with the same four values enqueue their kernels and return without waiting for the stream.  A writer the library does
+ * not see (the caller's own kernel, hipMemcpy, an allocator that hands the same address to another matrix) makes such a call
+ * multiply by the OLD weights: that is why nothing is kept unless the caller asks for it.
+ * pcmm_weights_static(.., 0) and pcmm_set_weight_cache(h, 0) take the promise back and drop what was kept under it. */
+int pcmm_weights_static(pcmm_ctx* h, const float* W_dev, size_t bytes, int is_static);
 int pcmm_set_weight_cache(pcmm_ctx* h, int enabled);
 int pcmm_weights_changed(pcmm_ctx* h, const float* W_dev);
 

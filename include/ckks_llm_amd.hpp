@@ -800,7 +800,12 @@ public:
         check(pcmm_info(handle, name, &v), "pcmm_info");
         return v;
     }
-    // digit planes of plaintext matrices are kept between PPMM calls (default); a matrix overwritten in place is announced
+    // By default every PPMM call reads its plaintext matrix afresh, as the reference does.  A matrix declared static (one that
+    // changes only through this library's copies) keeps its digit planes between calls; set_weight_cache(true) declares every
+    // matrix static; a static matrix overwritten in place by other means is announced with weights_changed.
+    void weights_static(const float* plain_mat, size_t bytes, bool is_static = true) {
+        check(pcmm_weights_static(handle, plain_mat, bytes, is_static ? 1 : 0), "pcmm_weights_static");
+    }
     void set_weight_cache(bool enabled) { check(pcmm_set_weight_cache(handle, enabled ? 1 : 0), "pcmm_set_weight_cache"); }
     void weights_changed(const float* plain_mat = nullptr) { check(pcmm_weights_changed(handle, plain_mat), "pcmm_weights_changed"); }
     // PCMM_Context.h: size-N1 transforms over the ring-pack primes, data = [mod_batch_size][mod_num][poly_num][N1]
@@ -876,7 +881,7 @@ public:
 
     // PCMM_Scheme::mlweCipherPacking (PCMM_Scheme.cuh:361-425): k MLWE samples -> 1 RLWE ciphertext with the repacking keys
     // (from addRepakcingKey, or installed by the caller in repackingKeys).
-    void mlweCipherPacking(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,
+    void mlweCipherPacking(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*> mlwe_cipher_decomposed, uint64_tt mlwe_num,
                            uint64_tt offset) {
         if (!repackingKeys) throw std::invalid_argument("mlweCipherPacking: repacking keys not exists");
         if (offset + mlwe_num > mlwe_cipher_decomposed.size()) throw std::invalid_argument("mlweCipherPacking: offset + mlwe_num exceeds the vector");
@@ -889,7 +894,7 @@ public:
     }
 
     // PCMM_Scheme::rlweCipherDecompose (PCMM_Scheme.cuh:90-125).  Shape errors print and return, as the reference (:103-106).
-    void rlweCipherDecompose(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, uint64_tt mlwe_num,
+    void rlweCipherDecompose(Ciphertext& rlwe_cipher, std::vector<MLWECiphertext*> mlwe_cipher_decomposed, uint64_tt mlwe_num,
                              uint64_tt offset) {
         if (mlwe_num > (uint64_tt)pcmm_context.mlwe_rank) {
             std::cout << "rlweCipherDecompose extract number muse <= mlwe_rank" << std::endl;
@@ -905,7 +910,7 @@ public:
     // PCMM_Scheme::PPMM (PPMM_kernel.cuh:254-349): plain_mat is a DEVICE pointer to mat_M x mat_N fp32, row-major.
     // scaler = (long)(q_ringpack[1] * 2^49 / scale) (:283-284); afterwards row i of the product (first modulus) is copied
     // back into mlwe_cipher_decomposed[i] and its scale becomes scale * scaler / q_ringpack[1] (:345-348).
-    void PPMM(float* plain_mat, std::vector<MLWECiphertext*>& mlwe_cipher_decomposed, int mat_M, int mat_N, int mat_K, int mlwe_num) {
+    void PPMM(float* plain_mat, std::vector<MLWECiphertext*> mlwe_cipher_decomposed, int mat_M, int mat_N, int mat_K, int mlwe_num) {
         if (mat_K != pcmm_context.N1) { std::cout << "matrix K should be equal to N1!" << std::endl; return; }
         if (mat_N != mlwe_num) { std::cout << "matrix N should be equal to mlwe number!" << std::endl; return; }
         const int mod_num = pcmm_context.ringpack_q_count;
@@ -947,7 +952,7 @@ public:
         check(pcmm_rlwe_decompose_packed(pcmm_context.handle, rlwe_cipher.cipher_device, (int)offset, (int)mlwe_num, (int)(take ? take : mlwe_num),
                                          rlwe_cipher.l), "rlweCipherDecomposePacked");
     }
-    void PPMMPacked(float* plain_mat, std::vector<MLWECiphertext*>& rows, int mat_M) {
+    void PPMMPacked(float* plain_mat, const std::vector<MLWECiphertext*>& rows, int mat_M) {
         const int mod_num = pcmm_context.ringpack_q_count;
         const size_t C = (size_t)pcmm_context.N1 * (pcmm_context.mlwe_rank + 1);
         const size_t need = (size_t)mat_M * mod_num * C;

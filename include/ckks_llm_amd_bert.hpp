@@ -189,6 +189,9 @@ public:
         return stop != second.c_str();
     }
 
+    // the device arrays this object allocated, in the order of `loaded`
+    const std::vector<float*>& tensors() const { return owned; }
+
 private:
     std::vector<float*> owned;
 };
@@ -226,9 +229,15 @@ public:
         for (uint64_tt q : pcmm_scheme.pcmm_context.q_ringpack) packed_gather = packed_gather && q - 1 <= 0x7f7f7f7f7full;      // five balanced residue digits
         for (int i = 0; i < decomp_num; i++)
             mlwe_cipher_buffer.push_back(new MLWECiphertext(PCMM_N1, q_ringpack_count - 1, q_ringpack_count - 1, mlwe_rank, 0));
+        // the model's tensors were uploaded by this object and are not written again: their digit planes are kept between calls
+        // (a caller that does overwrite one says so: pcmm_scheme.pcmm_context.weights_changed)
+        for (size_t i = 0; i < model_weights.tensors().size() && i < model_weights.loaded.size(); i++)
+            if (model_weights.loaded[i].second) pcmm_scheme.pcmm_context.weights_static(model_weights.tensors()[i], model_weights.loaded[i].second);
     }
     Bert(const Bert&) = delete;
     ~Bert() {
+        for (size_t i = 0; i < model_weights.tensors().size() && i < model_weights.loaded.size(); i++)
+            if (model_weights.loaded[i].second) pcmm_weights_static(pcmm_scheme.pcmm_context.handle, model_weights.tensors()[i], model_weights.loaded[i].second, 0);
         for (MLWECiphertext* m : mlwe_cipher_buffer) delete m;
     }
 

@@ -164,10 +164,13 @@ def test_ppmm_reference_form_on_mlwe_ciphertexts():
         dev.PPMM(DeviceBuffer.from_numpy(W), mlwe, M, Kin, 64, Kin)
 
 
-def test_ppmm_prepared_weights_follow_the_buffer():
-    """The digit planes of a plaintext matrix are kept under (device address, shape, scaler).  A second call with the same matrix
-    reuses them; a matrix overwritten through the library's copy, a freed and reallocated buffer, an announced in-place change and
-    a switched-off cache must all give the product of what the buffer holds now."""
+def test_ppmm_reads_the_weights_in_every_call_unless_declared_static():
+    """As the reference (PPMM_kernel.cuh:148 quantises W inside the call), a PPMM call multiplies by what the weight buffer holds
+    when the call is made, also when a writer the library cannot see (a raw HIP copy here) has changed it.  A matrix declared
+    static keeps its digit planes under (device address, shape, scaler): a second call reuses them; a matrix overwritten through
+    the library's copy, a freed and reallocated buffer, an announced in-place change and a withdrawn declaration must all give
+    the product of what the buffer holds now."""
+    import ctypes
     q = CFG2_Q[:2]
     pair, dev, orc, rank = make(10, 128, list(q) + CFG2_Q[2:3], CFG3_P[:1], [CFG3_P[0]], list(q))
     C = (rank + 1) * 128
@@ -175,6 +178,10 @@ def test_ppmm_prepared_weights_follow_the_buffer():
     rng = np.random.default_rng(77)
     mlwe = [limbs_uniform(900 + n, q, 1, C)[0] for n in range(Kin)]
     bufs = [to_dev(m) for m in mlwe]
+    hip = ctypes.CDLL("/opt/rocm/lib/libamdhip64.so")
+
+    def raw_copy(dst, src, nbytes):                                   # device to device, not through the library
+        assert hip.hipMemcpy(ctypes.c_void_p(dst.ptr), ctypes.c_void_p(src.ptr), ctypes.c_size_t(nbytes), 3) == 0
 
     def want_for(W):
         out = np.zeros((M, 2, C), dtype=np.uint64)
@@ -190,29 +197,46 @@ def test_ppmm_prepared_weights_follow_the_buffer():
     W1 = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
     W2 = rng.normal(0, 0.02, (M, Kin)).astype(np.float32)
     W3 = rng.normal(0, 0.3, (M, Kin)).astype(np.float32)             # four plaintext digits: another kernel instance
+    pc = dev.pcmm_context
+    # default settings: nothing is kept
     dW = DeviceBuffer.from_numpy(W1)
+    second, third = DeviceBuffer.from_numpy(W2), DeviceBuffer.from_numpy(W3)
     assert np.array_equal(run(dW), want_for(W1))
-    assert np.array_equal(run(dW), want_for(W1))                      # prepared planes
-    dW.upload(W2)                                                     # overwritten in place through the library
-    assert np.array_equal(run(dW), want_for(W2))
-    dW.upload(W3)
-    assert np.array_equal(run(dW), want_for(W3)) and dev.pcmm_context.info("last_DW") == 4
-    addr = dW.ptr
-    dW.free()
-    dW = DeviceBuffer.from_numpy(W1)                                  # usually the same address again
-    assert np.array_equal(run(dW), want_for(W1)), ("reallocated at the same address", dW.ptr == addr)
-    # a change the library cannot see (another writer): announced by the caller
-    other = DeviceBuffer.from_numpy(W2)
-    import ctypes
-    hip = ctypes.CDLL("/opt/rocm/lib/libamdhip64.so")
-    assert hip.hipMemcpy(ctypes.c_void_p(dW.ptr), ctypes.c_void_p(other.ptr), ctypes.c_size_t(W2.nbytes), 3) == 0   # device to device
-    dev.pcmm_context.weights_changed(dW)
-    assert np.array_equal(run(dW), want_for(W2))
-    dev.pcmm_context.set_weight_cache(False)
-    first = DeviceBuffer.from_numpy(W1)
-    assert hip.hipMemcpy(ctypes.c_void_p(dW.ptr), ctypes.c_void_p(first.ptr), ctypes.c_size_t(W1.nbytes), 3) == 0
-    assert np.array_equal(run(dW), want_for(W1))                      # no cache: every call reads the matrix
-    dev.pcmm_context.set_weight_cache(True)
+    raw_copy(dW, second, W2.nbytes)
+    assert np.array_equal(run(dW), want_for(W2))                      # the new weights, unannounced
+    raw_copy(dW, third, W3.nbytes)
+    assert np.array_equal(run(dW), want_for(W3)) and pc.info("last_DW") == 4
+    dW.upload(W1)
+    assert np.array_equal(run(dW), want_for(W1)) and pc.info("last_DW") == 3
+    # declared static: planes kept
+    for declare in ("matrix", "handle"):
+        if declare == "matrix":
+            pc.weights_static(dW)
+        else:
+            pc.set_weight_cache(True)
+        dW.upload(W1)
+        assert np.array_equal(run(dW), want_for(W1))
+        assert np.array_equal(run(dW), want_for(W1))                  # prepared planes
+        raw_copy(dW, second, W2.nbytes)
+        assert np.array_equal(run(dW), want_for(W1))                  # the promise was broken: the kept planes answer (documented)
+        pc.weights_changed(dW)                                        # ... until the change is announced
+        assert np.array_equal(run(dW), want_for(W2))
+        dW.upload(W3)                                                 # overwritten in place through the library
+        assert np.array_equal(run(dW), want_for(W3)) and pc.info("last_DW") == 4
+        addr = dW.ptr
+        dW.free()                                                     # ends the declaration of the matrix, drops its planes
+        dW = DeviceBuffer.from_numpy(W1)                              # usually the same address again
+        assert np.array_equal(run(dW), want_for(W1)), ("reallocated at the same address", dW.ptr == addr)
+        if declare == "matrix":
+            raw_copy(dW, second, W2.nbytes)
+            assert np.array_equal(run(dW), want_for(W2))              # not static any more: read afresh
+            pc.weights_static(dW)
+            assert np.array_equal(run(dW), want_for(W2))
+            pc.weights_static(dW, is_static=False)
+        else:
+            pc.set_weight_cache(False)
+        raw_copy(dW, third, W3.nbytes)
+        assert np.array_equal(run(dW), want_for(W3))                  # declaration withdrawn: every call reads the matrix
 
 
 @pytest.mark.parametrize("wide", [False, True])

@@ -45,6 +45,69 @@ def test_two_calls_in_a_row_second_smaller():
     _both_ways(pair, CFG2_Q, 2, seed=73)
 
 
+def _free_device_bytes(hip):
+    import ctypes
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_the_entry_allocates_nothing_and_leaves_the_context_alone():
+    """On a fresh context (whose inter-pass buffer does not exist yet) the first call, at the largest batch the entry takes, leaves
+    the device's free memory and the context's own buffer as they were, and does not touch the context's launch mode.  The same
+    call recorded into a HIP graph (a capture refuses every allocation) replays with the ordinary entry point's result."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    # another context first: the runtime loads the kernels' code on the first launch of a process, which is not this entry's doing
+    warm = Pair(16, [], CFG2_Q[:2])
+    tiny = to_dev(limbs_uniform(80, CFG2_Q[:2], 1, warm.N))
+    warm.dev.ntt_noalloc(tiny, 0, 0, 1, 2, 2, False)
+    warm.dev.sync()
+    pair = Pair(16, [], CFG2_Q)
+    d, N = pair.dev, pair.N
+    cap = d.ntt_noalloc_max_limbs()
+    polys, mods = 2, min(len(CFG2_Q), cap // 2)
+    data = limbs_uniform(81, CFG2_Q[:mods], polys, N)
+    got, ref = to_dev(data), to_dev(data)
+    d.sync()
+    assert d.info("ntt_mid_bytes") == 0
+    d.set_ntt_mode(1)
+    before = _free_device_bytes(hip)
+    d.ntt_noalloc(got, 0, 0, polys, mods, mods, False)
+    d.sync()
+    assert _free_device_bytes(hip) == before
+    assert d.info("ntt_mid_bytes") == 0 and d.info("ntt_mode") == 1
+    d.set_ntt_mode(0)
+    d.ToNTTInplace(ref, 0, 0, polys, mods, mods)
+    want = from_dev(ref, data.shape)
+    assert np.array_equal(from_dev(got, data.shape), want)
+    # under capture
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+    d.set_stream(stream)
+    graph, gexec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0
+    d.ntt_noalloc(got, 0, 0, polys, mods, mods, False)
+    assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, ctypes.c_size_t(0)) == 0
+    for rep in range(3):
+        fresh = limbs_uniform(90 + rep, CFG2_Q[:mods], polys, N)
+        got.upload(fresh)
+        ref.upload(fresh)
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        assert hip.hipStreamSynchronize(stream) == 0
+        d.set_stream(None)
+        d.ToNTTInplace(ref, 0, 0, polys, mods, mods)          # eager work between the replays
+        d.sync()
+        d.set_stream(stream)
+        assert np.array_equal(from_dev(got, data.shape), from_dev(ref, data.shape)), rep
+    assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
+    d.set_stream(None)
+    assert hip.hipStreamDestroy(stream) == 0
+    got.free()
+    ref.free()
+
+
 def test_limit_is_reported():
     pair = Pair(16, [], CFG2_Q)
     cap = pair.dev.ntt_noalloc_max_limbs()
