@@ -9,6 +9,7 @@
 //     out_k = Barrett( sum_j y_j * ((D/d_j) mod r_k)  -  v * (D mod r_k) ) [ + r_k - sub_k, one conditional subtract ]
 // All of these kernels stream every limb once; they are HBM bound (read nsrc + write ntgt limbs per block).
 #include "context.hpp"
+#include "f64_exact.hpp"
 
 namespace ckks {
 
@@ -65,20 +66,11 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel(ConvArgs a) {
 // value is an exact integer held in a double (|.| < 2^53 throughout) and a*w mod q is the two-product form used by the NTT, so
 // the words written are the same.  y_j is brought to its canonical representative before it enters v and the sum, because the
 // reference's v = (int) sum y_j / d_j and sum y_j * hat_j are functions of that representative.
-__device__ __forceinline__ double u2d(u64 x) {                       // exact for x < 2^52
-    return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0;
-}
-__device__ __forceinline__ u64 d2u(double x) {                       // exact integer 0 <= x < 2^52
-    return (u64)__double_as_longlong(x + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
-}
-__device__ __forceinline__ double mulmod_d(double a, double w, double q, double qinv) {      // in (-0.51 q, 0.51 q)
-    const double h = a * w, l = __builtin_fma(a, w, -h), c = __builtin_rint(h * qinv);
-    return __builtin_fma(-c, q, h) + l;
-}
-__device__ __forceinline__ double canon_d(double r, double q, double qinv) {                 // any |r| < 2^52 -> [0, q)
-    r = __builtin_fma(-__builtin_rint(r * qinv), q, r);
-    return r < 0.0 ? r + q : r;
-}
+// (the arithmetic and the per-coefficient sums are in f64_exact.hpp, where a host build checks their ranges)
+__device__ __forceinline__ double u2d(u64 x) { return exact_u2d(x); }                        // exact for x < 2^52
+__device__ __forceinline__ u64 d2u(double x) { return bits52(x); }                           // exact integer 0 <= x < 2^52
+__device__ __forceinline__ double mulmod_d(double a, double w, double q, double qinv) { return mulmod_f64(a, w, q, qinv); }      // in (-0.51 q, 0.51 q)
+__device__ __forceinline__ double canon_d(double r, double q, double qinv) { return canon_f64(r, q, qinv); }                     // any |r| < 2^52 -> [0, q)
 
 // The targets of a block are shared out over CONV_TGT_PARTS workgroups (each recomputes the cheap y_j): a lane that walked
 // through all 24+ targets alone left the launch with too few, too long lanes to cover the memory latency.
@@ -100,7 +92,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel_f64(ConvArgs a) {
             const PrimeConst& ps = a.primes[b.src_prime[j]];
             const u64 xin = in[(long)b.src_limb[j] * a.N + x];
             if (j < b.ncopy && part == 0) out[(long)b.copy_limb[j] * a.N + x] = xin;
-            y[j] = canon_d(mulmod_d(u2d(xin), b.hatinv_d[j], ps.qd, ps.qinv_d), ps.qd, ps.qinv_d);
+            y[j] = conv_f64_scale(xin, b.hatinv_d[j], ps.qd, ps.qinv_d);
             vv += y[j] / ps.qd;
         }
     }
@@ -108,11 +100,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel_f64(ConvArgs a) {
     const int per = (b.ntgt + CONV_TGT_PARTS - 1) / CONV_TGT_PARTS, k_end = min(b.ntgt, (part + 1) * per);
     for (int k = part * per; k < k_end; k++) {
         const PrimeConst& pr = a.primes[b.tgt_prime[k]];
-        double acc = -v * b.dmod_d[k];                               // |v| <= nsrc, |dmod| <= q/2: exact
-#pragma unroll
-        for (int j = 0; j < MAXS; j++)
-            if (j < nsrc) acc += mulmod_d(y[j], b.hat_d[k][j], pr.qd, pr.qinv_d);
-        out[(long)b.tgt_limb[k] * a.N + x] = d2u(canon_d(acc, pr.qd, pr.qinv_d));
+        out[(long)b.tgt_limb[k] * a.N + x] = conv_f64_target<MAXS>(y, nsrc, b.hat_d[k], v, b.dmod_d[k], pr.qd, pr.qinv_d);
     }
 }
 
@@ -145,8 +133,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel_split(ConvArgs a, in
             xin += b.add_in[j];
             const u64 y = mul_shoup(xin, b.hatinv[j], b.hatinv_s[j], d);
             vv += (double)y / (double)d;
-            yl[j] = u2d(y & 0x7fffffffull);
-            yh[j] = u2d(y >> 31);
+            conv_split_parts(y, yl[j], yh[j]);
         }
     }
     const double v = (double)(int)vv;
@@ -154,14 +141,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_kernel_split(ConvArgs a, in
     for (int k = part * per; k < k_end; k++) {
         const PrimeConst& pr = a.primes[b.tgt_prime[k]];
         const double q = pr.qd, qinv = pr.qinv_d;
-        double acc = -mulmod_d(v, b.dmod_d[k], q, qinv);
-#pragma unroll
-        for (int j = 0; j < MAXS; j++)
-            if (j < nsrc) {
-                acc += mulmod_d(yl[j], b.hat_d[k][j], q, qinv) + mulmod_d(yh[j], b.hat31_d[k][j], q, qinv);
-                if ((j & 3) == 3) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
-            }
-        double r = canon_d(acc, q, qinv);
+        double r = conv_split_target<MAXS>(yl, yh, nsrc, b.hat_d[k], b.hat31_d[k], v, b.dmod_d[k], q, qinv);
         if (a.centred) {
             r -= u2d(b.sub_out[k]);
             r = r < 0.0 ? r + q : r;

@@ -878,14 +878,8 @@ struct KsModDownArgs {
     int K;
     int pre_scaled;              // the special-prime limbs already hold [c_p_i * pHat_i^-1]_p_i (canonical)
 };
-__device__ __forceinline__ double exact_u2d(u64 x) {                  // x < 2^52
-    return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0;
-}
 template <class AR>
-__device__ __forceinline__ double canon_f(const AR& ar, double r) {               // any |r| < 2^52 -> [0, q)
-    r = ar.balance(r);
-    return r < 0.0 ? r + ar.q : r;
-}
+__device__ __forceinline__ double canon_f(const AR& ar, double r) { return canon_f64(r, ar.q, ar.qinv); }               // any |r| < 2^52 -> [0, q)
 // With the wide arithmetic every constant enters balanced and at most 8 special primes are admitted: a term of the sum lies within
 // 0.88 q of zero (its operand, a residue modulo p_i, may be up to twice q), so eight of them stay below 2^53.
 template <class AR, class MID>

@@ -4,6 +4,7 @@
 #include <type_traits>
 
 #include "context.hpp"
+#include "f64_exact.hpp"
 
 namespace ckks {
 
@@ -52,57 +53,62 @@ struct F64Arith {
     typedef double TW;
     double q, qinv, hqinv, n_inv, w1n;
     bool lazy40;               // q < 2^36.5: the values between the passes of a forward transform (|x| < 5.1 q) fit 40 bits as they are
-    __device__ __forceinline__ F64Arith(const PrimeConst& pc)
+    CKKS_HD F64Arith(const PrimeConst& pc)
         : q(pc.qd), qinv(pc.qinv_d), hqinv(0.5 * pc.qinv_d), n_inv(pc.n_inv_d), w1n(pc.w1n_d), lazy40(pc.qd < 97184015999.0) {}
     // canonical residue (below 2^52) -> double: the word is the mantissa of 2^52 + x
-    __device__ __forceinline__ V from_canonical(u64 x) const { return __longlong_as_double((long long)(0x4330000000000000ull | x)) - 4503599627370496.0; }
-    __device__ __forceinline__ V from_mid(u64 x) const { return __longlong_as_double((long long)x); }
-    __device__ __forceinline__ u64 to_mid_fwd(V x) const { return (u64)__double_as_longlong(x); }
-    __device__ __forceinline__ V mulmod(V a, TW w) const {          // result in (-0.51 q, 0.51 q)
-        double h = a * w;
-        double l = __builtin_fma(a, w, -h);
-        double c = __builtin_rint(h * qinv);
-        return __builtin_fma(-c, q, h) + l;
-    }
-    __device__ __forceinline__ V balance(V x) const { return __builtin_fma(-__builtin_rint(x * qinv), q, x); }
-    // integer in [0, 2^52) held in a double -> the integer: the mantissa of 2^52 + r
-    __device__ __forceinline__ static u64 bits52(V r) { return (u64)__double_as_longlong(r + 4503599627370496.0) & 0xFFFFFFFFFFFFFull; }
-    __device__ __forceinline__ u64 canon(V r) const {               // r in (-q, q) -> [0, q)
+    CKKS_HD V from_canonical(u64 x) const { return exact_u2d(x); }
+    CKKS_HD V from_mid(u64 x) const { return f64_from_bits(x); }
+    CKKS_HD u64 to_mid_fwd(V x) const { return f64_bits(x); }
+    CKKS_HD V mulmod(V a, TW w) const { return mulmod_f64(a, w, q, qinv); }          // result in (-0.51 q, 0.51 q)
+    CKKS_HD V balance(V x) const { return balance_f64(x, q, qinv); }
+    CKKS_HD static u64 bits52(V r) { return ::ckks::bits52(r); }
+    CKKS_HD u64 canon(V r) const {               // r in (-q, q) -> [0, q)
         r = r < 0.0 ? r + q : r;
         return bits52(r);
     }
     // any integer |x| < 2^10 q -> [0, q) without a sign fix-up: (x + 1/2) / q is at least 1/(2q) > 2^-42 away from every integer
     // and the product is off by less than 2^-42, so the floor is exactly floor(x / q)
-    __device__ __forceinline__ u64 canon_any(V x) const {
+    CKKS_HD u64 canon_any(V x) const {
         const double c = __builtin_floor(__builtin_fma(x, qinv, hqinv));
-        return bits52(__builtin_fma(-c, q, x));
+        const u64 res = bits52(__builtin_fma(-c, q, x));
+        CKKS_RANGE(canonical(x, q, res, "F64Arith::canon_any"));
+        return res;
     }
-    __device__ __forceinline__ u64 to_mid_inv(V x) const { return (u64)__double_as_longlong(balance(x)); }
+    CKKS_HD u64 to_mid_inv(V x) const { return f64_bits(balance(x)); }
     // 40-bit form of a balanced value (q < 2^39, so |r| < 2^38.1): r + 2^39 read from the low mantissa bits of r + 2^52 + 2^39
-    __device__ __forceinline__ u64 enc40(V x) const { return (u64)__double_as_longlong(balance(x) + 4504149383184384.0) & 0xFFFFFFFFFFull; }
-    __device__ __forceinline__ u64 enc40_raw(V x) const { return (u64)__double_as_longlong(x + 4504149383184384.0) & 0xFFFFFFFFFFull; }   // |x| < 2^39
+    CKKS_HD u64 enc40(V x) const { return enc40_raw(balance(x)); }
+    CKKS_HD u64 enc40_raw(V x) const {                                                 // |x| < 2^39
+        CKKS_RANGE(below(x, 549755813888.0, "F64Arith::enc40_raw"));
+        return f64_bits(x + 4504149383184384.0) & 0xFFFFFFFFFFull;
+    }
     // 36-bit form of a balanced value (q < 2^36, so |r| < 2^35): r + 2^35 read from the low mantissa bits of r + 2^52 + 2^35
-    __device__ __forceinline__ u64 enc36(V x) const { return (u64)__double_as_longlong(balance(x) + 4503633987108864.0) & 0xFFFFFFFFFull; }
-    __device__ __forceinline__ V dec36(unsigned lo, unsigned hi4) const {
-        return __longlong_as_double((long long)(0x4330000000000000ull | ((u64)hi4 << 32) | lo)) - 4503633987108864.0;
+    CKKS_HD u64 enc36(V x) const {
+        const V r = balance(x);
+        CKKS_RANGE(below(r, 34359738368.0, "F64Arith::enc36"));
+        return f64_bits(r + 4503633987108864.0) & 0xFFFFFFFFFull;
     }
-    __device__ __forceinline__ V dec40(unsigned lo, unsigned hi8) const {
-        return __longlong_as_double((long long)(0x4330000000000000ull | ((u64)hi8 << 32) | lo)) - 4504149383184384.0;
-    }
-    __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon_any(x); }
-    template <int R> __device__ __forceinline__ void round_end(V (&)[R]) const {}          // q < 2^41: the ranges hold for a whole pass
-    __device__ __forceinline__ void ct(V& x, V& y, TW w) const {
+    CKKS_HD V dec36(unsigned lo, unsigned hi4) const { return f64_from_bits(0x4330000000000000ull | ((u64)hi4 << 32) | lo) - 4503633987108864.0; }
+    CKKS_HD V dec40(unsigned lo, unsigned hi8) const { return f64_from_bits(0x4330000000000000ull | ((u64)hi8 << 32) | lo) - 4504149383184384.0; }
+    CKKS_HD u64 to_canonical_fwd(V x) const { return canon_any(x); }
+    template <int R> CKKS_HD void round_end(V (&)[R]) const {}          // q < 2^41: the ranges hold for a whole pass
+    CKKS_HD void ct(V& x, V& y, TW w) const {
         double t = mulmod(y, w);
         y = x - t;
         x = x + t;
+        CKKS_RANGE(value(x, "F64Arith::ct sum"));
+        CKKS_RANGE(value(y, "F64Arith::ct difference"));
     }
-    __device__ __forceinline__ void gs(V& x, V& y, TW w) const {
+    CKKS_HD void gs(V& x, V& y, TW w) const {
         double s = x + y, d = x - y;
+        CKKS_RANGE(value(s, "F64Arith::gs sum"));
+        CKKS_RANGE(value(d, "F64Arith::gs difference"));
         x = s;
         y = mulmod(d, w);
     }
-    __device__ __forceinline__ void gs_last(V& x, V& y, u64& ox, u64& oy) const {
+    CKKS_HD void gs_last(V& x, V& y, u64& ox, u64& oy) const {
         double s = x + y, d = x - y;
+        CKKS_RANGE(value(s, "F64Arith::gs_last sum"));
+        CKKS_RANGE(value(d, "F64Arith::gs_last difference"));
         ox = canon_any(mulmod(s, n_inv));
         oy = canon_any(mulmod(d, w1n));
     }
@@ -119,23 +125,27 @@ struct F64Arith {
 //   of at most 8 q (results within 2 q of zero) and canonicalises by a balance and one conditional addition.
 struct F64WideArith : F64Arith {
     double half;
-    __device__ __forceinline__ F64WideArith(const PrimeConst& pc) : F64Arith(pc), half(0.5 * pc.qd) {}
-    __device__ __forceinline__ V from_canonical(u64 x) const {
+    CKKS_HD F64WideArith(const PrimeConst& pc) : F64Arith(pc), half(0.5 * pc.qd) {}
+    CKKS_HD V from_canonical(u64 x) const {
         const double d = F64Arith::from_canonical(x);
         return d > half ? d - q : d;
     }
-    __device__ __forceinline__ u64 canon_wide(V x) const {            // any integer |x| < 2^53 -> [0, q)
+    CKKS_HD u64 canon_wide(V x) const {            // any integer |x| < 2^53 -> [0, q)
         const double r = balance(x);                                   // within (q + 1) / 2 of zero
-        return bits52(r < 0.0 ? r + q : r);
+        const u64 res = bits52(r < 0.0 ? r + q : r);
+        CKKS_RANGE(canonical(x, q, res, "F64WideArith::canon_wide"));
+        return res;
     }
-    __device__ __forceinline__ u64 to_mid_fwd(V x) const { return (u64)__double_as_longlong(balance(x)); }
-    __device__ __forceinline__ u64 to_canonical_fwd(V x) const { return canon_wide(x); }
-    template <int R> __device__ __forceinline__ void round_end(V (&v)[R]) const {
+    CKKS_HD u64 to_mid_fwd(V x) const { return f64_bits(balance(x)); }
+    CKKS_HD u64 to_canonical_fwd(V x) const { return canon_wide(x); }
+    template <int R> CKKS_HD void round_end(V (&v)[R]) const {
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = balance(v[j]);
     }
-    __device__ __forceinline__ void gs_last(V& x, V& y, u64& ox, u64& oy) const {
+    CKKS_HD void gs_last(V& x, V& y, u64& ox, u64& oy) const {
         double s = x + y, d = x - y;
+        CKKS_RANGE(value(s, "F64WideArith::gs_last sum"));
+        CKKS_RANGE(value(d, "F64WideArith::gs_last difference"));
         ox = canon_wide(mulmod(s, n_inv));
         oy = canon_wide(mulmod(d, w1n));
     }
@@ -149,7 +159,7 @@ struct F64WideArith : F64Arith {
 //   tw[(tw_off << s) + (e >> (S - s))],  tw_off = 1 for the strided pass, N1 + row for the row pass.
 // ------------------------------------------------------------------------------------------------------------
 template <class AR, int S, int S1>
-__device__ __forceinline__ void fwd_spread(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
+CKKS_HD void fwd_spread(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
                                            const AR& ar) {
     constexpr int R = 1 << S1;
 #pragma unroll
@@ -165,7 +175,7 @@ __device__ __forceinline__ void fwd_spread(typename AR::V (&v)[1 << S1], const t
     }
 }
 template <class AR, int S, int S1>
-__device__ __forceinline__ void fwd_packed(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
+CKKS_HD void fwd_packed(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
                                            unsigned g, const AR& ar) {
     constexpr int R = 1 << S1;
 #pragma unroll
@@ -182,7 +192,7 @@ __device__ __forceinline__ void fwd_packed(typename AR::V (&v)[1 << S1], const t
 }
 // inverse: same index structure, stages in the opposite order, Gentleman-Sande butterflies
 template <class AR, int S, int S1>
-__device__ __forceinline__ void inv_packed(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
+CKKS_HD void inv_packed(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
                                            unsigned g, const AR& ar) {
     constexpr int R = 1 << S1;
 #pragma unroll
@@ -198,7 +208,7 @@ __device__ __forceinline__ void inv_packed(typename AR::V (&v)[1 << S1], const t
     }
 }
 template <class AR, int S, int S1, int S_STOP>
-__device__ __forceinline__ void inv_spread(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
+CKKS_HD void inv_spread(typename AR::V (&v)[1 << S1], const typename AR::TW* __restrict__ tw, unsigned tw_off,
                                            const AR& ar) {
     constexpr int R = 1 << S1;
 #pragma unroll

@@ -15,6 +15,7 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "f64_exact.hpp"
 #include "pcmm.hpp"
 
 namespace ckks {
@@ -35,15 +36,8 @@ __device__ __forceinline__ void async_copy16(const void* g, void* lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory", "m0");
 }
 
-__device__ __forceinline__ double mulmod_f64(double a, double w, double q, double qinv) {
-    double h = a * w;
-    double l = __builtin_fma(a, w, -h);
-    double c = __builtin_rint(h * qinv);
-    return __builtin_fma(-c, q, h) + l;
-}
-__device__ __forceinline__ double balance_f64(double x, double q, double qinv) {
-    return __builtin_fma(-__builtin_rint(x * qinv), q, x);
-}
+// mulmod_f64, balance_f64 and the per-output statement of the epilogue (ppmm_recombine, ppmm_recombine_wide) are in f64_exact.hpp,
+// where a host build checks their ranges
 
 // ------------------------------------------------------------------------------------------------------------
 // Pass 1: residue digit planes.  Every residue is read ONCE, split into DC balanced base-256 digits and written in the
@@ -353,7 +347,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                     for (int r = 0; r < 4; r++) {
                         const double res = t[r] < 0.0 ? t[r] + q : t[r];
                         if (LAST) rl_wide[WIDE ? mt : 0][WIDE ? nt : 0][WIDE ? r : 0] = res;
-                        const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
+                        const u64 ures = f64_bits(res + 4503599627370496.0) & 0xFFFFFFFFFFFFFull;
                         if (LAST && !store_last) {}                           // a tail job other than the first: the residues are only needed in registers
                         else if (FULL) orow[r][nt * 16] = ures;
                         else if (mrow + mt * 16 + r < a.M) orow[r][nt * 16] = ures;
@@ -363,7 +357,8 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                 // The four outputs of a lane in one MFMA tile advance together, one operation at a time: every operation below is
                 // a chain link of one output, and four independent links in flight hide the FP64 pipeline latency.
                 // Horner inside each group of four diagonals: y_g = sum_{i<4} 256^i S_{4g+i}; |S_e| <= DW * Kpad * 2^14 and the
-                // launcher admits DW * Kpad < 2^15 only, so |y_g| < 2^53 and every step is exact
+                // launcher admits DW * Kpad <= 2^14 only, so |S_e| <= 2^28, |y_g| < 2^53 and every step is exact (ppmm_recombine in
+                // f64_exact.hpp is this sequence for one output; a host build checks its ranges)
                 double y0[4], y1[4], t[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) { y0[r] = (double)acc[3][mt][nt][r]; y1[r] = (double)acc[ND - 1][mt][nt][r]; }
@@ -413,7 +408,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                 for (int r = 0; r < 4; r++) {
                     const double res = t[r] < 0.0 ? t[r] + q : t[r];
                     // res is an integer in [0, q): adding 2^52 leaves it in the low mantissa bits
-                    const u64 ures = (u64)__double_as_longlong(res + 4503599627370496.0) & 0xFFFFFFFFFFull;
+                    const u64 ures = f64_bits(res + 4503599627370496.0) & 0xFFFFFFFFFFull;
                     if (LAST) {
                         rl_lo[mt][r][nt] = (unsigned)ures;
                         rl_hi[mt][nt] = (r == 0 ? 0u : rl_hi[mt][nt]) | ((unsigned)(ures >> 32) << (8 * r));
@@ -430,9 +425,9 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
         const int im = prime_of(it);
         q = a.pq[a.np + im].qd;
         qinv = a.pq[a.np + im].qinv_d;
-        c32 = __longlong_as_double((long long)a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
-        if (WIDE) c64 = __longlong_as_double((long long)a.consts[3 * PPMM_MAX_MODS + im]);   // 2^64 mod q (balanced)
-        qli = __longlong_as_double((long long)a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
+        c32 = f64_from_bits(a.consts[2 * PPMM_MAX_MODS + im]);   // 2^32 mod q (balanced)
+        if (WIDE) c64 = f64_from_bits(a.consts[3 * PPMM_MAX_MODS + im]);   // 2^64 mod q (balanced)
+        qli = f64_from_bits(a.consts[4 * PPMM_MAX_MODS + im]);   // q_last^-1 mod q
 #pragma unroll
         for (int e = 0; e < ND; e++)
 #pragma unroll
