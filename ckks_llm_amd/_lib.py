@@ -38,6 +38,7 @@ def _declare(L):
         "ckks_ctx_create": (i, [C.POINTER(vp), i, u64p, i, u64p, i, u64p, i, i]), "ckks_ctx_destroy": (i, [vp]),
         "ckks_set_stream": (i, [vp, vp]), "ckks_ctx_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "ckks_ctx_set_arith_mode": (i, [vp, i]), "ckks_ctx_set_ntt_mode": (i, [vp, i]), "ckks_ctx_check": (i, [vp]), "ckks_ctx_set_ntt_chain": (i, [vp, i, i]),
+        "ckks_ctx_set_option": (i, [vp, C.c_char_p, l]), "pcmm_set_option": (i, [vp, C.c_char_p, l]),
         "ckks_ctx_table": (i, [vp, C.c_char_p, u64p, sz, C.POINTER(sz)]),
         "ckks_ntt_fwd": (i, [vp, vp, i, i, i, i, i]), "ckks_ntt_inv": (i, [vp, vp, i, i, i, i, i]),
         "ckks_ntt_timed": (i, [vp, vp, i, i, i, i, i, i, C.POINTER(C.c_float), C.POINTER(C.c_float)]),

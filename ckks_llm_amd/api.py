@@ -145,6 +145,10 @@ class Context_23:
         batches of up to 128 limbs), 5: as 4 with a limb's tiles spread over all XCDs (mode 0 above 40 limbs).  All give the same residues."""
         _check(self.L_.ckks_ctx_set_ntt_mode(self.h, mode), "ckks_ctx_set_ntt_mode")
 
+    def set_option(self, name, value=1):
+        """Test / tuning switch by name: ks_split, ks_back_split, conv_int, ntt_no_reverse, ntt_chunk (see ckks_hip.h)."""
+        _check(self.L_.ckks_ctx_set_option(self.h, name.encode(), int(value)), "ckks_ctx_set_option")
+
     def set_ntt_chain(self, skew=0, spin_max=-1):
         """Tuning / test hook of the chained transform (ntt_mode 2); spin_max = 0 sends every second-pass tile to the finishing launch."""
         _check(self.L_.ckks_ctx_set_ntt_chain(self.h, skew, spin_max), "ckks_ctx_set_ntt_chain")
@@ -616,6 +620,10 @@ class PCMM_Context:
         v = C.c_long()
         _check(self.L_.pcmm_info(self.h, name.encode(), C.byref(v)), "pcmm_info")
         return v.value
+
+    def set_option(self, name, value=1):
+        """Test / tuning switch by name: gather_plain, ppmm_generic, ppmm_no_tail (see ckks_hip.h)."""
+        _check(self.L_.pcmm_set_option(self.h, name.encode(), int(value)), "pcmm_set_option")
 
     def weights_static(self, plain_mat, nbytes=None, is_static=True):
         """Declare a weight matrix static (it changes only through this library's copies): its digit planes are kept between PPMM

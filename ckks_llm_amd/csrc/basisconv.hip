@@ -166,8 +166,7 @@ static int launch_conv(ckks_ctx* c, const ConvPlan& plan, u64* out, const u64* i
         CKKS_HIP_TRY(hipGetLastError());
         return CKKS_OK;
     }
-    static const bool no_split = getenv("CKKS_CONV_INT") != nullptr;
-    if (plan.split_ok && c->arith_mode == 0 && !no_split) {
+    if (plan.split_ok && c->arith_mode == 0 && !c->conv_int) {
         const int parts = plan.max_tgt <= 8 ? 1 : plan.max_tgt <= 16 ? 2 : 4;
         grid.y *= parts;
         if (max_src <= 4) hipLaunchKernelGGL(conv_kernel_split<4>, grid, block, 0, c->stream, a, parts);

@@ -422,6 +422,11 @@ extern "C" int ckks_ctx_info(const ckks_ctx* c, const char* name, long* value) {
     else if (n == "ntt_mid_bytes") *value = (long)c->ntt_mid_cap;      // size of the inter-pass buffer the ordinary entry points have grown so far
     else if (n == "ntt_resident_round") *value = c->logN == 16 ? ckks::ntt_resident_round(c) : 0;      // limbs per round of the resident transform (0: it never applies)
     else if (n == "ntt_chain_deferred_tiles") return ckks::ntt_chain_deferred(const_cast<ckks_ctx*>(c), value);
+    else if (n == "ntt_pair_deferred_tiles") return ckks::ntt_pair_deferred(const_cast<ckks_ctx*>(c), value);
+    else if (n == "ntt_pair_stolen_tiles") return ckks::ntt_pair_deferred(const_cast<ckks_ctx*>(c), value, true);
+    else if (n == "ntt_pair_resident_blocks") *value = c->pair_resident_blocks[ckks::PAIR_KIND_F64];      // of the FP64 transform kernel
+    else if (n == "ntt_pair_resident_blocks_int") *value = c->pair_resident_blocks[ckks::PAIR_KIND_INT];
+    else if (n == "ntt_extra_forms") *value = ckks::ntt_extra_forms();
     else { ckks::set_error("ckks_ctx_info: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
@@ -441,6 +446,20 @@ extern "C" int ckks_ctx_set_arith_mode(ckks_ctx* c, int mode) {
 extern "C" int ckks_ctx_set_ntt_mode(ckks_ctx* c, int mode) {
     if (!c || mode < 0 || mode > 6) return CKKS_E_INVALID;
     c->ntt_mode = mode;
+    return CKKS_OK;
+}
+
+// test / tuning switches of a context, by name
+extern "C" int ckks_ctx_set_option(ckks_ctx* c, const char* name, long value) {
+    if (!c || !name) return CKKS_E_INVALID;
+    const std::string n(name);
+    if (n == "ks_split") c->ks_split = value != 0;
+    else if (n == "ks_back_split") c->ks_back_split = value != 0;
+    else if (n == "conv_int") c->conv_int = value != 0;
+    else if (n == "ntt_no_reverse") c->ntt_no_reverse = value != 0;
+    else if (n == "pair_no_steal") c->pair_no_steal = value != 0;
+    else if (n == "ntt_chunk") { if (value < 0 || value > 65535) return CKKS_E_INVALID; c->ntt_chunk = (int)value; }
+    else { ckks::set_error("ckks_ctx_set_option: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
 

@@ -99,6 +99,12 @@ struct ckks_ctx {
     std::vector<DecodeTab> decode_tabs;   // CRT tables of decode_coeffs, one per level, built on first use
     int chain_skew = 0, chain_spin = -1;  // chained transform: limbs a chain's first pass runs ahead of its second (0: default), poll limit of a wait (-1: default)
     void* d_ntt_pair = nullptr;           // completion words of the paired (one-launch, small-batch) transform, one per 128-byte line
+    unsigned pair_resident_blocks[6] = {}; // workgroups of each one-launch kernel that fit the chip at once (occupancy x compute units), by PAIR_KIND_*
+    // test / tuning switches (ckks_ctx_set_option): the fused key-switch, rescale and ring-packing launches off; the key switch's
+    // last steps as separate launches; conversions into primes below 2^50 in 128-bit integers; the second launch of a transform
+    // takes the limbs in forward order; limbs per trip through the inter-pass buffer (0: all)
+    bool ks_split = false, ks_back_split = false, conv_int = false, ntt_no_reverse = false, pair_no_steal = false;
+    int ntt_chunk = 0;
     unsigned* h_pair_fail = nullptr;      // pinned host word that a paired transform raises when one of its waits ran out
     void* d_ntt_chain = nullptr;          // completion words of the chained (one-launch) transform, allocated on its first use; zero between transforms
 };
@@ -116,7 +122,10 @@ int hip_fail(hipError_t e, const char* what);
 // chained (one-launch) transform: tiles left to its finishing launch so far, and the host view of its slot order (for tests)
 int ntt_chain_deferred(ckks_ctx* c, long* tiles);
 // 1 once a paired (one-launch) transform of the context has given up a wait: its output is incomplete and the context unusable
+enum { PAIR_KIND_F64 = 0, PAIR_KIND_WIDE, PAIR_KIND_INT, PAIR_KIND_RESCALE, PAIR_KIND_RESCALE_WIDE, PAIR_KIND_KS_BACK };
 int ntt_pair_failed(const ckks_ctx* c);
+int ntt_pair_deferred(ckks_ctx* c, long* tiles, bool stolen = false);        // second-pass tiles that paired launches have left to their limb's last workgroup (synchronises)
+int ntt_extra_forms();                                  // 1 if the library was built with launch forms 2 and 3
 int ntt_pair_init(ckks_ctx* c);
 void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile);
 unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew);

@@ -31,6 +31,7 @@
 
 #include "context.hpp"
 #include "ntt_core.hpp"
+#include "pair_protocol.hpp"
 
 namespace ckks {
 
@@ -39,11 +40,35 @@ namespace ckks {
 // strided pass (first SA forward stages / last SA inverse stages): one tile = CW adjacent columns, all N1 rows
 // ------------------------------------------------------------------------------------------------------------
 
+// The two questions that a workgroup of a paired launch asks of its limb's protocol words (pair_protocol.hpp) with atomics that
+// return an answer - the claim of its own first-pass tile and its counting out - ride inside a tile: lane 0 asks behind the
+// tile's own loads (memory operations return in the order of their issue, so an answer that queues behind the other workgroups'
+// atomics on the same words does not hold the loads up) and publishes the answer in LDS, the claim just ahead of the tile's
+// first barrier, the count at the tile's end.  Behind that barrier every lane knows whether a claimed tile is this workgroup's;
+// up to there a tile only reads global memory and writes LDS, so a tile that turns out to be another's leaves no trace.
+// Default: nothing to ask.
+struct TileClaim {
+    unsigned* lds = nullptr;       // where the answer is published (nullptr: nothing to ask)
+    unsigned* words = nullptr;     // the limb's protocol words
+    unsigned tile = 0;
+    bool counting_out = false;     // false: the claim of a first-pass tile; true: the counting out, inside a second-pass tile
+    __device__ __forceinline__ unsigned start(unsigned tid) const {
+        unsigned v = tile;
+        if (lds && tid == 0) {
+            asm volatile("" ::: "memory");
+            v = counting_out ? pair::leave(words) : pair::claim_own(words, tile, true);
+        }
+        return v;
+    }
+    __device__ __forceinline__ void publish(unsigned tid, unsigned value) const { if (lds && tid == 0) *lds = value; }
+    __device__ __forceinline__ bool lost() const { return lds && !counting_out && *lds == pair::LEAVE; }
+};
+
 // PAIRED: the tile is one half of a paired transform - what it hands to or takes from the other pass moves as shared accesses
 template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool EMBED = false, bool PAIRED = false>
 __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
                                              typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const NttArgs* ea = nullptr,
-                                             unsigned poly = 0, bool lift = false) {
+                                             unsigned poly = 0, bool lift = false, const TileClaim& claim = TileClaim()) {
     typedef StridedCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     typedef typename AR::V V;
@@ -95,11 +120,14 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
 #pragma unroll
             for (int j = 0; j < R; j++) v[j] = ar.from_canonical(load_word<COHERENT>(col + (long)(g + j * G) * N2));
         }
+        const unsigned claimed = claim.start(tid);
         fwd_spread<AR, SA, S1>(v, tw, 1u, ar);
         ar.round_end(v);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+        claim.publish(tid, claimed);
         __syncthreads();
+        if (claim.lost()) return;                       // uniform: another workgroup has taken this tile; nothing was stored yet
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
         fwd_packed<AR, SA, S1>(v, tw, 1u, g, ar);
@@ -120,6 +148,7 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
 #pragma unroll
             for (int j = 0; j < R; j++) v[j] = ar.from_mid(PAIRED ? get<true>(col + (long)(g * R + j) * N2) : load_word<COHERENT>(col + (long)(g * R + j) * N2));
         }
+        const unsigned counted = claim.start(tid);
         inv_packed<AR, SA, S1>(v, tw, 1u, g, ar);
         ar.round_end(v);
 #pragma unroll
@@ -136,6 +165,7 @@ __device__ __forceinline__ void strided_tile(u64* limb, unsigned tile, const typ
             store_word<COHERENT>(col + (long)(g + j * G) * N2, ox);
             store_word<COHERENT>(col + (long)(g + (j + R / 2) * G) * N2, oy);
         }
+        claim.publish(tid, counted);
     }
 }
 
@@ -158,7 +188,7 @@ __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pas
 
 template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool PAIRED = false>
 __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                         typename AR::V* lds, unsigned tid, char* mid_limb = nullptr) {
+                                         typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const TileClaim& claim = TileClaim()) {
     typedef RowCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     typedef typename AR::V V;
@@ -180,6 +210,7 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
 #pragma unroll
             for (int j = 0; j < R; j++) v[j] = ar.from_mid(PAIRED ? get<true>(rp + u + j * U) : load_word<COHERENT>(rp + u + j * U));
         }
+        const unsigned counted = claim.start(tid);
         fwd_spread<AR, SB, S1>(v, tw, tw_off, ar);
         ar.round_end(v);
 #pragma unroll
@@ -195,10 +226,17 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; j++) store_word<COHERENT>(rp + u + j * U, ar.to_canonical_fwd(lrow[padded(u + j * U)]));
+        claim.publish(tid, counted);
     } else {
+        u64 raw[R];
 #pragma unroll
-        for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = ar.from_canonical(load_word<COHERENT>(rp + u + j * U));
+        for (int j = 0; j < R; j++) raw[j] = load_word<COHERENT>(rp + u + j * U);
+        const unsigned claimed = claim.start(tid);
+#pragma unroll
+        for (int j = 0; j < R; j++) lrow[padded(u + j * U)] = ar.from_canonical(raw[j]);
+        claim.publish(tid, claimed);
         __syncthreads();
+        if (claim.lost()) return;                       // uniform: another workgroup has taken this tile; nothing was stored yet
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
         inv_packed<AR, SB, S1>(v, tw, tw_off, u, ar);
@@ -233,85 +271,7 @@ __global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass(NttArg
                                                   COMPACT ? a.mid + l * MID_LIMB_BYTES : nullptr);
 }
 
-// ------------------------------------------------------------------------------------------------------------
-// Whole-limb transform: one workgroup carries one limb through both passes in one launch.
-//
-// The workgroup is GROUPS groups of 256 lanes; each group takes every GROUPS-th tile of the first pass, the workgroup waits
-// until all its stores have left the compute unit, then the groups take the tiles of the second pass.  Nothing is exchanged
-// between workgroups, so there is no synchronisation beyond the workgroup barrier.  Between the passes the limb is not
-// read back from HBM: its lines are still in the XCD's L2 or, once displaced from there, in the memory-side cache, because
-// only (resident workgroups) x N x 8 bytes are in that state at any time.  The second-pass loads bypass the L1, which may
-// still hold pre-transform copies of the same lines from the first pass of this very workgroup.
-// ------------------------------------------------------------------------------------------------------------
-template <class AR, int SA, int SB, bool INVERSE, int GROUPS>
-__global__ __launch_bounds__(256 * GROUPS) void ntt_limb_kernel(NttArgs a) {
-    typedef StridedCfg<SA, SB> CS;
-    typedef RowCfg<SA, SB> CR;
-    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES, "whole-limb kernel: tile shapes must agree");
-    static_assert(CS::TILES % GROUPS == 0, "whole-limb kernel: tiles must divide among the groups");
-    constexpr int TILES = CS::TILES;
-    constexpr long N = 1l << (SA + SB);
-    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
-    typedef typename AR::TW TW;
-    __shared__ typename AR::V lds_all[GROUPS][LDS_WORDS];
-    const unsigned grp = threadIdx.x / 256, tid = threadIdx.x % 256;
-    typename AR::V* lds = lds_all[grp];
-    int prime;
-    u64* limb = limb_ptr(a, blockIdx.x, N, prime);
-    const AR ar(a.primes[prime]);
-    const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
-#pragma unroll 1
-    for (int t = grp; t < TILES; t += GROUPS) {
-        if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, t, tw, ar, lds, tid);
-        else row_tile<AR, SA, SB, true, false>(limb, t, tw, ar, lds, tid);
-        __syncthreads();
-    }
-    // every store of the first pass has been acknowledged by the L2 before any lane starts the second pass
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-#pragma unroll 1
-    for (int t = grp; t < TILES; t += GROUPS) {
-        if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, t, tw, ar, lds, tid);
-        else strided_tile<AR, SA, SB, true, true>(limb, t, tw, ar, lds, tid);
-        __syncthreads();
-    }
-}
-
-// ------------------------------------------------------------------------------------------------------------
-// Chained transform: both passes in ONE launch, the data between them held in the XCD's L2.
-//
-// A two-launch transform moves every limb through HBM twice.  Here the second pass of a limb runs on the same XCD as its first
-// pass, a few microseconds later, while the limb's lines (512 KiB at N = 2^16, written in place by the first pass) are still
-// dirty in that XCD's 4 MiB L2: HBM sees one read and one write per limb.
-//
-// Order of work.  The grid is one-dimensional and not persistent.  Workgroup b belongs to chain x = b mod 8 and takes slot
-// s = b / 8 of that chain; the hardware hands consecutive workgroups of a grid to the XCDs in turn, so a chain's workgroups all
-// run on one XCD.  A chain works through the limbs x, x + 8, x + 16, .. in entries of TILES workgroups (one pass of one limb):
-//     P1(k=0) .. P1(k=skew-1) | P1(k=skew) P2(k=0) | P1(k=skew+1) P2(k=1) | ...
-// so that the second pass of a limb is dispatched while later limbs' first passes keep the compute units busy.
-//
-// Synchronisation.  A first-pass workgroup waits for nothing; when its stores have reached the L2 it adds 1 to the limb's
-// completion word.  A second-pass workgroup waits until that word reads TILES.  Workgroups of a grid start in the order of their
-// index, so what it waits for has started before it; the wait is bounded by a poll count all the same.
-// Nothing depends on the placement or on the wait for correctness: every workgroup reads the XCD it really runs on from the
-// hardware register; a first-pass workgroup that finds itself on another XCD than its chain's adds a mark to the completion word
-// instead of the plain 1, and a second-pass workgroup that is on the wrong XCD, sees a mark, or runs out of polls does not touch
-// the data: it records its tile in the limb's `todo` word and leaves.  A second launch (ntt_chain_finish_kernel, one workgroup
-// per limb) runs the recorded tiles - after the kernel boundary every store is visible everywhere - and returns both words to
-// zero for the next transform.  Every workgroup of both launches ends after a bounded number of steps.
-// ------------------------------------------------------------------------------------------------------------
-constexpr unsigned CHAIN_XCDS = 8;
-constexpr unsigned CHAIN_MARK = 0x10000u;          // added by a first-pass workgroup that ran on an unexpected XCD
-struct ChainArgs {
-    unsigned* done;            // [limb] completion word of the first pass
-    unsigned* todo;            // [limb] bit t: second-pass tile t was left to the finishing launch
-    unsigned* stats;           // [0]: tiles left to the finishing launch since the context was created
-    unsigned limbs, kmax, skew, spin_max;
-    unsigned zero;             // 0, but not known to the compiler: "add zero" stays a read-modify-write executed at the L2
-    unsigned long long xcc_of; // nibble x: the XCD that runs chain x
-};
-
+// order of work of the chained transform (mode 2, ntt_extra_forms.hpp); pure arithmetic, also exported for its host-side test
 // slot s of a chain -> pass (0 / 1), index k of the limb within the chain, tile.  k >= kmax: an empty slot.
 __host__ __device__ inline void chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned& second, unsigned& k, unsigned& tile) {
     const unsigned e = s / tiles;
@@ -321,93 +281,14 @@ __host__ __device__ inline void chain_slot(unsigned s, unsigned tiles, unsigned 
 }
 __host__ __device__ inline unsigned chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return (skew + 2 * kmax) * tiles; }
 
-template <class AR, int SA, int SB, bool INVERSE>
-__global__ __launch_bounds__(256) void ntt_chain_kernel(NttArgs a, ChainArgs ch) {
-    typedef StridedCfg<SA, SB> CS;
-    typedef RowCfg<SA, SB> CR;
-    static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES && CS::TILES <= 16, "chained kernel: tile shapes");
-    constexpr unsigned TILES = CS::TILES;
-    constexpr long N = 1l << (SA + SB);
-    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
-    typedef typename AR::TW TW;
-    __shared__ typename AR::V lds[LDS_WORDS];
-    __shared__ unsigned go;
-    const unsigned x = blockIdx.x % CHAIN_XCDS;
-    unsigned second, k, tile;
-    chain_slot(blockIdx.x / CHAIN_XCDS, TILES, ch.skew, second, k, tile);
-    const unsigned limb_id = x + CHAIN_XCDS * k;
-    if (k >= ch.kmax || limb_id >= ch.limbs) return;                            // uniform over the workgroup
-    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;       // XCC_ID[3:0]
-    const bool placed = xcc == (unsigned)((ch.xcc_of >> (4 * x)) & 15u);
-    int prime;
-    u64* limb = limb_ptr(a, limb_id, N, prime);
-    const AR ar(a.primes[prime]);
-    const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
-    if (!second) {
-        if (!INVERSE) strided_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
-        else row_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
-        // every store of this tile has been acknowledged by the L2 before the completion word moves
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (threadIdx.x == 0) atomicAdd(&ch.done[limb_id], placed ? 1u : CHAIN_MARK + 1u);
-        return;
-    }
-    if (threadIdx.x == 0) {
-        unsigned ok = placed ? 1u : 0u;
-        if (ok) {
-            unsigned v = 0;
-            for (unsigned n = 0; n < ch.spin_max; n++) {
-                v = atomicAdd(&ch.done[limb_id], ch.zero);
-                if (v >= TILES) break;
-                __builtin_amdgcn_s_sleep(8);
-            }
-            ok = v == TILES ? 1u : 0u;
-        }
-        if (!ok) atomicOr(&ch.todo[limb_id], 1u << tile);
-        go = ok;
-    }
-    __syncthreads();
-    if (!go) return;
-    // second-pass loads bypass this compute unit's L1 (which may hold pre-transform copies of the same lines) and are served by the L2
-    if (!INVERSE) row_tile<AR, SA, SB, false, true>(limb, tile, tw, ar, lds, threadIdx.x);
-    else strided_tile<AR, SA, SB, true, true>(limb, tile, tw, ar, lds, threadIdx.x);
-}
-
-// One workgroup per limb: runs the second-pass tiles that the chained launch left behind, then clears the limb's words.
-template <class AR, int SA, int SB, bool INVERSE>
-__global__ __launch_bounds__(256) void ntt_chain_finish_kernel(NttArgs a, ChainArgs ch) {
-    typedef StridedCfg<SA, SB> CS;
-    typedef RowCfg<SA, SB> CR;
-    constexpr long N = 1l << (SA + SB);
-    constexpr int LDS_WORDS = CS::LDS_WORDS > CR::LDS_WORDS ? CS::LDS_WORDS : CR::LDS_WORDS;
-    typedef typename AR::TW TW;
-    __shared__ typename AR::V lds[LDS_WORDS];
-    __shared__ unsigned mask_s;
-    const unsigned limb_id = blockIdx.x;
-    if (limb_id >= ch.limbs) return;
-    if (threadIdx.x == 0) mask_s = ch.todo[limb_id];
-    __syncthreads();
-    const unsigned mask = mask_s;
-    if (mask) {
-        int prime;
-        u64* limb = limb_ptr(a, limb_id, N, prime);
-        const AR ar(a.primes[prime]);
-        const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
-#pragma unroll 1
-        for (unsigned tile = 0; tile < (unsigned)CS::TILES; tile++) {
-            if (!((mask >> tile) & 1u)) continue;
-            if (!INVERSE) row_tile<AR, SA, SB, false, false>(limb, tile, tw, ar, lds, threadIdx.x);
-            else strided_tile<AR, SA, SB, true, false>(limb, tile, tw, ar, lds, threadIdx.x);
-            __syncthreads();
-        }
-    }
-    if (threadIdx.x == 0) {
-        ch.done[limb_id] = 0;
-        ch.todo[limb_id] = 0;
-        if (mask) atomicAdd(ch.stats, (unsigned)__builtin_popcount(mask));
-    }
-}
+#ifdef CKKS_NTT_EXTRA_FORMS
+#include "ntt_extra_forms.hpp"
+#else
+int ntt_chain_deferred(ckks_ctx*, long* tiles) { *tiles = 0; return CKKS_OK; }
+#endif
+// host view of the slot order, for tests
+void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile) { chain_slot(s, tiles, skew, *second, *k, *tile); }
+unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return chain_slots(kmax, tiles, skew); }
 
 // ------------------------------------------------------------------------------------------------------------
 // Paired transform for small batches: both passes in one launch, one workgroup per (limb, tile) that runs the tile of the
@@ -415,29 +296,31 @@ __global__ __launch_bounds__(256) void ntt_chain_finish_kernel(NttArgs a, ChainA
 // A launch of a few hundred workgroups is over before the chip has ramped up, so for one ciphertext the second launch's
 // ramp and the drain between the launches cost as much as the work; here they fall away.
 //
-// Synchronisation is that of the programming model, with no assumption about where a workgroup runs: every wave releases its
-// first-pass stores at agent scope, the workgroup adds 1 to the limb's completion word, polls it (agent-scope loads) until
-// it reads a multiple of TILES, and every wave acquires at agent scope before the second pass loads.  The word is a
-// multiple of TILES between launches (launches of one context are ordered on its stream and each adds TILES to the words of
-// its limbs), so nothing has to be cleared; a workgroup has added its own 1 before it polls, so a multiple of TILES can only
-// be the completed count.
-// Progress: a waiting workgroup waits for workgroups that wait for nothing.  Workgroups start in the order of their index and
-// the sixteen of a limb lie within 128 consecutive indices, so at most 128 resident workgroups can be waiting for one that has not
-// started; the launcher only uses this kernel where the chip holds more than that many at once.  The wait is bounded all the
-// same (about two seconds of polls): a workgroup that runs out of polls leaves its tile undone and raises the context's
-// host-visible failure word, which fails the next call or synchronisation on the context.
+// Synchronisation (pair_protocol.hpp has the protocol and its reasoning): what the first pass hands to the second moves as
+// relaxed atomic accesses at agent scope - on this hardware ordinary stores that are written through to, and loads that are
+// served from, the level of the memory system that all compute units share.  Every wave waits until its stores have been
+// acknowledged (s_waitcnt 0 behind a workgroup-scope release fence), the workgroup meets at a barrier, and one lane then counts
+// the tile done with a relaxed atomic at agent scope.  A reader has seen the full count, by an access of the same kind, before
+// it issues its loads.  This rests on the hardware's behaviour for these access kinds, which is what the programming model's
+// agent-scope release/acquire pair would also compile to for them; no cache maintenance is asked for beyond it.
+// Progress does not depend on which workgroups are resident or in what order they start: a workgroup whose wait outlasts a few
+// tens of polls takes over first-pass tiles whose workgroups have not started, every wait is bounded, and what a workgroup
+// leaves undone the last workgroup of the limb to leave completes; the launch returns its words to zero.
 // Blocks are numbered so that the tiles of a limb go to one XCD (workgroup b of a grid goes to XCD b mod 8): the inter-pass
 // data then stays in that XCD's L2.  Placement only matters for speed.
 // ------------------------------------------------------------------------------------------------------------
 constexpr unsigned PAIR_XCDS = 8;
-constexpr int PAIR_MAX_LIMBS = 4096;               // completion words per context
+constexpr int PAIR_MAX_LIMBS = 4096;               // protocol words per context
 constexpr int PAIR_GROUPED_LIMBS = 40;             // ... and up to this many with a limb's tiles on one XCD, above it spread over all
-constexpr int PAIR_WORD_STRIDE = 32;               // one completion word per 128-byte line: atomics on one line are carried out one after the other
-constexpr int PAIR_AUTO_LIMBS = 128;                // automatic mode: batches up to this many limbs take the paired kernel
+constexpr int PAIR_WORD_STRIDE = pair::WORDS;      // protocol words per limb (pair_protocol.hpp)
+constexpr int PAIR_AUTO_LIMBS = 128;               // automatic mode: batches up to this many limbs take the paired kernel (while the grid fits the chip)
 struct PairArgs {
-    unsigned* done;            // [limb * PAIR_WORD_STRIDE] first-pass completion count, a multiple of TILES between launches
-    unsigned* fail;            // host-visible word: nonzero once a wait has run out
-    unsigned limbs, spin_max;
+    unsigned* done;            // [limb * PAIR_WORD_STRIDE] the limb's protocol words (pair_protocol.hpp), zero between launches
+    unsigned* fail;            // host-visible word: nonzero once a wait of the key switch's last launch has run out
+    unsigned limbs;
+    unsigned spin_steal;       // polls after which a waiting workgroup takes over tiles whose workgroups have not started
+    unsigned spin_max;         // polls after which it leaves its second-pass tiles to the last workgroup out
+    unsigned steal;            // 0: no workgroup takes over another's tile (a test setting)
     unsigned spread;           // the tiles of a limb go to consecutive workgroups, i.e. to all XCDs (larger batches, and a test setting)
 };
 // (limb, tile) of workgroup b of a paired launch
@@ -446,25 +329,67 @@ __device__ __forceinline__ void pair_block(const PairArgs& p, unsigned b, unsign
     limb_id = p.spread ? b / tiles : b % PAIR_XCDS + PAIR_XCDS * (idx / tiles);
     tile = p.spread ? b % tiles : idx % tiles;
 }
-// Between the two tiles of a workgroup: this workgroup's shared stores are complete, the limb's count moves, and the workgroup
-// waits for the count to read a multiple of `tiles`.  false: the wait ran out (the failure word is raised), the caller leaves.
-__device__ __forceinline__ bool pair_hand_over(const PairArgs& p, unsigned limb_id, unsigned tiles, unsigned* go) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);                                              // every shared store of this wave has been acknowledged
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned* word = p.done + (size_t)limb_id * PAIR_WORD_STRIDE;
-        (void)__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned ok = 0;
-        for (unsigned n = 0; n < p.spin_max; n++) {
-            if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) % tiles == 0) { ok = 1; break; }
-            __builtin_amdgcn_s_sleep(4);
-        }
-        if (!ok) __hip_atomic_store(p.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        *go = ok;
+// The two passes of (limb_id, tile) under the protocol.  pass1(t) and pass2(t) run tile t on the whole workgroup (t is the
+// workgroup's own tile unless it has taken over others; uniform over the workgroup).  stealing = false: a workgroup only ever
+// runs its own tile (the first pass is work that only this workgroup can do, already under way when this is called).
+template <class P1, class P2>
+__device__ __forceinline__ void pair_run(const PairArgs& p, unsigned limb_id, unsigned tile, unsigned* sh, bool stealing, P1 pass1, P2 pass2) {
+    static_assert(pair::TILES == 16, "sixteen tiles per limb");
+    unsigned* w = p.done + (size_t)limb_id * PAIR_WORD_STRIDE;
+    // The claim of the own tile travels while the tile's loads do (see TileClaim); a tile taken over later is claimed before it starts.
+    TileClaim own;
+    own.lds = stealing ? sh : nullptr;
+    own.words = w;
+    own.tile = tile;
+    unsigned mine = 0, act = tile;
+    for (bool first = true;; first = false) {
+        pass1(act, first ? own : TileClaim());
+        if (first && own.lost()) { act = pair::LEAVE; break; }                  // uniform: behind the tile's first barrier every lane reads the same word
+        mine |= 1u << act;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);                                          // every shared store of this wave has been acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0) *sh = pair::tile_done_then_decide(w, stealing, p.spin_steal, p.spin_max);
+        // The deciding lane's LDS write is complete before its wave reaches the barrier: said explicitly, because a barrier in a
+        // loop has been seen compiled with no wait for a write that reaches it over the loop's back edge.
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        act = *sh;
+        __syncthreads();
+        if (act >= pair::TILES) break;
     }
+    // Counting out does not wait for the own second pass: nothing that the last workgroup out does (the second pass of tiles that
+    // others have left, the reset of the words) depends on it.  It rides inside the first second-pass tile (see TileClaim); a
+    // workgroup with no second pass to run counts out here.
+    unsigned todo = act == pair::GO ? mine : 0u;
+    TileClaim out;
+    out.lds = sh;
+    out.words = w;
+    out.counting_out = true;
+    if (todo == 0u && threadIdx.x == 0) {
+        if (act == pair::DEFER) pair::defer(w, mine);
+        *sh = pair::leave(w);
+    }
+    for (bool first = true; todo; first = false) {
+        const unsigned t = (unsigned)__builtin_ctz(todo);
+        todo &= todo - 1u;
+        __syncthreads();                                                        // the tile before is done with the LDS
+        pass2(t, first ? out : TileClaim());
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);                                         // lgkmcnt(0) only: the LDS write above, not the tile's last stores
     __syncthreads();
-    return *go != 0;
+    unsigned last = *sh;
+    if (!(last & 0x80000000u)) return;
+    // last out: every first-pass tile of the limb is complete; what the others left undone, then the words back to zero
+    const unsigned finished = last & pair::ALL;
+    todo = finished;
+    while (todo) {
+        const unsigned t = (unsigned)__builtin_ctz(todo);
+        todo &= todo - 1u;
+        __syncthreads();
+        pass2(t, TileClaim());
+    }
+    if (threadIdx.x == 0) pair::reset(w, finished);
 }
 template <class AR, int SA, int SB, bool INVERSE, bool COMPACT>
 __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
@@ -485,32 +410,57 @@ __global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     const AR ar(a.primes[prime]);
     const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * N;
     char* mid_limb = COMPACT ? a.mid + (long)limb_id * MID_LIMB_BYTES : nullptr;
-    if (!INVERSE) strided_tile<AR, SA, SB, false, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
-    else row_tile<AR, SA, SB, true, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
-    if (!pair_hand_over(p, limb_id, TILES, &go)) return;
-    if (COMPACT) limb += a.out_delta;
-    if (!INVERSE) row_tile<AR, SA, SB, false, false, COMPACT, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
-    else strided_tile<AR, SA, SB, true, false, COMPACT, false, true>(limb, tile, tw, ar, lds, threadIdx.x, mid_limb);
+    u64* out_limb = COMPACT ? limb + a.out_delta : limb;
+    pair_run(p, limb_id, tile, &go, p.steal != 0,
+             [&](unsigned t, const TileClaim& claim) {
+                 if (!INVERSE) strided_tile<AR, SA, SB, false, false, COMPACT, false, true>(limb, t, tw, ar, lds, threadIdx.x, mid_limb, nullptr, 0, false, claim);
+                 else row_tile<AR, SA, SB, true, false, COMPACT, true>(limb, t, tw, ar, lds, threadIdx.x, mid_limb, claim);
+             },
+             [&](unsigned t, const TileClaim& out) {
+                 if (!INVERSE) row_tile<AR, SA, SB, false, false, COMPACT, true>(out_limb, t, tw, ar, lds, threadIdx.x, mid_limb, out);
+                 else strided_tile<AR, SA, SB, true, false, COMPACT, false, true>(out_limb, t, tw, ar, lds, threadIdx.x, mid_limb, nullptr, 0, false, out);
+             });
 }
 
 static int ensure_mid(ckks_ctx* c, size_t need);
 
-// Completion words and failure word of the paired transform, once per context (at its creation, so that no transform allocates).
+static void pair_resident_blocks(ckks_ctx* c);      // defined behind the kernels it asks about
+
+// Protocol words and failure word of the paired transform, once per context (at its creation, so that no transform allocates).
 int ntt_pair_init(ckks_ctx* c) {
     if (c->d_ntt_pair) return CKKS_OK;
     if (hipHostMalloc((void**)&c->h_pair_fail, sizeof(unsigned), hipHostMallocMapped) != hipSuccess) { set_error("NTT: cannot allocate the failure word of the paired transform"); return CKKS_E_NOMEM; }
     *c->h_pair_fail = 0;
     const size_t bytes = ((size_t)PAIR_MAX_LIMBS + 64) * PAIR_WORD_STRIDE * sizeof(unsigned);      // the last 64: counters of ks_back_kernel
     if (hipMalloc(&c->d_ntt_pair, bytes) != hipSuccess) { set_error("NTT: cannot allocate the completion words of the paired transform"); return CKKS_E_NOMEM; }
-    CKKS_HIP_TRY(hipMemsetAsync(c->d_ntt_pair, 0, bytes, c->stream));
+    CKKS_HIP_TRY(hipMemset(c->d_ntt_pair, 0, bytes));          // complete before the caller can launch anything on any stream
+    pair_resident_blocks(c);
     return CKKS_OK;
 }
 int ntt_pair_failed(const ckks_ctx* c) { return c->h_pair_fail && *(volatile unsigned*)c->h_pair_fail ? 1 : 0; }
+int ntt_pair_deferred(ckks_ctx* c, long* tiles, bool stolen) {
+    *tiles = 0;
+    if (!c->d_ntt_pair) return CKKS_OK;
+    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
+    std::vector<unsigned> w((size_t)PAIR_MAX_LIMBS * PAIR_WORD_STRIDE);
+    CKKS_HIP_TRY(hipMemcpy(w.data(), c->d_ntt_pair, w.size() * sizeof(unsigned), hipMemcpyDeviceToHost));
+    for (int i = 0; i < PAIR_MAX_LIMBS; i++) *tiles += w[(size_t)i * PAIR_WORD_STRIDE + (stolen ? pair::STOLEN_TOTAL : pair::DEFERRED_TOTAL)];
+    return CKKS_OK;
+}
+int ntt_extra_forms() {
+#ifdef CKKS_NTT_EXTRA_FORMS
+    return 1;
+#else
+    return 0;
+#endif
+}
 
 static PairArgs pair_args(const ckks_ctx* c, int limbs) {
     PairArgs p;
     p.done = (unsigned*)c->d_ntt_pair; p.fail = c->h_pair_fail; p.limbs = (unsigned)limbs;
     p.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : 4000000u;
+    p.spin_steal = c->chain_spin >= 0 && c->chain_spin < 32 ? (unsigned)c->chain_spin : 32u;
+    p.steal = c->pair_no_steal ? 0u : 1u;
     p.spread = c->ntt_mode == 5 || (c->ntt_mode == 0 && limbs > PAIR_GROUPED_LIMBS) ? 1u : 0u;
     return p;
 }
@@ -558,9 +508,8 @@ static void launch_passes(ckks_ctx* c, const NttArgs& args_in, int n, bool inver
     typedef RowCfg<SA, SB> CR;
     // The second launch walks the limbs backwards: what the first launch wrote last is still in the memory-side cache (256 MiB)
     // when the second starts, and what the second writes last is what a following transform of the same data reads first.
-    static const bool rev_env = getenv("CKKS_NTT_NO_REVERSE") == nullptr;
     NttArgs args = args_in, args2 = args_in;
-    args2.reverse = rev_env ? 1 : 0;
+    args2.reverse = c->ntt_no_reverse ? 0 : 1;
     dim3 gs(CS::TILES, n), bs(CS::THREADS);
     dim3 gr(CR::TILES, n), br(CR::THREADS);
     if (!inverse) {
@@ -579,8 +528,7 @@ template <class AR, int SA, int SB>
 static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, bool compact_ok, int first = 0, const NttFixedArea* fixed = nullptr) {
     // first: the limbs before it have been taken by another launch form (the resident transform takes whole rounds of a batch)
     constexpr bool CAN_COMPACT = std::is_same<AR, F64Arith>::value && SA == 8 && SB == 8;
-    static const int chunk_env = getenv("CKKS_NTT_CHUNK") ? atoi(getenv("CKKS_NTT_CHUNK")) : 0;
-    int chunk = (chunk_env > 0 && !c->ev_mid_armed) ? chunk_env : limbs - first;
+    int chunk = (c->ntt_chunk > 0 && !c->ev_mid_armed) ? c->ntt_chunk : limbs - first;
     const bool compact = CAN_COMPACT && compact_ok && (fixed || c->ntt_mode != 1);
     if (compact) {
         // the inter-pass buffer is kept at or below 1 GiB; larger batches go through it in chunks (stream order keeps them apart)
@@ -612,91 +560,19 @@ static int launch_two_pass(ckks_ctx* c, NttArgs args, int limbs, bool inverse, b
     return CKKS_OK;
 }
 
-constexpr unsigned CHAIN_MAX_LIMBS = 65536;
-static int ensure_chain(ckks_ctx* c) {
-    if (c->d_ntt_chain) return CKKS_OK;
-    const size_t bytes = (2 * (size_t)CHAIN_MAX_LIMBS + 16) * sizeof(unsigned);
-    if (hipMalloc(&c->d_ntt_chain, bytes) != hipSuccess) { set_error("NTT: cannot allocate the completion words of the chained transform"); return CKKS_E_NOMEM; }
-    CKKS_HIP_TRY(hipMemsetAsync(c->d_ntt_chain, 0, bytes, c->stream));
-    return CKKS_OK;
-}
-
-template <class AR, int SA, int SB>
-static int launch_chain(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
-    static const int skew_env = getenv("CKKS_NTT_SKEW") ? atoi(getenv("CKKS_NTT_SKEW")) : 0;
-    static const int spin_env = getenv("CKKS_NTT_SPIN") ? atoi(getenv("CKKS_NTT_SPIN")) : 0;
-    static const int lds_env = getenv("CKKS_NTT_CHAIN_LDS") ? atoi(getenv("CKKS_NTT_CHAIN_LDS")) : 0;      // extra LDS per workgroup: fewer resident workgroups
-    int rc = ensure_chain(c);
-    if (rc) return rc;
-    args.limb_base = 0;
-    args.limbs_total = (unsigned)limbs;
-    args.mid = nullptr;
-    ChainArgs ch;
-    ch.done = (unsigned*)c->d_ntt_chain;
-    ch.todo = ch.done + CHAIN_MAX_LIMBS;
-    ch.stats = ch.todo + CHAIN_MAX_LIMBS;
-    ch.limbs = (unsigned)limbs;
-    ch.kmax = ((unsigned)limbs + CHAIN_XCDS - 1) / CHAIN_XCDS;
-    ch.skew = c->chain_skew > 0 ? (unsigned)c->chain_skew : skew_env > 0 ? (unsigned)skew_env : 1u;
-    if (ch.skew > ch.kmax) ch.skew = ch.kmax;
-    // about 5 ms of polls by default, far beyond any wait of a healthy launch; 0 polls (a test setting) leaves every second-pass
-    // tile to the finishing launch
-    ch.spin_max = c->chain_spin >= 0 ? (unsigned)c->chain_spin : spin_env > 0 ? (unsigned)spin_env : 20000u;
-    ch.zero = 0;
-    ch.xcc_of = 0x76543210ull;
-    const unsigned blocks = chain_slots(ch.kmax, StridedCfg<SA, SB>::TILES, ch.skew) * CHAIN_XCDS;
-    if (!inverse) {
-        hipLaunchKernelGGL((ntt_chain_kernel<AR, SA, SB, false>), dim3(blocks), dim3(256), (size_t)lds_env, c->stream, args, ch);
-        hipLaunchKernelGGL((ntt_chain_finish_kernel<AR, SA, SB, false>), dim3((unsigned)limbs), dim3(256), 0, c->stream, args, ch);
-    } else {
-        hipLaunchKernelGGL((ntt_chain_kernel<AR, SA, SB, true>), dim3(blocks), dim3(256), (size_t)lds_env, c->stream, args, ch);
-        hipLaunchKernelGGL((ntt_chain_finish_kernel<AR, SA, SB, true>), dim3((unsigned)limbs), dim3(256), 0, c->stream, args, ch);
-    }
-    CKKS_HIP_TRY(hipGetLastError());
-    return CKKS_OK;
-}
-// tiles that second-pass workgroups of chained transforms have left to the finishing launch so far (synchronises the stream)
-int ntt_chain_deferred(ckks_ctx* c, long* tiles) {
-    *tiles = 0;
-    if (!c->d_ntt_chain) return CKKS_OK;
-    CKKS_HIP_TRY(hipStreamSynchronize(c->stream));
-    unsigned v = 0;
-    CKKS_HIP_TRY(hipMemcpy(&v, (unsigned*)c->d_ntt_chain + 2 * (size_t)CHAIN_MAX_LIMBS, sizeof(v), hipMemcpyDeviceToHost));
-    *tiles = v;
-    return CKKS_OK;
-}
-// host view of the slot order, for tests
-void ntt_chain_slot(unsigned s, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile) { chain_slot(s, tiles, skew, *second, *k, *tile); }
-unsigned ntt_chain_slots(unsigned kmax, unsigned tiles, unsigned skew) { return chain_slots(kmax, tiles, skew); }
-
-template <class AR, int SA, int SB>
-static int launch_whole_limb(ckks_ctx* c, NttArgs args, int limbs, bool inverse) {
-    static const int groups_env = getenv("CKKS_NTT_GROUPS") ? atoi(getenv("CKKS_NTT_GROUPS")) : 0;
-    args.limb_base = 0;
-    args.limbs_total = (unsigned)limbs;
-    args.mid = nullptr;
-    if (groups_env == 2) {
-        if (!inverse) hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, false, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
-        else hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, true, 2>), dim3(limbs), dim3(512), 0, c->stream, args);
-    } else {
-        if (!inverse) hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, false, 4>), dim3(limbs), dim3(1024), 0, c->stream, args);
-        else hipLaunchKernelGGL((ntt_limb_kernel<AR, SA, SB, true, 4>), dim3(limbs), dim3(1024), 0, c->stream, args);
-    }
-    CKKS_HIP_TRY(hipGetLastError());
-    return CKKS_OK;
-}
-
-// Whether a transform of `limbs` limbs runs as the paired kernel: always in modes 4 and 5 while its completion words suffice, in
-// the automatic mode up to the batch at which two launches are as fast (CKKS_NTT_PAIR_MAX overrides that limit).  Measured
+// Whether a transform of `limbs` limbs runs as the paired kernel: always in modes 4 and 5 while its protocol words suffice, in
+// the automatic mode up to the batch at which two launches are as fast and only while every workgroup of the launch fits the chip
+// at once (the protocol completes without that, but workgroups that wait for ones that cannot start yet gain nothing).  Measured
 // against two launches: with a limb's tiles on one XCD 9.5 us against 15.7 us at 16 limbs, 15 against 22.5 at 32, level at 48 and
 // behind above; with the tiles spread over the XCDs 14.4 us at 16 limbs, 20.5 against 22.5 at 48, 34.8 against 36 at 96,
 // 49.5 against 48 at 144.  Hence: one XCD per limb up to 40 limbs, spread from there to 128.
-static bool pair_applies(const ckks_ctx* c, int limbs) {
-    static const int max_env = getenv("CKKS_NTT_PAIR_MAX") ? atoi(getenv("CKKS_NTT_PAIR_MAX")) : -1;
-    if (limbs > PAIR_MAX_LIMBS || c->cu_count < 64) return false;            // the progress argument needs more than 128 resident workgroups
+// kind: which kernel would run (PAIR_KIND_*): its own occupancy decides what fits the chip
+static bool pair_applies(const ckks_ctx* c, int limbs, int kind) {
+    if (limbs > PAIR_MAX_LIMBS) return false;
     if (c->ntt_mode == 4 || c->ntt_mode == 5) return true;
-    return c->ntt_mode == 0 && limbs <= (max_env >= 0 ? max_env : PAIR_AUTO_LIMBS);
+    return c->ntt_mode == 0 && limbs <= PAIR_AUTO_LIMBS && pair_blocks(limbs, 16u) <= c->pair_resident_blocks[kind];
 }
+template <class AR> constexpr int pair_kind_of() { return std::is_same<AR, F64Arith>::value ? PAIR_KIND_F64 : std::is_same<AR, F64WideArith>::value ? PAIR_KIND_WIDE : PAIR_KIND_INT; }
 
 template <class AR>
 static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inverse, bool compact_ok, bool res36_ok = false,
@@ -705,10 +581,12 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
     // changed for it: other threads' calls on the same context see the mode they set).
     const int mode = fixed ? 1 : c->ntt_mode;
     // mode 2: both passes in one launch, the limb held in the XCD's L2 between them (N >= 2^15)
+#ifdef CKKS_NTT_EXTRA_FORMS
     if (!c->ev_mid_armed && mode == 2 && !args.embed_mlwe) {
         if (c->logN == 16) return launch_chain<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_chain<AR, 8, 7>(c, args, limbs, inverse);
     }
+#endif
     // The resident transform - one persistent workgroup per compute unit carries whole limbs through both passes in its registers
     // (N = 2^16, primes below 2^36) - takes the whole rounds of a batch (one limb per compute unit and round) and a last round that is
     // at least three quarters full; what is left goes out as two launches behind it.  Mode 6 asks for it wherever it applies, the
@@ -723,13 +601,15 @@ static int dispatch_logn(ckks_ctx* c, const NttArgs& args, int limbs, bool inver
         return launch_two_pass<AR, 8, 8>(c, args, limbs, inverse, compact_ok, whole);
     }
     // mode 4, and the automatic mode for small batches: both passes in one launch of one workgroup per (limb, tile)
-    if (!c->ev_mid_armed && !fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs)) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
+    if (!c->ev_mid_armed && !fixed && !args.embed_mlwe && c->logN == 16 && pair_applies(c, limbs, pair_kind_of<AR>())) return launch_pair<AR, 8, 8>(c, args, limbs, inverse, compact_ok);
     // mode 3: one workgroup per limb, both passes in one launch.  Measured slower than two launches at the full batch size
     // (the limbs in flight, 0.5 MiB per resident workgroup, exceed the L2 by far), so the automatic mode does not pick it.
+#ifdef CKKS_NTT_EXTRA_FORMS
     if (!c->ev_mid_armed && mode == 3) {
         if (c->logN == 16) return launch_whole_limb<AR, 8, 8>(c, args, limbs, inverse);
         if (c->logN == 15) return launch_whole_limb<AR, 8, 7>(c, args, limbs, inverse);
     }
+#endif
     switch (c->logN) {
         case 8:  return launch_two_pass<AR, 4, 4>(c, args, limbs, inverse, compact_ok, 0, fixed);
         case 9:  return launch_two_pass<AR, 5, 4>(c, args, limbs, inverse, compact_ok, 0, fixed);
@@ -1062,18 +942,18 @@ __global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
     fwd_packed<F64Arith, 8, S1>(v, twf, 1u, g, ar);
     char* mid_limb = a.mid_out + ((long)li * 2 + z) * MID_LIMB_BYTES;
     mid_store_columns<F64Arith, true>(mid_limb, tile, g, cl, v, ar);
-    // second pass of the result's forward transform, once the limb's sixteen first-pass tiles are there
-    if (!pair_hand_over(a.pair, li * 2u + z, 16u, &go)) return;
-    row_tile<F64Arith, 8, 8, false, false, true, true>(a.out + (long)z * a.out_z_stride + (long)li * N, tile, twf, ar, lds, tid, mid_limb);
+    // second pass of the result's forward transform, once the limb's sixteen first-pass tiles are there (each of them is the
+    // work above of one workgroup: nothing to take over)
+    pair_run(a.pair, li * 2u + z, tile, &go, false, [](unsigned, const TileClaim&) {},
+             [&](unsigned t, const TileClaim& out) { row_tile<F64Arith, 8, 8, false, false, true, true>(a.out + (long)z * a.out_z_stride + (long)li * N, t, twf, ar, lds, tid, mid_limb, out); });
 }
 
 // The stage-fusing launches below keep data in the 5-byte inter-pass form and compute in FP64: N = 2^16, automatic back end and
-// transform modes, every prime involved below 2^39.  CKKS_KS_SPLIT (any value) in the environment switches them off, for tuning.
+// transform modes, every prime involved below 2^39.  The context option "ks_split" switches them off, for tuning and tests.
 // How the stage-fused launches can run on primes first_prime .. first_prime + prime_count - 1: 0 not at all, 1 with the 5-byte
 // inter-pass pieces (all primes below 2^39), 2 with whole limbs between the passes and the wide FP64 arithmetic (all below 2^50).
 static int stage_fusion_form(const ckks_ctx* c, int first_prime, int prime_count) {
-    static const bool off = getenv("CKKS_KS_SPLIT") != nullptr;
-    if (off || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed) return 0;
+    if (c->ks_split || c->logN != 16 || c->arith_mode != 0 || c->ntt_mode != 0 || c->ev_mid_armed) return 0;
     if (first_prime < 0 || prime_count < 1 || first_prime + prime_count > c->nprimes) return 0;
     int form = 1;
     for (int j = first_prime; j < first_prime + prime_count; j++) {
@@ -1193,7 +1073,7 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     KsModUpArgs u;
     u.y = (const u64*)work; u.v = (signed char*)(work + (size_t)(l + 1) * N); u.mid = mid; u.blocks = c->d_conv + plan.first;
     u.primes = c->d_primes; u.tw_fwd = c->d_twd_fwd; u.ndigits = ndigits; u.p_num = P;
-    if (pair_applies(c, l + 1)) {
+    if (pair_applies(c, l + 1, PAIR_KIND_F64)) {
         // one launch: the constants that differ between the two tables (N^-1 and the last twiddle) only enter the second pass
         args.primes = c->d_primes_modup + (size_t)l * c->nprimes;
         args.out_delta = (long)((u64*)work - (u64*)in_ntt);
@@ -1213,8 +1093,10 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
     k.tw_fwd = c->d_twd_fwd; k.tw_inv = c->d_twd_inv; k.ndigits = ndigits; k.key_digit_stride = W; k.key_z_stride = (long)dnum * W;
     k.in_ntt = (const u64*)in_ntt; k.p_num = P;
     hipLaunchKernelGGL(ks_row_fused_kernel, dim3(CR::TILES, mod_num), dim3(256), 0, c->stream, k);
-    static const bool back_split = getenv("CKKS_KS_BACK_SPLIT") != nullptr;
-    if (out && finished && !back_split && c->d_ntt_pair && pair_applies(c, 2 * mod_num)) {
+    // The last launch's ModDown workgroups wait for the special-prime workgroups at the front of the same grid, which is only sound
+    // while the whole grid is resident at once; otherwise (and with the tuning switch set) the steps go out as separate launches.
+    const bool back_fits = (unsigned)(P + l + 1) * 32u <= c->pair_resident_blocks[PAIR_KIND_KS_BACK];
+    if (out && finished && !c->ks_back_split && back_fits && c->d_ntt_pair && pair_applies(c, 2 * mod_num, PAIR_KIND_KS_BACK)) {
         // last pass of the sums' inverse transform, ModDown and both passes of the results' forward transform in one launch
         KsBackArgs bk;
         bk.mid_in = k.mid_out; bk.sums = (u64*)sums; bk.z_stride = (long)W * N; bk.mid_out = mid;
@@ -1404,7 +1286,7 @@ struct RescaleArgs {
 };
 // SHARED: the two tiles are the halves of one paired launch (what the first hands to the second moves as shared accesses)
 template <class AR, class MID, bool SHARED>
-__device__ __forceinline__ void rescale_strided_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds) {
+__device__ __forceinline__ void rescale_strided_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds, const TileClaim& claim = TileClaim()) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     constexpr long N = 1l << 16;
@@ -1416,19 +1298,22 @@ __device__ __forceinline__ void rescale_strided_tile(const RescaleArgs& a, unsig
     double v[R];
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = ar.balance(exact_u2d(col[(long)(g + j * G) * N2]));      // x mod q_i, |.| <= q_i / 2
+    const unsigned claimed = claim.start(tid);
     const double* tw = a.tw_fwd + (long)prime * N;
     fwd_spread<AR, 8, S1>(v, tw, 1u, ar);
     ar.round_end(v);
 #pragma unroll
     for (int j = 0; j < R; j++) lds[(g + j * G) * CW + cl] = v[j];
+    claim.publish(tid, claimed);
     __syncthreads();
+    if (claim.lost()) return;
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = lds[(g * R + j) * CW + cl];
     fwd_packed<AR, 8, S1>(v, tw, 1u, g, ar);
     MID::template store_columns<AR, SHARED>(a.mid + (long)limb * MID::LIMB_BYTES, tile, g, cl, v, ar);
 }
 template <class AR, class MID, bool SHARED>
-__device__ __forceinline__ void rescale_row_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds) {
+__device__ __forceinline__ void rescale_row_tile(const RescaleArgs& a, unsigned limb, unsigned tile, double* lds, const TileClaim& claim = TileClaim()) {
     typedef RowCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     constexpr long N = 1l << 16;
@@ -1446,6 +1331,7 @@ __device__ __forceinline__ void rescale_row_tile(const RescaleArgs& a, unsigned 
     u64 c[R];                                            // the limb's own words, needed after the butterflies
 #pragma unroll
     for (int j = 0; j < R; j++) c[j] = rp[j * U];
+    const unsigned counted = claim.start(tid);
     double v[R];
 #pragma unroll
     for (int j = 0; j < R; j++) v[j] = MID::decode(ar, raw, j, rl);
@@ -1467,6 +1353,7 @@ __device__ __forceinline__ void rescale_row_tile(const RescaleArgs& a, unsigned 
         const double x = ar.balance(lrow[padded(u + j * U)]);
         rp[j * U] = ar.canon(ar.mulmod(exact_u2d(c[j]) - x, inv));          // |c - x| < 1.5 q
     }
+    claim.publish(tid, counted);
 }
 template <class AR, class MID>
 __global__ __launch_bounds__(256) void rescale_strided_kernel(RescaleArgs a) {
@@ -1489,9 +1376,8 @@ __global__ __launch_bounds__(256) void rescale_pair_kernel(RescaleArgs a, PairAr
     unsigned limb, tile;
     pair_block(p, blockIdx.x, TILES, limb, tile);
     if (limb >= p.limbs) return;
-    rescale_strided_tile<AR, MID, true>(a, limb, tile, lds);
-    if (!pair_hand_over(p, limb, TILES, &go)) return;
-    rescale_row_tile<AR, MID, true>(a, limb, tile, lds);
+    pair_run(p, limb, tile, &go, true, [&](unsigned t, const TileClaim& claim) { rescale_strided_tile<AR, MID, true>(a, limb, t, lds, claim); },
+             [&](unsigned t, const TileClaim& out) { rescale_row_tile<AR, MID, true>(a, limb, t, lds, out); });
 }
 // cipher: [2][poly_mod_len] limbs over q_0 .. (prime indices K + i); limb l already in the coefficient domain.
 // *done = false (nothing launched) where it does not apply.
@@ -1507,7 +1393,7 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
     r.cipher = (u64*)cipher; r.mid = (char*)c->d_ntt_mid; r.primes = c->d_primes; r.tw_fwd = c->d_twd_fwd; r.inv = (const u64*)inv;
     r.l = l; r.poly_mod_len = c->L + 1; r.prime0 = c->K;
     const dim3 gs(limbs, StridedCfg<8, 8>::TILES), gr(RowCfg<8, 8>::TILES, limbs);
-    if (pair_applies(c, limbs) && c->d_ntt_pair) {
+    if (pair_applies(c, limbs, form == 1 ? PAIR_KIND_RESCALE : PAIR_KIND_RESCALE_WIDE) && c->d_ntt_pair) {
         const PairArgs p = pair_args(c, limbs);
         const dim3 gp(pair_blocks(limbs, StridedCfg<8, 8>::TILES));
         if (form == 1) hipLaunchKernelGGL((rescale_pair_kernel<F64Arith, MidPieces>), gp, dim3(256), 0, c->stream, r, p);
@@ -1558,6 +1444,29 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
     return CKKS_OK;
+}
+
+// Workgroups of each one-launch kernel that the chip holds at once: its occupancy times the compute units.
+static void pair_resident_blocks(ckks_ctx* c) {
+    const unsigned cus = (unsigned)(c->cu_count > 0 ? c->cu_count : 1);
+    auto ask = [&](int kind, auto kernel) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess) { (void)hipGetLastError(); n = 1; }
+        if (n < 1) n = 1;
+        const unsigned blocks = (unsigned)n * cus;
+        if (c->pair_resident_blocks[kind] == 0 || blocks < c->pair_resident_blocks[kind]) c->pair_resident_blocks[kind] = blocks;
+    };
+    ask(PAIR_KIND_F64, ntt_pair_kernel<F64Arith, 8, 8, false, true>);
+    ask(PAIR_KIND_F64, ntt_pair_kernel<F64Arith, 8, 8, true, true>);
+    ask(PAIR_KIND_F64, ntt_pair_kernel<F64Arith, 8, 8, false, false>);
+    ask(PAIR_KIND_F64, ntt_pair_kernel<F64Arith, 8, 8, true, false>);
+    ask(PAIR_KIND_WIDE, ntt_pair_kernel<F64WideArith, 8, 8, false, false>);
+    ask(PAIR_KIND_WIDE, ntt_pair_kernel<F64WideArith, 8, 8, true, false>);
+    ask(PAIR_KIND_INT, ntt_pair_kernel<IntArith, 8, 8, false, false>);
+    ask(PAIR_KIND_INT, ntt_pair_kernel<IntArith, 8, 8, true, false>);
+    ask(PAIR_KIND_RESCALE, rescale_pair_kernel<F64Arith, MidPieces>);
+    ask(PAIR_KIND_RESCALE_WIDE, rescale_pair_kernel<F64WideArith, MidLimb>);
+    ask(PAIR_KIND_KS_BACK, ks_back_kernel);
 }
 
 static int launch_ntt_from(ckks_ctx* c, uint64_t* dev, int start_poly_idx, int start_mod_idx, int poly_num, int mod_num,

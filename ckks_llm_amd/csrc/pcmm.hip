@@ -348,7 +348,7 @@ extern "C" int pcmm_rlwe_decompose(pcmm_ctx* h, const uint64_t* rlwe, uint64_t* 
     a.rlwe = rlwe; a.mlwe = h->d_ptrs; a.primes = c->d_primes; a.N = c->N; a.N1 = h->N1; a.rank = h->rank; a.mlwe_num = mlwe_num;
     a.L = c->L; a.p_num = c->p_num;
     const int k = h->rank;
-    const bool force_plain = getenv("CKKS_GATHER_PLAIN") != nullptr;              // test hook: the one-lane-per-word kernel
+    const bool force_plain = h->gather_plain;                                     // test hook: the one-lane-per-word kernel
     // 16-word row segments (one 128-byte line) when the window fits the LDS a workgroup may ask for, else 8-word segments
     static const bool big_lds = hipFuncSetAttribute(reinterpret_cast<const void*>(rlwe_gather_tiled_kernel<16>),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess;
@@ -763,7 +763,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     // the bytes of x + 0x80..80 must not carry into byte d.  DW digits must hold +-|A|max, DC digits every residue 0 .. qmax - 1.
     auto top = [](int d) { unsigned long long v = 0; for (int i = 0; i < d; i++) v = (v << 8) | 0x7f; return v; };
     int DC = 1; while (DC < 8 && qmax - 1 > top(DC)) DC++;
-    static const bool force_generic = getenv("CKKS_PPMM_GENERIC") != nullptr;     // test hook: exercise the generic kernel
+    const bool force_generic = h->ppmm_generic;                                   // test hook: exercise the generic kernel
     // what the matrix of a given |A|max runs on.  Residues in 5 digits (q < 2^39) with up to 4 plaintext digits, or in 7 digits
     // (q < 2^50) with up to 3; wider plaintext matrices (any int64) go through the same kernels in slices of three digits.
     struct Plan { int DW, slices, planes; bool mfma; };
@@ -850,7 +850,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
     PpmmArgs a;
     a.A = we->d_A; a.Adig = we->d_Adig; a.mlwe = (const u64* const*)h->d_ptrs; a.mlwe_base = nullptr;
     a.mlwe_stride = (long)mod_num * C; a.out = out; a.pq = h->d_pq; a.consts = d_cst; a.C = C; a.M = M; a.Kin = Kin;
-    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np; a.raw_all = 0;
+    a.Mpad = Mpad; a.Kpad = Kpad; a.mod_num = mod_num; a.np = h->np; a.raw_all = 0; a.no_tail = h->ppmm_no_tail ? 1 : 0;
     if (packed && !mfma_ok) { set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
     h->last_path = mfma_ok ? 1 : 0; h->last_DW = DW; h->last_DC = DC; h->last_absmax = absmax; h->last_slices = mfma_ok ? slices : 0;
     if (mfma_ok) {
@@ -907,6 +907,16 @@ extern "C" int pcmm_info(const pcmm_ctx* h, const char* name, long* value) {
     else if (n == "last_slices") *value = h->last_slices;
     else if (n == "last_absmax") *value = (long)h->last_absmax; else if (n == "N1") *value = h->N1; else if (n == "mlwe_rank") *value = h->rank;
     else { set_error("pcmm_info: unknown name " + n); return CKKS_E_INVALID; }
+    return CKKS_OK;
+}
+// test / tuning switches of a ring-pack handle, by name (value 0: off, anything else: on)
+extern "C" int pcmm_set_option(pcmm_ctx* h, const char* name, long value) {
+    if (!h || !name) return CKKS_E_INVALID;
+    const std::string n(name);
+    if (n == "gather_plain") h->gather_plain = value != 0;          // rlweCipherDecompose with the one-lane-per-word gather
+    else if (n == "ppmm_generic") h->ppmm_generic = value != 0;     // PPMM on the generic 128-bit kernel instead of the MFMA one
+    else if (n == "ppmm_no_tail") h->ppmm_no_tail = value != 0;     // PPMM runs the remainder column panels whole instead of as jobs by prime
+    else { set_error("pcmm_set_option: unknown name " + n); return CKKS_E_INVALID; }
     return CKKS_OK;
 }
 extern "C" int pcmm_set_weight_cache(pcmm_ctx* h, int enabled) {

@@ -42,6 +42,7 @@ struct pcmm_ctx {
     };
     std::vector<Weights> weights;
     bool weights_cached = false;
+    bool gather_plain = false, ppmm_generic = false, ppmm_no_tail = false;      // test / tuning switches (pcmm_set_option)
     std::vector<std::pair<uintptr_t, size_t>> static_ranges;    // device address ranges whose matrices the caller has declared static
     // work space of the calls that keep nothing: the quantised matrix and its digit planes of the call in flight
     long long* d_workA = nullptr;
@@ -83,6 +84,7 @@ struct PpmmArgs {
     long C;
     int M, Kin, Mpad, Kpad, mod_num, np;
     int raw_all;                  // MFMA kernel: store every modulus' residue as it is (no fused rescale); the caller combines slices
+    int no_tail = 0;              // MFMA kernel: run the remainder column panels whole instead of as jobs by prime (tuning switch)
 };
 
 size_t ppmm_bdig_bytes(const PpmmArgs& a, int DC);

@@ -462,7 +462,7 @@ static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool p
     unsigned blocks = (unsigned)((c_tiles + 7) / 8) * 8u * (unsigned)m_tiles;
     // The column panels beyond the last full group of eight (one per XCD) are cut into jobs by prime where that pays: a single patch
     // of row tiles (small M), enough primes to share, and the fused rescale (a job needs the last prime only then).
-    static const bool no_tail = getenv("CKKS_PPMM_NO_TAIL") != nullptr;        // test / tuning hook
+    const bool no_tail = a.no_tail != 0;                                       // test / tuning switch
     int main_blocks = (int)blocks, tail_jobs = 0;
     const int rest = c_tiles % 8;
     if (!no_tail && rest != 0 && c_tiles >= 8 && m_block == m_tiles && a.mod_num >= 8 && !a.raw_all) {

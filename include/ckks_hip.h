@@ -59,6 +59,11 @@ int ckks_ctx_create(ckks_ctx** out, int logN, const uint64_t* p, int p_num, cons
 int ckks_ctx_destroy(ckks_ctx* ctx);
 int ckks_set_stream(ckks_ctx* ctx, void* hip_stream);
 /* scalar facts: "N","logN","p_num","q_num","t_num","gamma","dnum","Ri_blockNum","Qj_blockNum","arith_mode","ntt_mode";
+ * "ntt_mid_bytes": size of the inter-pass buffer that the ordinary transforms have grown so far;
+ * "ntt_pair_deferred_tiles" (synchronises): second-pass tiles that paired transforms have left to the last workgroup of their limb;
+ * "ntt_pair_resident_blocks" / "ntt_pair_resident_blocks_int": workgroups of the paired transform kernel (FP64 / integer back end) that the chip
+ * holds at once; "ntt_pair_stolen_tiles" (synchronises): first-pass tiles taken over from workgroups that had not started; "ntt_extra_forms": 1 if
+ * modes 2 and 3 are built in;
  * "ntt_chain_deferred_tiles" (synchronises): second-pass tiles that chained transforms have left to their finishing launch;
  * "ntt_resident_round": limbs that one round of the resident transform takes (one per compute unit; 0 where it never applies) */
 int ckks_ctx_info(const ckks_ctx* ctx, const char* name, long* value);
@@ -73,8 +78,11 @@ int ckks_ctx_set_arith_mode(ckks_ctx* ctx, int mode);
  * takes this form for batches of up to 128 limbs, where it is faster than two launches); 5: as 4 with the tiles of a limb spread
  * over all XCDs (what mode 0 does above 40 limbs); 6: resident - one persistent workgroup per compute unit carries whole limbs
  * through both passes in its registers, so that a limb crosses HBM once in and once out (N = 2^16, primes below 2^36, at least one
- * limb per compute unit; mode 0 takes it there too, for the whole rounds of a batch).  All give the same residues.  Should a wait of the paired form ever run out (about two
- * seconds), the transform's output is incomplete, ckks_ctx_check and every later transform of the context return CKKS_E_UNAVAILABLE.
+ * limb per compute unit; mode 0 takes it there too, for the whole rounds of a batch).  All give the same residues.  Modes 2 and 3
+ * exist only in a library built with CKKS_NTT_EXTRA_FORMS (they lose to two launches at every size; the default build leaves
+ * them out and runs two launches where they are asked for).  The paired form completes whatever part of its grid the chip holds
+ * at once and in whatever order its workgroups start: a workgroup that waits too long takes over the tiles of workgroups that have
+ * not started, and what it leaves undone the last workgroup of the limb completes.
  * No counterpart in the reference (its transforms are always two launches, Context_23.cuh:847-889). */
 int ckks_ctx_set_ntt_mode(ckks_ctx* ctx, int mode);
 /* Synchronises the context's stream and returns what HIP reports for the launches so far.  Plays the part of the reference's
@@ -83,8 +91,19 @@ int ckks_ctx_check(ckks_ctx* ctx);
 /* Test / tuning hook of the chained transform (mode 2).  skew: limbs that a chain's first pass runs ahead of its second pass
  * (0 = default); spin_max: polls that a second-pass workgroup spends waiting for its limb's first pass before it leaves its tile
  * to the finishing launch (-1 = default; 0 sends every tile there).  Results do not depend on either.  spin_max also bounds
- * the wait of the paired transform (modes 0, 4, 5), which has no finishing launch: there a wait that runs out is an error. */
+ * the waits of the paired transform (modes 0, 4, 5): 0 makes every workgroup take over what it can at once and leave its second
+ * pass to the last workgroup of its limb ("ntt_pair_deferred_tiles" of ckks_ctx_info counts those), with the same results.
+ * The one wait that can still fail is in the last launch of the fused hybrid key switch (its ModDown workgroups wait for the
+ * special-prime workgroups of the same grid, which the launcher only uses while the whole grid fits the chip): should it run
+ * out, ckks_ctx_check and every later call on the context return CKKS_E_UNAVAILABLE. */
 int ckks_ctx_set_ntt_chain(ckks_ctx* ctx, int skew, int spin_max);
+/* Test / tuning switches of a context, by name (value 0 = off, the default).  Results do not depend on any of them.
+ *   "ks_split"        the hybrid key switch, the rescale and the ring packing run their stages as separate launches
+ *   "ks_back_split"   the hybrid key switch runs its last three steps as separate launches
+ *   "conv_int"        basis conversions into primes below 2^50 accumulate in 128-bit integers instead of FP64
+ *   "ntt_no_reverse"  the second launch of a two-launch transform takes the limbs in forward order
+ *   "ntt_chunk"       value = limbs per trip through the inter-pass buffer of a two-launch transform (0: the whole batch) */
+int ckks_ctx_set_option(ckks_ctx* ctx, const char* name, long value);
 /* Order of work of the chained transform, for tests: slot `slot` of a chain of `tiles` workgroups per pass -> pass (0 / 1),
  * index k of the limb within the chain and tile; ckks_ntt_chain_slots = slots of a chain of kmax limbs.  Pure host functions. */
 int ckks_ntt_chain_slot(unsigned slot, unsigned tiles, unsigned skew, unsigned* second, unsigned* k, unsigned* tile);
@@ -354,6 +373,10 @@ int pcmm_ppmm_strided(pcmm_ctx* h, const float* W_dev, const uint64_t* mlwe_dev,
  * pcmm_weights_static(.., 0) and pcmm_set_weight_cache(h, 0) take the promise back and drop what was kept under it. */
 int pcmm_weights_static(pcmm_ctx* h, const float* W_dev, size_t bytes, int is_static);
 int pcmm_set_weight_cache(pcmm_ctx* h, int enabled);
+/* Test / tuning switches of a ring-pack handle, by name (value 0 = off, the default; results do not depend on them):
+ * "gather_plain" (rlweCipherDecompose with the one-lane-per-word gather), "ppmm_generic" (PPMM on the generic 128-bit kernel),
+ * "ppmm_no_tail" (PPMM runs the remainder column panels whole instead of as jobs by prime). */
+int pcmm_set_option(pcmm_ctx* h, const char* name, long value);
 int pcmm_weights_changed(pcmm_ctx* h, const float* W_dev);
 
 /* ---- the gather writing PPMM's operand directly.  No counterpart in the reference, where rlweCipherDecompose materialises every

@@ -32,6 +32,13 @@ def check_fwd_inv(pair, primes_idx0, primes, poly_num, seed, mode=None):
     buf.free()
 
 
+
+def needs_extra_forms(dev):
+    """Launch forms 2 (chained) and 3 (one workgroup per limb) exist only in a library built with EXTRA_FORMS=1."""
+    if not dev.info("ntt_extra_forms"):
+        pytest.skip("library built without the extra launch forms (make EXTRA_FORMS=1)")
+
+
 def test_config1_n4096_4primes_batch16():
     """BASELINE config 1: N = 2^12, 4 primes < 2^36, batch of 16 polynomials, seed 1."""
     pair = Pair(12, [], CFG1_Q)
@@ -172,6 +179,7 @@ def test_one_launch_transform_matches_two_launch_and_oracle(logN, polys, mode):
     q = CFG2_Q[:5]
     pair = Pair(logN, [], q)
     N, L1 = pair.N, len(q)
+    needs_extra_forms(pair.dev)
     pair.dev.set_arith_mode(mode)
     data = limbs_uniform(40 + logN, q, polys, N)
     want = data.copy()
@@ -205,6 +213,7 @@ def test_whole_limb_transform_matches_oracle(logN, polys, mode):
     q = CFG2_Q[:5]
     pair = Pair(logN, [], q)
     N, L1 = pair.N, len(q)
+    needs_extra_forms(pair.dev)
     pair.dev.set_arith_mode(mode)
     data = limbs_uniform(40 + logN, q, polys, N)
     want = data.copy()
@@ -294,29 +303,58 @@ def test_paired_transform_matches_oracle(primes, polys, arith, mode):
     buf.free()
 
 
-def test_paired_transform_reports_a_wait_that_ran_out():
-    """With a poll limit of zero no second-pass tile of the paired transform may start unless its limb is already complete at the
-    first look; every workgroup still ends normally, the context's failure word is raised, check() and every later transform of
-    the context report it.  Another context is not affected."""
-    from ckks_llm_amd import CkksError
+@pytest.mark.parametrize("mode,arith,polys", [(4, 0, 2), (5, 0, 3), (4, 1, 2), (0, 0, 6)])
+def test_paired_transform_completes_when_every_wait_runs_out(mode, arith, polys):
+    """With a poll limit of zero a workgroup of the paired transform never waits: it takes over whatever first-pass tiles nobody
+    has claimed and, unless its limb is complete at the first look, leaves its second-pass tiles to the last workgroup of the limb
+    to leave.  The transform must still come out right, in place and through the 5-byte form, on both back ends, again and again
+    on the same protocol words, and the context stays usable; the counter of left-over tiles says that the path was taken."""
     q = CFG2_Q[:3]
     pair = Pair(16, [], q)
-    data = limbs_uniform(5, q, 2, pair.N)
-    buf = to_dev(data)
-    pair.dev.set_ntt_mode(4)
-    pair.dev.set_ntt_chain(0, 0)
-    pair.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
-    with pytest.raises(CkksError):
-        pair.dev.check()
-    with pytest.raises(CkksError):
-        pair.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
-    other = Pair(16, [], q)
+    pair.dev.set_arith_mode(arith)
+    data = limbs_uniform(5, q, polys, pair.N)
     want = data.copy()
-    other.orc.ToNTTInplace(want.reshape(-1), 0, 0, 2, 3, 3)
-    buf.upload(data)
-    other.dev.ToNTTInplace(buf, 0, 0, 2, 3, 3)
-    other.dev.check()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, 3, 3)
+    buf = to_dev(data)
+    pair.dev.set_ntt_mode(mode)
+    pair.dev.set_ntt_chain(0, 0)
+    before = pair.dev.info("ntt_pair_deferred_tiles")
+    for rep in range(3):
+        pair.dev.ToNTTInplace(buf, 0, 0, polys, 3, 3)
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), want), rep
+        pair.dev.FromNTTInplace(buf, 0, 0, polys, 3, 3)
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), data), rep
+    assert pair.dev.info("ntt_pair_deferred_tiles") > before
+    # back to the default limits: same words, nothing left over from the forced runs
+    pair.dev.set_ntt_chain(0, -1)
+    pair.dev.ToNTTInplace(buf, 0, 0, polys, 3, 3)
+    pair.dev.check()
     assert np.array_equal(from_dev(buf, data.shape), want)
+    buf.free()
+
+
+def test_paired_transform_larger_than_the_chip_holds():
+    """A paired launch with several times more workgroups than fit the chip at once (mode 4 forces the form at any size): the
+    protocol does not need the workgroups of a limb to be resident together."""
+    q = CFG2_Q[:6]
+    pair = Pair(16, [], q)
+    polys = 2 * (pair.dev.info("ntt_pair_resident_blocks") // 16) // len(q) + 3
+    assert 16 * polys * len(q) > pair.dev.info("ntt_pair_resident_blocks")
+    data = limbs_uniform(17, q, polys, pair.N)
+    want = data.copy()
+    pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, polys, len(q), len(q))
+    buf = to_dev(data)
+    for mode in (4, 5):
+        pair.dev.set_ntt_mode(mode)
+        buf.upload(data)
+        pair.dev.ToNTTInplace(buf, 0, 0, polys, len(q), len(q))
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), want), mode
+        pair.dev.FromNTTInplace(buf, 0, 0, polys, len(q), len(q))
+        pair.dev.check()
+        assert np.array_equal(from_dev(buf, data.shape), data), mode
     buf.free()
 
 
@@ -370,6 +408,7 @@ def test_chained_transform_finishing_launch_and_skews(skew, spin):
     data = limbs_uniform(77, q, 1, N)
     want = data.copy()
     pair.orc.ToNTTInplace(want.reshape(-1), 0, 0, 1, L1, L1)
+    needs_extra_forms(pair.dev)
     pair.dev.set_ntt_mode(2)
     pair.dev.set_ntt_chain(skew, spin)
     buf = to_dev(data)
@@ -449,8 +488,8 @@ def test_full_size_properties_batch32():
     pair.dev.FromNTTInplace(d, 0, 0, 2 * B, L1, L1)
     pair.dev.check()
     assert np.array_equal(from_dev(d, data.shape), data)
-    # the two-launch path and the whole-limb path give the same residues on the whole batch
-    for m in (1, 2, 3):
+    # the other launch forms give the same residues on the whole batch (the paired form far beyond what the chip holds at once)
+    for m in (1, 4, 5) + ((2, 3) if pair.dev.info("ntt_extra_forms") else ()):
         pair.dev.set_ntt_mode(m)
         pair.dev.ToNTTInplace(d, 0, 0, 2 * B, L1, L1)
         assert np.array_equal(from_dev(d, data.shape), got), m

@@ -24,13 +24,13 @@ def make(logN, N1, q_ctx, p_ctx, p_rp, q_rp):
 @pytest.mark.parametrize("plain", [False, True])
 @pytest.mark.parametrize("logN,N1,mlwe_num", [(10, 128, 8), (10, 128, 2), (12, 256, 16), (10, 64, 1), (14, 32, 512), (14, 32, 64),
                                               (12, 8, 512), (10, 4, 256)])
-def test_rlwe_decompose(logN, N1, mlwe_num, plain, monkeypatch):
+def test_rlwe_decompose(logN, N1, mlwe_num, plain):
     """Both gather kernels (LDS-tiled with 16- or 8-word row segments, and one lane per word - forced through the launcher's
     test hook, and taken anyway when N1 is not a multiple of 8) against the oracle."""
-    if plain:
-        monkeypatch.setenv("CKKS_GATHER_PLAIN", "1")
     q = CFG2_Q[:3]
     pair, dev, orc, rank = make(logN, N1, q, CFG3_P[:1], [CFG3_P[0]], q[:2])
+    if plain:
+        dev.pcmm_context.set_option("gather_plain")
     N, L = pair.N, len(q) - 1
     for l in (L, 0):
         rlwe = limbs_uniform(l + 1, q, 2, N)                                  # [2][L+1][N], coefficient domain
