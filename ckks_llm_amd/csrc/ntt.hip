@@ -52,15 +52,20 @@ struct TileClaim {
     unsigned* words = nullptr;     // the limb's protocol words
     unsigned tile = 0;
     bool counting_out = false;     // false: the claim of a first-pass tile; true: the counting out, inside a second-pass tile
+    // start() only issues the atomic and returns what it will bring, untouched: anything computed from it here would make the
+    // wave wait for it at this point; publish() is where it is first looked at
     __device__ __forceinline__ unsigned start(unsigned tid) const {
-        unsigned v = tile;
+        unsigned v = 0;
         if (lds && tid == 0) {
             asm volatile("" ::: "memory");
-            v = counting_out ? pair::leave(words) : pair::claim_own(words, tile, true);
+            v = counting_out ? pair::Atomics::fetch_add(words + pair::LEFT, 1u) : pair::Atomics::fetch_or(words + pair::CLAIM, 1u << tile);
         }
         return v;
     }
-    __device__ __forceinline__ void publish(unsigned tid, unsigned value) const { if (lds && tid == 0) *lds = value; }
+    // claim: the tile, or LEAVE if it was taken; counting out: how many had left before (the last one out sees TILES - 1)
+    __device__ __forceinline__ void publish(unsigned tid, unsigned raw) const {
+        if (lds && tid == 0) *lds = counting_out ? raw : ((raw >> tile) & 1u ? pair::LEAVE : tile);
+    }
     __device__ __forceinline__ bool lost() const { return lds && !counting_out && *lds == pair::LEAVE; }
 };
 
@@ -368,7 +373,7 @@ __device__ __forceinline__ void pair_run(const PairArgs& p, unsigned limb_id, un
     out.counting_out = true;
     if (todo == 0u && threadIdx.x == 0) {
         if (act == pair::DEFER) pair::defer(w, mine);
-        *sh = pair::leave(w);
+        *sh = pair::Atomics::fetch_add(w + pair::LEFT, 1u);
     }
     for (bool first = true; todo; first = false) {
         const unsigned t = (unsigned)__builtin_ctz(todo);
@@ -378,10 +383,13 @@ __device__ __forceinline__ void pair_run(const PairArgs& p, unsigned limb_id, un
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);                                         // lgkmcnt(0) only: the LDS write above, not the tile's last stores
     __syncthreads();
-    unsigned last = *sh;
-    if (!(last & 0x80000000u)) return;
+    if (*sh + 1u != pair::TILES) return;                                        // how many had counted out before this workgroup
     // last out: every first-pass tile of the limb is complete; what the others left undone, then the words back to zero
-    const unsigned finished = last & pair::ALL;
+    __syncthreads();
+    if (threadIdx.x == 0) *sh = pair::Atomics::load(w + pair::TODO) & pair::ALL;
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __syncthreads();
+    const unsigned finished = *sh;
     todo = finished;
     while (todo) {
         const unsigned t = (unsigned)__builtin_ctz(todo);
@@ -392,7 +400,7 @@ __device__ __forceinline__ void pair_run(const PairArgs& p, unsigned limb_id, un
     if (threadIdx.x == 0) pair::reset(w, finished);
 }
 template <class AR, int SA, int SB, bool INVERSE, bool COMPACT>
-__global__ __launch_bounds__(256) void ntt_pair_kernel(NttArgs a, PairArgs p) {
+__global__ __launch_bounds__(256, 4) void ntt_pair_kernel(NttArgs a, PairArgs p) {
     typedef StridedCfg<SA, SB> CS;
     typedef RowCfg<SA, SB> CR;
     static_assert(CS::THREADS == 256 && CR::THREADS == 256 && CS::TILES == CR::TILES && CS::TILES == 16, "paired kernel: tile shapes");
@@ -844,7 +852,7 @@ struct KsBackArgs {
     unsigned* count;             // [2 * 16] pairs (done, seen), one pair per 128-byte line; zero between launches
     int K, nq;
 };
-__global__ __launch_bounds__(256) void ks_back_kernel(KsBackArgs a) {
+__global__ __launch_bounds__(256, 4) void ks_back_kernel(KsBackArgs a) {
     typedef StridedCfg<8, 8> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, G = C::G, CW = C::CW;
     constexpr long N = 1l << 16;
@@ -1367,7 +1375,7 @@ __global__ __launch_bounds__(256) void rescale_row_kernel(RescaleArgs a) {
 }
 // both in one launch, paired like ntt_pair_kernel
 template <class AR, class MID>
-__global__ __launch_bounds__(256) void rescale_pair_kernel(RescaleArgs a, PairArgs p) {
+__global__ __launch_bounds__(256, 4) void rescale_pair_kernel(RescaleArgs a, PairArgs p) {
     constexpr int LDS_WORDS = StridedCfg<8, 8>::LDS_WORDS > RowCfg<8, 8>::LDS_WORDS ? StridedCfg<8, 8>::LDS_WORDS : RowCfg<8, 8>::LDS_WORDS;
     constexpr unsigned TILES = StridedCfg<8, 8>::TILES;
     static_assert(TILES == RowCfg<8, 8>::TILES, "tile counts");
