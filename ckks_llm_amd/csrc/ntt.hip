@@ -914,32 +914,38 @@ __global__ __launch_bounds__(256, 4) void ks_back_kernel(KsBackArgs a) {
     if (!go) return;
     // ModDown (BasisConv.cuh:257-326) on the scaled special-prime coefficients, as in ks_moddown_strided_kernel with pre_scaled
     const u64* col = a.sums + (long)z * a.z_stride + tile * CW + cl;
+    // The sum starts from minus the limb's own coefficient (the ModDown is (own - sum) P^-1 mod q): the sixteen coefficients need
+    // no registers of their own from here on, which is what lets four of these workgroups share a compute unit.
     double acc[R];
 #pragma unroll
-    for (int j = 0; j < R; j++) acc[j] = 0.0;
-    u64 x[R], xn[R];
+    for (int j = 0; j < R; j++) acc[j] = -exact_u2d(own[j]);
+    // half a limb ahead: the loads of one half of the rows are in flight while the other half is multiplied
+    u64 xa[R / 2], xb[R / 2];
 #pragma unroll
-    for (int j = 0; j < R; j++) x[j] = get<true>(col + (long)(g + j * G) * N2);
+    for (int j = 0; j < R / 2; j++) xa[j] = get<true>(col + (long)(g + j * G) * N2);
     for (int i = 0; i < a.K; i++) {
         const double hat = exact_u2d(a.pHatVecModq[(long)li * a.K + i]);
-        if (i + 1 < a.K) {
-            const u64* nl = col + (long)(i + 1) * N;
+        const u64* cur = col + (long)i * N;
 #pragma unroll
-            for (int j = 0; j < R; j++) xn[j] = get<true>(nl + (long)(g + j * G) * N2);
-        }
+        for (int j = 0; j < R / 2; j++) xb[j] = get<true>(cur + (long)(g + (j + R / 2) * G) * N2);
 #pragma unroll
-        for (int j = 0; j < R; j++) {
-            if (a.K == 1) acc[j] = exact_u2d(x[j]);                                                  // BasisConv.cuh:274
-            else acc[j] += ar.mulmod(exact_u2d(x[j]), hat);
+        for (int j = 0; j < R / 2; j++) {
+            if (a.K == 1) acc[j] += exact_u2d(xa[j]);                                                // BasisConv.cuh:274
+            else acc[j] += ar.mulmod(exact_u2d(xa[j]), hat);
         }
         if (i + 1 < a.K) {
 #pragma unroll
-            for (int j = 0; j < R; j++) x[j] = xn[j];
+            for (int j = 0; j < R / 2; j++) xa[j] = get<true>(cur + N + (long)(g + j * G) * N2);
+        }
+#pragma unroll
+        for (int j = 0; j < R / 2; j++) {
+            if (a.K == 1) acc[j + R / 2] += exact_u2d(xb[j]);
+            else acc[j + R / 2] += ar.mulmod(exact_u2d(xb[j]), hat);
         }
     }
     const double pinv = exact_u2d(a.PinvModq[li]);
 #pragma unroll
-    for (int j = 0; j < R; j++) v[j] = ar.mulmod(ar.q - canon_f(ar, acc[j]) + exact_u2d(own[j]), pinv);      // in (-0.51 q, 0.51 q)
+    for (int j = 0; j < R; j++) v[j] = ar.mulmod(ar.q - canon_f(ar, acc[j]), pinv);      // (own - sum) P^-1, in (-0.51 q, 0.51 q)
     const double* twf = a.tw_fwd + (long)prime * N;
     fwd_spread<F64Arith, 8, S1>(v, twf, 1u, ar);
 #pragma unroll

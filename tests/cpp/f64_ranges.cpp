@@ -305,6 +305,7 @@ int f64r_conv_split(int nsrc, int ntgt, const uint64_t* d, const uint64_t* r, co
 // p_i (which may exceed q), own [count] residues modulo q.
 int f64r_moddown(int wide, uint64_t q, int K, const uint64_t* x, const uint64_t* phat, uint64_t pinv, const uint64_t* own, uint64_t* out, long count) {
     const PrimeConst pc = prime_const(q, 1, 1);
+    bool failed = false;
     auto run = [&](const auto& ar) {
         for (long n = 0; n < count; n++) {
             double acc = 0.0;
@@ -317,11 +318,21 @@ int f64r_moddown(int wide, uint64_t q, int K, const uint64_t* x, const uint64_t*
             range::value(t, "moddown: own - sum");
             const double v = ar.mulmod(t, wide ? balanced_double(pinv, q) : exact_u2d(pinv));
             out[n] = wide ? F64WideArith(pc).canon_wide(v) : ar.canon_any(v);
+            // the form of the key switch's last launch: the sum starts from minus the own coefficient
+            double acc2 = -exact_u2d(own[n]);
+            for (int i = 0; i < K; i++) {
+                if (K == 1) acc2 += exact_u2d(x[n]);
+                else acc2 += ar.mulmod(exact_u2d(x[(long)i * count + n]), wide ? balanced_double(phat[i], q) : exact_u2d(phat[i]));
+                range::value(acc2, "moddown: running sum from -own");
+            }
+            const double v2 = ar.mulmod(ar.q - canon_f64(acc2, ar.q, ar.qinv), wide ? balanced_double(pinv, q) : exact_u2d(pinv));
+            const uint64_t out2 = wide ? F64WideArith(pc).canon_wide(v2) : ar.canon_any(v2);
+            if (out2 != out[n]) { failed = true; return; }
         }
     };
     if (wide) run(F64WideArith(pc));
     else run(F64Arith(pc));
-    return 0;
+    return failed ? 2 : 0;
 }
 
 // Recombination of the digit-plane PPMM: S [count][ND] anti-diagonal sums, r_last [count] residues of the last prime (ignored when
