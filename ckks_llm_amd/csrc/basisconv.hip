@@ -432,8 +432,12 @@ extern "C" int ckks_keyswitch_23(ckks_ctx* c, uint64_t* out, uint64_t* d2, const
     if ((rc = launch_ntt(c, d2, 0, K, 1, l + 1, L + 1, 0, 1, true))) return rc;                     // :219
     if ((rc = ckks_modup_qj_to_t(c, up, d2, l, 1))) return rc;                                      // :221
     if ((rc = launch_ntt(c, up, 0, K + L + 1, cipher_blockNum, T, T, 0, 1, false))) return rc;      // :223
-    if ((rc = ckks_external_product_t(c, ext, up, swk, l))) return rc;                              // :225
-    if ((rc = launch_ntt(c, ext, 0, K + L + 1, swk_blockNum, T, T, (long)RB * T, 2, true))) return rc;   // :226
+    bool ext_fused = false;
+    if ((rc = launch_ext_product_inverse_fused(c, ext, up, swk, l, &ext_fused))) return rc;       // :225 and :226 in two launches
+    if (!ext_fused) {
+        if ((rc = ckks_external_product_t(c, ext, up, swk, l))) return rc;                          // :225
+        if ((rc = launch_ntt(c, ext, 0, K + L + 1, swk_blockNum, T, T, (long)RB * T, 2, true))) return rc;   // :226
+    }
     if ((rc = ckks_modup_t_to_pql(c, buf, ext, l, 2))) return rc;                                   // :228
     bool fused = false;
     if ((rc = launch_ks_moddown_fused(c, out, buf, (long)RB * T * c->N, l, L + 1, false, &fused))) return rc;  // :229 and :231 in two launches

@@ -164,6 +164,10 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
 // pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
                             bool* done);
+// Key switch through the T basis: external product of the digits `up` (NTT domain over T) with the key `swk` and inverse transform
+// of the sums into `ext` (coefficient domain on return), the product and the first pass of the transform in one launch;
+// *done = false where it does not apply (nothing launched: the caller runs the separate steps).
+int launch_ext_product_inverse_fused(ckks_ctx* c, uint64_t* ext, const uint64_t* up, const uint64_t* swk, int l, bool* done);
 // Forward transform whose first pass reads its input from MLWE samples (the embedding of the ring packing) instead of dev:
 // coefficient pos of polynomial y = coefficient pos >> logk of row y of sample (pos mod 2^logk) >> loggap, zero where pos mod 2^logk
 // is no multiple of 2^loggap; on the limbs of prime start_mod_idx the value is lifted around zero from q0 to p0.

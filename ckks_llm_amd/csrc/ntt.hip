@@ -747,6 +747,92 @@ __global__ __launch_bounds__(256, 2) void ks_row_fused_kernel(KsRowArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// Key switch through the T basis (KeySwitch_23.cuh:225-226): the external product with the key (external_product_T,
+// ExternalProduct.cuh:56-83: out[z][o] = sum over the digits d of c[d][o mod T] * key[z][d][o], 128-bit sums, one reduction) and
+// the row pass of the inverse transform of every sum in one launch.  A workgroup forms one tile of 16 rows of one output limb in
+// the lane layout in which the row pass loads (so the key and the digits are read in full lines) and runs the row pass on it; the
+// strided pass follows as a launch of its own.  Against the separate launches this saves one write and one read of every sum.
+// N = 2^16, integer back end (the T primes of the reference's sets have 60 bits).
+// Order of the workgroups: consecutive workgroups go to the eight XCDs in turn; numbered as below, those of one XCD take the
+// output blocks and polynomials of one (tile, T prime) one after the other, so the digit tiles they share (and the prime's
+// twiddles) are read from that XCD's L2.
+// ------------------------------------------------------------------------------------------------------------
+struct ExtRowArgs {
+    const u64* c;                // digits over T, NTT domain: limb d * t_num + t
+    const u64* key;              // limb z * key_z_stride + d * key_digit_stride + o
+    u64* out;                    // limb z * out_z_stride + o: as an in-place inverse transform leaves it between its passes
+    const PrimeConst* primes;
+    const ulonglong2* tw_inv;    // [prime][N]
+    int ndigits, t_num, blocks, prime0;
+    long key_digit_stride, key_z_stride, out_z_stride;
+};
+__global__ __launch_bounds__(256, 4) void ext_row_fused_kernel(ExtRowArgs a) {
+    typedef RowCfg<8, 8> C;
+    constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
+    constexpr long N = 1l << 16;
+    static_assert(R == 16 && U == 16 && ROWS == 16, "tile shape");
+    __shared__ u64 lds[C::LDS_WORDS];
+    const unsigned tid = threadIdx.x;
+    unsigned w = blockIdx.x;
+    const unsigned t = w % (unsigned)a.t_num; w /= (unsigned)a.t_num;
+    const unsigned z = w & 1u; w >>= 1;
+    const unsigned blk = w % (unsigned)a.blocks, tile = w / (unsigned)a.blocks;
+    const unsigned o = blk * (unsigned)a.t_num + t;
+    const int prime = a.prime0 + (int)t;
+    const PrimeConst& pr = a.primes[prime];
+    const IntArith ar(pr);
+    const ulonglong2* tw = a.tw_inv + (long)prime * N;
+    const unsigned u = tid % U, rl = tid / U;
+    const unsigned row = tile * ROWS + rl;
+    u64* lrow = lds + rl * C::PITCH;
+    const unsigned tw_off = N1 + row;
+    const long at = (long)row * N2 + u;
+    const u64* cp = a.c + (long)t * N + at;
+    const u64* kp = a.key + ((long)z * a.key_z_stride + o) * N + at;
+    // The sums of a lane's sixteen words, four at a time: the 128-bit sums of all sixteen would take half of the registers that
+    // let four workgroups share a compute unit.  The reduced sums go where the row pass exchanges its data.
+    constexpr int CH = 4;
+    const long c_step = (long)a.t_num * N, k_step = a.key_digit_stride * N;
+#pragma unroll 1
+    for (int j0 = 0; j0 < R; j0 += CH) {
+        u128w acc[CH];
+        u64 x[CH], k[CH], xn[CH], kn[CH];
+#pragma unroll
+        for (int j = 0; j < CH; j++) { acc[j] = u128w{0, 0}; x[j] = cp[(j0 + j) * U]; k[j] = kp[(j0 + j) * U]; }
+        for (int d = 0; d < a.ndigits; d++) {
+            if (d + 1 < a.ndigits) {                        // the next digit's words are on their way while this one's are multiplied
+#pragma unroll
+                for (int j = 0; j < CH; j++) { xn[j] = cp[(d + 1) * c_step + (j0 + j) * U]; kn[j] = kp[(d + 1) * k_step + (j0 + j) * U]; }
+            }
+#pragma unroll
+            for (int j = 0; j < CH; j++) mac128(acc[j], x[j], k[j]);
+            if (d + 1 < a.ndigits) {
+#pragma unroll
+                for (int j = 0; j < CH; j++) { x[j] = xn[j]; k[j] = kn[j]; }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CH; j++) lrow[padded(u + (j0 + j) * U)] = barrett128(acc[j], pr.q, pr.mu_hi, pr.mu_lo);
+    }
+    // the row pass of the inverse transform (row_tile, inverse branch) on the sums
+    __syncthreads();
+    u64 v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lrow[padded(u * R + j)];
+    inv_packed<IntArith, 8, S1>(v, tw, tw_off, u, ar);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; j++) v[j] = lrow[padded(u + j * U)];
+    inv_spread<IntArith, 8, S1, 0>(v, tw, tw_off, ar);
+    u64* rp = a.out + ((long)z * a.out_z_stride + o) * N + at;
+#pragma unroll
+    for (int j = 0; j < R; j++) rp[j * U] = ar.to_mid_inv(v[j]);
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // End of a key switch: ModDown and the first pass of the forward transform of its result in one launch.  The strided pass
 // of limb q_i of polynomial z takes each of its inputs from the K special-prime limbs and limb q_i of the extended
 // polynomial (BasisConv.cuh:257-326: out = (c_q - sum_i [c_p_i * pHat_i^-1]_p_i * pHat_i) * P^-1 mod q) instead of reading
@@ -1455,6 +1541,34 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
         hipLaunchKernelGGL((ks_moddown_strided_kernel<F64WideArith, MidLimb>), gs, dim3(256), 0, c->stream, m);
         hipLaunchKernelGGL((ntt_row_pass<F64WideArith, 8, 8, false, false>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
     }
+    CKKS_HIP_TRY(hipGetLastError());
+    *done = true;
+    return CKKS_OK;
+}
+
+// External product with the switching key and inverse transform of the sums (KeySwitch_23.cuh:225-226) in two launches where the
+// separate steps take three (or two with a write and a read of every sum between them); *done = false where it does not apply.
+int launch_ext_product_inverse_fused(ckks_ctx* c, uint64_t* ext, const uint64_t* up, const uint64_t* swk, int l, bool* done) {
+    *done = false;
+    if (c->ks_split || c->logN != 16 || c->ntt_mode != 0 || c->ev_mid_armed || c->t_num <= 0 || c->gamma <= 0 || c->p_num <= 0) return CKKS_OK;
+    const int T = c->t_num, prime0 = c->p_num + c->q_num;
+    // the integer back end is what the transforms over T would run on: every T prime too wide for the FP64 forms, or the context set to integers
+    for (int j = 0; j < T; j++)
+        if (c->arith_mode == 0 && c->pqt[prime0 + j] < (1ull << 50)) return CKKS_OK;
+    const int ndigits = (l + 1 + c->p_num - 1) / c->p_num;                                   // cipher_blockNum, ExternalProduct.cuh:87
+    if (ndigits > c->dnum) { set_error("external_product_T: the level needs more digits than the key holds (q_num is no multiple of p_num)"); return CKKS_E_INVALID; }
+    const int blocks = (c->p_num + l + 1 + c->gamma - 1) / c->gamma;                         // :88
+    ExtRowArgs a;
+    a.c = (const u64*)up; a.key = (const u64*)swk; a.out = (u64*)ext; a.primes = c->d_primes; a.tw_inv = (const ulonglong2*)c->d_tw_inv;
+    a.ndigits = ndigits; a.t_num = T; a.blocks = blocks; a.prime0 = prime0;
+    a.key_digit_stride = (long)T * c->Ri_blockNum; a.key_z_stride = (long)c->Ri_blockNum * T * c->dnum; a.out_z_stride = (long)c->Ri_blockNum * T;
+    const int limbs = 2 * blocks * T;
+    hipLaunchKernelGGL(ext_row_fused_kernel, dim3((unsigned)(RowCfg<8, 8>::TILES * limbs)), dim3(256), 0, c->stream, a);
+    NttArgs args;
+    args.data = (u64*)ext; args.primes = c->d_primes; args.tw = c->d_tw_inv;
+    args.start_poly_idx = 0; args.start_mod_idx = prime0; args.poly_num = blocks; args.mod_num = T; args.poly_mod_len = T;
+    args.batch_stride_limbs = a.out_z_stride; args.limb_base = 0; args.limbs_total = (unsigned)limbs; args.mid = nullptr;
+    hipLaunchKernelGGL((ntt_strided_pass<IntArith, 8, 8, true, false>), dim3(StridedCfg<8, 8>::TILES, limbs), dim3(StridedCfg<8, 8>::THREADS), 0, c->stream, args);
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
     return CKKS_OK;

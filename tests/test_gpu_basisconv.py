@@ -119,9 +119,11 @@ def test_external_product_and_keyswitch_23(params):
 @pytest.mark.parametrize("primes", ["36", "49"])
 def test_keyswitch_23_full_ring(primes):
     """The T-basis switch at N = 2^16 with the reference's 60-bit T primes over P and Q primes below 2^39 (36- and 37-bit) and over
-    the reference's own 49- and 50-bit P and Q primes: at this size its ModDown runs inside the first pass of the final transform
-    (handing over 5-byte values below 2^39, whole limbs on the wide FP64 arithmetic above); same words as the oracle's separate
-    steps, and as the device's own separate steps (ntt mode 1)."""
+    the reference's own 49- and 50-bit P and Q primes: at this size its external product runs in one launch with the row pass of
+    the sums' inverse transform, and its ModDown inside the first pass of the final transform (handing over 5-byte values below
+    2^39, whole limbs on the wide FP64 arithmetic above); same words as the oracle's separate steps, and as the device's own
+    separate steps (ntt mode 1).  Three T primes here: the launch's numbering of its workgroups is exercised away from the
+    eight primes it is laid out for."""
     q, p, t = CFG2_Q[:6], CFG3_P[:2], REF_PARAMS[16]["t"][:3]      # q_num a multiple of p_num, as in every set of the reference
     if primes == "49":
         q, p = REF_PARAMS[16]["q"][:6], REF_PARAMS[16]["p"][:2]
