@@ -98,14 +98,31 @@ def bench_ntt(args, P):
         ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
         ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
 
+    # The timed steps carry a mark (an event record on the launch stream, nothing waits for it) in front of every transform, as long
+    # as the marks last: the intervals between them, read after the region, are the transforms' durations inside the timed region.
+    marked = min(args.steps, 2000)
+
+    def marked_step(i):
+        ctx.timer_mark(2 * i)
+        ctx.FromNTTInplace(buf, 0, 0, polys, L1, L1)
+        ctx.timer_mark(2 * i + 1)
+        ctx.ToNTTInplace(buf, 0, 0, polys, L1, L1)
+
     for _ in range(args.warmup):
         step()
     ctx.sync()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        if i < marked:
+            marked_step(i)
+        else:
+            step()
+    ctx.timer_mark(2 * marked)          # behind the last marked step's forward transform when every step is marked
     ctx.sync()
     dt = time.perf_counter() - t0
+    inv_in_region = sum(ctx.timer_between(2 * i, 2 * i + 1) for i in range(marked)) / marked
+    n_fwd = marked if marked == args.steps else marked - 1          # the last mark sits behind the unmarked steps, if there are any
+    fwd_in_region = sum(ctx.timer_between(2 * i + 1, 2 * i + 2) for i in range(n_fwd)) / max(1, n_fwd)
     # round trip must give the data back (bit-exact) - cheap end-to-end sanity on the timed buffer
     back = buf.download(np.uint64, one.size).reshape(one.shape)
     assert np.array_equal(back, one), "NTT round trip changed the data"
@@ -115,7 +132,7 @@ def bench_ntt(args, P):
     # Per-kernel durations, HIP events on the launch stream.  Where the library takes the resident transform (one launch per
     # transform: N = 2^16, primes below 2^36, at least a limb per compute unit) the launch is the transform; otherwise a transform
     # is two launches and the events sit between them.
-    reps = max(5, args.steps)
+    reps = max(5, min(20, args.steps))
     per_round = ctx.info("ntt_resident_round")
     resident = args.ntt_mode in (0, 6) and per_round > 0 and limbs >= per_round and max(primes) < (1 << 36)
     one_launch = resident or args.ntt_mode in (2, 3, 4, 5)
@@ -142,13 +159,18 @@ def bench_ntt(args, P):
     ctx.set_ntt_mode(args.ntt_mode)
     passes = [("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2), ("ntt_row_pass(inv)", i1), ("ntt_strided_pass(inv)", i2)]
     pass_ms = {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)}
+    same_kernel_ms = None
     if one_launch:
-        fwd_ms, inv_ms = timed(ctx.ToNTTInplace, 2 * reps), timed(ctx.FromNTTInplace, 2 * reps)
+        # one launch per transform: the intervals between the marks of the timed region are the launches' durations
+        fwd_ms, inv_ms = fwd_in_region, inv_in_region
         name = "ntt_resident_kernel" if resident else "one-launch transform (ntt_mode %d)" % args.ntt_mode
         dom_name, dom_ms = max([(name + "(fwd)", fwd_ms), (name + "(inv)", inv_ms)], key=lambda x: x[1])
         alg_bytes_launch = alg_bytes_transform
         key = "ntt_resident_fwd_1536_limbs" if dom_name.endswith("(fwd)") else "ntt_resident_inv_1536_limbs"
         kernel_ms = {"fwd": round(fwd_ms, 4), "inv": round(inv_ms, 4)}
+        # beside it: ten launches of the same kernel in a row (a launch that follows its own kind runs faster than one that
+        # follows the other direction, as every launch of the timed region does)
+        same_kernel_ms = {"fwd": round(timed(ctx.ToNTTInplace, 10), 4), "inv": round(timed(ctx.FromNTTInplace, 10), 4)}
     else:
         fwd_ms, inv_ms = f1 + f2, i1 + i2
         dom_name, dom_ms = max(passes, key=lambda x: x[1])          # the slowest of all four passes
@@ -160,6 +182,10 @@ def bench_ntt(args, P):
     roofline = {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic.get(key) if limbs == 1536 and resident == (args.ntt_mode in (0, 6)) else None,
                 "traffic_source": traffic_note, "launches_per_transform": 1 if one_launch else 2, "kernel_ms": kernel_ms,
+                "kernel_ms_is": "average over the launches of the timed region (marks on the launch stream between them)" if one_launch
+                                else "average over %d transforms with events between the two launches, behind the timed region" % reps,
+                "transform_ms_in_timed_region": {"fwd": round(fwd_in_region, 4), "inv": round(inv_in_region, 4)},
+                "kernel_ms_same_kernel_back_to_back": same_kernel_ms,
                 "two_launch_form_pass_ms": pass_ms,
                 "transform_algorithmic_GBps": {"fwd": round(alg_bytes_transform / (fwd_ms * 1e-3) / 1e9, 1),
                                                "inv": round(alg_bytes_transform / (inv_ms * 1e-3) / 1e9, 1)},
@@ -247,8 +273,10 @@ def bench_cpu_baseline(P, seconds_target=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults: 30 warm-up steps (about 30 ms) carry the run past the clock ramp that follows an idle GPU (the first 15 ms or so
+    # run about 8 % slower); 100 timed steps then take a tenth of a second
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--batch", type=int, default=32, help="ciphertexts per step (BASELINE configs[1]: 32)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--ntt-mode", type=int, default=0, help="profiling aid: launch form of the transforms (ckks_ctx_set_ntt_mode); with a "

@@ -35,6 +35,7 @@ def _declare(L):
         "ckks_memset": (i, [vp, i, sz]), "ckks_sync": (i, []), "ckks_device_count": (i, [C.POINTER(i)]),
         "ckks_measure_mfma_i8_peak": (i, [vp, C.POINTER(d)]),
         "ckks_timer_start": (i, [vp]), "ckks_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
+        "ckks_timer_mark": (i, [vp, i]), "ckks_timer_between": (i, [vp, i, i, C.POINTER(C.c_float)]),
         "ckks_ctx_create": (i, [C.POINTER(vp), i, u64p, i, u64p, i, u64p, i, i]), "ckks_ctx_destroy": (i, [vp]),
         "ckks_set_stream": (i, [vp, vp]), "ckks_ctx_info": (i, [vp, C.c_char_p, C.POINTER(l)]),
         "ckks_ctx_set_arith_mode": (i, [vp, i]), "ckks_ctx_set_ntt_mode": (i, [vp, i]), "ckks_ctx_check": (i, [vp]), "ckks_ctx_set_ntt_chain": (i, [vp, i, i]),

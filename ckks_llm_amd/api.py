@@ -163,6 +163,16 @@ class Context_23:
     def sync(self):
         _check(self.L_.ckks_sync(), "ckks_sync")
 
+    def timer_mark(self, slot):
+        """Record mark `slot` (0 .. 4095) on the context's stream; returns at once."""
+        _check(self.L_.ckks_timer_mark(self.h, slot), "ckks_timer_mark")
+
+    def timer_between(self, slot_a, slot_b):
+        """Milliseconds from mark slot_a to mark slot_b (waits for slot_b)."""
+        ms = C.c_float()
+        _check(self.L_.ckks_timer_between(self.h, slot_a, slot_b, C.byref(ms)), "ckks_timer_between")
+        return ms.value
+
     def timer_start(self):
         _check(self.L_.ckks_timer_start(self.h), "ckks_timer_start")
 

@@ -398,6 +398,7 @@ extern "C" int ckks_ctx_destroy(ckks_ctx* c) {
     if (c->d_ntt_pair) (void)hipFree(c->d_ntt_pair);
     if (c->h_pair_fail) (void)hipHostFree(c->h_pair_fail);
     for (auto& e : c->decode_tabs) (void)hipFree(e.dev);
+    for (hipEvent_t e : c->ev_marks) if (e) (void)hipEventDestroy(e);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->ev_mid) (void)hipEventDestroy(c->ev_mid);
@@ -543,6 +544,24 @@ extern "C" int ckks_timer_stop(ckks_ctx* c, float* ms) {
     CKKS_HIP_TRY(hipEventRecord(c->ev1, c->stream));
     CKKS_HIP_TRY(hipEventSynchronize(c->ev1));
     CKKS_HIP_TRY(hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return CKKS_OK;
+}
+
+// Marks on the context's stream, read back in pairs: a caller that queues many launches back to back puts a mark between them
+// (an event record; nothing waits) and asks for the intervals once the work is done.
+constexpr int TIMER_MAX_MARKS = 4096;
+extern "C" int ckks_timer_mark(ckks_ctx* c, int slot) {
+    if (!c || slot < 0 || slot >= TIMER_MAX_MARKS) { ckks::set_error("timer_mark: slot outside 0 .. 4095"); return CKKS_E_INVALID; }
+    if ((size_t)slot >= c->ev_marks.size()) c->ev_marks.resize((size_t)slot + 1, nullptr);
+    if (!c->ev_marks[slot]) CKKS_HIP_TRY(hipEventCreate(&c->ev_marks[slot]));
+    CKKS_HIP_TRY(hipEventRecord(c->ev_marks[slot], c->stream));
+    return CKKS_OK;
+}
+extern "C" int ckks_timer_between(ckks_ctx* c, int slot_a, int slot_b, float* ms) {
+    if (!c || !ms || slot_a < 0 || slot_b < 0 || (size_t)slot_a >= c->ev_marks.size() || (size_t)slot_b >= c->ev_marks.size() ||
+        !c->ev_marks[slot_a] || !c->ev_marks[slot_b]) { ckks::set_error("timer_between: a slot that was never marked"); return CKKS_E_INVALID; }
+    CKKS_HIP_TRY(hipEventSynchronize(c->ev_marks[slot_b]));
+    CKKS_HIP_TRY(hipEventElapsedTime(ms, c->ev_marks[slot_a], c->ev_marks[slot_b]));
     return CKKS_OK;
 }
 

@@ -58,6 +58,7 @@ struct ckks_ctx {
     long N = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr, ev_mid = nullptr;
+    std::vector<hipEvent_t> ev_marks;          // ckks_timer_mark: created on first use, destroyed with the context
     bool ev_mid_armed = false;           // record ev_mid between the two passes of the next NTT (per-kernel timing)
 
     // host copies (reference names, reference layouts) for ckks_ctx_table and for launch-time decisions

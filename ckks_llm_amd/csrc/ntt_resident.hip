@@ -19,6 +19,14 @@
 // row 16 m + k, which is exactly the set of rows (forward: that a lane of the column pass ends with; inverse: that a lane of
 // the column pass starts from).
 //
+// One twiddle table serves both directions.  The tables hold the powers of psi in bit-reversed order; psi^-k = -psi^(N-k), and in
+// that order the exponent N - k sits, within each power-of-two block of the table, at the mirrored index: inverse[j] =
+// -forward[3 * 2^s - 1 - j] for 2^s <= j < 2^(s+1), the same bits (the entries are balanced residues, so the sign flips exactly).
+// The inverse transform therefore reads the forward table at mirrored places - a contiguous group of twiddles stays a contiguous
+// group, of the mirrored row and lane group, in reverse order - and negates what it reads (a source modifier, no instruction).
+// Alternating forward and inverse launches then keep one table warm in the memory-side cache instead of displacing each other's
+// (measured: a launch that follows the other direction lost 25 - 55 us of 465 us to that).
+//
 // Vector memory operations complete in the order of their issue and share one counter.  The asynchronous loads are issued
 // from inline assembly, invisible to the compiler's own bookkeeping, so a step is written such that no load the compiler
 // waits for is older than an asynchronous load still in flight: the twiddles of a step are in registers (drain()) before the
@@ -118,6 +126,12 @@ struct SpreadTwiddles {
             for (int k = 0; k < (1 << s); k++) t[(1 << s) - 1 + k] = tw[(off << s) + k];
     }
 };
+// inverse twiddle j (1 <= j) from the forward table: the negative of the entry at the mirrored place of j's power-of-two block
+template <class TW>
+__device__ __forceinline__ TW mirrored(const TW* __restrict__ fwd, unsigned j) {
+    const unsigned top = 1u << (31 - __builtin_clz(j));
+    return -fwd[3u * top - 1u - j];
+}
 struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 // after(s) runs behind the butterflies of the round's stage s (the asynchronous loads of the next tile go out there, one per stage)
 template <class AR, class F, class H = NoHook>
@@ -220,6 +234,27 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     };
     coordinates();
 
+    // The kernel's own code, fetched as data.  The code (about 100 KiB, unrolled over the 32 steps of a limb) exceeds the instruction
+    // cache, so instruction fetch leans on the L2; a launch that follows a different kernel finds none of its code there and would
+    // fetch it line by line, in execution order, from memory - with two waves per SIMD nothing hides that (measured: 20 us of 465 for a
+    // launch that follows a copy of itself under another name).  Here every lane reads one word per 128-byte line of the stretch of
+    // code between this point and the label in front of the kernel's end, all lines at once: one memory latency, and the
+    // instruction fetches that follow hit the L2.  Both labels lie inside this function, so every address between them is this
+    // function's code.
+    {
+        int code_bytes;
+        if constexpr (INVERSE) asm volatile("ckks_res_inv_code_begin:\n\ts_mov_b32 %0, ckks_res_inv_code_end-ckks_res_inv_code_begin" : "=s"(code_bytes));
+        else asm volatile("ckks_res_fwd_code_begin:\n\ts_mov_b32 %0, ckks_res_fwd_code_end-ckks_res_fwd_code_begin" : "=s"(code_bytes));
+        const char* pc = reinterpret_cast<const char*>(__builtin_amdgcn_s_getpc());
+        code_bytes -= 1024;                              // the program counter was read a few instructions behind the first label
+        if (code_bytes > 0 && code_bytes < (1 << 18)) {
+            unsigned seen = 0;
+            for (int at = (int)threadIdx.x * 128; at < code_bytes; at += RES_LANES * 128)
+                seen |= __hip_atomic_load(reinterpret_cast<const unsigned*>(pc + at), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // served by the L2
+            asm volatile("" : : "v"(seen));
+        }
+    }
+
     // Requests tile (2 s + grp) of the first pass of `limb`.  Inverse transforms: with it the twiddles of the tile's last four
     // stages, which depend on the row only: 15 per row = 8 chunks of 16 bytes (stage 3: 4, stage 2: 2, stage 1: 1, stage 0: the
     // chunk that holds its one twiddle), 4 rows per wave, into this wave's 512 bytes of the twiddle staging of the step's parity.
@@ -236,7 +271,8 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             // every lane takes part (the upper half of the wave repeats the lower half's chunks into the second half of the wave's
             // 1 KiB): no branch; the staging is single: the step's own reads of it are over (they come before this in the last round)
             const unsigned i = (lane >> 3) & 3, c = lane & 7;
-            const unsigned off = 256 + 16 * (4 * wq + i) + tile;
+            const unsigned trow_id = 16 * (4 * wq + i) + tile;
+            const unsigned off = 256 + (INVERSE ? 255 - trow_id : trow_id);          // inverse: the mirrored row of the forward table
             // chunk c: 0..3 stage 3 (twiddles 8 off + 2 c ..), 4..5 stage 2 (4 off + 2 (c - 4) ..), 6 stage 1 (2 off ..), 7 the pair that holds stage 0's (off)
             const unsigned sh = (0x01223333u >> (4 * c)) & 15u, add = (0x00206420u >> (4 * c)) & 15u;
             const TW* src = tw + (((off << sh) + add) & ~1u);
@@ -307,7 +343,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     PackedTwiddles<AR> wp;                               // second-round twiddles of a row-pass step, fetched a step ahead
     TW w_col = 0.0;                                      // this lane's entry of the column pass's twiddle table, fetched ahead
     if (!INVERSE && threadIdx.x < 256) w_col = ((const TW*)a.tw + (long)prime * RES_N)[threadIdx.x];
-    if (INVERSE) wp.load_ordered((const TW*)a.tw + (long)prime * RES_N, 256 + 16 * g + grp, cl);
+    if (INVERSE) wp.load_ordered((const TW*)a.tw + (long)prime * RES_N, 511 - (16 * g + grp), 15 - cl);
     for (;;) {
         const AR ar(a.primes[prime]);
         const TW* __restrict__ tw = (const TW*)a.tw + (long)prime * RES_N;
@@ -416,16 +452,17 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 V v[16];
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl * 16 + j)];
-                inv_round<AR, 0>(v, ar, [&](int d, int k) { return wp.t[(1 << d) - 1 + k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, 3 - d); });
+                // (mirrored groups: twiddle k of stage d is the negative of entry 2^d - 1 - k of the group that was fetched)
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return -wp.t[(2 << d) - 2 - k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, 3 - d); });
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
-                if (s == 7 && threadIdx.x < 256) w_col = tw[threadIdx.x];
+                if (s == 7 && threadIdx.x < 256) w_col = mirrored(tw, threadIdx.x ? threadIdx.x : 1u);      // (entry 0 of the table is not a twiddle and is never used)
                 wave_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl + 16 * j)];
-                inv_round<AR, 0>(v, ar, [&](int d, int k) { return d == 3 ? trow[k] : d == 2 ? trow[8 + k] : d == 1 ? trow[12 + k] : trow[14 + (tw_off & 1u)]; },
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return d == 3 ? -trow[7 - k] : d == 2 ? -trow[11 - k] : d == 1 ? -trow[13 - k] : -trow[15 - (tw_off & 1u)]; },
                                  [&](int d) { if (s < 7) { request_part(limb, tw, s + 1, 7 - d); if (d == 0) request_part(limb, tw, s + 1, 8); } });
-                if (s < 7) wp.load_ordered(tw, tw_off + 2, cl);         // the next step's, behind the requests: they arrive together
+                if (s < 7) wp.load_ordered(tw, 511 - (row + 2), 15 - cl);         // the next step's, behind the requests: they arrive together
                 hand_over(v, ar, s);                    // balanced to (-q/2, q/2] between the passes, as in the two-launch form
             }
             if (threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
@@ -443,9 +480,9 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 col_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = col_area[(g + 16 * j) * 16 + cl];
-                inv_round<AR, 1>(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; },        // scalar loads
+                inv_round<AR, 1>(v, ar, [&](int d, int k) { return -tw[(2u << d) - 1 - k]; },        // scalar loads, mirrored
                                  [&](int d) { if (s == 7 && more) { request_part(next_limb, next_tw, 0, 9 - 3 * d); request_part(next_limb, next_tw, 0, 10 - 3 * d); request_part(next_limb, next_tw, 0, 11 - 3 * d); } });
-                if (s == 7 && more) wp.load_ordered(next_tw, 256 + 16 * g + grp, cl);
+                if (s == 7 && more) wp.load_ordered(next_tw, 511 - (16 * g + grp), 15 - cl);
                 u64* col = limb + (2 * s + grp) * 16 + cl;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -463,6 +500,9 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
         limb = next_limb;
         prime = next_prime;
     }
+    // end of the stretch of code that the kernel's first instructions fetch as data
+    if constexpr (INVERSE) asm volatile("ckks_res_inv_code_end:");
+    else asm volatile("ckks_res_fwd_code_end:");
 }
 
 }  // namespace
@@ -482,6 +522,7 @@ int launch_ntt_resident(ckks_ctx* c, const NttArgs& args_in, int limbs, int coun
     args.limb_base = 0;
     args.limbs_total = (unsigned)limbs;
     args.mid = nullptr;
+    args.tw = c->d_twd_fwd;                             // both directions read the forward table
     const dim3 g(resident_grid(c)), b(RES_LANES);
     // Successive launches of a context walk the rounds in opposite directions: where the same batch goes through several
     // transforms in a row, each starts on the limbs that the one before wrote last.  The order of the limbs has no effect

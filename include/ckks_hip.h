@@ -50,6 +50,11 @@ int ckks_device_count(int* count);
 /* HIP-event timing on the context's stream (replaces CUDATimer, TimeUtils.cuh:10-35) */
 int ckks_timer_start(ckks_ctx* ctx);
 int ckks_timer_stop(ckks_ctx* ctx, float* elapsed_ms);
+/* Marks between launches queued back to back: ckks_timer_mark records event `slot` (0 .. 4095) on the context's stream and
+ * returns at once; ckks_timer_between waits for mark slot_b and gives the time from mark slot_a to it.  A measurement aid with
+ * no counterpart in the reference (its CUDATimer brackets one region). */
+int ckks_timer_mark(ckks_ctx* ctx, int slot);
+int ckks_timer_between(ckks_ctx* ctx, int slot_a, int slot_b, float* elapsed_ms);
 
 /* ---- context: Context_23::Context_23 + getPrimeCKKS + preComputeOnCPU + copyMemoryToGPU
  *      (Context_23.cuh:12-472, 475-701; Params.cuh).  Primes are passed explicitly; gamma is the block width of
