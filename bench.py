@@ -159,7 +159,6 @@ def bench_ntt(args, P):
     ctx.set_ntt_mode(args.ntt_mode)
     passes = [("ntt_strided_pass(fwd)", f1), ("ntt_row_pass(fwd)", f2), ("ntt_row_pass(inv)", i1), ("ntt_strided_pass(inv)", i2)]
     pass_ms = {"fwd_strided": round(f1, 4), "fwd_row": round(f2, 4), "inv_row": round(i1, 4), "inv_strided": round(i2, 4)}
-    same_kernel_ms = None
     if one_launch:
         # one launch per transform: the intervals between the marks of the timed region are the launches' durations
         fwd_ms, inv_ms = fwd_in_region, inv_in_region
@@ -168,9 +167,6 @@ def bench_ntt(args, P):
         alg_bytes_launch = alg_bytes_transform
         key = "ntt_resident_fwd_1536_limbs" if dom_name.endswith("(fwd)") else "ntt_resident_inv_1536_limbs"
         kernel_ms = {"fwd": round(fwd_ms, 4), "inv": round(inv_ms, 4)}
-        # beside it: ten launches of the same kernel in a row (a launch that follows its own kind runs faster than one that
-        # follows the other direction, as every launch of the timed region does)
-        same_kernel_ms = {"fwd": round(timed(ctx.ToNTTInplace, 10), 4), "inv": round(timed(ctx.FromNTTInplace, 10), 4)}
     else:
         fwd_ms, inv_ms = f1 + f2, i1 + i2
         dom_name, dom_ms = max(passes, key=lambda x: x[1])          # the slowest of all four passes
@@ -185,7 +181,7 @@ def bench_ntt(args, P):
                 "kernel_ms_is": "average over the launches of the timed region (marks on the launch stream between them)" if one_launch
                                 else "average over %d transforms with events between the two launches, behind the timed region" % reps,
                 "transform_ms_in_timed_region": {"fwd": round(fwd_in_region, 4), "inv": round(inv_in_region, 4)},
-                "kernel_ms_same_kernel_back_to_back": same_kernel_ms,
+
                 "two_launch_form_pass_ms": pass_ms,
                 "transform_algorithmic_GBps": {"fwd": round(alg_bytes_transform / (fwd_ms * 1e-3) / 1e9, 1),
                                                "inv": round(alg_bytes_transform / (inv_ms * 1e-3) / 1e9, 1)},
