@@ -296,7 +296,10 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
         // the row pointers alive across the loop).
         long row_stride = (long)a.mod_num * a.C;
         asm volatile("" : "+s"(row_stride));
-        const int mrow = m0 + wm * 32 + 4 * lg;
+        // (so do the row numbers: formed ahead of the loop over the primes, their 64-bit forms would be kept, or spilled to memory
+        // and fetched back one by one, across the K loops)
+        int mrow = m0 + wm * 32 + 4 * lg;
+        asm volatile("" : "+v"(mrow));
         u64* obase = a.out + (long)im * a.C + c0 + wc * 32 + lr;
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) {
@@ -392,8 +395,12 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void ppmm_mfma_kernel(PpmmArgs a, c
                     double h[4], l[4], c[4];
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        const unsigned hi = (rl_hi[mt][nt] >> (8 * r)) & 0xff;
-                        t[r] -= __builtin_fma((double)hi, 4294967296.0, (double)rl_lo[mt][r][nt]);
+                        // read through values the optimiser cannot see through: the conversions are the same for every prime but
+                        // the last, and hoisted out of the loop over the primes they would occupy 32 registers across the K loops
+                        unsigned lo = rl_lo[mt][r][nt], hw = rl_hi[mt][nt];
+                        asm volatile("" : "+v"(lo), "+v"(hw));
+                        const unsigned hi = (hw >> (8 * r)) & 0xff;
+                        t[r] -= __builtin_fma((double)hi, 4294967296.0, (double)lo);
                     }
 #pragma unroll
                     for (int r = 0; r < 4; r++) h[r] = t[r] * qli;
