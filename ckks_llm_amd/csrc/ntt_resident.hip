@@ -126,12 +126,6 @@ struct SpreadTwiddles {
             for (int k = 0; k < (1 << s); k++) t[(1 << s) - 1 + k] = tw[(off << s) + k];
     }
 };
-// inverse twiddle j (1 <= j) from the forward table: the negative of the entry at the mirrored place of j's power-of-two block
-template <class TW>
-__device__ __forceinline__ TW mirrored(const TW* __restrict__ fwd, unsigned j) {
-    const unsigned top = 1u << (31 - __builtin_clz(j));
-    return -fwd[3u * top - 1u - j];
-}
 struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 // after(s) runs behind the butterflies of the round's stage s (the asynchronous loads of the next tile go out there, one per stage)
 template <class AR, class F, class H = NoHook>
@@ -207,13 +201,13 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     __shared__ __align__(16) unsigned char lds_r[RES_R_BYTES];
     __shared__ __align__(16) unsigned lds_s[RES_S_BYTES / 4];
     __shared__ __align__(16) unsigned char lds_t[RES_T_BYTES];
-    __shared__ TW lds_w[256];                            // twiddles 1 .. 255 of the limb's prime: the column pass's, the same for every column
+    __shared__ __align__(16) TW lds_w[256];              // entries 0 .. 255 of the prime's table: twiddles 1 .. 255 are the column pass's, the same for every column
     unsigned grp = threadIdx.x >> 8;
     unsigned tid = threadIdx.x & 255, cl = tid & 15, g = tid >> 4;    // column pass: column within the tile, group of rows; row pass: lane within the row (u = cl), row group (rl = g)
-    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wq = wave & 3;
+    unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wq = wave & 3;
     unsigned lane = threadIdx.x & 63;
     // this wave's part of the staging area, and where this lane reads its sixteen words from (word j at + 512 j)
-    const unsigned p_wave = (unsigned)(size_t)(lptr_t)lds_p + wave * 8192;
+    unsigned p_wave = (unsigned)(size_t)(lptr_t)lds_p + wave * 8192;
     const u64* p_lane;
     // asynchronous load m (0..7) of a tile moves 1 KiB: words 2m and 2m+1 of every lane of the wave
     unsigned d_chunk, d_i, d_jl;
@@ -226,6 +220,11 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
     auto coordinates = [&]() __attribute__((always_inline)) {
         unsigned x = threadIdx.x;
         asm volatile("" : "+v"(x));
+        // (the wave's number too: the scalar registers are as short as the vector ones, and the addresses that hang on it - staging
+        // areas, LDS bases of the asynchronous loads - would otherwise all be formed ahead of the limb and kept)
+        asm volatile("" : "+s"(wave));
+        wq = wave & 3;
+        p_wave = (unsigned)(size_t)(lptr_t)lds_p + wave * 8192;
         grp = x >> 8; tid = x & 255; cl = x & 15; g = tid >> 4; lane = x & 63;
         d_chunk = lane & 7; d_i = (lane >> 3) & 3; d_jl = lane >> 5;
         p_lane = reinterpret_cast<const u64*>(lds_p + wave * 8192 + lane * 8);
@@ -341,8 +340,12 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
 #endif
     request(limb, (const TW*)a.tw + (long)prime * RES_N, 0);
     PackedTwiddles<AR> wp;                               // second-round twiddles of a row-pass step, fetched a step ahead
-    TW w_col = 0.0;                                      // this lane's entry of the column pass's twiddle table, fetched ahead
-    if (!INVERSE && threadIdx.x < 256) w_col = ((const TW*)a.tw + (long)prime * RES_N)[threadIdx.x];
+    // The first 2 KiB of a prime's table go to lds_w by the same asynchronous loads as the tiles (waves 0 and 1, 1 KiB each), at a
+    // point where no wave reads lds_w any more and with a vmcnt(0) of every wave and a barrier between them and the first read.
+    auto request_col_twiddles = [&](const TW* t) __attribute__((always_inline)) {
+        if (wave < 2) dma16(t + (wave * 64 + lane) * 2, (unsigned)(size_t)(lptr_t)lds_w + wave * 1024);
+    };
+    if (!INVERSE) request_col_twiddles((const TW*)a.tw + (long)prime * RES_N);
     if (INVERSE) wp.load_ordered((const TW*)a.tw + (long)prime * RES_N, 511 - (16 * g + grp), 15 - cl);
     for (;;) {
         const AR ar(a.primes[prime]);
@@ -364,7 +367,6 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 V v[16];
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = ar.from_canonical(p_lane[j * 64]);
-                if (s == 0 && threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
                 // the same twiddles for every lane: scalar loads; behind each stage one eighth of the next tile is requested
                 fwd_round(v, ar, [&](int d, int k) { return tw[(1u << d) + k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, d); });
 #pragma unroll
@@ -420,7 +422,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
                 wave_sync();
                 RES_TICK(64 + 8 * s + 7);
-                if (s == 6 && more && threadIdx.x < 256) w_col = next_tw[threadIdx.x];
+                if (s == 6 && more) request_col_twiddles(next_tw);      // the next limb's: nobody has read lds_w since the first pass ended
                 if (s < 7) {
                     wp.load_ordered(tw, tw_off + 2, cl);
                     request_part(limb, tw, s + 1, 8);
@@ -445,6 +447,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 const unsigned row = 16 * g + 2 * s + grp;
                 const unsigned tw_off = 256 + row;
                 wait_all_vmem();                        // this wave's part of the tile, its row twiddles and the lane's twiddles have arrived
+                if (s == 0) request_col_twiddles(tw);   // for the second pass: the workgroup has left the last limb's second pass behind
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl + 16 * j)] = ar.from_canonical(p_lane[j * 64]);
                 const TW* trow = reinterpret_cast<const TW*>(lds_t + wave * 1024 + (lane >> 4) * 128);
@@ -456,7 +459,6 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 inv_round<AR, 0>(v, ar, [&](int d, int k) { return -wp.t[(2 << d) - 2 - k]; }, [&](int d) { if (s < 7) request_part(limb, tw, s + 1, 3 - d); });
 #pragma unroll
                 for (int j = 0; j < 16; j++) row_area[padded(cl * 16 + j)] = v[j];
-                if (s == 7 && threadIdx.x < 256) w_col = mirrored(tw, threadIdx.x ? threadIdx.x : 1u);      // (entry 0 of the table is not a twiddle and is never used)
                 wave_sync();
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = row_area[padded(cl + 16 * j)];
@@ -465,15 +467,15 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 if (s < 7) wp.load_ordered(tw, 511 - (row + 2), 15 - cl);         // the next step's, behind the requests: they arrive together
                 hand_over(v, ar, s);                    // balanced to (-q/2, q/2] between the passes, as in the two-launch form
             }
-            if (threadIdx.x < 256) lds_w[threadIdx.x] = w_col;
-            __syncthreads();
+            __syncthreads();                            // (every wave has waited for its loads since the column twiddles were requested)
             // ---------------- pass 2: columns (stages 7 .. 0) ----------------
 #pragma unroll
             for (int s = 0; s < 8; s++) {
                 coordinates();
                 V v[16];
                 take(v, ar, s);
-                inv_round<AR, 0>(v, ar, [&](int d, int k) { return lds_w[(16u << d) + (g << d) + k]; });
+                // (mirrored within the power-of-two block, negated: the table in lds_w is the forward one)
+                inv_round<AR, 0>(v, ar, [&](int d, int k) { return -lds_w[(16u << d) + ((15u - g) << d) + ((1u << d) - 1u - k)]; });
                 col_sync();                             // the exchange area is free
 #pragma unroll
                 for (int j = 0; j < 16; j++) col_area[(g * 16 + j) * 16 + cl] = v[j];
