@@ -459,6 +459,27 @@ def test_edge_cases_and_errors():
     assert np.array_equal(from_dev(d, data.shape), want)
 
 
+def test_marks_between_launches():
+    """ckks_timer_mark / ckks_timer_between: marks recorded between launches queued back to back give each launch's duration
+    afterwards; the intervals add up, and a slot that was never marked or lies outside the range is refused."""
+    from ckks_llm_amd import CkksError
+    pair = Pair(16, [], CFG2_Q[:4])
+    d = to_dev(limbs_uniform(5, CFG2_Q[:4], 2, pair.N))
+    for i in range(4):
+        pair.dev.timer_mark(i)
+        (pair.dev.ToNTTInplace if i % 2 == 0 else pair.dev.FromNTTInplace)(d, 0, 0, 2, 4, 4)
+    pair.dev.timer_mark(4)
+    parts = [pair.dev.timer_between(i, i + 1) for i in range(4)]
+    assert all(0.0 < t < 50.0 for t in parts), parts
+    assert abs(sum(parts) - pair.dev.timer_between(0, 4)) < 0.02 * len(parts) + 0.05 * sum(parts)
+    with pytest.raises(CkksError):
+        pair.dev.timer_between(0, 9)                 # never marked
+    with pytest.raises(CkksError):
+        pair.dev.timer_mark(4096)                    # outside 0 .. 4095
+    with pytest.raises(CkksError):
+        pair.dev.timer_mark(-1)
+
+
 def test_full_size_properties_batch32():
     """BASELINE config 2 at batch 32 (768 MiB): size-independent properties instead of a full oracle run:
     round trip, linearity on a sampled pair, and oracle parity on one sampled ciphertext."""
