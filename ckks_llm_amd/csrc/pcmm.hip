@@ -320,6 +320,8 @@ extern "C" int pcmm_ctx_destroy(pcmm_ctx* h) {
     for (auto& w : h->weights) { if (w.d_A) (void)hipFree(w.d_A); if (w.d_Adig) (void)hipFree(w.d_Adig); }
     if (h->pin) (void)hipHostFree(h->pin);
     if (h->pin_ev) (void)hipEventDestroy(h->pin_ev);
+    if (h->h_absmax) (void)hipHostFree(h->h_absmax);
+    if (h->ev_absmax) (void)hipEventDestroy(h->ev_absmax);
     if (h->small) ckks_ctx_destroy(h->small);
     delete h;
     return CKKS_OK;
@@ -796,6 +798,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         if (pl.mfma ? !we->d_Adig || we->planes != pl.planes : !we->d_A) { drop_weights(h, we); we = nullptr; }   // prepared for the other kernel
     }
     pcmm_ctx::Weights fresh;
+    bool packed_early = false;
     if (!we) {
         const long count = (long)M * Kin;
         fresh.W = W; fresh.M = M; fresh.Kin = Kin; fresh.scaler = scaler;
@@ -818,10 +821,37 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         (void)hipMemsetAsync(h->d_absmax, 0, sizeof(unsigned long long), c->stream);
         hipLaunchKernelGGL(quantise_kernel, dim3((unsigned)((count + 256 * QUANT_PER_LANE - 1) / (256 * QUANT_PER_LANE))), dim3(256), 0, c->stream, W,
                            fresh.d_A, h->d_absmax, count, scaler);
-        // the one host round trip of a matrix: its digit count selects the kernel instance
-        hipError_t e2 = hipMemcpyAsync(&fresh.absmax, h->d_absmax, sizeof(fresh.absmax), hipMemcpyDeviceToHost, c->stream);
-        if (e2 == hipSuccess) e2 = hipStreamSynchronize(c->stream);
+        // The one host round trip of a matrix: its digit count selects the kernel instance.  The host waits for the copy alone (an event
+        // behind it), and where the MFMA path is in reach the pack pass of the residues, which does not depend on the matrix, is
+        // already queued behind the copy: the GPU works through it while the answer travels.
+        hipError_t e2 = hipSuccess;
+        if (!h->h_absmax) e2 = hipHostMalloc((void**)&h->h_absmax, sizeof(unsigned long long), hipHostMallocDefault);
+        if (e2 == hipSuccess && !h->ev_absmax) e2 = hipEventCreateWithFlags(&h->ev_absmax, hipEventDisableTiming);
+        if (e2 == hipSuccess) e2 = hipMemcpyAsync(h->h_absmax, h->d_absmax, sizeof(unsigned long long), hipMemcpyDeviceToHost, c->stream);
+        if (e2 == hipSuccess) e2 = hipEventRecord(h->ev_absmax, c->stream);
         if (e2 != hipSuccess) { release(); return hip_fail(e2, "PPMM: |A| maximum"); }
+        if (!packed && !force_generic && aligned16 && (C % 64 == 0) && (DC <= 5 || (DC <= 7 && qmax < (1ull << 50))) && (long)Kpad * 3 <= 16384 &&
+            qmin > (1ull << 25)) {
+            PpmmArgs pa;
+            pa.A = nullptr; pa.Adig = nullptr; pa.mlwe = (const u64* const*)h->d_ptrs; pa.mlwe_base = nullptr; pa.mlwe_stride = (long)mod_num * C;
+            pa.out = out; pa.pq = h->d_pq; pa.consts = d_cst; pa.C = C; pa.M = M; pa.Kin = Kin; pa.Mpad = Mpad; pa.Kpad = Kpad; pa.mod_num = mod_num;
+            pa.np = h->np; pa.raw_all = 0;
+            const size_t need = ppmm_bdig_bytes(pa, DC);
+            bool room = need <= h->Bdig_cap;
+            if (!room) {
+                if (h->d_Bdig) { (void)hipDeviceSynchronize(); (void)hipFree(h->d_Bdig); h->d_Bdig = nullptr; h->Bdig_cap = 0; }
+                if (hipMalloc((void**)&h->d_Bdig, need) == hipSuccess) { h->Bdig_cap = need; room = true; }
+                else (void)hipGetLastError();                 // the later, checked allocation reports it
+            }
+            if (room) {
+                h->packed_K = h->packed_mods = 0;             // the planes now hold this call's operands
+                if ((rc = launch_ppmm_pack(c->stream, pa, DC, h->d_Bdig))) { release(); return rc; }
+                packed_early = true;
+            }
+        }
+        e2 = hipEventSynchronize(h->ev_absmax);
+        if (e2 != hipSuccess) { release(); return hip_fail(e2, "PPMM: |A| maximum"); }
+        fresh.absmax = *h->h_absmax;
         const Plan pl = plan_for(fresh.absmax);
         if (packed && !pl.mfma) { release(); set_error("PPMM on digit planes: the plaintext matrix or the primes are outside what the MFMA kernel takes"); return CKKS_E_INVALID; }
         fresh.bytes = (size_t)count * sizeof(long long);
@@ -864,7 +894,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
         }
         if (!packed) h->packed_K = h->packed_mods = 0;     // the planes now hold this call's operands
         if (slices == 1) {
-            rc = launch_ppmm_mfma_impl(c->stream, a, DW, DC, h->d_Bdig, !packed);
+            rc = launch_ppmm_mfma_impl(c->stream, a, DW, DC, h->d_Bdig, !packed && !packed_early);
             if (rc) return rc;
         } else {
             const size_t per_slice = (size_t)M * mod_num * C;
@@ -879,7 +909,7 @@ static int ppmm_common(pcmm_ctx* h, const float* W, const uint64_t* const* ptrs_
             for (int sl = 0; sl < slices; sl++) {
                 sa.Adig = we->d_Adig + (size_t)3 * sl * Mpad * Kpad;
                 sa.out = sl == 0 ? out : h->d_slices + (size_t)(sl - 1) * per_slice;
-                rc = launch_ppmm_mfma_impl(c->stream, sa, 3, DC, h->d_Bdig, !packed && sl == 0);      // the residue planes are packed once
+                rc = launch_ppmm_mfma_impl(c->stream, sa, 3, DC, h->d_Bdig, !packed && !packed_early && sl == 0);      // the residue planes are packed once
                 if (rc) return rc;
             }
             PpmmCombineArgs ca;

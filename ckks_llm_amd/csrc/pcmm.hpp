@@ -26,6 +26,8 @@ struct pcmm_ctx {
     uint64_t* d_small_tw = nullptr;          // tables of the size-N1 transform when N1 < 256: [prime][forward | inverse][N1]
     uint64_t small_n_inv[8] = {};            // N1^-1 modulo each ring-pack prime (N1 < 256)
     unsigned long long* d_absmax = nullptr;  // |A| maximum word, followed by the per-call constant table (PPMM_CONST_WORDS)
+    unsigned long long* h_absmax = nullptr;  // pinned host word the maximum is copied to, and the event behind that copy
+    hipEvent_t ev_absmax = nullptr;
     // Prepared plaintext matrices (only while the caller has switched the cache on: pcmm_set_weight_cache).  The first PPMM call
     // with a given (device pointer, shape, scaler) quantises the matrix, measures |A|max (the one host round trip) and splits it
     // into digit planes; later calls with the same key reuse the planes and issue no host synchronisation at all.
@@ -89,5 +91,6 @@ struct PpmmArgs {
 
 size_t ppmm_bdig_bytes(const PpmmArgs& a, int DC);
 int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC, int8_t* bdig, bool pack);
+int launch_ppmm_pack(hipStream_t stream, const PpmmArgs& a, int DC, int8_t* bdig);
 
 }  // namespace ckks

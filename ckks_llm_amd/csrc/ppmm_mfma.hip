@@ -482,6 +482,16 @@ static int launch_dw(hipStream_t stream, const PpmmArgs& a, int8_t* bdig, bool p
     return CKKS_OK;
 }
 
+// The pack pass on its own: the entry point starts it ahead of the host round trip that selects the contraction's instance (the
+// residue planes do not depend on the plaintext matrix) and then calls the contraction with pack = false.
+int launch_ppmm_pack(hipStream_t stream, const PpmmArgs& a, int DC, int8_t* bdig) {
+    const dim3 grid((unsigned)(a.C / CT), (unsigned)(a.Kpad / KS), (unsigned)a.mod_num);
+    if (DC <= 5) hipLaunchKernelGGL(ppmm_pack_kernel<5>, grid, dim3(256), 0, stream, a, bdig);
+    else hipLaunchKernelGGL(ppmm_pack_kernel<7>, grid, dim3(256), 0, stream, a, bdig);
+    CKKS_HIP_TRY(hipGetLastError());
+    return CKKS_OK;
+}
+
 // pack = false: the digit planes were written by the caller (the gather that emits them directly; 5 residue digits only)
 int launch_ppmm_mfma_impl(hipStream_t stream, const PpmmArgs& a, int DW, int DC, int8_t* bdig, bool pack) {
     if (DC > 5) {
