@@ -66,9 +66,12 @@ __device__ __forceinline__ unsigned resident_limb(unsigned b, unsigned grid, uns
 }
 
 // 16 bytes per lane from global memory into LDS at lds_addr + 16 * lane (lds_addr wave-uniform)
+// STREAM: a load of data that is read once (the caches need not keep the line)
+template <bool STREAM = false>
 __device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
     const unsigned base = __builtin_amdgcn_readfirstlane(lds_addr);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory", "m0");
+    if (STREAM) asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(g), "s"(base) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory", "m0");
 }
 // Ordering point for what a wave exchanges with itself through LDS (the hardware carries out a wave's LDS accesses in order; this
 // keeps the compiler from reordering them: as one thread sees it, the lane that writes and the lane that reads are unrelated).
@@ -265,7 +268,9 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             const u64* src;
             if (!INVERSE) src = limb + (long)(4 * wq + d_i + 16 * (2 * m + d_jl)) * 256 + tile * 16 + 2 * d_chunk;      // rows g + 16 j of 16 columns
             else src = limb + (long)(16 * (4 * wq + d_i) + tile) * 256 + 16 * (2 * m + d_jl) + 2 * d_chunk;             // columns u + 16 j of row 16 rl + tile
-            dma16(src, p_wave + m * 1024);
+            // the rows of an inverse transform's tile are read as streaming loads (434 -> 427 us per launch); for the columns of a forward
+            // transform's tile, 128 bytes per row, the same costs 37 us per launch
+            dma16<INVERSE>(src, p_wave + m * 1024);
         } else {
             // every lane takes part (the upper half of the wave repeats the lower half's chunks into the second half of the wave's
             // 1 KiB): no branch; the staging is single: the step's own reads of it are over (they come before this in the last round)
@@ -434,7 +439,10 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
 #ifdef CKKS_RES_EXP_NOSTORE
                     if (o == 0x123456789abcull) rp[cl + 16 * j] = o;
 #else
-                    rp[cl + 16 * j] = o;
+                    // (streaming stores: the results are not read again in this launch, and lines that linger in the caches as written
+                    // data cost the loads of this launch and of the next more than the next launch's hits on them would save:
+                    // 437 -> 417 us per forward launch, 453 -> 434 us per inverse launch, 474 -> 433 us for an inverse that follows a forward)
+                    __builtin_nontemporal_store(o, &rp[cl + 16 * j]);
 #endif
                 }
             }
@@ -490,8 +498,8 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
                 for (int j = 0; j < 8; j++) {
                     u64 ox, oy;
                     ar.gs_last(v[j], v[j + 8], ox, oy);
-                    col[(long)(g + 16 * j) * 256] = ox;
-                    col[(long)(g + 16 * (j + 8)) * 256] = oy;
+                    __builtin_nontemporal_store(ox, &col[(long)(g + 16 * j) * 256]);          // streaming stores, as in the forward direction
+                    __builtin_nontemporal_store(oy, &col[(long)(g + 16 * (j + 8)) * 256]);
                 }
             }
         }
