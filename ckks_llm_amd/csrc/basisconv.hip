@@ -423,6 +423,12 @@ extern "C" int ckks_rescale(ckks_ctx* c, uint64_t* cipher, uint64_t* scratch, in
     return CKKS_OK;
 }
 extern "C" int ckks_keyswitch_23(ckks_ctx* c, uint64_t* out, uint64_t* d2, const uint64_t* swk, int l, uint64_t* up, uint64_t* ext, uint64_t* buf) {
+    bool added;
+    return ckks::keyswitch_23_add(c, out, d2, swk, l, up, ext, buf, nullptr, 0, &added);
+}
+int ckks::keyswitch_23_add(ckks_ctx* c, uint64_t* out, uint64_t* d2, const uint64_t* swk, int l, uint64_t* up, uint64_t* ext, uint64_t* buf,
+                           const uint64_t* addend, long addend_poly_stride, bool* added) {
+    *added = false;
     if (!c || !out || !d2 || !up || !ext || !buf) return CKKS_E_INVALID;
     if (!swk) { set_error("rotKey_23 not exists"); return CKKS_E_STATE; }                           // KeySwitch_23.cuh:198-201
     if (!level_ok(c, l) || c->t_num == 0 || c->gamma == 0 || c->p_num == 0) { set_error("keyswitch_23: bad level or basis"); return CKKS_E_INVALID; }
@@ -440,8 +446,8 @@ extern "C" int ckks_keyswitch_23(ckks_ctx* c, uint64_t* out, uint64_t* d2, const
     }
     if ((rc = ckks_modup_t_to_pql(c, buf, ext, l, 2))) return rc;                                   // :228
     bool fused = false;
-    if ((rc = launch_ks_moddown_fused(c, out, buf, (long)RB * T * c->N, l, L + 1, false, &fused))) return rc;  // :229 and :231 in two launches
-    if (fused) return CKKS_OK;
+    if ((rc = launch_ks_moddown_fused(c, out, buf, (long)RB * T * c->N, l, L + 1, false, &fused, addend, addend_poly_stride))) return rc;  // :229 and :231 in two launches
+    if (fused) { *added = addend != nullptr; return CKKS_OK; }
     if ((rc = ckks_moddown_pql_to_ql(c, out, buf, l, 2))) return rc;                                // :229
     return launch_ntt(c, out, 0, K, 2, l + 1, L + 1, 0, 1, false);                                  // :231
 }

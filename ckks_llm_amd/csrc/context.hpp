@@ -162,9 +162,13 @@ int launch_hybrid_front_fused(ckks_ctx* c, const uint64_t* in_ntt, uint64_t* wor
 // it does not apply.
 int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* inv, bool* done);
 // End of a key switch (ModDown of two extended polynomials, forward transform of the results) with the ModDown inside the first
-// pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).
+// pass of the transform; *done = false where it does not apply (the caller then runs the separate steps).  With addend set, limb
+// i of result z leaves as its sum with addend[(z * addend_poly_stride + i) * N ...] (NTT domain, canonical).
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
-                            bool* done);
+                            bool* done, const uint64_t* addend = nullptr, long addend_poly_stride = 0);
+// ckks_keyswitch_23 with the option of adding addend (as above) to the result inside the last launch; *added tells whether it was.
+int keyswitch_23_add(ckks_ctx* c, uint64_t* out, uint64_t* d2, const uint64_t* swk, int l, uint64_t* up, uint64_t* ext, uint64_t* buf,
+                     const uint64_t* addend, long addend_poly_stride, bool* added);
 // Key switch through the T basis: external product of the digits `up` (NTT domain over T) with the key `swk` and inverse transform
 // of the sums into `ext` (coefficient domain on return), the product and the first pass of the transform in one launch;
 // *done = false where it does not apply (nothing launched: the caller runs the separate steps).

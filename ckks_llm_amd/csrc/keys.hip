@@ -205,7 +205,11 @@ extern "C" int ckks_mult_23(ckks_ctx* c, uint64_t* out, const uint64_t* c1, cons
     hipLaunchKernelGGL(tensor_kernel, dim3(N / THREADS, l + 1), dim3(THREADS), 0, c->stream, axbx, axax, bxbx, (const u64*)c1, (const u64*)c2,
                        (const u64*)c1 + N * L1, (const u64*)c2 + N * L1, c->d_primes, N, K);
     CKKS_HIP_TRY(hipGetLastError());
-    if ((rc = ckks_keyswitch_23(c, out, axax, rlk, l, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer))) return rc;
+    // out = KeySwitch(axax) + (axbx, bxbx) (:233-234): the additions ride on the last launch of the key switch where that is one of
+    // the fused forms (axbx and bxbx lie 2 (L+1) limbs apart in the work area)
+    bool added = false;
+    if ((rc = keyswitch_23_add(c, out, axax, rlk, l, modUp_QjtoT_temp, exProduct_T_temp, modUp_TtoQj_buffer, (const uint64_t*)axbx, 2l * L1, &added))) return rc;
+    if (added) return CKKS_OK;
     hipLaunchKernelGGL(add_pair_kernel, dim3(N / THREADS, l + 1), dim3(THREADS), 0, c->stream, (u64*)out, (u64*)out + N * L1, (const u64*)axbx,
                        (const u64*)bxbx, c->d_primes, N, K);
     CKKS_HIP_TRY(hipGetLastError());

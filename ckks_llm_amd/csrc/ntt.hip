@@ -193,7 +193,8 @@ __global__ __launch_bounds__((StridedCfg<SA, SB>::THREADS)) void ntt_strided_pas
 
 template <class AR, int SA, int SB, bool INVERSE, bool COHERENT, bool COMPACT = false, bool PAIRED = false>
 __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typename AR::TW* __restrict__ tw, const AR& ar,
-                                         typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const TileClaim& claim = TileClaim()) {
+                                         typename AR::V* lds, unsigned tid, char* mid_limb = nullptr, const TileClaim& claim = TileClaim(),
+                                         const u64* addend = nullptr, u64 addend_q = 0) {
     typedef RowCfg<SA, SB> C;
     constexpr int S1 = C::S1, R = C::R, N2 = C::N2, U = C::U, N1 = C::N1, ROWS = C::ROWS;
     typedef typename AR::V V;
@@ -230,7 +231,12 @@ __device__ __forceinline__ void row_tile(u64* limb, unsigned tile, const typenam
         for (int j = 0; j < R; j++) lrow[padded(u * R + j)] = v[j];
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < R; j++) store_word<COHERENT>(rp + u + j * U, ar.to_canonical_fwd(lrow[padded(u + j * U)]));
+        for (int j = 0; j < R; j++) {
+            u64 w = ar.to_canonical_fwd(lrow[padded(u + j * U)]);
+            // a forward transform whose result is added to a limb in the NTT domain (null for every plain transform: folded away)
+            if (addend) w = csub(w + addend[(long)row * N2 + u + j * U], addend_q);
+            store_word<COHERENT>(rp + u + j * U, w);
+        }
         claim.publish(tid, counted);
     } else {
         u64 raw[R];
@@ -274,6 +280,22 @@ __global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass(NttArg
     const AR ar(a.primes[prime]);
     row_tile<AR, SA, SB, INVERSE, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
                                                   COMPACT ? a.mid + l * MID_LIMB_BYTES : nullptr);
+}
+
+// The row pass of a forward transform that adds its result to a second operand in the NTT domain: limb (polynomial y, modulus j)
+// of the launch receives addend[(y * addend_poly_stride + j) * N ...] (the closing additions of a multiplication,
+// KeySwitch_23.cuh:233-234, without a launch, a read and a write of their own).
+template <class AR, int SA, int SB, bool COMPACT>
+__global__ __launch_bounds__((RowCfg<SA, SB>::THREADS)) void ntt_row_pass_add(NttArgs a, const u64* addend, long addend_poly_stride) {
+    constexpr long N = 1l << (SA + SB);
+    __shared__ typename AR::V lds[RowCfg<SA, SB>::LDS_WORDS];
+    int prime;
+    const unsigned l = blockIdx.y;
+    u64* limb = limb_ptr(a, l, N, prime);
+    const AR ar(a.primes[prime]);
+    const u64* add = addend + ((long)limb_poly(a, l) * addend_poly_stride + (prime - a.start_mod_idx)) * N;
+    row_tile<AR, SA, SB, false, false, COMPACT>(limb, blockIdx.x, (const typename AR::TW*)a.tw + (long)prime * N, ar, lds, threadIdx.x,
+                                                COMPACT ? a.mid + l * MID_LIMB_BYTES : nullptr, TileClaim(), add, a.primes[prime].q);
 }
 
 // order of work of the chained transform (mode 2, ntt_extra_forms.hpp); pure arithmetic, also exported for its host-side test
@@ -787,32 +809,57 @@ __global__ __launch_bounds__(256, 4) void ext_row_fused_kernel(ExtRowArgs a) {
     u64* lrow = lds + rl * C::PITCH;
     const unsigned tw_off = N1 + row;
     const long at = (long)row * N2 + u;
-    const u64* cp = a.c + (long)t * N + at;
-    const u64* kp = a.key + ((long)z * a.key_z_stride + o) * N + at;
-    // The sums of a lane's sixteen words, four at a time: the 128-bit sums of all sixteen would take half of the registers that
-    // let four workgroups share a compute unit.  The reduced sums go where the row pass exchanges its data.
-    constexpr int CH = 4;
-    const long c_step = (long)a.t_num * N, k_step = a.key_digit_stride * N;
+    // The product phase.  Its sums go through LDS before the row pass, so its lanes need not own the words that the pass gives
+    // them: lane tid takes words 2 (tid % 128) and the next of rows tid / 128 + 2 r, r = 0 .. 7, with 16-byte loads - a wave reads
+    // 1 KiB of a key row in one instruction, where eight-byte loads on the pass's own assignment read four 128-byte pieces.
+    // Four words (two loads) at a time: the 128-bit sums of all sixteen would take half of the registers that let four workgroups
+    // share a compute unit.  Two digits' words are in flight: (x, k) holds the even digits, (xn, kn) the odd ones, each
+    // refilled right after its use.
+    {
+        const unsigned pu = (tid & 127u) * 2u, pr0 = tid >> 7;
+        const long pat = (long)(tile * ROWS + pr0) * N2 + pu;
+        const ulonglong2* cp2 = reinterpret_cast<const ulonglong2*>(a.c + (long)t * N + pat);
+        const ulonglong2* kp2 = reinterpret_cast<const ulonglong2*>(a.key + ((long)z * a.key_z_stride + o) * N + pat);
+        const long c_step = (long)a.t_num * (N / 2), k_step = a.key_digit_stride * (N / 2);       // in 16-byte words
+        constexpr int H = 2;                                    // loads per chunk; a load's two rows apart = N2 16-byte words
 #pragma unroll 1
-    for (int j0 = 0; j0 < R; j0 += CH) {
-        u128w acc[CH];
-        u64 x[CH], k[CH], xn[CH], kn[CH];
+        for (int j0 = 0; j0 < ROWS / 2; j0 += H) {
+            u128w acc[2 * H];
+            ulonglong2 x[H], k[H], xn[H], kn[H];
 #pragma unroll
-        for (int j = 0; j < CH; j++) { acc[j] = u128w{0, 0}; x[j] = cp[(j0 + j) * U]; k[j] = kp[(j0 + j) * U]; }
-        for (int d = 0; d < a.ndigits; d++) {
-            if (d + 1 < a.ndigits) {                        // the next digit's words are on their way while this one's are multiplied
+            for (int j = 0; j < H; j++) {
+                acc[2 * j] = u128w{0, 0};
+                acc[2 * j + 1] = u128w{0, 0};
+                x[j] = cp2[(j0 + j) * N2];
+                k[j] = kp2[(j0 + j) * N2];
+            }
+            if (a.ndigits > 1) {
 #pragma unroll
-                for (int j = 0; j < CH; j++) { xn[j] = cp[(d + 1) * c_step + (j0 + j) * U]; kn[j] = kp[(d + 1) * k_step + (j0 + j) * U]; }
+                for (int j = 0; j < H; j++) { xn[j] = cp2[c_step + (j0 + j) * N2]; kn[j] = kp2[k_step + (j0 + j) * N2]; }
+            }
+            for (int d = 0; d < a.ndigits; d += 2) {
+#pragma unroll
+                for (int j = 0; j < H; j++) { mac128(acc[2 * j], x[j].x, k[j].x); mac128(acc[2 * j + 1], x[j].y, k[j].y); }
+                if (d + 2 < a.ndigits) {
+#pragma unroll
+                    for (int j = 0; j < H; j++) { x[j] = cp2[(d + 2) * c_step + (j0 + j) * N2]; k[j] = kp2[(d + 2) * k_step + (j0 + j) * N2]; }
+                }
+                if (d + 1 < a.ndigits) {
+#pragma unroll
+                    for (int j = 0; j < H; j++) { mac128(acc[2 * j], xn[j].x, kn[j].x); mac128(acc[2 * j + 1], xn[j].y, kn[j].y); }
+                    if (d + 3 < a.ndigits) {
+#pragma unroll
+                        for (int j = 0; j < H; j++) { xn[j] = cp2[(d + 3) * c_step + (j0 + j) * N2]; kn[j] = kp2[(d + 3) * k_step + (j0 + j) * N2]; }
+                    }
+                }
             }
 #pragma unroll
-            for (int j = 0; j < CH; j++) mac128(acc[j], x[j], k[j]);
-            if (d + 1 < a.ndigits) {
-#pragma unroll
-                for (int j = 0; j < CH; j++) { x[j] = xn[j]; k[j] = kn[j]; }
+            for (int j = 0; j < H; j++) {
+                u64* srow = lds + (pr0 + 2 * (j0 + j)) * C::PITCH;
+                srow[padded(pu)] = barrett128(acc[2 * j], pr.q, pr.mu_hi, pr.mu_lo);
+                srow[padded(pu + 1)] = barrett128(acc[2 * j + 1], pr.q, pr.mu_hi, pr.mu_lo);
             }
         }
-#pragma unroll
-        for (int j = 0; j < CH; j++) lrow[padded(u + (j0 + j) * U)] = barrett128(acc[j], pr.q, pr.mu_hi, pr.mu_lo);
     }
     // the row pass of the inverse transform (row_tile, inverse branch) on the sums
     __syncthreads();
@@ -1513,7 +1560,7 @@ int launch_rescale_fused(ckks_ctx* c, uint64_t* cipher, int l, const uint64_t* i
 // in: two extended polynomials [P | Q_l] in the coefficient domain, in_z_stride words apart; out: two polynomials of
 // out_poly_mod_len limbs, written in the NTT domain on limbs 0 .. l.  *done = false (nothing launched) where it does not apply.
 int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long in_z_stride, int l, int out_poly_mod_len, bool pre_scaled,
-                            bool* done) {
+                            bool* done, const uint64_t* addend, long addend_poly_stride) {
     *done = false;
     const int form = c->p_num <= 0 || l < 0 || l > c->L ? 0 : stage_fusion_form(c, 0, c->K + l + 1);
     if (form == 0 || (form == 2 && c->K > 8)) return CKKS_OK;
@@ -1533,13 +1580,15 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
         m.mid = (char*)c->d_ntt_mid; m.mid_stride_i = 2 * MidPieces::LIMB_BYTES; m.mid_stride_z = MidPieces::LIMB_BYTES;
         args.mid = (char*)c->d_ntt_mid;
         hipLaunchKernelGGL((ks_moddown_strided_kernel<F64Arith, MidPieces>), gs, dim3(256), 0, c->stream, m);
-        hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+        if (addend) hipLaunchKernelGGL((ntt_row_pass_add<F64Arith, 8, 8, true>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args, (const u64*)addend, addend_poly_stride);
+        else hipLaunchKernelGGL((ntt_row_pass<F64Arith, 8, 8, false, true>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
     } else {
         // wide primes: the first pass writes the output limbs themselves, as an in-place transform leaves them between its passes
         m.mid = (char*)out; m.mid_stride_i = N * (long)sizeof(u64); m.mid_stride_z = (long)out_poly_mod_len * N * (long)sizeof(u64);
         args.mid = nullptr;
         hipLaunchKernelGGL((ks_moddown_strided_kernel<F64WideArith, MidLimb>), gs, dim3(256), 0, c->stream, m);
-        hipLaunchKernelGGL((ntt_row_pass<F64WideArith, 8, 8, false, false>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
+        if (addend) hipLaunchKernelGGL((ntt_row_pass_add<F64WideArith, 8, 8, false>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args, (const u64*)addend, addend_poly_stride);
+        else hipLaunchKernelGGL((ntt_row_pass<F64WideArith, 8, 8, false, false>), gr, dim3(RowCfg<8, 8>::THREADS), 0, c->stream, args);
     }
     CKKS_HIP_TRY(hipGetLastError());
     *done = true;
@@ -1551,6 +1600,7 @@ int launch_ks_moddown_fused(ckks_ctx* c, uint64_t* out, const uint64_t* in, long
 int launch_ext_product_inverse_fused(ckks_ctx* c, uint64_t* ext, const uint64_t* up, const uint64_t* swk, int l, bool* done) {
     *done = false;
     if (c->ks_split || c->logN != 16 || c->ntt_mode != 0 || c->ev_mid_armed || c->t_num <= 0 || c->gamma <= 0 || c->p_num <= 0) return CKKS_OK;
+    if ((((uintptr_t)up | (uintptr_t)swk) & 15u) != 0) return CKKS_OK;                      // the product phase reads 16 bytes at a time
     const int T = c->t_num, prime0 = c->p_num + c->q_num;
     // the integer back end is what the transforms over T would run on: every T prime too wide for the FP64 forms, or the context set to integers
     for (int j = 0; j < T; j++)

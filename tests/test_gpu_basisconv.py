@@ -122,7 +122,7 @@ def test_keyswitch_23_full_ring(primes):
     the reference's own 49- and 50-bit P and Q primes: at this size its external product runs in one launch with the row pass of
     the sums' inverse transform, and its ModDown inside the first pass of the final transform (handing over 5-byte values below
     2^39, whole limbs on the wide FP64 arithmetic above); same words as the oracle's separate steps, and as the device's own
-    separate steps (ntt mode 1).  Three T primes here: the launch's numbering of its workgroups is exercised away from the
+    separate steps (ntt mode 1); the same for a whole multiplication, whose additions then leave with the last launch.  Three T primes here: the launch's numbering of its workgroups is exercised away from the
     eight primes it is laid out for."""
     q, p, t = CFG2_Q[:6], CFG3_P[:2], REF_PARAMS[16]["t"][:3]      # q_num a multiple of p_num, as in every set of the reference
     if primes == "49":
@@ -144,6 +144,17 @@ def test_keyswitch_23_full_ring(primes):
             s1.zero(); s2.zero(); s3.zero()
             d.keyswitch_23(do, dd2, dswk, l, s1, s2, s3)
             assert np.array_equal(from_dev(do, wout.shape)[:, :l + 1], wout[:, :l + 1]), (l, mode)
+        # the whole multiplication (KeySwitch_23.cuh:192-236): at this size its two closing additions ride on the last launch of
+        # the key switch (mode 0) or run as a launch of their own (mode 1)
+        c1, c2 = limbs_uniform(40 + l, q, 2, N), limbs_uniform(50 + l, q, 2, N)
+        wm = np.zeros((2, Q, N), dtype=np.uint64)
+        o.mult_23(wm.reshape(-1), c1.reshape(-1), c2.reshape(-1), swk.reshape(-1), l)
+        dc1, dc2 = to_dev(c1), to_dev(c2)
+        for mode in (0, 1):
+            d.set_ntt_mode(mode)
+            dm, work = to_dev(np.zeros_like(wm)), DeviceBuffer(8 * N * Q * 3)
+            assert d.L_.ckks_mult_23(d.h, dm.ptr, dc1.ptr, dc2.ptr, dswk.ptr, l, work.ptr, s1.ptr, s2.ptr, s3.ptr) == 0
+            assert np.array_equal(from_dev(dm, wm.shape)[:, :l + 1], wm[:, :l + 1]), ("mult_23", l, mode)
     # a context whose q_num is no multiple of p_num has keys of q_num / p_num digits (Context_23.cuh:29): levels that need more are refused
     odd = Pair(10, p, CFG2_Q[:5], t, 3)
     with pytest.raises(Exception):
