@@ -132,7 +132,7 @@ def test_keyswitch_23_full_ring(primes):
     Q, T, RB, QB, dnum, L = o.q_num, o.t_num, o.Ri_blockNum, o.Qj_blockNum, o.dnum, o.L
     swk = limbs_uniform(7, t, 2 * dnum * RB, N)
     dswk = to_dev(swk)
-    for l in (L, 2):
+    for l in (L, 2, 1):                                            # three digits, two, one (the product's two-deep read-ahead at its ends)
         d2 = np.zeros((Q, N), dtype=np.uint64)
         d2[:l + 1] = limbs_uniform(20 + l, q[:l + 1], 1, N)[0]
         wout = np.zeros((2, Q, N), dtype=np.uint64)
