@@ -56,7 +56,7 @@ constexpr int RES_PITCH = RowCfg<8, 8>::PITCH;                       // 272: pad
 constexpr int RES_P_BYTES = 65536;                                   // staging of the tiles that arrive: 8 KiB per wave
 constexpr int RES_R_BYTES = 2 * 16 * RES_PITCH * 8;                  // exchange area of a step: one tile per group (69632 bytes)
 constexpr int RES_S_BYTES = 9 * RES_LANES * 4;                       // hand-over between the groups: 9 words per lane
-constexpr int RES_T_BYTES = 8 * 1024;                                // inverse transforms: row twiddles of a step, 512 bytes per wave (written twice over by the wave's 64 lanes)
+constexpr int RES_T_BYTES = 8 * 1024;                                // row twiddles of a step: the first 512 bytes of 1 KiB per wave
 
 // limb of workgroup b in round `it`: consecutive workgroups of a grid go to the eight XCDs in turn, and the workgroups of one
 // XCD take consecutive limbs - limbs are ordered prime-major, so one XCD's compute units read one prime's twiddles from its L2.
@@ -282,8 +282,9 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             // transform's tile, 128 bytes per row, the same costs 37 us per launch
             dma16<INVERSE>(src, p_wave + m * 1024);
         } else {
-            // every lane takes part (the upper half of the wave repeats the lower half's chunks into the second half of the wave's
-            // 1 KiB): no branch; the staging is single: the step's own reads of it are over (they come before this in the last round)
+            // the lower half of the wave fetches the 512 bytes (the upper half would only repeat them into the second half of the
+            // wave's 1 KiB, which nobody reads: 433 -> 428 us per inverse launch without); the staging is single: the step's own
+            // reads of it are over (they come before this in the last round)
             const unsigned i = (lane >> 3) & 3, c = lane & 7;
             const unsigned trow_id = 16 * (4 * wq + i) + tile;
             const unsigned off = 256 + (INVERSE ? 255 - trow_id : trow_id);          // inverse: the mirrored row of the forward table
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(RES_LANES) void ntt_resident_kernel(NttArgs a, unsi
             const unsigned sh = (0x01223333u >> (4 * c)) & 15u, add = (0x00206420u >> (4 * c)) & 15u;
             const TW* src = tw + (((off << sh) + add) & ~1u);
             asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-            dma16(src, (unsigned)(size_t)(lptr_t)lds_t + wave * 1024);
+            if (lane < 32) dma16(src, (unsigned)(size_t)(lptr_t)lds_t + wave * 1024);
         }
     };
     auto request = [&](const u64* limb, const TW* tw, int s) __attribute__((always_inline)) {
